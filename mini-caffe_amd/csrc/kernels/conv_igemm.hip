@@ -1,0 +1,585 @@
+// Implicit-GEMM Convolution / Deconvolution for gfx950 (fp32 MFMA).
+//
+// The contraction the reference performs per image as im2col + sgemm
+// (reference src/layers/base_conv_layer.cpp:254-271, src/util/im2col.cpp:19-55)
+// and, for Deconvolution, as sgemm(A^T) + col2im (base_conv_layer.cpp:280-296,
+// im2col.cpp:153-187) is done here for the whole batch in one launch with no
+// column buffer:
+//
+//   Y[g][m][p] = sum_k Wt[g][k][m] * X(p, k)      m = output channel in group
+//                                                 p = (image, qh, qw) "pixel"
+//                                                 k = (input channel, tap)
+//
+// X(p, k) is gathered straight from the NCHW bottom blob through a per-k tap
+// table {element offset, dh, dw}; zero padding is a bounds test.  A
+// Deconvolution with stride s is split into s_h*s_w output-parity classes, each
+// of which is a stride-1 gather with its own tap table, so no scatter-add and
+// no wasted multiply by inserted zeros.
+//
+// Tiling: 256 threads = 4 wavefronts per workgroup, BM x BN output tile,
+// K step 16, LDS double buffer filled from registers (global loads for tile
+// t+1 are in flight while tile t is multiplied).  Each wavefront owns a grid of
+// 32x32 accumulators fed by v_mfma_f32_32x32x2_f32.  Filters are repacked once
+// into K-major, zero-padded [g][Kpad][Mpad] so that A-tile loads are aligned
+// float4 rows and need no predicates.
+#include "mc_common.h"
+#include "mchip/kernels.h"
+
+#include <algorithm>
+#include <cstring>
+#include <vector>
+
+namespace mchip {
+namespace {
+
+constexpr int BK = 16;
+
+typedef float acc16 __attribute__((ext_vector_type(16)));
+
+struct IgemmArgs {
+  const float* __restrict__ x;
+  const float* __restrict__ wt;
+  float* __restrict__ y;
+  const int4* __restrict__ ktab;  // [Kpad] {element offset, dh, dw, unused}
+  const float* __restrict__ scale;
+  const float* __restrict__ shift;
+  const float* __restrict__ residual;
+  int P;              // pixels = num * Hq * Wq
+  int Hq, Wq, HqWq;   // iteration grid of this sub-problem
+  int H, W;           // bottom height / width
+  int q_sh, q_sw;     // bottom origin of pixel (qh,qw): qh*q_sh + in_oh
+  int in_oh, in_ow;
+  int x_nstride;      // Cin*H*W
+  int x_gstride;      // (Cin/g)*H*W
+  int M;              // output channels per group
+  int Mpad, Kpad;
+  int wt_gstride;     // Kpad*Mpad
+  int Wo;             // top width
+  int y_cstride;      // Ho*Wo
+  int y_nstride;      // Cout*Ho*Wo
+  int out_sh, out_sw, out_oh, out_ow;  // top row = qh*out_sh + out_oh
+  int MT, NT;         // tile counts
+  int act;
+  float slope;
+};
+
+__device__ __forceinline__ float apply_act(float v, int act, float slope) {
+  switch (act) {
+    case MC_ACT_RELU:
+      return v > 0.f ? v : v * slope;
+    case MC_ACT_TANH:
+      return static_cast<float>(tanh(static_cast<double>(v)));
+    case MC_ACT_SIGMOID:
+      return static_cast<float>(1. / (1. + exp(-static_cast<double>(v))));
+    default:
+      return v;
+  }
+}
+
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(256) void igemm_kernel(const IgemmArgs a) {
+  static_assert(WM * WN == 4, "four wavefronts per workgroup");
+  static_assert(BN >= 64 && 256 % BN == 0, "BN must be 64, 128 or 256");
+  constexpr int TM = BM / WM / 32;
+  constexpr int TN = BN / WN / 32;
+  static_assert(TM >= 1 && TN >= 1, "wave tile must hold a 32x32 block");
+  constexpr int ROWS_PER_PASS = 256 / BN;
+  constexpr int B_PER_THREAD = BK / ROWS_PER_PASS;
+  constexpr int A_F4 = BM * BK / 4;               // float4 per A tile
+  constexpr int A_VEC = (A_F4 + 255) / 256;
+
+  __shared__ __attribute__((aligned(16))) float As[2][BK][BM];
+  __shared__ __attribute__((aligned(16))) float Bs[2][BK][BN];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int g = blockIdx.y;
+
+  // XCD-aware tile order: workgroup ids are dealt round-robin to the 8 XCDs, so
+  // give each XCD a contiguous run of logical tiles (m fastest): the tiles that
+  // share one pixel tile, and neighbouring pixel tiles, then hit the same L2.
+  int mt, nt;
+  {
+    const int total = a.MT * a.NT;
+    const int bid = blockIdx.x;
+    const int q = total / kNumXcd, r = total % kNumXcd;
+    const int xcd = bid % kNumXcd, local = bid / kNumXcd;
+    const int logical = xcd * q + (xcd < r ? xcd : r) + local;
+    mt = logical % a.MT;
+    nt = logical / a.MT;
+  }
+
+  // The pixel this thread gathers for the B tile (fixed over the K loop).
+  const int pj = tid % BN;
+  const int prow = tid / BN;  // wave-uniform because BN >= 64
+  int hi0, wi0, xbase;
+  {
+    const int p = nt * BN + pj;
+    if (p < a.P) {
+      const int n = p / a.HqWq;
+      const int rem = p - n * a.HqWq;
+      const int qh = rem / a.Wq;
+      const int qw = rem - qh * a.Wq;
+      hi0 = qh * a.q_sh + a.in_oh;
+      wi0 = qw * a.q_sw + a.in_ow;
+      xbase = n * a.x_nstride + g * a.x_gstride + hi0 * a.W + wi0;
+    } else {
+      hi0 = -(1 << 24);  // fails every bounds test -> contributes zeros
+      wi0 = 0;
+      xbase = 0;
+    }
+  }
+  const float* __restrict__ wt_tile = a.wt + (size_t)g * a.wt_gstride + mt * BM;
+
+  float4 areg[A_VEC];
+  float breg[B_PER_THREAD];
+
+  auto load_tiles = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < A_VEC; ++i) {
+      const int f = tid + 256 * i;
+      if (A_F4 % 256 == 0 || f < A_F4) {
+        const int row = f / (BM / 4);
+        const int c4 = f % (BM / 4);
+        areg[i] = *reinterpret_cast<const float4*>(
+            wt_tile + (size_t)(kt * BK + row) * a.Mpad + c4 * 4);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < B_PER_THREAD; ++i) {
+      const int krow = __builtin_amdgcn_readfirstlane(kt * BK + i * ROWS_PER_PASS + prow);
+      const int4 t = a.ktab[krow];
+      const int hi = hi0 + t.y;
+      const int wi = wi0 + t.z;
+      const bool ok = static_cast<unsigned>(hi) < static_cast<unsigned>(a.H) &&
+                      static_cast<unsigned>(wi) < static_cast<unsigned>(a.W);
+      breg[i] = ok ? a.x[xbase + t.x] : 0.f;
+    }
+  };
+  auto store_tiles = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < A_VEC; ++i) {
+      const int f = tid + 256 * i;
+      if (A_F4 % 256 == 0 || f < A_F4) {
+        const int row = f / (BM / 4);
+        const int c4 = f % (BM / 4);
+        *reinterpret_cast<float4*>(&As[buf][row][c4 * 4]) = areg[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < B_PER_THREAD; ++i) {
+      Bs[buf][i * ROWS_PER_PASS + prow][pj] = breg[i];
+    }
+  };
+
+  acc16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int wm0 = (wave % WM) * (BM / WM);
+  const int wn0 = (wave / WM) * (BN / WN);
+  const int l32 = lane & 31;
+  const int lhi = lane >> 5;
+
+  const int KT = a.Kpad / BK;
+  if (KT > 0) {
+    load_tiles(0);
+    store_tiles(0);
+  }
+  __syncthreads();
+  for (int kt = 0; kt < KT; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < KT) load_tiles(kt + 1);
+#pragma unroll
+    for (int kk = 0; kk < BK / 2; ++kk) {
+      float av[TM], bv[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) av[i] = As[buf][kk * 2 + lhi][wm0 + i * 32 + l32];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) bv[j] = Bs[buf][kk * 2 + lhi][wn0 + j * 32 + l32];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < KT) store_tiles(buf ^ 1);
+    __syncthreads();
+  }
+
+  // Epilogue.  Accumulator register r of lane l holds row 8*(r/4)+4*(l/32)+r%4,
+  // column l%32 of its 32x32 block; a half-wave therefore stores 32 consecutive
+  // pixels of one output channel.
+  const bool has_scale = a.scale != nullptr;
+  const bool has_shift = a.shift != nullptr;
+  const bool has_res = a.residual != nullptr;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int p = nt * BN + wn0 + j * 32 + l32;
+    if (p >= a.P) continue;
+    const int n = p / a.HqWq;
+    const int rem = p - n * a.HqWq;
+    const int qh = rem / a.Wq;
+    const int qw = rem - qh * a.Wq;
+    const int ybase = n * a.y_nstride + (qh * a.out_sh + a.out_oh) * a.Wo +
+                      qw * a.out_sw + a.out_ow;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = mt * BM + wm0 + i * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+        if (m < a.M) {
+          const int c = g * a.M + m;
+          float v = acc[i][j][r];
+          if (has_scale) v *= a.scale[c];
+          if (has_shift) v += a.shift[c];
+          const int yo = ybase + c * a.y_cstride;
+          if (has_res) v += a.residual[yo];
+          a.y[yo] = apply_act(v, a.act, a.slope);
+        }
+      }
+    }
+  }
+}
+
+// wt[g][k][m] = w[g*wg_stride + wk_off[k] + m*wm_stride] for k<K, m<M, else 0.
+__global__ void pack_weights_kernel(const float* __restrict__ w, float* __restrict__ wt,
+                                    const int* __restrict__ wk_off, int G, int K, int Kpad,
+                                    int M, int Mpad, int wm_stride, int wg_stride) {
+  const long total = (long)G * Kpad * Mpad;
+  for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total;
+       i += (long)gridDim.x * blockDim.x) {
+    const int m = static_cast<int>(i % Mpad);
+    const long t = i / Mpad;
+    const int k = static_cast<int>(t % Kpad);
+    const int g = static_cast<int>(t / Kpad);
+    float v = 0.f;
+    if (k < K && m < M) v = w[(long)g * wg_stride + wk_off[k] + (long)m * wm_stride];
+    wt[i] = v;
+  }
+}
+
+struct TileConfig {
+  int bm, bn;
+  const char* name;
+  void (*kernel)(const IgemmArgs);
+};
+
+const TileConfig kConfigs[] = {
+    {128, 128, "igemm_f32_128x128", igemm_kernel<128, 128, 2, 2>},
+    {128, 64, "igemm_f32_128x64", igemm_kernel<128, 64, 2, 2>},
+    {64, 128, "igemm_f32_64x128", igemm_kernel<64, 128, 2, 2>},
+    {64, 64, "igemm_f32_64x64", igemm_kernel<64, 64, 2, 2>},
+    {32, 128, "igemm_f32_32x128", igemm_kernel<32, 128, 1, 4>},
+    {32, 256, "igemm_f32_32x256", igemm_kernel<32, 256, 1, 4>},
+    {64, 256, "igemm_f32_64x256", igemm_kernel<64, 256, 1, 4>},
+};
+constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
+
+// One stride-1 gather problem: the whole Convolution, or one output-parity
+// class of a Deconvolution.
+struct SubProblem {
+  int K = 0, Kpad = 0;
+  int Hq = 0, Wq = 0;
+  int q_sh = 1, q_sw = 1, in_oh = 0, in_ow = 0;
+  int out_sh = 1, out_sw = 1, out_oh = 0, out_ow = 0;
+  std::vector<int4> ktab;    // host copy
+  std::vector<int> wk_off;   // host copy
+  int4* ktab_dev = nullptr;
+  int* wk_off_dev = nullptr;
+  float* wt_dev = nullptr;
+};
+
+}  // namespace
+}  // namespace mchip
+
+using namespace mchip;
+
+struct mcConvPlan {
+  mcConvGeom geom;
+  int Ho = 0, Wo = 0;
+  int M = 0;        // output channels per group
+  int Cin_g = 0;
+  int Mpad = 0;
+  int wm_stride = 0, wg_stride = 0;
+  int forced_config = -1;
+  std::vector<SubProblem> subs;
+};
+
+namespace {
+
+int pick_config(const mcConvPlan* plan, long pixels) {
+  if (plan->forced_config >= 0) return plan->forced_config;
+  const int M = plan->M;
+  int bm = M > 64 ? 128 : (M > 32 ? 64 : 32);
+  int bn = 128;
+  auto blocks = [&](int bm_, int bn_) {
+    return (long)ceil_div(M, bm_) * ceil_div(pixels, bn_) * plan->geom.group;
+  };
+  if (bm == 128 && blocks(128, 128) < 2 * kNumCu) {
+    bm = (M % 128 != 0 && M % 128 <= 64) || blocks(128, 64) < 2 * kNumCu ? 64 : 128;
+    bn = 64;
+  } else if (bm == 64 && blocks(64, 128) < 2 * kNumCu) {
+    bn = 64;
+  } else if (bm == 32) {
+    bn = blocks(32, 256) >= 4 * kNumCu ? 256 : 128;
+  }
+  for (int i = 0; i < kNumConfigs; ++i)
+    if (kConfigs[i].bm == bm && kConfigs[i].bn == bn) return i;
+  return 0;
+}
+
+int free_sub(SubProblem& s) {
+  if (s.ktab_dev) (void)hipFree(s.ktab_dev);
+  if (s.wk_off_dev) (void)hipFree(s.wk_off_dev);
+  if (s.wt_dev) (void)hipFree(s.wt_dev);
+  s.ktab_dev = nullptr;
+  s.wk_off_dev = nullptr;
+  s.wt_dev = nullptr;
+  return 0;
+}
+
+// floor division for possibly negative numerators
+inline int floordiv(int a, int b) { return (a >= 0) ? a / b : -((-a + b - 1) / b); }
+
+}  // namespace
+
+extern "C" {
+
+int mcConvPlanCreate(const mcConvGeom* gp, mcConvPlan** out) {
+  MC_REQUIRE(gp && out, "mcConvPlanCreate: null argument");
+  const mcConvGeom& g = *gp;
+  MC_REQUIRE(g.channels_in > 0 && g.channels_out > 0 && g.height_in > 0 && g.width_in > 0,
+             "mcConvPlanCreate: non-positive blob dimension");
+  MC_REQUIRE(g.kernel_h > 0 && g.kernel_w > 0, "Filter dimensions must be nonzero.");
+  MC_REQUIRE(g.stride_h > 0 && g.stride_w > 0, "Stride dimensions must be nonzero.");
+  MC_REQUIRE(g.dilation_h > 0 && g.dilation_w > 0, "Dilation dimensions must be nonzero.");
+  MC_REQUIRE(g.pad_h >= 0 && g.pad_w >= 0, "Padding must be non-negative.");
+  MC_REQUIRE(g.group > 0 && g.channels_in % g.group == 0 && g.channels_out % g.group == 0,
+             "Number of channels and of outputs must be multiples of group.");
+  MC_REQUIRE(g.height_in < 16384 && g.width_in < 16384 && g.kernel_h * g.dilation_h < 16384 &&
+                 g.kernel_w * g.dilation_w < 16384,
+             "mcConvPlanCreate: spatial extent too large for the tap table");
+
+  mcConvPlan* plan = new mcConvPlan();
+  plan->geom = g;
+  const int ext_h = g.dilation_h * (g.kernel_h - 1) + 1;
+  const int ext_w = g.dilation_w * (g.kernel_w - 1) + 1;
+  if (!g.transposed) {
+    plan->Ho = (g.height_in + 2 * g.pad_h - ext_h) / g.stride_h + 1;
+    plan->Wo = (g.width_in + 2 * g.pad_w - ext_w) / g.stride_w + 1;
+  } else {
+    plan->Ho = g.stride_h * (g.height_in - 1) + ext_h - 2 * g.pad_h;
+    plan->Wo = g.stride_w * (g.width_in - 1) + ext_w - 2 * g.pad_w;
+  }
+  if (plan->Ho <= 0 || plan->Wo <= 0) {
+    const int ho = plan->Ho, wo = plan->Wo;
+    delete plan;
+    return fail("mcConvPlanCreate: empty output (%d x %d)", ho, wo);
+  }
+  plan->M = g.channels_out / g.group;
+  plan->Cin_g = g.channels_in / g.group;
+  plan->Mpad = ceil_div(plan->M, 128) * 128;
+  const int HW = g.height_in * g.width_in;
+  const int khkw = g.kernel_h * g.kernel_w;
+
+  if (!g.transposed) {
+    SubProblem s;
+    s.K = plan->Cin_g * khkw;
+    s.Hq = plan->Ho;
+    s.Wq = plan->Wo;
+    s.q_sh = g.stride_h;
+    s.q_sw = g.stride_w;
+    s.in_oh = -g.pad_h;
+    s.in_ow = -g.pad_w;
+    for (int c = 0; c < plan->Cin_g; ++c)
+      for (int i = 0; i < g.kernel_h; ++i)
+        for (int j = 0; j < g.kernel_w; ++j) {
+          const int dh = i * g.dilation_h, dw = j * g.dilation_w;
+          s.ktab.push_back(make_int4(c * HW + dh * g.width_in + dw, dh, dw, 0));
+          s.wk_off.push_back((c * g.kernel_h + i) * g.kernel_w + j);
+        }
+    plan->wm_stride = s.K;
+    plan->wg_stride = plan->M * s.K;
+    plan->subs.push_back(std::move(s));
+  } else {
+    plan->wm_stride = khkw;
+    plan->wg_stride = plan->Cin_g * plan->M * khkw;
+    for (int rh = 0; rh < g.stride_h; ++rh)
+      for (int rw = 0; rw < g.stride_w; ++rw) {
+        if (rh >= plan->Ho || rw >= plan->Wo) continue;
+        SubProblem s;
+        s.Hq = (plan->Ho - rh + g.stride_h - 1) / g.stride_h;
+        s.Wq = (plan->Wo - rw + g.stride_w - 1) / g.stride_w;
+        s.out_sh = g.stride_h;
+        s.out_sw = g.stride_w;
+        s.out_oh = rh;
+        s.out_ow = rw;
+        // top row oh = s*q + rh receives bottom row ih with oh = ih*s - p + kh*d,
+        // i.e. ih = q + (rh + p - kh*d)/s whenever that quotient is exact.
+        std::vector<int> tap_h, off_h, tap_w, off_w;
+        for (int i = 0; i < g.kernel_h; ++i) {
+          const int num = rh + g.pad_h - i * g.dilation_h;
+          if (((num % g.stride_h) + g.stride_h) % g.stride_h == 0) {
+            tap_h.push_back(i);
+            off_h.push_back(floordiv(num, g.stride_h));
+          }
+        }
+        for (int j = 0; j < g.kernel_w; ++j) {
+          const int num = rw + g.pad_w - j * g.dilation_w;
+          if (((num % g.stride_w) + g.stride_w) % g.stride_w == 0) {
+            tap_w.push_back(j);
+            off_w.push_back(floordiv(num, g.stride_w));
+          }
+        }
+        for (int c = 0; c < plan->Cin_g; ++c)
+          for (size_t i = 0; i < tap_h.size(); ++i)
+            for (size_t j = 0; j < tap_w.size(); ++j) {
+              s.ktab.push_back(
+                  make_int4(c * HW + off_h[i] * g.width_in + off_w[j], off_h[i], off_w[j], 0));
+              s.wk_off.push_back(c * plan->M * khkw + tap_h[i] * g.kernel_w + tap_w[j]);
+            }
+        s.K = static_cast<int>(s.ktab.size());
+        plan->subs.push_back(std::move(s));
+      }
+  }
+
+  for (auto& s : plan->subs) {
+    s.Kpad = ceil_div(s.K, BK) * BK;
+    // Padding rows multiply zero weights; give them a tap that fails the
+    // bounds test so nothing is fetched.
+    while (static_cast<int>(s.ktab.size()) < s.Kpad) s.ktab.push_back(make_int4(0, 1 << 20, 0, 0));
+    if (s.Kpad == 0) continue;
+    hipError_t e = hipMalloc(&s.ktab_dev, sizeof(int4) * s.Kpad);
+    if (e == hipSuccess) e = hipMalloc(&s.wk_off_dev, sizeof(int) * s.K);
+    if (e == hipSuccess)
+      e = hipMalloc(&s.wt_dev, sizeof(float) * (size_t)g.group * s.Kpad * plan->Mpad);
+    if (e == hipSuccess)
+      e = hipMemcpy(s.ktab_dev, s.ktab.data(), sizeof(int4) * s.Kpad, hipMemcpyHostToDevice);
+    if (e == hipSuccess)
+      e = hipMemcpy(s.wk_off_dev, s.wk_off.data(), sizeof(int) * s.K, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+      for (auto& t : plan->subs) free_sub(t);
+      delete plan;
+      return fail("mcConvPlanCreate: device set-up failed: %s", hipGetErrorString(e));
+    }
+  }
+  *out = plan;
+  return 0;
+}
+
+int mcConvPlanDestroy(mcConvPlan* plan) {
+  if (!plan) return 0;
+  for (auto& s : plan->subs) free_sub(s);
+  delete plan;
+  return 0;
+}
+
+int mcConvPlanOutputShape(const mcConvPlan* plan, int* ho, int* wo) {
+  MC_REQUIRE(plan, "mcConvPlanOutputShape: null plan");
+  if (ho) *ho = plan->Ho;
+  if (wo) *wo = plan->Wo;
+  return 0;
+}
+
+int mcConvPlanSetWeights(mcConvPlan* plan, const float* weights, void* stream) {
+  MC_REQUIRE(plan && weights, "mcConvPlanSetWeights: null argument");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  for (auto& s : plan->subs) {
+    if (s.Kpad == 0) continue;
+    const long total = (long)plan->geom.group * s.Kpad * plan->Mpad;
+    pack_weights_kernel<<<ew_blocks(total, 256), 256, 0, st>>>(
+        weights, s.wt_dev, s.wk_off_dev, plan->geom.group, s.K, s.Kpad, plan->M, plan->Mpad,
+        plan->wm_stride, plan->wg_stride);
+    MC_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+int mcConvPlanForceConfig(mcConvPlan* plan, int config) {
+  MC_REQUIRE(plan, "mcConvPlanForceConfig: null plan");
+  MC_REQUIRE(config >= -1 && config < kNumConfigs, "mcConvPlanForceConfig: no such configuration");
+  plan->forced_config = config;
+  return 0;
+}
+
+int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* top,
+                  const mcEpilogue* ep, void* stream) {
+  MC_REQUIRE(plan && bottom && top, "mcConvForward: null argument");
+  MC_REQUIRE(num > 0, "mcConvForward: batch must be positive");
+  const mcConvGeom& g = plan->geom;
+  const long in_count = (long)num * g.channels_in * g.height_in * g.width_in;
+  const long out_count = (long)num * g.channels_out * plan->Ho * plan->Wo;
+  MC_REQUIRE(in_count < (1L << 31) && out_count < (1L << 31),
+             "mcConvForward: blob exceeds 2^31 elements");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  for (const auto& s : plan->subs) {
+    const long pixels = (long)num * s.Hq * s.Wq;
+    if (pixels == 0) continue;
+    MC_REQUIRE(pixels < (1L << 31), "mcConvForward: too many output pixels");
+    const TileConfig& cfg = kConfigs[pick_config(plan, pixels)];
+    IgemmArgs a;
+    a.x = bottom;
+    a.wt = s.wt_dev;
+    a.y = top;
+    a.ktab = s.ktab_dev;
+    a.scale = ep ? ep->scale : nullptr;
+    a.shift = ep ? ep->shift : nullptr;
+    a.residual = ep ? ep->residual : nullptr;
+    a.P = static_cast<int>(pixels);
+    a.Hq = s.Hq;
+    a.Wq = s.Wq;
+    a.HqWq = s.Hq * s.Wq;
+    a.H = g.height_in;
+    a.W = g.width_in;
+    a.q_sh = s.q_sh;
+    a.q_sw = s.q_sw;
+    a.in_oh = s.in_oh;
+    a.in_ow = s.in_ow;
+    a.x_nstride = g.channels_in * g.height_in * g.width_in;
+    a.x_gstride = plan->Cin_g * g.height_in * g.width_in;
+    a.M = plan->M;
+    a.Mpad = plan->Mpad;
+    a.Kpad = s.Kpad;
+    a.wt_gstride = s.Kpad * plan->Mpad;
+    a.Wo = plan->Wo;
+    a.y_cstride = plan->Ho * plan->Wo;
+    a.y_nstride = g.channels_out * plan->Ho * plan->Wo;
+    a.out_sh = s.out_sh;
+    a.out_sw = s.out_sw;
+    a.out_oh = s.out_oh;
+    a.out_ow = s.out_ow;
+    a.MT = ceil_div(plan->M, cfg.bm);
+    a.NT = ceil_div(pixels, cfg.bn);
+    a.act = ep ? ep->activation : MC_ACT_NONE;
+    a.slope = ep ? ep->negative_slope : 0.f;
+    const long blocks = (long)a.MT * a.NT;
+    MC_REQUIRE(blocks < (1L << 31), "mcConvForward: grid too large");
+    dim3 grid(static_cast<unsigned>(blocks), g.group, 1);
+    cfg.kernel<<<grid, 256, 0, st>>>(a);
+    MC_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+double mcConvPlanFlops(const mcConvPlan* plan, int num) {
+  if (!plan) return 0.;
+  const mcConvGeom& g = plan->geom;
+  const double taps = (double)g.kernel_h * g.kernel_w;
+  if (!g.transposed)
+    return 2. * num * g.channels_out * plan->Ho * plan->Wo * (g.channels_in / g.group) * taps;
+  return 2. * num * g.channels_in * g.height_in * g.width_in * (g.channels_out / g.group) * taps;
+}
+
+const char* mcConvPlanKernelName(const mcConvPlan* plan, int num) {
+  if (!plan || plan->subs.empty()) return "";
+  const auto& s = plan->subs[0];
+  return kConfigs[pick_config(plan, (long)num * s.Hq * s.Wq)].name;
+}
+
+}  // extern "C"

@@ -1,0 +1,91 @@
+"""ctypes prototypes of the kernel-level C ABI (include/mchip/kernels.h).
+
+Pointers are raw device addresses (ints); torch is only used by callers to own
+device memory and streams.
+"""
+import ctypes
+
+from .base import LIB, check_mc
+
+c_void_p = ctypes.c_void_p
+c_int = ctypes.c_int
+c_float = ctypes.c_float
+
+ACT_NONE, ACT_RELU, ACT_TANH, ACT_SIGMOID = 0, 1, 2, 3
+
+
+class ConvGeom(ctypes.Structure):
+    _fields_ = [(n, c_int) for n in (
+        "channels_in", "height_in", "width_in", "channels_out", "kernel_h", "kernel_w",
+        "stride_h", "stride_w", "pad_h", "pad_w", "dilation_h", "dilation_w", "group",
+        "transposed")]
+
+
+class Epilogue(ctypes.Structure):
+    _fields_ = [("scale", c_void_p), ("shift", c_void_p), ("residual", c_void_p),
+                ("activation", c_int), ("negative_slope", c_float)]
+
+
+LIB.mcConvPlanCreate.argtypes = [ctypes.POINTER(ConvGeom), ctypes.POINTER(c_void_p)]
+LIB.mcConvPlanDestroy.argtypes = [c_void_p]
+LIB.mcConvPlanOutputShape.argtypes = [c_void_p, ctypes.POINTER(c_int), ctypes.POINTER(c_int)]
+LIB.mcConvPlanSetWeights.argtypes = [c_void_p, c_void_p, c_void_p]
+LIB.mcConvForward.argtypes = [c_void_p, c_int, c_void_p, c_void_p, ctypes.POINTER(Epilogue),
+                              c_void_p]
+LIB.mcConvPlanFlops.argtypes = [c_void_p, c_int]
+LIB.mcConvPlanFlops.restype = ctypes.c_double
+LIB.mcConvPlanKernelName.argtypes = [c_void_p, c_int]
+LIB.mcConvPlanKernelName.restype = ctypes.c_char_p
+LIB.mcConvPlanForceConfig.argtypes = [c_void_p, c_int]
+
+
+def conv_geom(cin, h, w, cout, kernel, stride=1, pad=0, dilation=1, group=1, transposed=False):
+    def two(v):
+        return (v, v) if isinstance(v, int) else tuple(v)
+    kh, kw = two(kernel)
+    sh, sw = two(stride)
+    ph, pw = two(pad)
+    dh, dw = two(dilation)
+    return ConvGeom(cin, h, w, cout, kh, kw, sh, sw, ph, pw, dh, dw, group, int(transposed))
+
+
+class ConvPlan(object):
+    """Owns one mcConvPlan."""
+
+    def __init__(self, geom):
+        self.geom = geom
+        self.handle = c_void_p()
+        check_mc(LIB.mcConvPlanCreate(ctypes.byref(geom), ctypes.byref(self.handle)))
+
+    def close(self):
+        if self.handle:
+            LIB.mcConvPlanDestroy(self.handle)
+            self.handle = c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def output_shape(self):
+        ho, wo = c_int(), c_int()
+        check_mc(LIB.mcConvPlanOutputShape(self.handle, ctypes.byref(ho), ctypes.byref(wo)))
+        return ho.value, wo.value
+
+    def set_weights(self, w_ptr, stream=0):
+        check_mc(LIB.mcConvPlanSetWeights(self.handle, w_ptr, stream))
+
+    def force_config(self, idx):
+        check_mc(LIB.mcConvPlanForceConfig(self.handle, idx))
+
+    def forward(self, num, x_ptr, y_ptr, scale=None, shift=None, residual=None,
+                activation=ACT_NONE, negative_slope=0.0, stream=0):
+        ep = Epilogue(scale, shift, residual, activation, negative_slope)
+        check_mc(LIB.mcConvForward(self.handle, num, x_ptr, y_ptr, ctypes.byref(ep), stream))
+
+    def flops(self, num):
+        return LIB.mcConvPlanFlops(self.handle, num)
+
+    def kernel_name(self, num):
+        return LIB.mcConvPlanKernelName(self.handle, num).decode()

@@ -1,0 +1,293 @@
+"""ctypes/numpy front end of the CPU checker (oracle/mc_oracle*.c).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by
+the cpu_baseline leg of bench.py.  The product package never imports it.
+
+Arrays are float32, C-contiguous, in the reference's NCHW blob layout.
+"""
+import ctypes
+import glob
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libmcoracle.so")
+
+c_float_p = ctypes.POINTER(ctypes.c_float)
+c_int_p = ctypes.POINTER(ctypes.c_int)
+
+
+def build(force=False):
+    """Compile the checker (and oracle/_ref when the reference checkout exists)."""
+    if force:
+        subprocess.check_call(["make", "-C", _HERE, "clean"], stdout=subprocess.DEVNULL)
+    subprocess.check_call(["make", "-C", _HERE], stdout=subprocess.DEVNULL)
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        build()
+    return ctypes.CDLL(_LIB_PATH)
+
+
+_lib = _load()
+
+
+def _fp(a):
+    return a.ctypes.data_as(c_float_p)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+class ConvGeom(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int) for n in (
+        "channels_in", "height_in", "width_in", "channels_out", "kernel_h", "kernel_w",
+        "stride_h", "stride_w", "pad_h", "pad_w", "dilation_h", "dilation_w", "group",
+        "transposed")]
+
+
+def conv_geom(cin, h, w, cout, kernel, stride=1, pad=0, dilation=1, group=1, transposed=False):
+    def two(v):
+        return (v, v) if isinstance(v, int) else tuple(v)
+    kh, kw = two(kernel)
+    sh, sw = two(stride)
+    ph, pw = two(pad)
+    dh, dw = two(dilation)
+    return ConvGeom(cin, h, w, cout, kh, kw, sh, sw, ph, pw, dh, dw, group, int(transposed))
+
+
+# ---- BLAS plug -------------------------------------------------------------
+
+_blas_handle = None
+
+
+def find_openblas():
+    """Path of the OpenBLAS bundled with scipy (CBLAS symbols prefixed scipy_), or None."""
+    try:
+        import scipy
+    except ImportError:
+        return None
+    root = os.path.dirname(os.path.dirname(scipy.__file__))
+    hits = sorted(glob.glob(os.path.join(root, "scipy.libs", "libscipy_openblas-*.so")))
+    return hits[0] if hits else None
+
+
+def use_openblas(enable=True, threads=None):
+    """Route orc_gemm through OpenBLAS's cblas_sgemm, as the reference does
+    (src/util/math_functions.cpp:8-16).  Returns the library path or None."""
+    global _blas_handle
+    if not enable:
+        _lib.orc_set_sgemm(None)
+        return None
+    path = find_openblas()
+    if path is None:
+        return None
+    if _blas_handle is None:
+        _blas_handle = ctypes.CDLL(path)
+    if threads is not None:
+        _blas_handle.scipy_openblas_set_num_threads(int(threads))
+    fn = ctypes.cast(_blas_handle.scipy_cblas_sgemm, ctypes.c_void_p)
+    _lib.orc_set_sgemm(fn)
+    return path
+
+
+def openblas_threads():
+    if _blas_handle is None:
+        return 0
+    return int(_blas_handle.scipy_openblas_get_num_threads())
+
+
+# ---- prototypes --------------------------------------------------------------
+
+_lib.orc_set_sgemm.argtypes = [ctypes.c_void_p]
+_lib.orc_gemm.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                          ctypes.c_float, c_float_p, c_float_p, ctypes.c_float, c_float_p]
+_lib.orc_im2col.argtypes = [c_float_p] + [ctypes.c_int] * 11 + [c_float_p]
+_lib.orc_col2im.argtypes = [c_float_p] + [ctypes.c_int] * 11 + [c_float_p]
+_lib.orc_conv_output_shape.argtypes = [ctypes.POINTER(ConvGeom), c_int_p, c_int_p]
+_lib.orc_conv_forward.argtypes = [ctypes.POINTER(ConvGeom), ctypes.c_int, c_float_p, c_float_p,
+                                  c_float_p, c_float_p]
+_lib.orc_deconv_forward.argtypes = _lib.orc_conv_forward.argtypes
+_lib.orc_inner_product.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, c_float_p, c_float_p,
+                                   c_float_p, ctypes.c_int, c_float_p]
+_lib.orc_exp.argtypes = [ctypes.c_int, c_float_p, c_float_p]
+_lib.orc_powx.argtypes = [ctypes.c_int, c_float_p, ctypes.c_float, c_float_p]
+_lib.orc_batch_norm.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, c_float_p, c_float_p,
+                                c_float_p, c_float_p, ctypes.c_int, ctypes.c_float, c_float_p]
+_lib.orc_scale.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, c_float_p, c_float_p,
+                           c_float_p, c_float_p]
+_lib.orc_bias.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, c_float_p, c_float_p,
+                          c_float_p]
+_lib.orc_relu.argtypes = [ctypes.c_size_t, c_float_p, ctypes.c_float, c_float_p]
+_lib.orc_tanh.argtypes = [ctypes.c_size_t, c_float_p, c_float_p]
+_lib.orc_sigmoid.argtypes = [ctypes.c_size_t, c_float_p, c_float_p]
+_lib.orc_pooling_output_shape.argtypes = [ctypes.c_int] * 8 + [c_int_p, c_int_p]
+_lib.orc_pooling.argtypes = [ctypes.c_int] * 10 + [c_float_p, c_float_p]
+_lib.orc_eltwise.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(c_float_p), c_float_p,
+                             ctypes.c_size_t, c_float_p]
+_lib.orc_softmax.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, c_float_p, c_float_p]
+
+
+# ---- numpy API ---------------------------------------------------------------
+
+def gemm(transa, transb, M, N, K, alpha, A, B, beta, C):
+    A, B = _f32(A), _f32(B)
+    _lib.orc_gemm(int(transa), int(transb), M, N, K, alpha, _fp(A), _fp(B), beta, _fp(C))
+    return C
+
+
+def im2col(im, kernel, pad, stride, dilation):
+    im = _f32(im)
+    C, H, W = im.shape
+    (kh, kw), (ph, pw), (sh, sw), (dh, dw) = kernel, pad, stride, dilation
+    Ho = (H + 2 * ph - (dh * (kh - 1) + 1)) // sh + 1
+    Wo = (W + 2 * pw - (dw * (kw - 1) + 1)) // sw + 1
+    col = np.empty((C * kh * kw, Ho, Wo), np.float32)
+    _lib.orc_im2col(_fp(im), C, H, W, kh, kw, ph, pw, sh, sw, dh, dw, _fp(col))
+    return col
+
+
+def col2im(col, C, H, W, kernel, pad, stride, dilation):
+    col = _f32(col)
+    (kh, kw), (ph, pw), (sh, sw), (dh, dw) = kernel, pad, stride, dilation
+    im = np.empty((C, H, W), np.float32)
+    _lib.orc_col2im(_fp(col), C, H, W, kh, kw, ph, pw, sh, sw, dh, dw, _fp(im))
+    return im
+
+
+def conv_output_shape(geom):
+    ho, wo = ctypes.c_int(), ctypes.c_int()
+    _lib.orc_conv_output_shape(ctypes.byref(geom), ctypes.byref(ho), ctypes.byref(wo))
+    return ho.value, wo.value
+
+
+def conv_forward(geom, x, w, bias=None):
+    """Convolution (geom.transposed == 0) or Deconvolution forward of x [N,Cin,H,W]."""
+    x, w = _f32(x), _f32(w)
+    b = _f32(bias) if bias is not None else None
+    ho, wo = conv_output_shape(geom)
+    y = np.empty((x.shape[0], geom.channels_out, ho, wo), np.float32)
+    fn = _lib.orc_deconv_forward if geom.transposed else _lib.orc_conv_forward
+    fn(ctypes.byref(geom), x.shape[0], _fp(x), _fp(w), _fp(b) if b is not None else None, _fp(y))
+    return y
+
+
+def inner_product(x, w, bias=None, transpose=False):
+    x, w = _f32(x), _f32(w)
+    M, K = x.shape[0], int(np.prod(x.shape[1:]))
+    N = w.shape[1] if transpose else w.shape[0]
+    b = _f32(bias) if bias is not None else None
+    y = np.empty((M, N), np.float32)
+    _lib.orc_inner_product(M, N, K, _fp(x), _fp(w), _fp(b) if b is not None else None,
+                           int(transpose), _fp(y))
+    return y
+
+
+def exp(a):
+    a = _f32(a)
+    y = np.empty_like(a)
+    _lib.orc_exp(a.size, _fp(a), _fp(y))
+    return y
+
+
+def powx(a, b):
+    a = _f32(a)
+    y = np.empty_like(a)
+    _lib.orc_powx(a.size, _fp(a), b, _fp(y))
+    return y
+
+
+def batch_norm(x, blob0, blob1, blob2, use_global_stats=True, eps=1e-5):
+    x = _f32(x)
+    num, ch = x.shape[0], (x.shape[1] if x.ndim > 1 else 1)
+    spatial = x.size // (num * ch)
+    y = np.empty_like(x)
+    b0, b1, b2 = _f32(blob0), _f32(blob1), _f32(blob2)
+    _lib.orc_batch_norm(num, ch, spatial, _fp(x), _fp(b0), _fp(b1), _fp(b2),
+                        int(use_global_stats), eps, _fp(y))
+    return y
+
+
+def scale(x, gamma, beta=None, axis=1):
+    x, gamma = _f32(x), _f32(gamma)
+    outer = int(np.prod(x.shape[:axis]))
+    inner = int(np.prod(x.shape[axis + gamma.ndim:]))
+    b = _f32(beta) if beta is not None else None
+    y = np.empty_like(x)
+    _lib.orc_scale(outer, gamma.size, inner, _fp(x), _fp(gamma),
+                   _fp(b) if b is not None else None, _fp(y))
+    return y
+
+
+def bias(x, beta, axis=1):
+    x, beta = _f32(x), _f32(beta)
+    outer = int(np.prod(x.shape[:axis]))
+    inner = int(np.prod(x.shape[axis + beta.ndim:]))
+    y = np.empty_like(x)
+    _lib.orc_bias(outer, beta.size, inner, _fp(x), _fp(beta), _fp(y))
+    return y
+
+
+def relu(x, negative_slope=0.0):
+    x = _f32(x)
+    y = np.empty_like(x)
+    _lib.orc_relu(x.size, _fp(x), negative_slope, _fp(y))
+    return y
+
+
+def tanh(x):
+    x = _f32(x)
+    y = np.empty_like(x)
+    _lib.orc_tanh(x.size, _fp(x), _fp(y))
+    return y
+
+
+def sigmoid(x):
+    x = _f32(x)
+    y = np.empty_like(x)
+    _lib.orc_sigmoid(x.size, _fp(x), _fp(y))
+    return y
+
+
+def pooling_output_shape(H, W, kernel, stride, pad):
+    ho, wo = ctypes.c_int(), ctypes.c_int()
+    _lib.orc_pooling_output_shape(H, W, kernel[0], kernel[1], stride[0], stride[1], pad[0], pad[1],
+                                  ctypes.byref(ho), ctypes.byref(wo))
+    return ho.value, wo.value
+
+
+def pooling(x, method, kernel, stride=(1, 1), pad=(0, 0), global_pooling=False):
+    """method: 'MAX' or 'AVE'; x [N,C,H,W]."""
+    x = _f32(x)
+    N, C, H, W = x.shape
+    if global_pooling:
+        kernel = (H, W)
+    ho, wo = pooling_output_shape(H, W, kernel, stride, pad)
+    y = np.empty((N, C, ho, wo), np.float32)
+    _lib.orc_pooling({"MAX": 0, "AVE": 1}[method], N * C, H, W, kernel[0], kernel[1], stride[0],
+                     stride[1], pad[0], pad[1], _fp(x), _fp(y))
+    return y
+
+
+def eltwise(bottoms, op="SUM", coeffs=None):
+    bs = [_f32(b) for b in bottoms]
+    arr = (c_float_p * len(bs))(*[_fp(b) for b in bs])
+    co = _f32(coeffs) if coeffs is not None and len(coeffs) else None
+    y = np.empty_like(bs[0])
+    _lib.orc_eltwise({"PROD": 0, "SUM": 1, "MAX": 2}[op], len(bs), arr,
+                     _fp(co) if co is not None else None, bs[0].size, _fp(y))
+    return y
+
+
+def softmax(x, axis=1):
+    x = _f32(x)
+    axis = axis % x.ndim
+    outer = int(np.prod(x.shape[:axis]))
+    inner = int(np.prod(x.shape[axis + 1:]))
+    y = np.empty_like(x)
+    _lib.orc_softmax(outer, x.shape[axis], inner, _fp(x), _fp(y))
+    return y
