@@ -33,6 +33,7 @@ namespace mchip {
 namespace {
 
 constexpr int BK = 16;
+constexpr int LDK = BK + 4;  // LDS row pitch in floats
 
 typedef float acc16 __attribute__((ext_vector_type(16)));
 
@@ -53,7 +54,6 @@ struct IgemmArgs {
   int x_gstride;      // (Cin/g)*H*W
   int M;              // output channels per group
   int Mpad, Kpad;
-  int wt_gstride;     // Kpad*Mpad
   int Wo;             // top width
   int y_cstride;      // Ho*Wo
   int y_nstride;      // Cout*Ho*Wo
@@ -62,6 +62,10 @@ struct IgemmArgs {
   int act;
   float slope;
 };
+
+__device__ __forceinline__ float f4at(const float4& v, int e) {
+  return e == 0 ? v.x : (e == 1 ? v.y : (e == 2 ? v.z : v.w));
+}
 
 __device__ __forceinline__ float apply_act(float v, int act, float slope) {
   switch (act) {
@@ -83,13 +87,18 @@ __global__ __launch_bounds__(256) void igemm_kernel(const IgemmArgs a) {
   constexpr int TM = BM / WM / 32;
   constexpr int TN = BN / WN / 32;
   static_assert(TM >= 1 && TN >= 1, "wave tile must hold a 32x32 block");
-  constexpr int ROWS_PER_PASS = 256 / BN;
-  constexpr int B_PER_THREAD = BK / ROWS_PER_PASS;
-  constexpr int A_F4 = BM * BK / 4;               // float4 per A tile
+  constexpr int QUADS = BK / 4;                   // float4 groups along K per tile
+  constexpr int ROWS_PER_PASS = 256 / BN;         // K quads gathered per pass
+  constexpr int B_Q = QUADS / ROWS_PER_PASS;      // quads per thread
+  static_assert(B_Q >= 1, "tile too narrow for 256 gathering threads");
+  constexpr int A_F4 = BM * QUADS;                // float4 per A tile
   constexpr int A_VEC = (A_F4 + 255) / 256;
 
-  __shared__ __attribute__((aligned(16))) float As[2][BK][BM];
-  __shared__ __attribute__((aligned(16))) float Bs[2][BK][BN];
+  // K runs fastest in LDS ([row][k], rows padded to LDK floats) so that one
+  // ds_read_b128 hands a lane four K steps of its MFMA operand; the 80-byte row
+  // pitch spreads eight consecutive rows over all 32 banks.
+  __shared__ __attribute__((aligned(16))) float As[2][BM][LDK];
+  __shared__ __attribute__((aligned(16))) float Bs[2][BN][LDK];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -130,48 +139,81 @@ __global__ __launch_bounds__(256) void igemm_kernel(const IgemmArgs a) {
       xbase = 0;
     }
   }
-  const float* __restrict__ wt_tile = a.wt + (size_t)g * a.wt_gstride + mt * BM;
+  const int KT = a.Kpad / BK;
+  // Packed filter: [g][K tile][m][16 k], so an A tile is one contiguous run.
+  const float* __restrict__ wt_tile =
+      a.wt + ((size_t)g * KT * a.Mpad + (size_t)mt * BM) * BK;
+  const size_t wt_kt_stride = (size_t)a.Mpad * BK;
 
   float4 areg[A_VEC];
-  float breg[B_PER_THREAD];
+  float4 breg[B_Q];
 
-  auto load_tiles = [&](int kt) {
-#pragma unroll
-    for (int i = 0; i < A_VEC; ++i) {
-      const int f = tid + 256 * i;
-      if (A_F4 % 256 == 0 || f < A_F4) {
-        const int row = f / (BM / 4);
-        const int c4 = f % (BM / 4);
-        areg[i] = *reinterpret_cast<const float4*>(
-            wt_tile + (size_t)(kt * BK + row) * a.Mpad + c4 * 4);
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < B_PER_THREAD; ++i) {
-      const int krow = __builtin_amdgcn_readfirstlane(kt * BK + i * ROWS_PER_PASS + prow);
-      const int4 t = a.ktab[krow];
-      const int hi = hi0 + t.y;
-      const int wi = wi0 + t.z;
-      const bool ok = static_cast<unsigned>(hi) < static_cast<unsigned>(a.H) &&
-                      static_cast<unsigned>(wi) < static_cast<unsigned>(a.W);
-      breg[i] = ok ? a.x[xbase + t.x] : 0.f;
-    }
-  };
-  auto store_tiles = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < A_VEC; ++i) {
-      const int f = tid + 256 * i;
-      if (A_F4 % 256 == 0 || f < A_F4) {
-        const int row = f / (BM / 4);
-        const int c4 = f % (BM / 4);
-        *reinterpret_cast<float4*>(&As[buf][row][c4 * 4]) = areg[i];
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < B_PER_THREAD; ++i) {
-      Bs[buf][i * ROWS_PER_PASS + prow][pj] = breg[i];
-    }
-  };
+  // Global -> registers for K tile kt.  Branch-free on purpose: tap entries are
+  // scalar loads, an out-of-image tap reads element 0 and is zeroed by a
+  // select, so all loads of a tile issue back to back.
+#define MC_GATHER1(dst, t)                                                                   \
+  {                                                                                          \
+    const int hi = hi0 + (t).y;                                                              \
+    const int wi = wi0 + (t).z;                                                              \
+    const bool ok = (static_cast<unsigned>(hi) < static_cast<unsigned>(a.H)) &               \
+                    (static_cast<unsigned>(wi) < static_cast<unsigned>(a.W));                \
+    const int off = ok ? xbase + (t).x : 0;                                                  \
+    const float v = a.x[off];                                                                \
+    dst = ok ? v : 0.f;                                                                      \
+  }
+#define MC_LOAD_TILES(kt)                                                                    \
+  {                                                                                          \
+    _Pragma("unroll") for (int i = 0; i < A_VEC; ++i) {                                      \
+      const int f = tid + 256 * i;                                                           \
+      if (A_F4 % 256 == 0 || f < A_F4)                                                       \
+        areg[i] = *reinterpret_cast<const float4*>(wt_tile + (kt)*wt_kt_stride + f * 4);     \
+    }                                                                                        \
+    _Pragma("unroll") for (int i = 0; i < B_Q; ++i) {                                        \
+      const int krow =                                                                       \
+          __builtin_amdgcn_readfirstlane((kt)*BK + (i * ROWS_PER_PASS + prow) * 4);          \
+      const int4 t0 = a.ktab[krow], t1 = a.ktab[krow + 1], t2 = a.ktab[krow + 2],            \
+                 t3 = a.ktab[krow + 3];                                                      \
+      MC_GATHER1(breg[i].x, t0);                                                             \
+      MC_GATHER1(breg[i].y, t1);                                                             \
+      MC_GATHER1(breg[i].z, t2);                                                             \
+      MC_GATHER1(breg[i].w, t3);                                                             \
+    }                                                                                        \
+  }
+#define MC_STORE_TILES(buf)                                                                  \
+  {                                                                                          \
+    _Pragma("unroll") for (int i = 0; i < A_VEC; ++i) {                                      \
+      const int f = tid + 256 * i;                                                           \
+      if (A_F4 % 256 == 0 || f < A_F4)                                                       \
+        *reinterpret_cast<float4*>(&As[buf][f / QUADS][(f % QUADS) * 4]) = areg[i];          \
+    }                                                                                        \
+    _Pragma("unroll") for (int i = 0; i < B_Q; ++i) {                                        \
+      *reinterpret_cast<float4*>(&Bs[buf][pj][(i * ROWS_PER_PASS + prow) * 4]) = breg[i];    \
+    }                                                                                        \
+  }
+  // One MFMA K step multiplies k-pairs; which two physical k rows form a pair
+  // is free as long as A and B agree, so half-wave 0 takes k = 8h+e and
+  // half-wave 1 takes k = 8h+4+e for step (h, e): four steps per b128 read.
+#define MC_COMPUTE(buf)                                                                      \
+  {                                                                                          \
+    float4 av[TM][2], bv[TN][2];                                                             \
+    _Pragma("unroll") for (int h = 0; h < 2; ++h) {                                          \
+      _Pragma("unroll") for (int i = 0; i < TM; ++i) av[i][h] =                              \
+          *reinterpret_cast<const float4*>(&As[buf][wm0 + i * 32 + l32][h * 8 + lhi * 4]);   \
+      _Pragma("unroll") for (int j = 0; j < TN; ++j) bv[j][h] =                              \
+          *reinterpret_cast<const float4*>(&Bs[buf][wn0 + j * 32 + l32][h * 8 + lhi * 4]);   \
+    }                                                                                        \
+    _Pragma("unroll") for (int h = 0; h < 2; ++h) {                                          \
+      _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                        \
+        _Pragma("unroll") for (int i = 0; i < TM; ++i) {                                     \
+          _Pragma("unroll") for (int j = 0; j < TN; ++j) {                                   \
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(f4at(av[i][h], e),              \
+                                                             f4at(bv[j][h], e), acc[i][j],   \
+                                                             0, 0, 0);                       \
+          }                                                                                  \
+        }                                                                                    \
+      }                                                                                      \
+    }                                                                                        \
+  }
 
   acc16 acc[TM][TN];
 #pragma unroll
@@ -186,31 +228,25 @@ __global__ __launch_bounds__(256) void igemm_kernel(const IgemmArgs a) {
   const int l32 = lane & 31;
   const int lhi = lane >> 5;
 
-  const int KT = a.Kpad / BK;
   if (KT > 0) {
-    load_tiles(0);
-    store_tiles(0);
-  }
-  __syncthreads();
-  for (int kt = 0; kt < KT; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < KT) load_tiles(kt + 1);
-#pragma unroll
-    for (int kk = 0; kk < BK / 2; ++kk) {
-      float av[TM], bv[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i) av[i] = As[buf][kk * 2 + lhi][wm0 + i * 32 + l32];
-#pragma unroll
-      for (int j = 0; j < TN; ++j) bv[j] = Bs[buf][kk * 2 + lhi][wn0 + j * 32 + l32];
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
-    }
-    if (kt + 1 < KT) store_tiles(buf ^ 1);
+    MC_LOAD_TILES(0);
+    MC_STORE_TILES(0);
     __syncthreads();
+    for (int kt = 0; kt < KT - 1; ++kt) {
+      const int buf = kt & 1;
+      MC_LOAD_TILES(kt + 1);
+      __builtin_amdgcn_sched_barrier(0);  // keep the global loads ahead of the MFMA block
+      MC_COMPUTE(buf);
+      __builtin_amdgcn_sched_barrier(0);
+      MC_STORE_TILES(buf ^ 1);
+      __syncthreads();
+    }
+    MC_COMPUTE((KT - 1) & 1);
   }
+#undef MC_GATHER1
+#undef MC_LOAD_TILES
+#undef MC_STORE_TILES
+#undef MC_COMPUTE
 
   // Epilogue.  Accumulator register r of lane l holds row 8*(r/4)+4*(l/32)+r%4,
   // column l%32 of its 32x32 block; a half-wave therefore stores 32 consecutive
@@ -247,17 +283,22 @@ __global__ __launch_bounds__(256) void igemm_kernel(const IgemmArgs a) {
   }
 }
 
-// wt[g][k][m] = w[g*wg_stride + wk_off[k] + m*wm_stride] for k<K, m<M, else 0.
+// Packed filter wt[g][kt][m][kl] = w[g*wg_stride + wk_off[k] + m*wm_stride] with
+// k = kt*16 + kl, zero where k >= K or m >= M.
 __global__ void pack_weights_kernel(const float* __restrict__ w, float* __restrict__ wt,
                                     const int* __restrict__ wk_off, int G, int K, int Kpad,
                                     int M, int Mpad, int wm_stride, int wg_stride) {
   const long total = (long)G * Kpad * Mpad;
+  const int KT = Kpad / BK;
   for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total;
        i += (long)gridDim.x * blockDim.x) {
-    const int m = static_cast<int>(i % Mpad);
-    const long t = i / Mpad;
-    const int k = static_cast<int>(t % Kpad);
-    const int g = static_cast<int>(t / Kpad);
+    const int kl = static_cast<int>(i % BK);
+    long t = i / BK;
+    const int m = static_cast<int>(t % Mpad);
+    t /= Mpad;
+    const int kt = static_cast<int>(t % KT);
+    const int g = static_cast<int>(t / KT);
+    const int k = kt * BK + kl;
     float v = 0.f;
     if (k < K && m < M) v = w[(long)g * wg_stride + wk_off[k] + (long)m * wm_stride];
     wt[i] = v;
@@ -313,21 +354,19 @@ struct mcConvPlan {
 
 namespace {
 
+// Tile choice.  With 256 CUs the tile count per CU is small for most layers, so
+// load balance (the last, partly filled round of tiles) dominates: measured on
+// ResNet-50 shapes the 64x64 tile, which runs 8 workgroups per CU, beats the
+// larger tiles everywhere their extra reuse could matter.  Narrow outputs
+// (<= 32 channels per group) use the 32-row tiles instead of padding M to 64.
 int pick_config(const mcConvPlan* plan, long pixels) {
   if (plan->forced_config >= 0) return plan->forced_config;
   const int M = plan->M;
-  int bm = M > 64 ? 128 : (M > 32 ? 64 : 32);
-  int bn = 128;
-  auto blocks = [&](int bm_, int bn_) {
-    return (long)ceil_div(M, bm_) * ceil_div(pixels, bn_) * plan->geom.group;
-  };
-  if (bm == 128 && blocks(128, 128) < 2 * kNumCu) {
-    bm = (M % 128 != 0 && M % 128 <= 64) || blocks(128, 64) < 2 * kNumCu ? 64 : 128;
-    bn = 64;
-  } else if (bm == 64 && blocks(64, 128) < 2 * kNumCu) {
-    bn = 64;
-  } else if (bm == 32) {
-    bn = blocks(32, 256) >= 4 * kNumCu ? 256 : 128;
+  int bm = 64, bn = 64;
+  if (M <= 32) {
+    bm = 32;
+    const long tiles256 = (long)ceil_div(pixels, 256) * plan->geom.group;
+    bn = tiles256 >= 8L * kNumCu ? 256 : 128;
   }
   for (int i = 0; i < kNumConfigs; ++i)
     if (kConfigs[i].bm == bm && kConfigs[i].bn == bn) return i;
@@ -546,7 +585,6 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
     a.M = plan->M;
     a.Mpad = plan->Mpad;
     a.Kpad = s.Kpad;
-    a.wt_gstride = s.Kpad * plan->Mpad;
     a.Wo = plan->Wo;
     a.y_cstride = plan->Ho * plan->Wo;
     a.y_nstride = g.channels_out * plan->Ho * plan->Wo;
