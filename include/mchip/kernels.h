@@ -75,6 +75,12 @@ typedef struct mcConvPlan mcConvPlan;
 int mcConvPlanCreate(const mcConvGeom* geom, mcConvPlan** plan);
 int mcConvPlanDestroy(mcConvPlan* plan);
 
+/* Plan for InnerProduct: top (M x N) = bottom (M x K) * W^T with W stored N x K,
+ * or K x N when transpose is set (inner_product_layer.cpp:80-93; replaces the
+ * caffe_gpu_gemv / caffe_gpu_gemm of inner_product_layer.cu:9-31).  It is the
+ * 1x1 convolution of a [M, K, 1, 1] blob: run it with mcConvForward(num = M). */
+int mcInnerProductPlanCreate(int K, int N, int transpose, mcConvPlan** plan);
+
 /* Output height/width for this geometry (conv_layer.cpp:12-25,
  * deconv_layer.cpp:11-25). */
 int mcConvPlanOutputShape(const mcConvPlan* plan, int* height_out, int* width_out);
@@ -101,6 +107,116 @@ const char* mcConvPlanKernelName(const mcConvPlan* plan, int num);
 /* Tuning/test knob: pin the tile configuration (index into the built-in table),
  * -1 restores the automatic choice.  No counterpart in the reference. */
 int mcConvPlanForceConfig(mcConvPlan* plan, int config);
+
+
+/* HIP stream of the calling thread's Mini-Caffe context (created on first use);
+ * lets a harness record events around Net::Forward.  NULL if no device. */
+void* mcCurrentStream(void);
+
+/* ---- per-channel transforms and activations (HBM-bound) ------------------- */
+
+/* One fused pass  v = x[o][c][i];  v -= sub[c];  v /= div[c];  v *= mul[c];
+ * v += add[c];  y = act(v)  with every vector optional (NULL skips the step).
+ * The step order is the reference's: BatchNorm subtracts the mean, then divides
+ * by sqrt(var+eps) (batch_norm_layer.cpp:103-135); Scale multiplies, its Bias
+ * adds (scale_layer.cpp:102-114, bias_layer.cpp:68-83); then ReLU / TanH /
+ * Sigmoid (relu_layer.cpp:12-30, tanh_layer.cpp:14-22, sigmoid_layer.cpp:12-24).
+ * Replaces ScaleForward/ScaleBiasForward (scale_layer.cu:9-25), BiasForward
+ * (bias_layer.cu:9-16), ReLUForward (relu_layer.cu:8-13), TanHForward,
+ * SigmoidForward and the ~10 passes of BatchNormLayer::Forward_gpu
+ * (batch_norm_layer.cu:9-73).  x == y (in place) is allowed. */
+typedef struct mcChannelOp {
+  const float* sub;
+  const float* div;
+  const float* mul;
+  const float* add;
+  int activation;        /* enum mcActivation */
+  float negative_slope;
+} mcChannelOp;
+int mcChannelTransform(const float* x, float* y, int outer, int channels, int inner,
+                       const mcChannelOp* op, void* stream);
+
+/* BatchNorm with stored statistics: mean[c] = blob0[c]*f, stdev[c] =
+ * sqrt(blob1[c]*f + eps) with f = (blob2[0] == 0 ? 0 : 1/blob2[0])
+ * (batch_norm_layer.cpp:83-90,123-126), computed on the device. */
+int mcBatchNormStored(const float* blob0, const float* blob1, const float* blob2, float eps,
+                      int channels, float* mean, float* stdev, void* stream);
+
+/* BatchNorm with batch statistics (use_global_stats: false): per channel, mean
+ * over num*spatial and stdev = sqrt(E[(x-mean)^2] + eps)
+ * (batch_norm_layer.cpp:91-126).  One workgroup per channel, two passes. */
+int mcBatchNormBatchStats(const float* x, int num, int channels, int spatial, float eps,
+                          float* mean, float* stdev, void* stream);
+
+/* Collapses a chain of up to 4 per-channel stages (same step order as
+ * mcChannelTransform, applied first to last) that follow a contraction into one
+ * scale/shift pair for its epilogue:  y = acc*scale[c] + shift[c].
+ * bias0 (optional) is the contraction's own bias, added before the first stage. */
+int mcFoldChannelOps(const float* bias0, const mcChannelOp* stages, int num_stages, int channels,
+                     float* scale, float* shift, void* stream);
+
+/* ---- Pooling ---------------------------------------------------------------- */
+
+enum mcPoolMethod { MC_POOL_MAX = 0, MC_POOL_AVE = 1 };
+
+/* Output extent with Caffe's ceil rule and last-window clip
+ * (pooling_layer.cpp:88-107). */
+int mcPoolingOutputShape(int height, int width, int kernel_h, int kernel_w, int stride_h,
+                         int stride_w, int pad_h, int pad_w, int* height_out, int* width_out);
+
+/* bottom [planes, H, W] -> top [planes, Ho, Wo] with planes = num*channels.
+ * MAX starts from -FLT_MAX over the window clipped to the image; AVE divides by
+ * the window area clipped to the padded extent (pooling_layer.cpp:127-189).
+ * Replaces MaxPoolForward / AvePoolForward (pooling_layer.cu:10-71). */
+int mcPooling(int method, const float* bottom, float* top, int planes, int height, int width,
+              int kernel_h, int kernel_w, int stride_h, int stride_w, int pad_h, int pad_w,
+              void* stream);
+
+/* ---- Eltwise ---------------------------------------------------------------- */
+
+enum mcEltwiseOp { MC_ELT_PROD = 0, MC_ELT_SUM = 1, MC_ELT_MAX = 2 };
+
+/* top = op over up to 8 bottoms of `count` floats; SUM is 0 + sum coeff_i*x_i in
+ * bottom order (eltwise_layer.cpp:38-78); coeffs may be NULL (all 1).  An
+ * activation can be fused on the result.  bottoms: host array of device
+ * pointers.  Replaces MaxForward and the caffe_gpu_axpy / caffe_gpu_mul chains
+ * of eltwise_layer.cu:10-50. */
+int mcEltwise(int op, int num_bottoms, const float* const* bottoms, const float* coeffs,
+              long count, float* top, int activation, float negative_slope, void* stream);
+
+/* ---- Softmax ---------------------------------------------------------------- */
+
+/* Softmax along an axis of extent `channels` with `inner` trailing elements:
+ * subtract the max, expf, sum in ascending channel order, divide
+ * (softmax_layer.cpp:28-63).  One launch instead of the five of
+ * softmax_layer.cu:77-111. */
+int mcSoftmax(const float* bottom, float* top, int outer, int channels, int inner, void* stream);
+
+/* ---- layout ----------------------------------------------------------------- */
+
+/* rows x width strided copy: dst[r*dst_pitch + i] = src[r*src_pitch + i].
+ * Concat and Slice are one such copy per bottom/top (concat_layer.cu:8-46,
+ * slice_layer.cu:8-46). */
+int mcCopy2D(const float* src, long src_pitch, float* dst, long dst_pitch, long width, long rows,
+             void* stream);
+
+/* Generic N-d transpose, top axis i = bottom axis order[i]
+ * (permute_layer.cpp:9-106, PermuteKernel permute_layer.cu:10-28).  The
+ * NCHW->NHWC order (0,2,3,1) and other "swap two adjacent axis groups" orders go
+ * through an LDS-tiled transpose so both sides are coalesced. shape/order: host. */
+int mcPermute(const float* bottom, float* top, int num_axes, const int* shape, const int* order,
+              void* stream);
+
+/* L2 normalisation (SSD's Normalize layer, normalize_layer.cpp:88-135; .cu:44-103).
+ * across_spatial == 0: per pixel, norm = sqrt(eps + sum_c x^2); y = (x / norm) * scale.
+ * across_spatial != 0: per image, norm = sqrt(sum x^2 + eps); y = (x * (1/norm)) * scale.
+ * scale holds one value when channel_shared, else one per channel. */
+int mcNormalize(const float* bottom, float* top, int num, int channels, int spatial,
+                int across_spatial, int channel_shared, float eps, const float* scale,
+                void* stream);
+
+/* Fill `count` floats with `value` (caffe_gpu_set, math_functions.cu:70-82). */
+int mcFill(float* dst, long count, float value, void* stream);
 
 #ifdef __cplusplus
 }

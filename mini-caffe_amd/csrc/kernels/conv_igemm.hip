@@ -512,6 +512,27 @@ int mcConvPlanCreate(const mcConvGeom* gp, mcConvPlan** out) {
   return 0;
 }
 
+int mcInnerProductPlanCreate(int K, int N, int transpose, mcConvPlan** out) {
+  MC_REQUIRE(K > 0 && N > 0 && out, "mcInnerProductPlanCreate: bad argument");
+  mcConvGeom g = {K, 1, 1, N, 1, 1, 1, 1, 0, 0, 1, 1, 1, 0};
+  if (mcConvPlanCreate(&g, out)) return -1;
+  if (transpose) {
+    // weights are K x N: element (k, m) sits at k*N + m
+    mcConvPlan* plan = *out;
+    SubProblem& s = plan->subs[0];
+    for (int k = 0; k < s.K; ++k) s.wk_off[k] = k * N;
+    plan->wm_stride = 1;
+    hipError_t e =
+        hipMemcpy(s.wk_off_dev, s.wk_off.data(), sizeof(int) * s.K, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+      mcConvPlanDestroy(plan);
+      *out = nullptr;
+      return fail("mcInnerProductPlanCreate: %s", hipGetErrorString(e));
+    }
+  }
+  return 0;
+}
+
 int mcConvPlanDestroy(mcConvPlan* plan) {
   if (!plan) return 0;
   for (auto& s : plan->subs) free_sub(s);

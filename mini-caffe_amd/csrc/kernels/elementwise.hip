@@ -1,0 +1,366 @@
+// HBM-bound per-channel and elementwise kernels: the fused BatchNorm / Scale /
+// Bias / activation pass, BatchNorm statistics, Eltwise, fill and strided copy.
+//
+// All of them move each element once: one global read per input and one global
+// write per output, 16-byte vector accesses whenever the shape allows it, and a
+// grid of a few waves per CU walking the blob with a grid stride.
+#include "mc_common.h"
+#include "mchip/kernels.h"
+
+#include <cfloat>
+
+namespace mchip {
+namespace {
+
+__device__ __forceinline__ float act_apply(float v, int act, float slope) {
+  switch (act) {
+    case MC_ACT_RELU:
+      // slope == 0 gives max(x,0); otherwise max(x,0) + slope*min(x,0)
+      // (reference relu_layer.cpp:18-28).
+      return v > 0.f ? v : v * slope;
+    case MC_ACT_TANH:
+      return static_cast<float>(tanh(static_cast<double>(v)));
+    case MC_ACT_SIGMOID:
+      return static_cast<float>(1. / (1. + exp(-static_cast<double>(v))));
+    default:
+      return v;
+  }
+}
+
+struct ChanArgs {
+  const float* __restrict__ x;
+  float* __restrict__ y;
+  const float* __restrict__ sub;
+  const float* __restrict__ div;
+  const float* __restrict__ mul;
+  const float* __restrict__ add;
+  long count;     // outer*channels*inner
+  int channels;
+  int inner;
+  int act;
+  float slope;
+};
+
+__device__ __forceinline__ float chan_one(float v, int c, const ChanArgs& a) {
+  if (a.sub) v -= a.sub[c];
+  if (a.div) v /= a.div[c];
+  if (a.mul) v *= a.mul[c];
+  if (a.add) v += a.add[c];
+  return act_apply(v, a.act, a.slope);
+}
+
+// VEC = 4 requires inner % 4 == 0, so the four lanes of a float4 share a channel.
+template <int VEC>
+__global__ __launch_bounds__(256) void channel_transform_kernel(const ChanArgs a) {
+  const long n = a.count / VEC;
+  for (long i = blockIdx.x * 256L + threadIdx.x; i < n; i += gridDim.x * 256L) {
+    const long e = i * VEC;
+    const int c = static_cast<int>((e / a.inner) % a.channels);
+    if (VEC == 4) {
+      float4 v = reinterpret_cast<const float4*>(a.x)[i];
+      v.x = chan_one(v.x, c, a);
+      v.y = chan_one(v.y, c, a);
+      v.z = chan_one(v.z, c, a);
+      v.w = chan_one(v.w, c, a);
+      reinterpret_cast<float4*>(a.y)[i] = v;
+    } else {
+      a.y[i] = chan_one(a.x[i], c, a);
+    }
+  }
+}
+
+__global__ void bn_stored_kernel(const float* __restrict__ b0, const float* __restrict__ b1,
+                                 const float* __restrict__ b2, float eps, int C,
+                                 float* __restrict__ mean, float* __restrict__ stdev) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const float f = b2[0] == 0.f ? 0.f : 1.f / b2[0];
+  mean[c] = f * b0[c];
+  stdev[c] = sqrtf(f * b1[c] + eps);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// Sum over a 256-thread workgroup; every thread gets the result.
+__device__ __forceinline__ float block_sum_256(float v, float* lds4) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds4[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return lds4[0] + lds4[1] + lds4[2] + lds4[3];
+}
+
+__global__ __launch_bounds__(256) void bn_batch_stats_kernel(const float* __restrict__ x, int num,
+                                                             int C, int spatial, float eps,
+                                                             float* __restrict__ mean,
+                                                             float* __restrict__ stdev) {
+  __shared__ float red[4];
+  const int c = blockIdx.x;
+  const long per_c = (long)num * spatial;
+  const float alpha = static_cast<float>(1. / (static_cast<double>(num) * spatial));
+  float s = 0.f;
+  for (long i = threadIdx.x; i < per_c; i += 256) {
+    const long n = i / spatial, sp = i - n * spatial;
+    s += x[(n * C + c) * spatial + sp];
+  }
+  const float m = alpha * block_sum_256(s, red);
+  float q = 0.f;
+  for (long i = threadIdx.x; i < per_c; i += 256) {
+    const long n = i / spatial, sp = i - n * spatial;
+    const float d = x[(n * C + c) * spatial + sp] - m;
+    q += d * d;
+  }
+  const float var = alpha * block_sum_256(q, red);
+  if (threadIdx.x == 0) {
+    mean[c] = m;
+    stdev[c] = sqrtf(var + eps);
+  }
+}
+
+struct FoldArgs {
+  const float* bias0;
+  mcChannelOp st[4];
+  int ns;
+  int C;
+  float* scale;
+  float* shift;
+};
+
+__global__ void fold_kernel(const FoldArgs a) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= a.C) return;
+  float s = 1.f, t = a.bias0 ? a.bias0[c] : 0.f;
+  for (int i = 0; i < a.ns; ++i) {
+    const mcChannelOp& o = a.st[i];
+    if (o.sub) t -= o.sub[c];
+    if (o.div) {
+      s /= o.div[c];
+      t /= o.div[c];
+    }
+    if (o.mul) {
+      s *= o.mul[c];
+      t *= o.mul[c];
+    }
+    if (o.add) t += o.add[c];
+  }
+  a.scale[c] = s;
+  a.shift[c] = t;
+}
+
+struct EltArgs {
+  const float* in[8];
+  float coeff[8];
+  float* out;
+  long count;
+  int nb;
+  int op;
+  int act;
+  float slope;
+};
+
+__device__ __forceinline__ float elt_combine(int op, float acc, float v, float coeff) {
+  if (op == MC_ELT_PROD) return acc * v;
+  if (op == MC_ELT_SUM) return coeff * v + acc;
+  return v > acc ? v : acc;
+}
+
+template <int VEC>
+__global__ __launch_bounds__(256) void eltwise_kernel(const EltArgs a) {
+  const long n = a.count / VEC;
+  for (long i = blockIdx.x * 256L + threadIdx.x; i < n; i += gridDim.x * 256L) {
+    if (VEC == 4) {
+      float4 acc;
+      if (a.op == MC_ELT_SUM) {
+        acc = make_float4(0.f, 0.f, 0.f, 0.f);
+      } else {
+        acc = reinterpret_cast<const float4*>(a.in[0])[i];
+      }
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        if (b >= a.nb) break;
+        if (b == 0 && a.op != MC_ELT_SUM) continue;
+        const float4 v = reinterpret_cast<const float4*>(a.in[b])[i];
+        acc.x = elt_combine(a.op, acc.x, v.x, a.coeff[b]);
+        acc.y = elt_combine(a.op, acc.y, v.y, a.coeff[b]);
+        acc.z = elt_combine(a.op, acc.z, v.z, a.coeff[b]);
+        acc.w = elt_combine(a.op, acc.w, v.w, a.coeff[b]);
+      }
+      acc.x = act_apply(acc.x, a.act, a.slope);
+      acc.y = act_apply(acc.y, a.act, a.slope);
+      acc.z = act_apply(acc.z, a.act, a.slope);
+      acc.w = act_apply(acc.w, a.act, a.slope);
+      reinterpret_cast<float4*>(a.out)[i] = acc;
+    } else {
+      float acc = a.op == MC_ELT_SUM ? 0.f : a.in[0][i];
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        if (b >= a.nb) break;
+        if (b == 0 && a.op != MC_ELT_SUM) continue;
+        acc = elt_combine(a.op, acc, a.in[b][i], a.coeff[b]);
+      }
+      a.out[i] = act_apply(acc, a.act, a.slope);
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void fill_kernel(float* __restrict__ dst, long count, float v) {
+  for (long i = blockIdx.x * 256L + threadIdx.x; i < count; i += gridDim.x * 256L) dst[i] = v;
+}
+
+template <int VEC>
+__global__ __launch_bounds__(256) void copy2d_kernel(const float* __restrict__ src, long src_pitch,
+                                                     float* __restrict__ dst, long dst_pitch,
+                                                     long width, long rows) {
+  const long wv = width / VEC;
+  const long n = wv * rows;
+  for (long i = blockIdx.x * 256L + threadIdx.x; i < n; i += gridDim.x * 256L) {
+    const long r = i / wv, c = (i - r * wv) * VEC;
+    if (VEC == 4) {
+      *reinterpret_cast<float4*>(dst + r * dst_pitch + c) =
+          *reinterpret_cast<const float4*>(src + r * src_pitch + c);
+    } else {
+      dst[r * dst_pitch + c] = src[r * src_pitch + c];
+    }
+  }
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace
+}  // namespace mchip
+
+using namespace mchip;
+
+extern "C" {
+
+int mcChannelTransform(const float* x, float* y, int outer, int channels, int inner,
+                       const mcChannelOp* op, void* stream) {
+  MC_REQUIRE(x && y && op, "mcChannelTransform: null argument");
+  MC_REQUIRE(outer >= 0 && channels > 0 && inner > 0, "mcChannelTransform: bad extents");
+  ChanArgs a;
+  a.x = x;
+  a.y = y;
+  a.sub = op->sub;
+  a.div = op->div;
+  a.mul = op->mul;
+  a.add = op->add;
+  a.count = (long)outer * channels * inner;
+  a.channels = channels;
+  a.inner = inner;
+  a.act = op->activation;
+  a.slope = op->negative_slope;
+  if (a.count == 0) return 0;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (inner % 4 == 0 && aligned16(x) && aligned16(y)) {
+    channel_transform_kernel<4><<<ew_blocks(a.count / 4, 256), 256, 0, st>>>(a);
+  } else {
+    channel_transform_kernel<1><<<ew_blocks(a.count, 256), 256, 0, st>>>(a);
+  }
+  MC_LAUNCH_CHECK();
+  return 0;
+}
+
+int mcBatchNormStored(const float* blob0, const float* blob1, const float* blob2, float eps,
+                      int channels, float* mean, float* stdev, void* stream) {
+  MC_REQUIRE(blob0 && blob1 && blob2 && mean && stdev, "mcBatchNormStored: null argument");
+  MC_REQUIRE(channels > 0, "mcBatchNormStored: bad channel count");
+  bn_stored_kernel<<<ceil_div(channels, 256), 256, 0, static_cast<hipStream_t>(stream)>>>(
+      blob0, blob1, blob2, eps, channels, mean, stdev);
+  MC_LAUNCH_CHECK();
+  return 0;
+}
+
+int mcBatchNormBatchStats(const float* x, int num, int channels, int spatial, float eps,
+                          float* mean, float* stdev, void* stream) {
+  MC_REQUIRE(x && mean && stdev, "mcBatchNormBatchStats: null argument");
+  MC_REQUIRE(num > 0 && channels > 0 && spatial > 0, "mcBatchNormBatchStats: bad extents");
+  bn_batch_stats_kernel<<<channels, 256, 0, static_cast<hipStream_t>(stream)>>>(
+      x, num, channels, spatial, eps, mean, stdev);
+  MC_LAUNCH_CHECK();
+  return 0;
+}
+
+int mcFoldChannelOps(const float* bias0, const mcChannelOp* stages, int num_stages, int channels,
+                     float* scale, float* shift, void* stream) {
+  MC_REQUIRE(scale && shift, "mcFoldChannelOps: null output");
+  MC_REQUIRE(num_stages >= 0 && num_stages <= 4, "mcFoldChannelOps: at most 4 stages");
+  MC_REQUIRE(num_stages == 0 || stages, "mcFoldChannelOps: null stages");
+  FoldArgs a;
+  a.bias0 = bias0;
+  for (int i = 0; i < num_stages; ++i) a.st[i] = stages[i];
+  a.ns = num_stages;
+  a.C = channels;
+  a.scale = scale;
+  a.shift = shift;
+  fold_kernel<<<ceil_div(channels, 256), 256, 0, static_cast<hipStream_t>(stream)>>>(a);
+  MC_LAUNCH_CHECK();
+  return 0;
+}
+
+int mcEltwise(int op, int num_bottoms, const float* const* bottoms, const float* coeffs,
+              long count, float* top, int activation, float negative_slope, void* stream) {
+  MC_REQUIRE(bottoms && top, "mcEltwise: null argument");
+  MC_REQUIRE(op >= MC_ELT_PROD && op <= MC_ELT_MAX, "Unknown elementwise operation.");
+  MC_REQUIRE(num_bottoms >= 1 && num_bottoms <= 8, "mcEltwise: 1..8 bottoms supported");
+  MC_REQUIRE(op == MC_ELT_SUM || num_bottoms >= 2, "mcEltwise: PROD/MAX need two bottoms");
+  if (count == 0) return 0;
+  EltArgs a;
+  bool vec = count % 4 == 0 && aligned16(top);
+  for (int i = 0; i < 8; ++i) {
+    a.in[i] = i < num_bottoms ? bottoms[i] : nullptr;
+    a.coeff[i] = (coeffs && i < num_bottoms) ? coeffs[i] : 1.f;
+    if (i < num_bottoms) {
+      MC_REQUIRE(bottoms[i], "mcEltwise: null bottom");
+      vec = vec && aligned16(bottoms[i]);
+    }
+  }
+  a.out = top;
+  a.count = count;
+  a.nb = num_bottoms;
+  a.op = op;
+  a.act = activation;
+  a.slope = negative_slope;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (vec) {
+    eltwise_kernel<4><<<ew_blocks(count / 4, 256), 256, 0, st>>>(a);
+  } else {
+    eltwise_kernel<1><<<ew_blocks(count, 256), 256, 0, st>>>(a);
+  }
+  MC_LAUNCH_CHECK();
+  return 0;
+}
+
+int mcFill(float* dst, long count, float value, void* stream) {
+  MC_REQUIRE(dst || count == 0, "mcFill: null argument");
+  if (count <= 0) return 0;
+  fill_kernel<<<ew_blocks(count, 256), 256, 0, static_cast<hipStream_t>(stream)>>>(dst, count,
+                                                                                    value);
+  MC_LAUNCH_CHECK();
+  return 0;
+}
+
+int mcCopy2D(const float* src, long src_pitch, float* dst, long dst_pitch, long width, long rows,
+             void* stream) {
+  MC_REQUIRE(src && dst, "mcCopy2D: null argument");
+  MC_REQUIRE(width >= 0 && rows >= 0 && src_pitch >= width && dst_pitch >= width,
+             "mcCopy2D: bad extents");
+  if (width == 0 || rows == 0) return 0;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool vec = width % 4 == 0 && src_pitch % 4 == 0 && dst_pitch % 4 == 0 && aligned16(src) &&
+                   aligned16(dst);
+  if (vec) {
+    copy2d_kernel<4><<<ew_blocks(width / 4 * rows, 256), 256, 0, st>>>(src, src_pitch, dst,
+                                                                       dst_pitch, width, rows);
+  } else {
+    copy2d_kernel<1><<<ew_blocks(width * rows, 256), 256, 0, st>>>(src, src_pitch, dst, dst_pitch,
+                                                                   width, rows);
+  }
+  MC_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // extern "C"

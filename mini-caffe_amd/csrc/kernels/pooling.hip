@@ -1,0 +1,144 @@
+// Max / average pooling (HBM-bound).
+//
+// Windowed pooling: one thread per output element, output width fastest, so a
+// wavefront reads a contiguous span of each input row it touches.  Global
+// pooling (window == image, one output per plane): one wavefront per plane with
+// a shuffle reduction.
+#include "mc_common.h"
+#include "mchip/kernels.h"
+
+#include <cfloat>
+#include <cmath>
+
+namespace mchip {
+namespace {
+
+struct PoolArgs {
+  const float* __restrict__ x;
+  float* __restrict__ y;
+  long total;  // planes*Ho*Wo
+  int H, W, Ho, Wo;
+  int kh, kw, sh, sw, ph, pw;
+};
+
+template <int METHOD>
+__global__ __launch_bounds__(256) void pool_kernel(const PoolArgs a) {
+  for (long i = blockIdx.x * 256L + threadIdx.x; i < a.total; i += gridDim.x * 256L) {
+    const int ow = static_cast<int>(i % a.Wo);
+    const long t = i / a.Wo;
+    const int oh = static_cast<int>(t % a.Ho);
+    const long plane = t / a.Ho;
+    const float* __restrict__ xp = a.x + plane * a.H * a.W;
+    int hs = oh * a.sh - a.ph, ws = ow * a.sw - a.pw;
+    if (METHOD == MC_POOL_MAX) {
+      const int he = min(hs + a.kh, a.H), we = min(ws + a.kw, a.W);
+      hs = max(hs, 0);
+      ws = max(ws, 0);
+      float m = -FLT_MAX;
+      for (int h = hs; h < he; ++h)
+        for (int w = ws; w < we; ++w) m = fmaxf(m, xp[h * a.W + w]);
+      a.y[i] = m;
+    } else {
+      int he = min(hs + a.kh, a.H + a.ph), we = min(ws + a.kw, a.W + a.pw);
+      const int area = (he - hs) * (we - ws);
+      hs = max(hs, 0);
+      ws = max(ws, 0);
+      he = min(he, a.H);
+      we = min(we, a.W);
+      float s = 0.f;
+      for (int h = hs; h < he; ++h)
+        for (int w = ws; w < we; ++w) s += xp[h * a.W + w];
+      a.y[i] = s / static_cast<float>(area);
+    }
+  }
+}
+
+// One wavefront per plane; 4 planes per 256-thread workgroup.
+template <int METHOD>
+__global__ __launch_bounds__(256) void global_pool_kernel(const float* __restrict__ x,
+                                                          float* __restrict__ y, long planes,
+                                                          int hw) {
+  const long plane = blockIdx.x * 4L + (threadIdx.x >> 6);
+  if (plane >= planes) return;
+  const int lane = threadIdx.x & 63;
+  const float* __restrict__ xp = x + plane * hw;
+  float v = METHOD == MC_POOL_MAX ? -FLT_MAX : 0.f;
+  for (int i = lane; i < hw; i += 64) {
+    if (METHOD == MC_POOL_MAX) v = fmaxf(v, xp[i]);
+    else v += xp[i];
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float u = __shfl_xor(v, o, 64);
+    if (METHOD == MC_POOL_MAX) v = fmaxf(v, u);
+    else v += u;
+  }
+  if (lane == 0) y[plane] = METHOD == MC_POOL_MAX ? v : v / static_cast<float>(hw);
+}
+
+}  // namespace
+}  // namespace mchip
+
+using namespace mchip;
+
+extern "C" {
+
+int mcPoolingOutputShape(int H, int W, int kh, int kw, int sh, int sw, int ph, int pw, int* Ho,
+                         int* Wo) {
+  MC_REQUIRE(kh > 0 && kw > 0, "Filter dimensions cannot be zero.");
+  MC_REQUIRE(sh > 0 && sw > 0, "Stride dimensions cannot be zero.");
+  MC_REQUIRE(ph >= 0 && pw >= 0 && ((ph == 0 && pw == 0) || (ph < kh && pw < kw)),
+             "pad must be smaller than the kernel");
+  int ho = static_cast<int>(std::ceil(static_cast<float>(H + 2 * ph - kh) / sh)) + 1;
+  int wo = static_cast<int>(std::ceil(static_cast<float>(W + 2 * pw - kw) / sw)) + 1;
+  if (ph || pw) {
+    // The last window must start strictly inside the image, not in the padding.
+    if ((ho - 1) * sh >= H + ph) --ho;
+    if ((wo - 1) * sw >= W + pw) --wo;
+  }
+  MC_REQUIRE(ho > 0 && wo > 0, "mcPoolingOutputShape: empty output");
+  if (Ho) *Ho = ho;
+  if (Wo) *Wo = wo;
+  return 0;
+}
+
+int mcPooling(int method, const float* bottom, float* top, int planes, int H, int W, int kh,
+              int kw, int sh, int sw, int ph, int pw, void* stream) {
+  MC_REQUIRE(bottom && top, "mcPooling: null argument");
+  MC_REQUIRE(method == MC_POOL_MAX || method == MC_POOL_AVE, "Unknown pooling method.");
+  MC_REQUIRE(planes >= 0 && H > 0 && W > 0, "mcPooling: bad extents");
+  int Ho, Wo;
+  if (mcPoolingOutputShape(H, W, kh, kw, sh, sw, ph, pw, &Ho, &Wo)) return -1;
+  if (planes == 0) return 0;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (Ho == 1 && Wo == 1 && kh >= H && kw >= W && ph == 0 && pw == 0) {
+    const int blocks = ceil_div(planes, 4);
+    if (method == MC_POOL_MAX)
+      global_pool_kernel<MC_POOL_MAX><<<blocks, 256, 0, st>>>(bottom, top, planes, H * W);
+    else
+      global_pool_kernel<MC_POOL_AVE><<<blocks, 256, 0, st>>>(bottom, top, planes, H * W);
+    MC_LAUNCH_CHECK();
+    return 0;
+  }
+  PoolArgs a;
+  a.x = bottom;
+  a.y = top;
+  a.total = (long)planes * Ho * Wo;
+  a.H = H;
+  a.W = W;
+  a.Ho = Ho;
+  a.Wo = Wo;
+  a.kh = kh;
+  a.kw = kw;
+  a.sh = sh;
+  a.sw = sw;
+  a.ph = ph;
+  a.pw = pw;
+  const int blocks = ew_blocks(a.total, 256);
+  if (method == MC_POOL_MAX) pool_kernel<MC_POOL_MAX><<<blocks, 256, 0, st>>>(a);
+  else pool_kernel<MC_POOL_AVE><<<blocks, 256, 0, st>>>(a);
+  MC_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // extern "C"

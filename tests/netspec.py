@@ -1,0 +1,243 @@
+"""Test-side network descriptions.
+
+A spec is a list of layer dicts:
+    {"name": ..., "type": ..., "bottom": [...], "top": [...],
+     "<x>_param": {...},            # rendered verbatim into the prototxt
+     "blobs": [np.ndarray, ...]}     # parameter values, in the layer's blob order
+
+From one spec this module produces (1) the prototxt text fed to the library
+through its C ABI, (2) the weights to inject through CaffeNetListParam, and
+(3) the expected result, by walking the same layers with the CPU oracle in the
+reference's execution order (reference src/net.cpp:212-233: layers in file
+order, in-place tops overwrite their bottoms).
+
+Test infrastructure only; nothing here is imported by the product package.
+"""
+import numpy as np
+
+import oracle
+
+
+class Enum(str):
+    """A prototxt enum identifier (rendered without quotes)."""
+
+
+def _render_value(v):
+    if isinstance(v, Enum):
+        return str(v)
+    if isinstance(v, bool):
+        return "true" if v else "false"
+    if isinstance(v, str):
+        return '"%s"' % v
+    if isinstance(v, float):
+        return repr(float(v))
+    return str(v)
+
+
+def _render_fields(d, indent):
+    pad = " " * indent
+    out = []
+    for k, v in d.items():
+        vals = v if isinstance(v, (list, tuple)) else [v]
+        for item in vals:
+            if isinstance(item, dict):
+                out.append("%s%s {" % (pad, k))
+                out.extend(_render_fields(item, indent + 2))
+                out.append("%s}" % pad)
+            else:
+                out.append("%s%s: %s" % (pad, k, _render_value(item)))
+    return out
+
+
+def to_prototxt(spec, name="net"):
+    lines = ['name: "%s"' % name]
+    for layer in spec:
+        lines.append("layer {")
+        fields = {k: v for k, v in layer.items() if k != "blobs"}
+        lines.extend(_render_fields(fields, 2))
+        lines.append("}")
+    return "\n".join(lines) + "\n"
+
+
+def input_layer(tops_shapes, name="input"):
+    tops = list(tops_shapes.keys())
+    return {"name": name, "type": "Input", "top": tops,
+            "input_param": {"shape": [{"dim": list(s)} for s in tops_shapes.values()]}}
+
+
+def load_weights(net, spec):
+    """Write every layer's blobs into the net's parameter blobs (in net order)."""
+    params = net.param_list
+    i = 0
+    for layer in spec:
+        for arr in layer.get("blobs", []):
+            name, blob = params[i]
+            assert name.startswith(layer["name"]), (name, layer["name"])
+            assert list(blob.shape) == list(arr.shape), (name, blob.shape, arr.shape)
+            if arr.size:
+                blob.data[...] = arr
+            i += 1
+    assert i == len(params), "spec lists %d blobs, net has %d" % (i, len(params))
+
+
+# --------------------------------------------------------------------------
+# oracle execution
+# --------------------------------------------------------------------------
+
+def _pair(p, rep, h, w, default):
+    if h in p or w in p:
+        return int(p.get(h, default)), int(p.get(w, default))
+    v = p.get(rep, default)
+    if isinstance(v, (list, tuple)):
+        return (int(v[0]), int(v[0])) if len(v) == 1 else (int(v[0]), int(v[1]))
+    return int(v), int(v)
+
+
+def _conv(layer, x, transposed):
+    p = layer["convolution_param"]
+    k = _pair(p, "kernel_size", "kernel_h", "kernel_w", 0)
+    s = _pair(p, "stride", "stride_h", "stride_w", 1)
+    pad = _pair(p, "pad", "pad_h", "pad_w", 0)
+    d = _pair(p, "dilation", "_", "_", 1)
+    g = oracle.conv_geom(x.shape[1], x.shape[2], x.shape[3], p["num_output"], k, s, pad, d,
+                         p.get("group", 1), transposed)
+    blobs = layer["blobs"]
+    bias = blobs[1] if p.get("bias_term", True) else None
+    return oracle.conv_forward(g, x, blobs[0], bias)
+
+
+def _canon(axis, ndim):
+    return axis + ndim if axis < 0 else axis
+
+
+def run_layer(layer, bottoms):
+    """Returns the list of top arrays of one layer."""
+    t = layer["type"]
+    x = bottoms[0] if bottoms else None
+    if t == "Convolution":
+        return [_conv(layer, x, False)]
+    if t == "Deconvolution":
+        return [_conv(layer, x, True)]
+    if t == "InnerProduct":
+        p = layer["inner_product_param"]
+        axis = _canon(p.get("axis", 1), x.ndim)
+        x2 = x.reshape(int(np.prod(x.shape[:axis])), -1)
+        b = layer["blobs"]
+        y = oracle.inner_product(x2, b[0], b[1] if p.get("bias_term", True) else None,
+                                 p.get("transpose", False))
+        return [y.reshape(tuple(x.shape[:axis]) + (p["num_output"],))]
+    if t == "BatchNorm":
+        p = layer.get("batch_norm_param", {})
+        b = layer["blobs"]
+        return [oracle.batch_norm(x, b[0], b[1], b[2], p.get("use_global_stats", True),
+                                  p.get("eps", 1e-5))]
+    if t == "Scale":
+        p = layer.get("scale_param", {})
+        b = layer["blobs"]
+        axis = _canon(p.get("axis", 1), x.ndim)
+        return [oracle.scale(x, b[0], b[1] if p.get("bias_term", False) else None, axis)]
+    if t == "Bias":
+        p = layer.get("bias_param", {})
+        return [oracle.bias(x, layer["blobs"][0], _canon(p.get("axis", 1), x.ndim))]
+    if t == "ReLU":
+        slope = layer.get("relu_param", {}).get("negative_slope", 0.0)
+        return [oracle.relu(x, slope)]
+    if t == "TanH":
+        return [oracle.tanh(x)]
+    if t == "Sigmoid":
+        return [oracle.sigmoid(x)]
+    if t == "Pooling":
+        p = layer["pooling_param"]
+        g = p.get("global_pooling", False)
+        k = (0, 0) if g else _pair(p, "kernel_size", "kernel_h", "kernel_w", 0)
+        return [oracle.pooling(x, str(p.get("pool", "MAX")), k,
+                               _pair(p, "stride", "stride_h", "stride_w", 1),
+                               _pair(p, "pad", "pad_h", "pad_w", 0), g)]
+    if t == "Eltwise":
+        p = layer.get("eltwise_param", {})
+        return [oracle.eltwise(bottoms, str(p.get("operation", "SUM")), p.get("coeff"))]
+    if t == "Softmax":
+        return [oracle.softmax(x, layer.get("softmax_param", {}).get("axis", 1))]
+    if t == "Concat":
+        axis = _canon(layer.get("concat_param", {}).get("axis", 1), x.ndim)
+        return [np.ascontiguousarray(np.concatenate(bottoms, axis=axis))]
+    if t == "Slice":
+        p = layer.get("slice_param", {})
+        axis = _canon(p.get("axis", 1), x.ndim)
+        pts = p.get("slice_point")
+        ntop = len(layer["top"])
+        if pts is None:
+            parts = np.split(x, ntop, axis=axis)
+        else:
+            parts = np.split(x, list(pts) if isinstance(pts, (list, tuple)) else [pts], axis=axis)
+        return [np.ascontiguousarray(a) for a in parts]
+    if t == "Flatten":
+        p = layer.get("flatten_param", {})
+        a0, a1 = _canon(p.get("axis", 1), x.ndim), _canon(p.get("end_axis", -1), x.ndim)
+        return [x.reshape(x.shape[:a0] + (-1,) + x.shape[a1 + 1:])]
+    if t == "Reshape":
+        p = layer["reshape_param"]
+        dims = list(p["shape"]["dim"])
+        axis = p.get("axis", 0)
+        start = axis if axis >= 0 else x.ndim + axis + 1
+        na = p.get("num_axes", -1)
+        end = x.ndim if na == -1 else start + na
+        new = [x.shape[start + i] if d == 0 else d for i, d in enumerate(dims)]
+        shape = list(x.shape[:start]) + new + list(x.shape[end:])
+        return [x.reshape(shape)]
+    if t == "Permute":
+        order = list(layer["permute_param"]["order"])
+        order += [i for i in range(x.ndim) if i not in order]
+        return [np.ascontiguousarray(np.transpose(x, order))]
+    if t == "Split":
+        return [x.copy() for _ in layer["top"]]
+    if t == "Normalize":
+        p = layer.get("norm_param", {})
+        return [oracle.normalize(x, layer["blobs"][0], p.get("across_spatial", True),
+                                 p.get("channel_shared", True), p.get("eps", 1e-10))]
+    if t == "PriorBox":
+        return [oracle.prior_box(layer["prior_box_param"], x.shape, bottoms[1].shape)]
+    if t == "Proposal":
+        return oracle.proposal(layer.get("proposal_param", {}), bottoms[0], bottoms[1], bottoms[2],
+                               len(layer["top"]))
+    if t == "DetectionOutput":
+        return [oracle.detection_output(layer["detection_output_param"], bottoms[0], bottoms[1],
+                                        bottoms[2])]
+    raise NotImplementedError(t)
+
+
+def oracle_forward(spec, inputs, keep=None):
+    """Run the spec on the CPU oracle.  inputs: dict blob name -> array.
+    Returns dict blob name -> final array (in-place layers overwrite).
+    keep: optional set of blob names to retain (all are kept when None)."""
+    blobs = {k: np.ascontiguousarray(v, dtype=np.float32) for k, v in inputs.items()}
+    for layer in spec:
+        if layer["type"] == "Input":
+            for name in layer["top"]:
+                assert name in blobs, "missing input %s" % name
+            continue
+        bottoms = [blobs[b] for b in layer.get("bottom", [])]
+        tops = run_layer(layer, bottoms)
+        for name, arr in zip(layer["top"], tops):
+            blobs[name] = np.ascontiguousarray(arr, dtype=np.float32)
+    if keep is not None:
+        blobs = {k: v for k, v in blobs.items() if k in keep}
+    return blobs
+
+
+def rel_err(got, want, floor=1e-2):
+    """max |got - want| / max(|want|, tau) with tau = floor * max|want|.
+
+    Plain elementwise relative error is ill-posed at ReLU zeros and wherever a
+    long fp32 sum cancels: two correct fp32 evaluations of the same K=576 dot
+    product that merely add in a different order (OpenBLAS vs. plain loops, see
+    tests/test_oracle.py::test_blas_order_noise) already differ by ~2e-4 of an
+    output that is 1e-3 of the blob's peak.  The floor keeps the metric about the
+    implementation rather than about summation order."""
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    if want.size == 0:
+        return 0.0
+    tau = floor * max(np.abs(want).max(), 1e-30)
+    return float((np.abs(got - want) / np.maximum(np.abs(want), tau)).max())
