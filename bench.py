@@ -1,0 +1,130 @@
+#!/usr/bin/env python3
+"""Headline benchmark: ResNet-50 v1 forward, fp32, batch 64, 3x224x224, on one MI355X.
+
+A step is one Net::Forward through the C ABI (CaffeNetForward) on a batch that
+already sits in HBM: seeded synthetic input, He-normal random weights of the
+real architecture.  Prints one JSON line with images/s, the roofline figures of
+the dominant kernel (the fp32 MFMA implicit-GEMM convolution) measured with HIP
+events on the library's stream, and the CPU baseline (the oracle's restatement
+of the reference's per-image im2col + OpenBLAS sgemm path) timed on a bounded
+sample on this box's host cores.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "mini-caffe_amd"))
+
+FP32_MFMA_PEAK_TFLOPS = 157.3
+# HBM bytes per convolution launch (mean over the 53 launches of one forward),
+# from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in
+# profiles/igemm_resnet50_b64_pmc.txt; None until measured.
+CONV_TRAFFIC_BYTES_PER_LAUNCH = None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-batch", type=int, default=8)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported "
+                 "(the forward path shards over the batch with no exchange)" % args.gpus)
+
+    import numpy as np
+    import minicaffe as mc
+    from minicaffe import craft, zoo
+    from minicaffe.base import LIB
+
+    if not mc.check_gpu_available():
+        sys.exit("bench.py: no HIP device visible")
+    mc.set_runtime_mode(1, 0)
+
+    spec, inputs = zoo.resnet50_spec(batch=args.batch, size=224, seed=0)
+    flops = zoo.conv_flops(spec, inputs)
+    net = mc.Net.from_buffers(craft.to_prototxt(spec, "ResNet-50"))
+    craft.load_weights(net, spec)
+    net.forward(**inputs)          # uploads input + weights, packs filters
+    for _ in range(max(0, args.warmup - 1)):
+        net.forward()
+
+    import torch
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        net.forward()              # ends with a stream synchronisation
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = 1e3 * elapsed / args.steps
+    prob = net.get_blob("prob").data
+    assert np.isfinite(prob).all() and abs(float(prob.sum()) - args.batch) < 1e-2 * args.batch
+
+    # Roofline of the dominant kernel: same steps again with every contraction
+    # launch bracketed by HIP events on the launch stream.
+    LIB.mcConvTimingEnable(1)
+    for _ in range(args.steps):
+        net.forward()
+    tot_ms, launches, fl = ctypes.c_double(), ctypes.c_long(), ctypes.c_double()
+    LIB.mcConvTimingCollect(ctypes.byref(tot_ms), ctypes.byref(launches), ctypes.byref(fl))
+    LIB.mcConvTimingEnable(0)
+    achieved = fl.value / (tot_ms.value * 1e-3) / 1e12 if tot_ms.value > 0 else 0.0
+    roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP32_MFMA_PEAK_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
+                "traffic": CONV_TRAFFIC_BYTES_PER_LAUNCH,
+                "kernel": "igemm_f32 (Convolution + InnerProduct, fused BN/Scale/ReLU epilogue)",
+                "launches_per_step": launches.value // max(1, args.steps),
+                "kernel_ms_per_step": round(tot_ms.value / max(1, args.steps), 3),
+                "gflop_per_step": round(fl.value / max(1, args.steps) / 1e9, 1)}
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(args.cpu_batch)
+
+    out = {"metric": "images/sec at 1 MI355X (ResNet-50 b64 fp32)",
+           "value": round(args.batch * args.steps / elapsed, 1), "unit": "images/s",
+           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "ResNet-50 v1 forward, batch %d, 3x224x224, fp32 "
+                                  "(BASELINE configs[1])" % args.batch,
+                      "conv_gflop_per_step": round(flops["conv"] / 1e9, 1),
+                      "api": "CaffeNetForward (Net::Forward(reshape=true))"},
+           "roofline": roofline, "cpu_baseline": cpu}
+    print(json.dumps(out))
+
+
+def cpu_baseline(batch):
+    """The reference algorithm (per-image im2col + sgemm, unfused BN/Scale/ReLU)
+    as restated by the oracle, sgemm from the OpenBLAS bundled with scipy."""
+    import oracle
+    from oracle import netrun
+    from minicaffe import zoo
+    blas = oracle.use_openblas(True)
+    spec, inputs = zoo.resnet50_spec(batch=batch, size=224, seed=0)
+    netrun.oracle_forward(spec, {k: v[:1] for k, v in inputs.items()}, keep={"prob"})  # warm
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        netrun.oracle_forward(spec, inputs, keep={"prob"})
+        reps += 1
+        if time.perf_counter() - t0 > 10.0 or reps >= 5:
+            break
+    dt = time.perf_counter() - t0
+    return {"value": round(batch * reps / dt, 2), "unit": "images/s",
+            "cores": oracle.openblas_threads() if blas else 1, "kind": "port",
+            "blas": os.path.basename(blas) if blas else "built-in loops",
+            "sample": "%d pass(es) of ResNet-50 forward at batch %d (same graph, same seeds)"
+                      % (reps, batch)}
+
+
+if __name__ == "__main__":
+    main()

@@ -109,6 +109,14 @@ const char* mcConvPlanKernelName(const mcConvPlan* plan, int num);
 int mcConvPlanForceConfig(mcConvPlan* plan, int config);
 
 
+/* Measurement hook (no counterpart in the reference): while enabled on the
+ * calling thread, every contraction kernel launch is bracketed by two HIP events
+ * recorded on the launch stream.  mcConvTimingCollect waits for them, returns
+ * the summed kernel time, the number of launches and their algorithmic FLOPs,
+ * and clears the list. */
+int mcConvTimingEnable(int on);
+int mcConvTimingCollect(double* total_ms, long* launches, double* flops);
+
 /* HIP stream of the calling thread's Mini-Caffe context (created on first use);
  * lets a harness record events around Net::Forward.  NULL if no device. */
 void* mcCurrentStream(void);

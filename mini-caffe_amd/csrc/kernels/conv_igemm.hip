@@ -354,6 +354,16 @@ struct mcConvPlan {
 
 namespace {
 
+// Optional per-launch timing: when enabled, every contraction launch is
+// bracketed by HIP events on the stream it runs on.
+struct TimedLaunch {
+  hipEvent_t start, stop;
+  double flops;
+  const char* name;
+};
+thread_local bool g_timing = false;
+thread_local std::vector<TimedLaunch> g_timed;
+
 // Tile choice.  With 256 CUs the tile count per CU is small for most layers, so
 // load balance (the last, partly filled round of tiles) dominates: measured on
 // ResNet-50 shapes the 64x64 tile, which runs 8 workgroups per CU, beats the
@@ -620,9 +630,44 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
     const long blocks = (long)a.MT * a.NT;
     MC_REQUIRE(blocks < (1L << 31), "mcConvForward: grid too large");
     dim3 grid(static_cast<unsigned>(blocks), g.group, 1);
+    TimedLaunch tl;
+    if (g_timing) {
+      MC_HIP(hipEventCreate(&tl.start));
+      MC_HIP(hipEventCreate(&tl.stop));
+      tl.flops = 2.0 * pixels * plan->M * g.group * s.K;
+      tl.name = cfg.name;
+      MC_HIP(hipEventRecord(tl.start, st));
+    }
     cfg.kernel<<<grid, 256, 0, st>>>(a);
     MC_LAUNCH_CHECK();
+    if (g_timing) {
+      MC_HIP(hipEventRecord(tl.stop, st));
+      g_timed.push_back(tl);
+    }
   }
+  return 0;
+}
+
+int mcConvTimingEnable(int on) {
+  g_timing = on != 0;
+  return 0;
+}
+
+int mcConvTimingCollect(double* total_ms, long* launches, double* flops) {
+  double ms = 0., fl = 0.;
+  for (auto& t : g_timed) {
+    MC_HIP(hipEventSynchronize(t.stop));
+    float e = 0.f;
+    MC_HIP(hipEventElapsedTime(&e, t.start, t.stop));
+    ms += e;
+    fl += t.flops;
+    (void)hipEventDestroy(t.start);
+    (void)hipEventDestroy(t.stop);
+  }
+  if (total_ms) *total_ms = ms;
+  if (launches) *launches = static_cast<long>(g_timed.size());
+  if (flops) *flops = fl;
+  g_timed.clear();
   return 0;
 }
 

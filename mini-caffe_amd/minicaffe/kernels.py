@@ -26,6 +26,34 @@ class Epilogue(ctypes.Structure):
                 ("activation", c_int), ("negative_slope", c_float)]
 
 
+class ChannelOp(ctypes.Structure):
+    _fields_ = [("sub", c_void_p), ("div", c_void_p), ("mul", c_void_p), ("add", c_void_p),
+                ("activation", c_int), ("negative_slope", c_float)]
+
+
+c_long = ctypes.c_long
+LIB.mcChannelTransform.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int,
+                                   ctypes.POINTER(ChannelOp), c_void_p]
+LIB.mcBatchNormStored.argtypes = [c_void_p, c_void_p, c_void_p, c_float, c_int, c_void_p, c_void_p,
+                                  c_void_p]
+LIB.mcBatchNormBatchStats.argtypes = [c_void_p, c_int, c_int, c_int, c_float, c_void_p, c_void_p,
+                                      c_void_p]
+LIB.mcFoldChannelOps.argtypes = [c_void_p, ctypes.POINTER(ChannelOp), c_int, c_int, c_void_p,
+                                 c_void_p, c_void_p]
+LIB.mcPoolingOutputShape.argtypes = [c_int] * 8 + [ctypes.POINTER(c_int), ctypes.POINTER(c_int)]
+LIB.mcPooling.argtypes = [c_int, c_void_p, c_void_p] + [c_int] * 9 + [c_void_p]
+LIB.mcEltwise.argtypes = [c_int, c_int, ctypes.POINTER(c_void_p), ctypes.POINTER(c_float), c_long,
+                          c_void_p, c_int, c_float, c_void_p]
+LIB.mcSoftmax.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]
+LIB.mcCopy2D.argtypes = [c_void_p, c_long, c_void_p, c_long, c_long, c_long, c_void_p]
+LIB.mcPermute.argtypes = [c_void_p, c_void_p, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int),
+                          c_void_p]
+LIB.mcFill.argtypes = [c_void_p, c_long, c_float, c_void_p]
+LIB.mcNormalize.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p,
+                            c_void_p]
+LIB.mcConvTimingCollect.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(c_long),
+                                    ctypes.POINTER(ctypes.c_double)]
+
 LIB.mcConvPlanCreate.argtypes = [ctypes.POINTER(ConvGeom), ctypes.POINTER(c_void_p)]
 LIB.mcConvPlanDestroy.argtypes = [c_void_p]
 LIB.mcConvPlanOutputShape.argtypes = [c_void_p, ctypes.POINTER(c_int), ctypes.POINTER(c_int)]

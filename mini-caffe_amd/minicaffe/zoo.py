@@ -1,13 +1,12 @@
-"""Builders for the benchmark configurations as netspec layer lists.
+"""Builders for the benchmark configurations as minicaffe.craft layer lists.
 
 Weights are drawn here from seeded numpy generators with the distributions the
 configurations name; mini-caffe's own fillers are all constant
 (reference src/filler.hpp:51-71), so weights are always injected.
-Test infrastructure only.
 """
 import numpy as np
 
-from netspec import Enum, input_layer
+from .craft import Enum, input_layer
 
 
 def _rng(seed, *names):
@@ -140,6 +139,15 @@ def resnet50_spec(batch=64, size=224, seed=0, num_classes=1000, stages=(3, 4, 6,
     return spec, {"data": x}
 
 
+def _pool_out(n, k, s, pad):
+    """Caffe's ceil-mode pooled extent with the last-window clip."""
+    import math
+    o = int(math.ceil(float(n + 2 * pad - k) / s)) + 1
+    if pad and (o - 1) * s >= n + pad:
+        o -= 1
+    return o
+
+
 def conv_flops(spec, inputs):
     """Algorithmic FLOPs of the Convolution / Deconvolution / InnerProduct layers of a
     spec: 2*N*Cout*Ho*Wo*(Cin/g)*kh*kw (deconv: 2*N*Cin*Hin*Win*(Cout/g)*kh*kw), 2*M*N*K."""
@@ -171,14 +179,13 @@ def conv_flops(spec, inputs):
             total["fc"] += 2.0 * m * n_out * kk
             shapes[layer["top"][0]] = (m, n_out)
         elif t == "Pooling":
-            import oracle
             p = layer["pooling_param"]
             n, c, h, w = b[0]
             if p.get("global_pooling", False):
                 ho = wo = 1
             else:
                 k, s, pad = p["kernel_size"], p.get("stride", 1), p.get("pad", 0)
-                ho, wo = oracle.pooling_output_shape(h, w, (k, k), (s, s), (pad, pad))
+                ho, wo = _pool_out(h, k, s, pad), _pool_out(w, k, s, pad)
             shapes[layer["top"][0]] = (n, c, ho, wo)
         elif t == "Reshape":
             dims = list(layer["reshape_param"]["shape"]["dim"])

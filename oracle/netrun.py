@@ -1,88 +1,12 @@
-"""Test-side network descriptions.
+"""Runs a net description (minicaffe.craft spec) on the CPU oracle.
 
-A spec is a list of layer dicts:
-    {"name": ..., "type": ..., "bottom": [...], "top": [...],
-     "<x>_param": {...},            # rendered verbatim into the prototxt
-     "blobs": [np.ndarray, ...]}     # parameter values, in the layer's blob order
-
-From one spec this module produces (1) the prototxt text fed to the library
-through its C ABI, (2) the weights to inject through CaffeNetListParam, and
-(3) the expected result, by walking the same layers with the CPU oracle in the
-reference's execution order (reference src/net.cpp:212-233: layers in file
-order, in-place tops overwrite their bottoms).
-
-Test infrastructure only; nothing here is imported by the product package.
+TEST INFRASTRUCTURE ONLY.  Walks the layers in file order as the reference's
+Net::Forward does (reference src/net.cpp:212-233: in-place tops overwrite their
+bottoms) and evaluates each with the restated CPU arithmetic of oracle/.
 """
 import numpy as np
 
 import oracle
-
-
-class Enum(str):
-    """A prototxt enum identifier (rendered without quotes)."""
-
-
-def _render_value(v):
-    if isinstance(v, Enum):
-        return str(v)
-    if isinstance(v, bool):
-        return "true" if v else "false"
-    if isinstance(v, str):
-        return '"%s"' % v
-    if isinstance(v, float):
-        return repr(float(v))
-    return str(v)
-
-
-def _render_fields(d, indent):
-    pad = " " * indent
-    out = []
-    for k, v in d.items():
-        vals = v if isinstance(v, (list, tuple)) else [v]
-        for item in vals:
-            if isinstance(item, dict):
-                out.append("%s%s {" % (pad, k))
-                out.extend(_render_fields(item, indent + 2))
-                out.append("%s}" % pad)
-            else:
-                out.append("%s%s: %s" % (pad, k, _render_value(item)))
-    return out
-
-
-def to_prototxt(spec, name="net"):
-    lines = ['name: "%s"' % name]
-    for layer in spec:
-        lines.append("layer {")
-        fields = {k: v for k, v in layer.items() if k != "blobs"}
-        lines.extend(_render_fields(fields, 2))
-        lines.append("}")
-    return "\n".join(lines) + "\n"
-
-
-def input_layer(tops_shapes, name="input"):
-    tops = list(tops_shapes.keys())
-    return {"name": name, "type": "Input", "top": tops,
-            "input_param": {"shape": [{"dim": list(s)} for s in tops_shapes.values()]}}
-
-
-def load_weights(net, spec):
-    """Write every layer's blobs into the net's parameter blobs (in net order)."""
-    params = net.param_list
-    i = 0
-    for layer in spec:
-        for arr in layer.get("blobs", []):
-            name, blob = params[i]
-            assert name.startswith(layer["name"]), (name, layer["name"])
-            assert list(blob.shape) == list(arr.shape), (name, blob.shape, arr.shape)
-            if arr.size:
-                blob.data[...] = arr
-            i += 1
-    assert i == len(params), "spec lists %d blobs, net has %d" % (i, len(params))
-
-
-# --------------------------------------------------------------------------
-# oracle execution
-# --------------------------------------------------------------------------
 
 def _pair(p, rep, h, w, default):
     if h in p or w in p:

@@ -1,0 +1,245 @@
+"""Host-side behaviour of libcaffe.so through its C ABI; no GPU needed.
+
+Covers what the reference's tests/run_net.c asserts on a CPU box (creation,
+blob shapes, listing, the -1 + CaffeGetLastError error convention) plus the
+prototxt / caffemodel reader that replaces protobuf.
+"""
+import ctypes
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+
+import minicaffe as mc
+from minicaffe import craft, zoo
+from minicaffe.base import LIB
+
+import wire
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+REF = "/root/reference"
+needs_ref = pytest.mark.skipif(not os.path.isdir(REF), reason="reference checkout not present")
+
+
+def declared_functions(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b((?:Caffe|mc)[A-Z]\w*)\s*\(", text)))
+
+
+@pytest.mark.parametrize("header", ["caffe/c_api.h", "mchip/kernels.h"])
+def test_library_exports_every_declared_symbol(header):
+    names = declared_functions(header)
+    assert len(names) >= 20
+    missing = [n for n in names if not hasattr(LIB, n)]
+    assert not missing, missing
+
+
+def test_c_api_has_the_reference_entry_points():
+    # the 25 functions of the reference's include/caffe/c_api.h:26-162
+    want = """CaffeBlobNum CaffeBlobChannels CaffeBlobHeight CaffeBlobWidth CaffeBlobData
+    CaffeBlobCount CaffeBlobReshape CaffeBlobShape CaffeNetCreate CaffeNetCreateFromBuffer
+    CaffeNetDestroy CaffeNetMarkOutput CaffeNetForward CaffeNetGetBlob CaffeNetListBlob
+    CaffeNetListParam CaffeProfilerEnable CaffeProfilerDisable CaffeProfilerScopeStart
+    CaffeProfilerScopeEnd CaffeProfilerDump CaffeGPUAvailable CaffeSetMode CaffeGetLastError
+    CaffeMemoryPoolClear""".split()
+    assert len(want) == 25
+    assert set(want) <= set(declared_functions("caffe/c_api.h"))
+
+
+TRICKY = """
+# comment line
+name: 'tricky'   # trailing comment
+input: "data"
+input_dim: 2
+input_dim: 3
+input_dim: 12
+input_dim: 10
+layer {
+  name: "conv1" type: "Convolution" bottom: "data" top: "conv1"
+  param { lr_mult: 1.0 decay_mult: 1.0 }
+  param { lr_mult: 2.0 decay_mult: 0 }
+  convolution_param: {
+    num_output: 8; kernel_h: 3, kernel_w: 2
+    stride_h: 2 stride_w: 1 pad_h: 1 pad_w: 0
+    weight_filler { type: "xavier" } bias_filler { type: "constant" value: 0.25 }
+  }
+}
+layer { name: "pool" type: "Pooling" bottom: "conv1" top: "pool"
+        pooling_param { pool: AVE kernel_size: 2 stride: 2 } include { phase: TEST } }
+layer { name: "relu" type: "ReLU" bottom: "pool" top: "pool" relu_param { negative_slope: 1e-1 } }
+layer { name: "ip" type: "InnerProduct" bottom: "pool" top: "ip"
+        inner_product_param { num_output: 5 bias_term: false } }
+layer { name: "prob" type: "Softmax" bottom: "ip" top: "prob" }
+"""
+
+
+def test_prototxt_reader_and_shape_inference():
+    net = mc.Net.from_buffers(TRICKY)
+    shapes = {k: v.shape for k, v in net.blobs.items()}
+    # conv: H (12+2-3)/2+1 = 6, W (10-2)/1+1 = 9; pool (ceil): 3 x 5
+    assert shapes == {"data": [2, 3, 12, 10], "conv1": [2, 8, 6, 9], "pool": [2, 8, 3, 5],
+                      "ip": [2, 5], "prob": [2, 5]}
+    params = net.param_list
+    assert [n for n, _ in params] == ["conv1_0", "conv1_1", "ip_0"]
+    assert params[0][1].shape == [8, 3, 3, 2] and params[2][1].shape == [5, 120]
+    # every filler is a constant fill; "xavier" without value gives zeros
+    assert np.all(params[0][1].data == 0) and np.all(params[1][1].data == 0.25)
+    blob = net.get_blob("data")
+    assert (LIB.CaffeBlobNum(blob.handle), LIB.CaffeBlobChannels(blob.handle),
+            LIB.CaffeBlobHeight(blob.handle), LIB.CaffeBlobWidth(blob.handle),
+            LIB.CaffeBlobCount(blob.handle)) == (2, 3, 12, 10, 720)
+
+
+def err(fn):
+    with pytest.raises(mc.MiniCaffeError) as e:
+        fn()
+    return str(e.value)
+
+
+def test_error_convention():
+    assert "Unknown layer type: Nope" in err(lambda: mc.Net.from_buffers(
+        'layer { name: "d" type: "Input" top: "d" input_param { shape { dim: 1 } } }'
+        'layer { name: "x" type: "Nope" bottom: "d" top: "x" }'))
+    # nonexistent files must give -1 and a message (reference tests/run_net.c:73-74)
+    assert "File not found" in err(lambda: mc.Net("/nonexistent.prototxt", "/nonexistent.caffemodel"))
+    assert "takes 1 bottom blob" in err(lambda: mc.Net.from_buffers(
+        'layer { name: "r" type: "ReLU" top: "r" }'))
+    two = ('layer { name: "d" type: "Input" top: "d" input_param { shape { dim: 1 dim: 2 } } }'
+           'layer { name: "a" type: "ReLU" bottom: "d" top: "x" }'
+           'layer { name: "b" type: "ReLU" bottom: "d" top: "x" }')
+    assert "produced by multiple sources" in err(lambda: mc.Net.from_buffers(two))
+    assert "Unknown bottom blob 'nope'" in err(lambda: mc.Net.from_buffers(
+        'layer { name: "d" type: "Input" top: "d" input_param { shape { dim: 1 } } }'
+        'layer { name: "a" type: "ReLU" bottom: "nope" top: "x" }'))
+    assert "parse error at 1:" in err(lambda: mc.Net.from_buffers('layer { name "x" }'))
+    assert "missing closing brace" in err(lambda: mc.Net.from_buffers('layer { name: "x" '))
+    net = mc.Net.from_buffers(TRICKY)
+    assert "is not availiable" in err(lambda: net.mark_output("nope"))
+    assert "Unknown blob name" in err(lambda: net.get_blob("nope"))
+    assert "mode must be 0" in err(lambda: mc.set_runtime_mode(7, 0))
+
+
+def test_forward_without_gpu_mode_fails_loudly():
+    mc.set_runtime_mode(0, -1)
+    net = mc.Net.from_buffers(TRICKY)
+    msg = err(lambda: net.forward())
+    assert "HIP device path only" in msg
+
+
+def test_caffemodel_reader_and_weight_copy():
+    rng = np.random.default_rng(0)
+    w = rng.standard_normal((8, 3, 3, 2)).astype(np.float32)
+    b = rng.standard_normal(8).astype(np.float32)
+    ipw = rng.standard_normal((5, 120)).astype(np.float32)
+    for kw in ({}, {"packed": False}, {"as_double": True}):
+        model = wire.net("m", [wire.layer("conv1", "Convolution", [w, b], **kw),
+                               wire.layer("not_in_net", "ReLU", []),
+                               wire.layer("ip", "InnerProduct", [ipw], **kw)])
+        net = mc.Net.from_buffers(TRICKY, model)
+        params = dict(net.param_list)
+        assert np.array_equal(params["conv1_0"].data, w)
+        assert np.array_equal(params["conv1_1"].data, b)
+        assert np.array_equal(params["ip_0"].data, ipw)
+    # legacy 4-D blob dims: bias (1,1,1,8) and ip weight (1,1,5,120) match N-d targets
+    model = wire.net("m", [wire.layer("conv1", "Convolution", [w, b], legacy=True),
+                           wire.layer("ip", "InnerProduct", [ipw], legacy=True)])
+    net = mc.Net.from_buffers(TRICKY, model)
+    assert np.array_equal(dict(net.param_list)["ip_0"].data, ipw)
+    # shape mismatch is fatal and names both shapes
+    bad = wire.net("m", [wire.layer("conv1", "Convolution", [w[:, :, :2], b])])
+    msg = err(lambda: mc.Net.from_buffers(TRICKY, bad))
+    assert "shape mismatch" in msg and "8 3 2 2" in msg and "8 3 3 2" in msg
+    bad = wire.net("m", [wire.layer("conv1", "Convolution", [w])])
+    assert "Incompatible number of blobs" in err(lambda: mc.Net.from_buffers(TRICKY, bad))
+    assert "truncated" in err(lambda: mc.Net.from_buffers(TRICKY, model[:-3]))
+
+
+def test_create_from_files(tmp_path):
+    w = np.arange(8 * 3 * 3 * 2, dtype=np.float32).reshape(8, 3, 3, 2)
+    b = np.ones(8, np.float32)
+    (tmp_path / "n.prototxt").write_text(TRICKY)
+    (tmp_path / "n.caffemodel").write_bytes(
+        wire.net("m", [wire.layer("conv1", "Convolution", [w, b])]))
+    net = mc.Net(str(tmp_path / "n.prototxt"), str(tmp_path / "n.caffemodel"))
+    assert np.array_equal(dict(net.param_list)["conv1_0"].data, w)
+
+
+def test_layer_argument_checks():
+    base = 'layer { name: "d" type: "Input" top: "d" input_param { shape { dim: 1 dim: 4 dim: 6 dim: 6 } } }'
+
+    def conv(body):
+        return base + 'layer { name: "c" type: "Convolution" bottom: "d" top: "c" convolution_param { %s } }' % body
+    assert "kernel_size must be specified" in err(lambda: mc.Net.from_buffers(conv("num_output: 2")))
+    assert "multiples of group" in err(lambda: mc.Net.from_buffers(conv("num_output: 3 kernel_size: 1 group: 2")))
+    assert "not both" in err(lambda: mc.Net.from_buffers(conv("num_output: 2 kernel_size: 3 kernel_h: 3")))
+    assert "Stride dimensions must be nonzero" in err(lambda: mc.Net.from_buffers(conv("num_output: 2 kernel_size: 3 stride: 0")))
+    pool = base + 'layer { name: "p" type: "Pooling" bottom: "d" top: "p" pooling_param { %s } }'
+    assert "Filter size cannot specified" in err(lambda: mc.Net.from_buffers(pool % "global_pooling: true kernel_size: 2"))
+    assert "Unknown pooling method" in err(lambda: mc.Net.from_buffers(pool % "pool: STOCHASTIC kernel_size: 2"))
+    elt = base + ('layer { name: "e" type: "Eltwise" bottom: "d" bottom: "d" top: "e" '
+                  'eltwise_param { operation: PROD coeff: 1 coeff: 2 } }')
+    assert "only takes coefficients for summation" in err(lambda: mc.Net.from_buffers(elt))
+    assert "takes at least 2 bottom" in err(lambda: mc.Net.from_buffers(
+        base + 'layer { name: "e" type: "Eltwise" bottom: "d" top: "e" }'))
+    assert "Unknown filler name" in err(lambda: mc.Net.from_buffers(
+        conv('num_output: 2 kernel_size: 1 weight_filler { type: "fancy" }')))
+    resh = base + 'layer { name: "r" type: "Reshape" bottom: "d" top: "r" reshape_param { shape { dim: 0 dim: -1 dim: 5 } } }'
+    assert "must be divisible" in err(lambda: mc.Net.from_buffers(resh))
+
+
+def test_resnet50_graph_builds_with_reference_shapes():
+    spec, inputs = zoo.resnet50_spec(batch=2, size=224)
+    assert len(spec) == 229   # Input, 53 conv/BN/Scale, 49 ReLU, 16 Eltwise, 2 pool, IP, softmax
+    net = mc.Net.from_buffers(craft.to_prototxt(spec))
+    shapes = {k: v.shape for k, v in net.blobs.items()}
+    assert shapes["conv1"] == [2, 64, 112, 112] and shapes["pool1"] == [2, 64, 56, 56]
+    assert shapes["res3a"] == [2, 512, 28, 28] and shapes["res5c"] == [2, 2048, 7, 7]
+    assert shapes["pool5"] == [2, 2048, 1, 1] and shapes["prob"] == [2, 1000]
+    # 7.712 GFLOP per image in the convolutions
+    assert abs(zoo.conv_flops(spec, inputs)["conv"] / 2 / 1e9 - 7.712) < 0.01
+
+
+def test_profiler_dump(tmp_path):
+    mc.Profiler.enable()
+    mc.Profiler.open_scope("outer")
+    mc.Profiler.open_scope("inner")
+    mc.Profiler.close_scope()
+    mc.Profiler.close_scope()
+    mc.Profiler.disable()
+    fn = str(tmp_path / "profile.json")
+    mc.Profiler.dump(fn)
+    events = json.load(open(fn))["traceEvents"]
+    names = [e["name"] for e in events if e["ph"] == "B"]
+    assert "outer" in names and "outer:inner" in names
+    assert "not running" in err(mc.Profiler.disable)
+
+
+def test_memory_pool_clear_and_gpu_flag():
+    mc.memory_pool_clear()
+    assert LIB.CaffeGPUAvailable() in (0, 1)
+
+
+@needs_ref
+@pytest.mark.parametrize("name", ["1_F", "2_LE1", "2_N2", "2_RM2"])
+def test_reads_the_reference_example_models(name):
+    """Real prototxt + binary caffemodel pairs shipped with the reference's
+    deeplandmark example (example/models/deeplandmark): only files in the tree
+    with trained weights.  They must load; weights must be finite and non-trivial."""
+    d = os.path.join(REF, "example", "models", "deeplandmark")
+    net = mc.Net(os.path.join(d, name + ".prototxt"), os.path.join(d, name + ".caffemodel"))
+    params = net.param_list
+    assert len(params) >= 6
+    for _, blob in params:
+        a = blob.data
+        assert np.isfinite(a).all()
+    assert any(np.abs(b.data).max() > 1e-3 for _, b in params)
+
+
+@needs_ref
+def test_reads_the_reference_wgan_prototxt():
+    net = mc.Net.from_buffers(open(os.path.join(REF, "example", "models", "wgan", "g.prototxt")).read())
+    shapes = {k: v.shape for k, v in net.blobs.items()}
+    assert list(shapes.values())[-1][1:] == [3, 64, 64]

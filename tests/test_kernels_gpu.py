@@ -1,0 +1,238 @@
+"""Kernel-level parity on the MI355X: every entry point of include/mchip/kernels.h is
+called through the C ABI with device pointers (torch only owns the memory) and
+compared with the CPU oracle on the same seeded inputs.
+
+Tolerances: the dense contraction differs from the oracle only by fp32 summation
+order (see netrun.rel_err): 1e-4.  Pure data movement (pooling MAX, copy,
+permute, concat) must be bit-exact.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+import oracle
+from oracle import netrun
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def K(gpu_mode):
+    from minicaffe import kernels
+    oracle.use_openblas(False)
+    return kernels
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def fptr(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+CONV_CASES = [
+    # cin, h, w, cout, k, s, p, d, g, transposed, batch
+    (64, 56, 56, 64, 3, 1, 1, 1, 1, False, 1),      # config 1
+    (3, 33, 31, 64, 7, 2, 3, 1, 1, False, 2),       # ResNet conv1 geometry, odd extents
+    (64, 14, 14, 256, 1, 1, 0, 1, 1, False, 3),     # 1x1
+    (256, 14, 14, 128, 1, 2, 0, 1, 1, False, 2),    # strided 1x1
+    (32, 19, 19, 64, 3, 1, 6, 6, 1, False, 2),      # dilated (SSD fc6 geometry)
+    (32, 20, 20, 64, 3, 1, 1, 1, 4, False, 2),      # groups
+    (8, 9, 11, 8, (3, 2), (2, 1), (1, 0), 1, 8, False, 2),   # depthwise, non-square
+    (16, 5, 5, 24, 3, 1, 1, 1, 1, False, 2),        # odd M (SSD head)
+    (100, 1, 1, 1000, 1, 1, 0, 1, 1, False, 7),     # inner-product shape
+    (40, 10, 10, 130, 3, 2, 1, 1, 1, False, 2),     # M and K not multiples of the tile
+    (1024, 4, 4, 512, 4, 2, 1, 1, 1, True, 2),      # DCGAN deconv 4 -> 8
+    (16, 5, 7, 3, 4, 2, 1, 1, 1, True, 3),          # deconv to 3 channels
+    (8, 6, 6, 8, 3, 1, 1, 1, 1, True, 2),           # stride-1 deconv
+    (8, 6, 6, 12, 2, 3, 0, 1, 1, True, 2),          # kernel < stride: tapless output classes
+    (8, 6, 6, 12, 5, 2, 2, 1, 2, True, 2),          # grouped deconv
+    (8, 6, 6, 12, 3, 2, 1, 2, 1, True, 2),          # dilated deconv
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+@pytest.mark.parametrize("cfg", [-1, 0, 3, 5])
+def test_conv_forward(K, case, cfg):
+    cin, h, w, cout, k, s, p, d, g, tr, n = case
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((n, cin, h, w)).astype(np.float32)
+    kk = (k, k) if isinstance(k, int) else k
+    wshape = (cin, cout // g) + kk if tr else (cout, cin // g) + kk
+    wt = (rng.standard_normal(wshape) * 0.1).astype(np.float32)
+    b = rng.standard_normal(cout).astype(np.float32)
+    want = oracle.conv_forward(oracle.conv_geom(cin, h, w, cout, k, s, p, d, g, tr), x, wt, b)
+    plan = K.ConvPlan(K.conv_geom(cin, h, w, cout, k, s, p, d, g, tr))
+    plan.force_config(cfg)
+    assert plan.output_shape() == want.shape[2:]
+    xd, wd, bd = dev(x), dev(wt), dev(b)
+    yd = torch.full(want.shape, float("nan"), device="cuda")
+    plan.set_weights(wd.data_ptr())
+    plan.forward(n, xd.data_ptr(), yd.data_ptr(), shift=bd.data_ptr())
+    torch.cuda.synchronize()
+    assert netrun.rel_err(yd.cpu().numpy(), want) < 1e-4
+
+
+def test_conv_epilogue_matches_unfused_chain(K):
+    """scale/shift/residual/activation of the epilogue against Conv -> BatchNorm ->
+    Scale -> (+residual) -> ReLU evaluated layer by layer on the oracle."""
+    rng = np.random.default_rng(2)
+    n, cin, cout, h = 2, 24, 40, 9
+    x = rng.standard_normal((n, cin, h, h)).astype(np.float32)
+    wt = (rng.standard_normal((cout, cin, 3, 3)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal(cout).astype(np.float32)
+    mean = rng.standard_normal(cout).astype(np.float32)
+    var = (rng.random(cout) + 0.5).astype(np.float32)
+    gamma = (rng.random(cout) + 0.5).astype(np.float32)
+    beta = rng.standard_normal(cout).astype(np.float32)
+    res = rng.standard_normal((n, cout, h, h)).astype(np.float32)
+    y = oracle.conv_forward(oracle.conv_geom(cin, h, h, cout, 3, 1, 1), x, wt, bias)
+    y = oracle.batch_norm(y, mean, var, np.ones(1, np.float32), True, 1e-5)
+    y = oracle.scale(y, gamma, beta)
+    want = oracle.relu(oracle.eltwise([y, res], "SUM"), 0.1)
+    # fold BN + Scale on the device
+    LIB = K.LIB
+    meand, stdd = torch.empty(cout, device="cuda"), torch.empty(cout, device="cuda")
+    b0, b1, b2 = dev(mean), dev(var), dev(np.ones(1, np.float32))   # keep the tensors alive
+    K.check_mc(LIB.mcBatchNormStored(fptr(b0), fptr(b1), fptr(b2),
+                                     ctypes.c_float(1e-5), cout, fptr(meand), fptr(stdd), None))
+    gd, bd, biasd = dev(gamma), dev(beta), dev(bias)
+    stages = (K.ChannelOp * 2)(K.ChannelOp(meand.data_ptr(), stdd.data_ptr(), None, None, 0, 0.0),
+                               K.ChannelOp(None, None, gd.data_ptr(), bd.data_ptr(), 0, 0.0))
+    sc, sh = torch.empty(cout, device="cuda"), torch.empty(cout, device="cuda")
+    K.check_mc(LIB.mcFoldChannelOps(fptr(biasd), stages, 2, cout, fptr(sc), fptr(sh), None))
+    plan = K.ConvPlan(K.conv_geom(cin, h, h, cout, 3, 1, 1))
+    wd, xd, rd = dev(wt), dev(x), dev(res)
+    yd = torch.empty(want.shape, device="cuda")
+    plan.set_weights(wd.data_ptr())
+    plan.forward(n, xd.data_ptr(), yd.data_ptr(), scale=sc.data_ptr(), shift=sh.data_ptr(),
+                 residual=rd.data_ptr(), activation=K.ACT_RELU, negative_slope=0.1)
+    torch.cuda.synchronize()
+    assert netrun.rel_err(yd.cpu().numpy(), want) < 1e-4
+
+
+def test_conv_rejects_bad_geometry(K):
+    from minicaffe import MiniCaffeError
+    with pytest.raises(MiniCaffeError, match="multiples of group"):
+        K.ConvPlan(K.conv_geom(6, 8, 8, 4, 3, group=4))
+    with pytest.raises(MiniCaffeError, match="empty output"):
+        K.ConvPlan(K.conv_geom(3, 2, 2, 4, 5))
+    with pytest.raises(MiniCaffeError, match="Stride"):
+        K.ConvPlan(K.conv_geom(3, 8, 8, 4, 3, stride=0))
+
+
+@pytest.mark.parametrize("shape", [(2, 5, 7, 8), (3, 4, 1, 1), (1, 6, 3, 5), (2, 3, 16, 16)])
+def test_channel_transform(K, shape):
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal(shape).astype(np.float32)
+    c = shape[1]
+    mean, var = rng.standard_normal(c).astype(np.float32), (rng.random(c) + 0.5).astype(np.float32)
+    gamma, beta = rng.standard_normal(c).astype(np.float32), rng.standard_normal(c).astype(np.float32)
+    want = oracle.relu(oracle.scale(oracle.batch_norm(x, mean, var, np.ones(1, np.float32), True, 1e-5),
+                                    gamma, beta), 0.2)
+    std = np.sqrt(var + np.float32(1e-5)).astype(np.float32)
+    xd, yd = dev(x), torch.empty(shape, device="cuda")
+    md, sd, gd, bd = dev(mean), dev(std), dev(gamma), dev(beta)
+    op = K.ChannelOp(md.data_ptr(), sd.data_ptr(), gd.data_ptr(), bd.data_ptr(), K.ACT_RELU, 0.2)
+    inner = int(np.prod(shape[2:]))
+    K.check_mc(K.LIB.mcChannelTransform(fptr(xd), fptr(yd), shape[0], c, inner, ctypes.byref(op), None))
+    torch.cuda.synchronize()
+    assert netrun.rel_err(yd.cpu().numpy(), want) < 1e-5
+    # activations alone, in place
+    for act, fn in ((K.ACT_TANH, oracle.tanh), (K.ACT_SIGMOID, oracle.sigmoid)):
+        zd = dev(x)
+        op = K.ChannelOp(None, None, None, None, act, 0.0)
+        K.check_mc(K.LIB.mcChannelTransform(fptr(zd), fptr(zd), 1, 1, x.size, ctypes.byref(op), None))
+        torch.cuda.synchronize()
+        assert np.abs(zd.cpu().numpy() - fn(x)).max() < 2e-7
+
+
+def test_batch_norm_batch_stats(K):
+    rng = np.random.default_rng(4)
+    x = (rng.standard_normal((16, 12, 8, 8)) * 2 + 1).astype(np.float32)
+    want = oracle.batch_norm(x, np.zeros(12), np.zeros(12), np.zeros(1), False, 1e-5)
+    xd, yd = dev(x), torch.empty(x.shape, device="cuda")
+    md, sd = torch.empty(12, device="cuda"), torch.empty(12, device="cuda")
+    K.check_mc(K.LIB.mcBatchNormBatchStats(fptr(xd), 16, 12, 64, ctypes.c_float(1e-5), fptr(md), fptr(sd), None))
+    op = K.ChannelOp(md.data_ptr(), sd.data_ptr(), None, None, 0, 0.0)
+    K.check_mc(K.LIB.mcChannelTransform(fptr(xd), fptr(yd), 16, 12, 64, ctypes.byref(op), None))
+    torch.cuda.synchronize()
+    assert netrun.rel_err(yd.cpu().numpy(), want) < 1e-5
+    assert np.abs(md.cpu().numpy() - x.mean(axis=(0, 2, 3))).max() < 1e-5
+
+
+@pytest.mark.parametrize("method", ["MAX", "AVE"])
+@pytest.mark.parametrize("hw,k,s,p", [((112, 112), 3, 2, 0), ((75, 75), 2, 2, 0), ((19, 19), 3, 1, 1),
+                                      ((7, 7), 7, 1, 0), ((6, 6), 2, 2, 1), ((9, 13), 3, 3, 1)])
+def test_pooling(K, method, hw, k, s, p):
+    x = np.random.default_rng(5).standard_normal((2, 5) + hw).astype(np.float32)
+    want = oracle.pooling(x, method, (k, k), (s, s), (p, p))
+    ho, wo = ctypes.c_int(), ctypes.c_int()
+    K.check_mc(K.LIB.mcPoolingOutputShape(hw[0], hw[1], k, k, s, s, p, p, ctypes.byref(ho), ctypes.byref(wo)))
+    assert (ho.value, wo.value) == want.shape[2:]
+    xd, yd = dev(x), torch.full(want.shape, float("nan"), device="cuda")
+    K.check_mc(K.LIB.mcPooling(0 if method == "MAX" else 1, fptr(xd), fptr(yd), 10, hw[0], hw[1],
+                               k, k, s, s, p, p, None))
+    torch.cuda.synchronize()
+    got = yd.cpu().numpy()
+    if method == "MAX":
+        assert np.array_equal(got, want)
+    else:
+        assert np.abs(got - want).max() < 1e-5
+
+
+@pytest.mark.parametrize("op,coeffs", [("SUM", None), ("SUM", [1.0, -2.0, 0.5]), ("PROD", None), ("MAX", None)])
+@pytest.mark.parametrize("count", [4096, 1001])
+def test_eltwise(K, op, coeffs, count):
+    rng = np.random.default_rng(6)
+    xs = [rng.standard_normal(count).astype(np.float32) for _ in range(3)]
+    want = oracle.eltwise(xs, op, coeffs)
+    ds = [dev(a) for a in xs]
+    ptrs = (ctypes.c_void_p * 3)(*[d.data_ptr() for d in ds])
+    co = (ctypes.c_float * 3)(*coeffs) if coeffs else None
+    yd = torch.empty(count, device="cuda")
+    K.check_mc(K.LIB.mcEltwise({"PROD": 0, "SUM": 1, "MAX": 2}[op], 3, ptrs, co, count, fptr(yd), 0,
+                               ctypes.c_float(0), None))
+    torch.cuda.synchronize()
+    assert np.abs(yd.cpu().numpy() - want).max() < 1e-6
+
+
+@pytest.mark.parametrize("shape,axis", [((64, 1000), 1), ((8, 873, 21), 2), ((1, 2, 342, 63), 1),
+                                        ((3, 5, 7), 1), ((4, 1500), 1)])
+def test_softmax(K, shape, axis):
+    x = (np.random.default_rng(7).standard_normal(shape) * 3).astype(np.float32)
+    want = oracle.softmax(x, axis)
+    outer, inner = int(np.prod(shape[:axis])), int(np.prod(shape[axis + 1:]))
+    xd, yd = dev(x), torch.empty(shape, device="cuda")
+    K.check_mc(K.LIB.mcSoftmax(fptr(xd), fptr(yd), outer, shape[axis], inner, None))
+    torch.cuda.synchronize()
+    assert np.abs(yd.cpu().numpy() - want).max() < 1e-6
+
+
+@pytest.mark.parametrize("shape,order", [((8, 84, 38, 38), (0, 2, 3, 1)), ((2, 3, 4, 5), (0, 3, 1, 2)),
+                                         ((2, 3, 4, 5), (3, 2, 1, 0)), ((2, 3, 4, 5), (0, 1, 2, 3)),
+                                         ((3, 70, 65), (0, 2, 1)), ((5, 6), (1, 0))])
+def test_permute_bit_exact(K, shape, order):
+    x = np.random.default_rng(8).standard_normal(shape).astype(np.float32)
+    want = np.ascontiguousarray(np.transpose(x, order))
+    xd, yd = dev(x), torch.full(want.shape, float("nan"), device="cuda")
+    sh = (ctypes.c_int * len(shape))(*shape)
+    od = (ctypes.c_int * len(order))(*order)
+    K.check_mc(K.LIB.mcPermute(fptr(xd), fptr(yd), len(shape), sh, od, None))
+    torch.cuda.synchronize()
+    assert np.array_equal(yd.cpu().numpy(), want)
+
+
+def test_copy2d_and_fill(K):
+    x = np.random.default_rng(9).standard_normal((7, 33)).astype(np.float32)
+    xd = dev(x)
+    yd = torch.zeros((7, 50), device="cuda")
+    K.check_mc(K.LIB.mcCopy2D(fptr(xd), 33, ctypes.c_void_p(yd.data_ptr() + 4 * 10), 50, 33, 7, None))
+    K.check_mc(K.LIB.mcFill(fptr(yd), 5, ctypes.c_float(2.5), None))
+    torch.cuda.synchronize()
+    got = yd.cpu().numpy()
+    assert np.array_equal(got[:, 10:43], x) and np.all(got[0, :5] == 2.5) and np.all(got[1:, :10] == 0)
