@@ -223,6 +223,56 @@ int mcNormalize(const float* bottom, float* top, int num, int channels, int spat
                 int across_spatial, int channel_shared, float eps, const float* scale,
                 void* stream);
 
+/* ---- detection tail (bit-exact kept indices) --------------------------------- */
+
+/* Bytes of device scratch mcProposal needs for this problem size. */
+int mcProposalWorkspaceSize(int num_proposals, int pre_nms_topn, int post_nms_topn,
+                            size_t* bytes);
+
+/* ProposalLayer::Forward (proposal_layer.cpp:261-322; device path .cu:212-276)
+ * without host round trips.  All pointers are device memory.
+ *   scores   [1, 2A, H, W]  (foreground = second half), bbox [1, 4A, H, W]
+ *   im_info  (height, width, scale); anchors [A, 4] from GenerateAnchors (:56-85)
+ *   rois     [post_nms_topn, 5] rows (0, x1, y1, x2, y2); roi_scores optional
+ *   num_rois number of valid rows (device int; the caller copies it back to
+ *            shape the top blob, as Forward_cpu's final Reshape does, :313-320)
+ *   tie_flag optional device int: set to 1 when two of the pre_nms_topn+1 best
+ *            scores are equal.  Tie-free inputs are ordered by one radix sort; with
+ *            ties the order is whatever the reference's quicksort SortBBox (:88-111)
+ *            leaves, so that quicksort is then replayed on the device, level by
+ *            level, to give the same row order. */
+int mcProposal(const float* scores, const float* bbox, const float* im_info, const float* anchors,
+               int A, int H, int W, int feat_stride, float min_size, int pre_nms_topn,
+               int post_nms_topn, float nms_thresh, void* workspace, size_t workspace_bytes,
+               float* rois, float* roi_scores, int* num_rois, int* tie_flag, void* stream);
+
+/* Bytes of device scratch mcDetectionOutput needs, and the row capacity that can
+ * never be exceeded for these parameters. */
+int mcDetectionOutputWorkspaceSize(int num, int num_priors, int num_classes, int share_location,
+                                   int top_k, size_t* bytes);
+int mcDetectionOutputMaxRows(int num, int num_priors, int num_classes, int top_k, int keep_top_k);
+
+/* DetectionOutputLayer::Forward (detection_output_layer.cpp:74-226) on the device.
+ *   loc   [num, P*loc_classes*4], conf [num, P*num_classes] (prior-major),
+ *   prior [1, 2, P*4] (boxes, then variances); code_type 1 CORNER, 2 CENTER_SIZE,
+ *   3 CORNER_SIZE (PriorBoxParameter.CodeType); top_k / keep_top_k -1 = unlimited;
+ *   confidence_threshold -FLT_MAX = none.
+ * Per image and non-background class: scores above the threshold in
+ * (score desc, prior asc) order (std::stable_sort, bbox_util.cpp:523-540), cut to
+ * top_k, greedy NMS with IoU <= threshold against every kept box and the adaptive
+ * eta rule (:681-716); then keep_top_k per image over all classes.
+ * out_rows receives [image, label, score, xmin, ymin, xmax, ymax] rows, images and
+ * labels ascending, each label's boxes in NMS order; *num_rows (device int) is the
+ * row count, or num rows of -1 when nothing was kept (:175-185).
+ * Equal scores at the keep_top_k cut are resolved by (label asc, NMS order); the
+ * reference leaves that to std::sort. */
+int mcDetectionOutput(const float* loc, const float* conf, const float* prior, int num,
+                      int num_priors, int num_classes, int share_location, int background_label,
+                      int code_type, int variance_encoded_in_target, int keep_top_k,
+                      float confidence_threshold, float nms_threshold, float eta, int top_k,
+                      void* workspace, size_t workspace_bytes, float* out_rows, int max_rows,
+                      int* num_rows, void* stream);
+
 /* Fill `count` floats with `value` (caffe_gpu_set, math_functions.cu:70-82). */
 int mcFill(float* dst, long count, float value, void* stream);
 

@@ -1,0 +1,409 @@
+// SSD DetectionOutput on the device: box decode, per-(image, class) candidate
+// ordering + greedy NMS, per-image keep_top_k, row emission.
+//
+// Restates DetectionOutputLayer::Forward_cpu (reference
+// src/layers/detection_output_layer.cpp:74-226) with the helpers of
+// src/util/bbox_util.cpp (DecodeBBox :242-330, GetMaxScoreIndex :523-540,
+// JaccardOverlap :184-204, ApplyNMSFast :681-716).  The reference's device path
+// (detection_output_layer.cu:14-152) decodes on the GPU and then runs the whole
+// selection on the host; here nothing but the final row count returns to the
+// host.
+//
+// Compiled with -ffp-contract=off so that decoded coordinates, overlaps and
+// therefore the kept indices equal the CPU path's bit for bit.
+#include "../mc_common.h"
+#include "block_sort.h"
+#include "mchip/kernels.h"
+
+namespace mchip {
+namespace {
+
+struct DBox {
+  float xmin, ymin, xmax, ymax, size;
+};
+
+__device__ __forceinline__ float dbox_size(float xmin, float ymin, float xmax, float ymax) {
+  if (xmax < xmin || ymax < ymin) return 0.f;
+  const float width = xmax - xmin;
+  const float height = ymax - ymin;
+  return width * height;
+}
+
+// One thread per (image, loc class, prior).  code_type 1 CORNER, 2 CENTER_SIZE,
+// 3 CORNER_SIZE.  exp() and the "/ 2." halvings are evaluated in double, as the
+// reference's expressions promote.
+__global__ __launch_bounds__(256) void det_decode_kernel(
+    const float* __restrict__ loc, const float* __restrict__ prior, int num, int P,
+    int loc_classes, int code_type, int var_in_target, DBox* __restrict__ out) {
+  const long total = (long)num * loc_classes * P;
+  const long t = blockIdx.x * 256L + threadIdx.x;
+  if (t >= total) return;
+  const int p = static_cast<int>(t % P);
+  const int c = static_cast<int>((t / P) % loc_classes);
+  const int i = static_cast<int>(t / ((long)P * loc_classes));
+  const float* l = loc + ((long)i * P + p) * loc_classes * 4 + c * 4;
+  const float* pr = prior + p * 4;
+  const float* var = prior + ((long)P + p) * 4;
+  const float pxmin = pr[0], pymin = pr[1], pxmax = pr[2], pymax = pr[3];
+  DBox b;
+  if (code_type == 1) {
+    if (var_in_target) {
+      b.xmin = pxmin + l[0];
+      b.ymin = pymin + l[1];
+      b.xmax = pxmax + l[2];
+      b.ymax = pymax + l[3];
+    } else {
+      b.xmin = pxmin + var[0] * l[0];
+      b.ymin = pymin + var[1] * l[1];
+      b.xmax = pxmax + var[2] * l[2];
+      b.ymax = pymax + var[3] * l[3];
+    }
+  } else if (code_type == 2) {
+    const float pw = pxmax - pxmin;
+    const float ph = pymax - pymin;
+    const float pcx = static_cast<float>((static_cast<double>(pxmin + pxmax)) / 2.);
+    const float pcy = static_cast<float>((static_cast<double>(pymin + pymax)) / 2.);
+    float cx, cy, w, h;
+    if (var_in_target) {
+      cx = l[0] * pw + pcx;
+      cy = l[1] * ph + pcy;
+      w = static_cast<float>(exp(static_cast<double>(l[2])) * static_cast<double>(pw));
+      h = static_cast<float>(exp(static_cast<double>(l[3])) * static_cast<double>(ph));
+    } else {
+      cx = var[0] * l[0] * pw + pcx;
+      cy = var[1] * l[1] * ph + pcy;
+      w = static_cast<float>(exp(static_cast<double>(var[2] * l[2])) * static_cast<double>(pw));
+      h = static_cast<float>(exp(static_cast<double>(var[3] * l[3])) * static_cast<double>(ph));
+    }
+    b.xmin = static_cast<float>(static_cast<double>(cx) - static_cast<double>(w) / 2.);
+    b.ymin = static_cast<float>(static_cast<double>(cy) - static_cast<double>(h) / 2.);
+    b.xmax = static_cast<float>(static_cast<double>(cx) + static_cast<double>(w) / 2.);
+    b.ymax = static_cast<float>(static_cast<double>(cy) + static_cast<double>(h) / 2.);
+  } else {
+    const float pw = pxmax - pxmin;
+    const float ph = pymax - pymin;
+    if (var_in_target) {
+      b.xmin = pxmin + l[0] * pw;
+      b.ymin = pymin + l[1] * ph;
+      b.xmax = pxmax + l[2] * pw;
+      b.ymax = pymax + l[3] * ph;
+    } else {
+      b.xmin = pxmin + var[0] * l[0] * pw;
+      b.ymin = pymin + var[1] * l[1] * ph;
+      b.xmax = pxmax + var[2] * l[2] * pw;
+      b.ymax = pymax + var[3] * l[3] * ph;
+    }
+  }
+  b.size = dbox_size(b.xmin, b.ymin, b.xmax, b.ymax);
+  out[t] = b;
+}
+
+// JaccardOverlap on normalised boxes with cached sizes (bbox_util.cpp:184-204).
+__device__ __forceinline__ float jaccard(const DBox& a, const DBox& b) {
+  float ixmin, iymin, ixmax, iymax;
+  if (b.xmin > a.xmax || b.xmax < a.xmin || b.ymin > a.ymax || b.ymax < a.ymin) {
+    ixmin = iymin = ixmax = iymax = 0.f;
+  } else {
+    ixmin = fmaxf(a.xmin, b.xmin);
+    iymin = fmaxf(a.ymin, b.ymin);
+    ixmax = fminf(a.xmax, b.xmax);
+    iymax = fminf(a.ymax, b.ymax);
+  }
+  const float iw = ixmax - ixmin, ih = iymax - iymin;
+  if (iw > 0.f && ih > 0.f) {
+    const float isz = iw * ih;
+    return isz / (a.size + b.size - isz);
+  }
+  return 0.f;
+}
+
+constexpr int kKeptLds = 512;  // kept boxes cached in LDS; further ones are read from memory
+
+// One workgroup per (image, class).  Candidates: scores above the confidence
+// threshold in (score desc, prior index asc) order, cut to top_k; then the
+// greedy pass of ApplyNMSFast with its adaptive threshold.
+__global__ __launch_bounds__(kSortThreads) void det_class_nms_kernel(
+    const float* __restrict__ conf, const DBox* __restrict__ boxes, int P, int C,
+    int loc_classes, int background, float conf_thr, float nms_thr, float eta, int top_k,
+    int max_cand, uint32_t* keys0, int* vals0, uint32_t* keys1, int* vals1,
+    int* __restrict__ kept_idx, int* __restrict__ kept_count) {
+  __shared__ BlockSortLds lds;
+  __shared__ DBox kept_box[kKeptLds];
+  __shared__ int s_valid;
+  const int c = blockIdx.x, i = blockIdx.y;
+  const int seg = i * C + c;
+  if (c == background) {
+    if (threadIdx.x == 0) kept_count[seg] = 0;
+    return;
+  }
+  uint32_t* k0 = keys0 + (size_t)seg * P;
+  int* v0 = vals0 + (size_t)seg * P;
+  uint32_t* k1 = keys1 + (size_t)seg * P;
+  int* v1 = vals1 + (size_t)seg * P;
+  if (threadIdx.x == 0) s_valid = 0;
+  __syncthreads();
+  // Contiguous runs per thread, as block_sort_desc expects.
+  const int per = (P + kSortThreads - 1) / kSortThreads;
+  const int begin = min(static_cast<int>(threadIdx.x) * per, P), end = min(begin + per, P);
+  int valid = 0;
+  for (int p = begin; p < end; ++p) {
+    const float s = conf[((size_t)i * P + p) * C + c];
+    const bool ok = s > conf_thr;
+    valid += ok;
+    k0[p] = ok ? desc_key(s) : 0xffffffffu;  // below-threshold scores sort last
+    v0[p] = p;
+  }
+  if (valid) atomicAdd(&s_valid, valid);
+  __syncthreads();
+  block_sort_desc(k0, v0, k1, v1, P, &lds);
+  int ncand = s_valid;
+  if (top_k > -1 && top_k < ncand) ncand = top_k;
+
+  if (threadIdx.x >= 64) return;  // the greedy pass is one wavefront
+  const int lane = threadIdx.x;
+  const DBox* cls_boxes = boxes + ((size_t)i * loc_classes + (loc_classes == 1 ? 0 : c)) * P;
+  int* kept = kept_idx + (size_t)seg * max_cand;
+  float adaptive = nms_thr;
+  int nkept = 0;
+  for (int r = 0; r < ncand; ++r) {
+    const int idx = v0[r];
+    const DBox b = cls_boxes[idx];
+    bool reject = false;
+    for (int base = 0; base < nkept && !reject; base += 64) {
+      const int k = base + lane;
+      bool over = false;
+      if (k < nkept) {
+        const DBox kb = k < kKeptLds ? kept_box[k] : cls_boxes[kept[k]];
+        over = !(jaccard(b, kb) <= adaptive);
+      }
+      reject = __any(over);
+    }
+    if (!reject) {
+      if (lane == 0) {
+        kept[nkept] = idx;
+        if (nkept < kKeptLds) kept_box[nkept] = b;
+      }
+      ++nkept;
+      if (eta < 1.f && adaptive > 0.5f) adaptive *= eta;
+      __builtin_amdgcn_wave_barrier();
+      __threadfence_block();
+    }
+  }
+  if (lane == 0) kept_count[seg] = nkept;
+}
+
+// One workgroup per image: applies keep_top_k over all classes and writes the
+// image's rows [image, label, score, xmin, ymin, xmax, ymax], labels ascending,
+// each label's boxes in NMS order.
+__global__ __launch_bounds__(kSortThreads) void det_select_kernel(
+    const float* __restrict__ conf, const DBox* __restrict__ boxes, int P, int C,
+    int loc_classes, int keep_top_k, int max_cand, const int* __restrict__ kept_idx,
+    const int* __restrict__ kept_count, uint32_t* keys0, int* vals0, uint32_t* keys1,
+    int* vals1, int* __restrict__ selected, float* __restrict__ rows_tmp,
+    int* __restrict__ rows_count) {
+  __shared__ BlockSortLds lds;
+  __shared__ int s_off[1024];  // start of each class in the image's entry list
+  const int i = blockIdx.x;
+  const int max_entries = C * max_cand;
+  uint32_t* k0 = keys0 + (size_t)i * max_entries;
+  int* v0 = vals0 + (size_t)i * max_entries;
+  uint32_t* k1 = keys1 + (size_t)i * max_entries;
+  int* v1 = vals1 + (size_t)i * max_entries;
+  int* sel = selected + (size_t)i * max_entries;
+  if (threadIdx.x == 0) {
+    int off = 0;
+    for (int c = 0; c < C; ++c) {
+      s_off[c] = off;
+      off += kept_count[i * C + c];
+    }
+    s_off[C] = off;
+  }
+  __syncthreads();
+  const int total = s_off[C];
+  // entry e = (label, position in that label's NMS order), labels ascending
+  for (int e = threadIdx.x; e < total; e += kSortThreads) sel[e] = 1;
+  __syncthreads();
+  if (keep_top_k > -1 && total > keep_top_k) {
+    const int per = (total + kSortThreads - 1) / kSortThreads;
+    const int begin = min(static_cast<int>(threadIdx.x) * per, total), end = min(begin + per, total);
+    int c = 0;
+    for (int e = begin; e < end; ++e) {
+      while (s_off[c + 1] <= e) ++c;
+      const int idx = kept_idx[(size_t)(i * C + c) * max_cand + (e - s_off[c])];
+      k0[e] = desc_key(conf[((size_t)i * P + idx) * C + c]);
+      v0[e] = e;
+    }
+    __syncthreads();
+    block_sort_desc(k0, v0, k1, v1, total, &lds);
+    for (int r = threadIdx.x; r < total; r += kSortThreads) sel[v0[r]] = r < keep_top_k;
+    __syncthreads();
+  }
+  // compact the selected entries in entry order (single pass by one thread per
+  // class would serialise; a block scan over `sel` keeps it parallel)
+  const int per = (total + kSortThreads - 1) / kSortThreads;
+  const int begin = min(static_cast<int>(threadIdx.x) * per, total), end = min(begin + per, total);
+  uint32_t mine = 0;
+  for (int e = begin; e < end; ++e) mine += sel[e];
+  uint32_t pos = block_exclusive_scan(mine, lds.wave_sum);
+  int c = 0;
+  for (int e = begin; e < end; ++e) {
+    if (!sel[e]) continue;
+    while (s_off[c + 1] <= e) ++c;
+    const int idx = kept_idx[(size_t)(i * C + c) * max_cand + (e - s_off[c])];
+    const DBox b = boxes[((size_t)i * loc_classes + (loc_classes == 1 ? 0 : c)) * P + idx];
+    float* row = rows_tmp + ((size_t)i * max_entries + pos) * 7;
+    row[0] = static_cast<float>(i);
+    row[1] = static_cast<float>(c);
+    row[2] = conf[((size_t)i * P + idx) * C + c];
+    row[3] = b.xmin;
+    row[4] = b.ymin;
+    row[5] = b.xmax;
+    row[6] = b.ymax;
+    ++pos;
+  }
+  __syncthreads();
+  if (threadIdx.x == kSortThreads - 1) rows_count[i] = static_cast<int>(pos);
+}
+
+// Concatenates the per-image rows; with no detection at all, one row of -1 per
+// image carrying the image index (detection_output_layer.cpp:175-185).
+__global__ __launch_bounds__(256) void det_emit_kernel(const float* __restrict__ rows_tmp,
+                                                       const int* __restrict__ rows_count,
+                                                       int num, int max_entries, int max_rows,
+                                                       float* __restrict__ out,
+                                                       int* __restrict__ num_rows) {
+  __shared__ int s_off[1025];
+  if (threadIdx.x == 0) {
+    int off = 0;
+    for (int i = 0; i < num; ++i) {
+      s_off[i] = off;
+      off += rows_count[i];
+    }
+    s_off[num] = off;
+  }
+  __syncthreads();
+  const int total = s_off[num];
+  if (total == 0) {
+    for (int t = threadIdx.x; t < num * 7 && t < max_rows * 7; t += 256)
+      out[t] = (t % 7 == 0) ? static_cast<float>(t / 7) : -1.f;
+    if (threadIdx.x == 0) *num_rows = num;
+    return;
+  }
+  for (int i = 0; i < num; ++i) {
+    const int cnt = rows_count[i];
+    const float* src = rows_tmp + (size_t)i * max_entries * 7;
+    float* dst = out + (size_t)s_off[i] * 7;
+    for (int t = threadIdx.x; t < cnt * 7; t += 256)
+      if (s_off[i] + t / 7 < max_rows) dst[t] = src[t];
+  }
+  if (threadIdx.x == 0) *num_rows = total < max_rows ? total : max_rows;
+}
+
+struct DetLayout {
+  size_t boxes, k0, v0, k1, v1, kept_idx, kept_count, sk0, sv0, sk1, sv1, selected, rows_tmp,
+      rows_count, total;
+};
+
+inline size_t det_align(size_t v) { return (v + 255) / 256 * 256; }
+
+DetLayout det_layout(int num, int P, int C, int loc_classes, int max_cand) {
+  DetLayout L;
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    const size_t at = off;
+    off += det_align(bytes);
+    return at;
+  };
+  const size_t segs = (size_t)num * C;
+  const size_t entries = (size_t)num * C * max_cand;
+  L.boxes = take(sizeof(DBox) * (size_t)num * loc_classes * P);
+  L.k0 = take(4 * segs * P);
+  L.v0 = take(4 * segs * P);
+  L.k1 = take(4 * segs * P);
+  L.v1 = take(4 * segs * P);
+  L.kept_idx = take(4 * entries);
+  L.kept_count = take(4 * segs);
+  L.sk0 = take(4 * entries);
+  L.sv0 = take(4 * entries);
+  L.sk1 = take(4 * entries);
+  L.sv1 = take(4 * entries);
+  L.selected = take(4 * entries);
+  L.rows_tmp = take(4 * 7 * entries);
+  L.rows_count = take(4 * (size_t)num);
+  L.total = off;
+  return L;
+}
+
+int det_max_cand(int P, int top_k) { return (top_k > -1 && top_k < P) ? top_k : P; }
+
+}  // namespace
+}  // namespace mchip
+
+using namespace mchip;
+
+extern "C" {
+
+int mcDetectionOutputWorkspaceSize(int num, int num_priors, int num_classes, int share_location,
+                                   int top_k, size_t* bytes) {
+  MC_REQUIRE(bytes && num > 0 && num_priors > 0 && num_classes > 0,
+             "mcDetectionOutputWorkspaceSize: bad argument");
+  *bytes = det_layout(num, num_priors, num_classes, share_location ? 1 : num_classes,
+                      det_max_cand(num_priors, top_k))
+               .total;
+  return 0;
+}
+
+int mcDetectionOutputMaxRows(int num, int num_priors, int num_classes, int top_k, int keep_top_k) {
+  long per_image = (long)num_classes * det_max_cand(num_priors, top_k);
+  if (keep_top_k > -1 && keep_top_k < per_image) per_image = keep_top_k;
+  long rows = per_image * num;
+  if (rows < num) rows = num;
+  return rows > 0x7fffffffL ? 0x7fffffff : static_cast<int>(rows);
+}
+
+int mcDetectionOutput(const float* loc, const float* conf, const float* prior, int num,
+                      int num_priors, int num_classes, int share_location, int background_label,
+                      int code_type, int variance_encoded_in_target, int keep_top_k,
+                      float confidence_threshold, float nms_threshold, float eta, int top_k,
+                      void* workspace, size_t workspace_bytes, float* out_rows, int max_rows,
+                      int* num_rows, void* stream) {
+  MC_REQUIRE(loc && conf && prior && workspace && out_rows && num_rows,
+             "mcDetectionOutput: null argument");
+  MC_REQUIRE(num > 0 && num <= 1024 && num_priors > 0 && num_classes > 0 && num_classes < 1024,
+             "mcDetectionOutput: bad extents");
+  MC_REQUIRE(code_type >= 1 && code_type <= 3, "Unknown LocLossType.");
+  MC_REQUIRE(nms_threshold >= 0.f, "nms_threshold must be non negative.");
+  MC_REQUIRE(eta > 0.f && eta <= 1.f, "eta must be in (0, 1]");
+  MC_REQUIRE(max_rows >= num, "mcDetectionOutput: output needs at least one row per image");
+  const int loc_classes = share_location ? 1 : num_classes;
+  const int max_cand = det_max_cand(num_priors, top_k);
+  const DetLayout L = det_layout(num, num_priors, num_classes, loc_classes, max_cand);
+  MC_REQUIRE(workspace_bytes >= L.total, "mcDetectionOutput: workspace too small (%zu < %zu)",
+             workspace_bytes, L.total);
+  char* ws = static_cast<char*>(workspace);
+  DBox* boxes = reinterpret_cast<DBox*>(ws + L.boxes);
+  auto u32 = [&](size_t off) { return reinterpret_cast<uint32_t*>(ws + off); };
+  auto i32 = [&](size_t off) { return reinterpret_cast<int*>(ws + off); };
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const long ndec = (long)num * loc_classes * num_priors;
+  det_decode_kernel<<<ceil_div(ndec, 256), 256, 0, st>>>(loc, prior, num, num_priors, loc_classes,
+                                                         code_type, variance_encoded_in_target,
+                                                         boxes);
+  MC_LAUNCH_CHECK();
+  det_class_nms_kernel<<<dim3(num_classes, num), kSortThreads, 0, st>>>(
+      conf, boxes, num_priors, num_classes, loc_classes, background_label, confidence_threshold,
+      nms_threshold, eta, top_k, max_cand, u32(L.k0), i32(L.v0), u32(L.k1), i32(L.v1),
+      i32(L.kept_idx), i32(L.kept_count));
+  MC_LAUNCH_CHECK();
+  det_select_kernel<<<num, kSortThreads, 0, st>>>(
+      conf, boxes, num_priors, num_classes, loc_classes, keep_top_k, max_cand, i32(L.kept_idx),
+      i32(L.kept_count), u32(L.sk0), i32(L.sv0), u32(L.sk1), i32(L.sv1), i32(L.selected),
+      reinterpret_cast<float*>(ws + L.rows_tmp), i32(L.rows_count));
+  MC_LAUNCH_CHECK();
+  det_emit_kernel<<<1, 256, 0, st>>>(reinterpret_cast<float*>(ws + L.rows_tmp), i32(L.rows_count),
+                                     num, num_classes * max_cand, max_rows, out_rows, num_rows);
+  MC_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // extern "C"

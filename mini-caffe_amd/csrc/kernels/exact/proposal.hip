@@ -1,0 +1,509 @@
+// Region-proposal tail on the device: anchor decode, top-N ordering, bitmask-IoU
+// NMS with a single-wavefront scan, roi gather.  No host round trips: the only
+// value that returns to the host is the roi count, which fixes the top's shape.
+//
+// Restates ProposalLayer::Forward_cpu (reference src/layers/proposal_layer.cpp:261-322);
+// replaces GenerataProposalsGPU / NMSKernel / RetrieveRoisGPU and the host-side
+// SortBBox + bit scan of the reference's device path (proposal_layer.cu:48-276).
+//
+// This file is compiled with -ffp-contract=off: the kept-box indices must equal
+// the CPU path's bit for bit, so every a*b+c here is two roundings like there.
+#include "../mc_common.h"
+#include "block_sort.h"
+#include "mchip/kernels.h"
+
+namespace mchip {
+namespace {
+
+// TransformBBox (proposal_layer.cpp:14-53).  exp() is evaluated in double and
+// the product with the extent is narrowed afterwards, as the reference's
+// unqualified exp(float) does.
+__device__ __forceinline__ float decode_and_clip(float* box, float dx, float dy, float dlw,
+                                                 float dlh, float img_w, float img_h,
+                                                 float min_size) {
+  const float w = box[2] - box[0] + 1;
+  const float h = box[3] - box[1] + 1;
+  const float ctr_x = box[0] + 0.5f * w;
+  const float ctr_y = box[1] + 0.5f * h;
+  const float pred_ctr_x = dx * w + ctr_x;
+  const float pred_ctr_y = dy * h + ctr_y;
+  const float pred_w = static_cast<float>(exp(static_cast<double>(dlw)) * static_cast<double>(w));
+  const float pred_h = static_cast<float>(exp(static_cast<double>(dlh)) * static_cast<double>(h));
+  box[0] = pred_ctr_x - 0.5f * pred_w;
+  box[1] = pred_ctr_y - 0.5f * pred_h;
+  box[2] = pred_ctr_x + 0.5f * pred_w;
+  box[3] = pred_ctr_y + 0.5f * pred_h;
+  box[0] = fmaxf(0.f, fminf(box[0], img_w - 1));
+  box[1] = fmaxf(0.f, fminf(box[1], img_h - 1));
+  box[2] = fmaxf(0.f, fminf(box[2], img_w - 1));
+  box[3] = fmaxf(0.f, fminf(box[3], img_h - 1));
+  const float box_w = box[2] - box[0] + 1;
+  const float box_h = box[3] - box[1] + 1;
+  return (box_w >= min_size && box_h >= min_size) ? 1.f : 0.f;
+}
+
+// One thread per proposal, index = (h*W + w)*A + k (proposal_layer.cpp:125-147).
+__global__ __launch_bounds__(256) void proposal_decode_kernel(
+    const float* __restrict__ fg, const float* __restrict__ bbox, const float* __restrict__ anchors,
+    const float* __restrict__ im_info, int A, int H, int W, int feat_stride, float min_size_param,
+    float4* __restrict__ boxes, uint32_t* __restrict__ keys, uint32_t* __restrict__ keys_orig,
+    int* __restrict__ vals, float* __restrict__ scores) {
+  const int n = A * H * W;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const int k = i % A;
+  const int pix = i / A;
+  const int w = pix % W, h = pix / W;
+  const int fm = H * W;
+  const float img_h = im_info[0], img_w = im_info[1];
+  const float min_size = min_size_param * im_info[2];
+  const float x = static_cast<float>(w * feat_stride), y = static_cast<float>(h * feat_stride);
+  float box[4] = {x + anchors[k * 4 + 0], y + anchors[k * 4 + 1], x + anchors[k * 4 + 2],
+                  y + anchors[k * 4 + 3]};
+  const float* b = bbox + h * W + w;
+  const float valid = decode_and_clip(box, b[(k * 4 + 0) * fm], b[(k * 4 + 1) * fm],
+                                      b[(k * 4 + 2) * fm], b[(k * 4 + 3) * fm], img_w, img_h,
+                                      min_size);
+  const float s = valid * fg[k * fm + h * W + w];
+  boxes[i] = make_float4(box[0], box[1], box[2], box[3]);
+  scores[i] = s;
+  keys[i] = desc_key(s);
+  keys_orig[i] = keys[i];
+  vals[i] = i;
+}
+
+// Orders all proposals by (score desc, index asc) and flags score ties that
+// reach into the first `pre` places.
+__global__ __launch_bounds__(kSortThreads) void proposal_sort_kernel(
+    uint32_t* k0, int* v0, uint32_t* k1, int* v1, int n, int pre, int* __restrict__ tie_flag) {
+  __shared__ BlockSortLds lds;
+  block_sort_desc(k0, v0, k1, v1, n, &lds);
+  int ties = 0;
+  // a tie between two of the first pre+1 keys leaves their order to the
+  // reference's quicksort; equal keys <=> equal scores
+  for (int i = threadIdx.x; i < pre; i += kSortThreads)
+    if (i + 1 < n && k0[i] == k0[i + 1]) ties = 1;
+  if (ties) atomicOr(tie_flag, 1);
+}
+
+// Boxes and scores of the first `pre` proposals in their final order.
+__global__ __launch_bounds__(256) void proposal_order_gather_kernel(
+    const int* __restrict__ order, int pre, const float4* __restrict__ boxes,
+    const float* __restrict__ scores, float4* __restrict__ sorted_boxes,
+    float* __restrict__ sorted_scores) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= pre) return;
+  const int src = order[i];
+  sorted_boxes[i] = boxes[src];
+  sorted_scores[i] = scores[src];
+}
+
+// Exact replay of the reference's SortBBox (proposal_layer.cpp:88-111) for inputs
+// with equal scores, where the final order is whatever that quicksort leaves.
+//
+// The recursion is replayed level by level: all partitions of one depth at once.
+// A partition with pivot K = a[lo] never moves elements equal to K; it swaps the
+// i-th larger element found from the right (position R_i) with the i-th smaller
+// one found from the left (L_i) through a moving hole:
+//     a[lo] <- a[R_1],  a[R_i] <- a[L_i],  a[L_i] <- a[R_(i+1)],  pivot -> last hole
+// for as long as L_i < R_i (resp. R_(i+1) > L_i).  Ranks come from one prefix
+// sum over the whole array, so a level costs a handful of passes regardless of
+// how many partitions it holds.  Keys are the order-preserving integer images
+// of the scores (smaller key = larger score).  One 1024-thread workgroup; runs
+// only when `flag` says ties reach into the first num_top places.
+constexpr int kQsThreads = 1024;
+
+__global__ __launch_bounds__(kQsThreads) void quicksort_replay_kernel(
+    const int* __restrict__ flag, const uint32_t* __restrict__ key_in, int n, int num_top,
+    uint32_t* __restrict__ kA, int* __restrict__ vA, uint32_t* __restrict__ kB,
+    int* __restrict__ vB, int* __restrict__ seg_lo, int* __restrict__ seg_hi,
+    unsigned long long* __restrict__ pref, int* __restrict__ posS, int* __restrict__ posB,
+    int* __restrict__ mS, int* __restrict__ mB, int* __restrict__ hole, int* __restrict__ dest,
+    int* __restrict__ nseg, unsigned char* __restrict__ cls, int* __restrict__ order_out) {
+  if (*flag == 0) return;
+  __shared__ unsigned long long wave_tot[kQsThreads / 64];
+  const int tid = threadIdx.x;
+  // Phases that only need "every element once" walk the array with a stride of
+  // the workgroup size (coalesced, iterations independent so loads overlap);
+  // the prefix sum needs contiguous per-thread runs.
+  const int per = (n + kQsThreads - 1) / kQsThreads;
+  const int begin = min(tid * per, n), end = min(begin + per, n);
+  for (int p = tid; p < n; p += kQsThreads) {
+    kA[p] = key_in[p];
+    vA[p] = p;
+    seg_lo[p] = 0;
+    seg_hi[p] = n - 1;
+  }
+  __syncthreads();
+  uint32_t* __restrict__ key = kA;
+  int* __restrict__ val = vA;
+  uint32_t* __restrict__ nkey = kB;
+  int* __restrict__ nval = vB;
+  for (;;) {
+    // 1. classify against the segment's pivot: 1 = smaller score, 2 = larger score
+#pragma unroll 8
+    for (int p = tid; p < n; p += kQsThreads) {
+      const int lo = seg_lo[p];
+      unsigned char f = 0;
+      if (lo >= 0 && p != lo) {
+        const uint32_t K = key[lo], k = key[p];
+        f = k > K ? 1 : (k < K ? 2 : 0);
+      }
+      if (lo == p) {
+        mS[p] = 0;
+        mB[p] = 0;
+      }
+      cls[p] = f;
+      dest[p] = p;
+    }
+    __syncthreads();
+    // inclusive prefix counts over the whole array (smaller: low word, larger: high word)
+    unsigned long long local = 0;
+    for (int p = begin; p < end; ++p) {
+      const unsigned char f = cls[p];
+      local += f == 1 ? 1ull : (f == 2 ? (1ull << 32) : 0ull);
+    }
+    unsigned long long inc = local;
+    {
+      const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const unsigned lo32 = __shfl_up(static_cast<unsigned>(inc), o, 64);
+        const unsigned hi32 = __shfl_up(static_cast<unsigned>(inc >> 32), o, 64);
+        if (lane >= o) inc += (static_cast<unsigned long long>(hi32) << 32) | lo32;
+      }
+      if (lane == 63) wave_tot[wave] = inc;
+      __syncthreads();
+      unsigned long long base = 0;
+      for (int w = 0; w < wave; ++w) base += wave_tot[w];
+      inc = base + inc - local;  // exclusive prefix of this thread's run
+    }
+    for (int p = begin; p < end; ++p) {
+      const unsigned char f = cls[p];
+      inc += f == 1 ? 1ull : (f == 2 ? (1ull << 32) : 0ull);
+      pref[p] = inc;
+    }
+    __syncthreads();
+    // 2. rank -> position tables
+#pragma unroll 8
+    for (int p = tid; p < n; p += kQsThreads) {
+      const unsigned char f = cls[p];
+      if (f == 0) continue;
+      const int lo = seg_lo[p];
+      const unsigned long long base = pref[lo], mine = pref[p];
+      if (f == 1) {
+        posS[lo + static_cast<int>((mine & 0xffffffffull) - (base & 0xffffffffull))] = p;
+      } else {
+        const int nB = static_cast<int>((pref[seg_hi[p]] >> 32) - (base >> 32));
+        posB[lo + nB - static_cast<int>((mine >> 32) - (base >> 32)) + 1] = p;
+      }
+    }
+    __syncthreads();
+    // 3. who moves where
+#pragma unroll 8
+    for (int p = tid; p < n; p += kQsThreads) {
+      const unsigned char f = cls[p];
+      if (f == 0) continue;
+      const int lo = seg_lo[p];
+      const unsigned long long base = pref[lo], top = pref[seg_hi[p]], mine = pref[p];
+      const int nS = static_cast<int>((top & 0xffffffffull) - (base & 0xffffffffull));
+      const int nB = static_cast<int>((top >> 32) - (base >> 32));
+      if (f == 1) {
+        const int i = static_cast<int>((mine & 0xffffffffull) - (base & 0xffffffffull));
+        if (i <= nB && p < posB[lo + i]) {
+          dest[p] = posB[lo + i];
+          const int nx = i + 1;
+          if (!(nx <= nS && nx <= nB && posS[lo + nx] < posB[lo + nx])) mS[lo] = i;
+        }
+      } else {
+        const int i = nB - static_cast<int>((mine >> 32) - (base >> 32)) + 1;
+        if (i == 1 || (i - 1 <= nS && p > posS[lo + i - 1])) {
+          dest[p] = i == 1 ? lo : posS[lo + i - 1];
+          const int nx = i + 1;
+          if (!(nx <= nB && nx - 1 <= nS && posB[lo + nx] > posS[lo + nx - 1])) mB[lo] = i;
+        }
+      }
+    }
+    __syncthreads();
+    // 4. pivots find the final hole; an all-equal segment is final as it stands
+#pragma unroll 8
+    for (int p = tid; p < n; p += kQsThreads) {
+      if (seg_lo[p] != p) continue;
+      const bool all_equal = pref[seg_hi[p]] == pref[p];
+      int h;
+      if (mB[p] == 0) h = p;
+      else if (mB[p] > mS[p]) h = posB[p + mB[p]];
+      else h = posS[p + mS[p]];
+      hole[p] = all_equal ? -1 : h;
+      dest[p] = h;
+    }
+    __syncthreads();
+    // 5. apply the moves, derive the next level's segments
+    int active = 0;
+#pragma unroll 8
+    for (int p = tid; p < n; p += kQsThreads) {
+      const int d = dest[p];
+      nkey[d] = key[p];
+      nval[d] = val[p];
+      const int lo = seg_lo[p];
+      int nlo = -1, nhi = -1;
+      if (lo >= 0) {
+        const int hi = seg_hi[p];
+        const int h = hole[lo];
+        if (h >= 0) {
+          if (p < h) {
+            if (lo < h - 1) {
+              nlo = lo;
+              nhi = h - 1;
+            }
+          } else if (p > h) {
+            if (h + 1 < num_top && h + 1 < hi) {
+              nlo = h + 1;
+              nhi = hi;
+            }
+          }
+        }
+      }
+      nseg[2 * p] = nlo;
+      nseg[2 * p + 1] = nhi;
+      active |= nlo >= 0;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int p = tid; p < n; p += kQsThreads) {
+      seg_lo[p] = nseg[2 * p];
+      seg_hi[p] = nseg[2 * p + 1];
+    }
+    uint32_t* tk = key; key = nkey; nkey = tk;
+    int* tv = val; val = nval; nval = tv;
+    if (!__syncthreads_or(active)) break;
+  }
+  for (int p = tid; p < num_top; p += kQsThreads) order_out[p] = val[p];
+}
+
+// mask[i][cb] bit j: box cb*64+j (> i) overlaps box i by more than thr, with
+// the +1 pixel extents of NonMaximumSuppressionCPU (proposal_layer.cpp:150-185).
+__global__ __launch_bounds__(64) void nms_mask_kernel(const float4* __restrict__ boxes, int n,
+                                                      float thr, int nb,
+                                                      unsigned long long* __restrict__ mask) {
+  const int rb = blockIdx.y, cb = blockIdx.x;
+  if (cb < rb) return;
+  __shared__ float4 cols[64];
+  const int cn = min(64, n - cb * 64);
+  if (static_cast<int>(threadIdx.x) < cn) cols[threadIdx.x] = boxes[cb * 64 + threadIdx.x];
+  __syncthreads();
+  const int i = rb * 64 + threadIdx.x;
+  if (i >= n) return;
+  const float4 a = boxes[i];
+  const float area_a = (a.z - a.x + 1) * (a.w - a.y + 1);
+  unsigned long long bits = 0;
+  for (int j = 0; j < cn; ++j) {
+    if (cb * 64 + j <= i) continue;
+    const float4 b = cols[j];
+    const float area_b = (b.z - b.x + 1) * (b.w - b.y + 1);
+    const float x1 = fmaxf(a.x, b.x), y1 = fmaxf(a.y, b.y);
+    const float x2 = fminf(a.z, b.z), y2 = fminf(a.w, b.w);
+    const float w = fmaxf(0.f, x2 - x1 + 1), h = fmaxf(0.f, y2 - y1 + 1);
+    const float inter = w * h;
+    const float ov = inter / (area_a + area_b - inter);
+    if (ov > thr) bits |= 1ull << j;
+  }
+  mask[(size_t)i * nb + cb] = bits;
+}
+
+// One wavefront walks the boxes in score order.  Lane l owns words l, l+64, ...
+// of the running "removed" bitmap.  Per block of 64 boxes: the block's removed
+// word and the 64 diagonal mask words are brought into lanes, the 64 greedy
+// decisions are taken with wave broadcasts (no memory in the loop), then the
+// rows of the boxes that were kept are OR-ed into the bitmap.
+__global__ __launch_bounds__(64) void nms_scan_kernel(const unsigned long long* __restrict__ mask,
+                                                      int n, int nb, int max_keep,
+                                                      int* __restrict__ kept,
+                                                      int* __restrict__ num_kept) {
+  extern __shared__ unsigned long long removed[];  // nb words
+  const int lane = threadIdx.x;
+  for (int w = lane; w < nb; w += 64) removed[w] = 0;
+  __syncthreads();
+  int count = 0;
+  for (int blk = 0; blk < nb && count < max_keep; ++blk) {
+    const int i = blk * 64 + lane;
+    unsigned long long diag = i < n ? mask[(size_t)i * nb + blk] : 0ull;
+    unsigned long long rem = removed[blk];
+    const int bn = min(64, n - blk * 64);
+    unsigned long long keep_bits = 0;
+    for (int j = 0; j < bn && count < max_keep; ++j) {
+      if (!((rem >> j) & 1ull)) {
+        keep_bits |= 1ull << j;
+        if (lane == 0) kept[count] = blk * 64 + j;
+        ++count;
+        // broadcast row j's diagonal word
+        const unsigned lo = __shfl(static_cast<unsigned>(diag), j, 64);
+        const unsigned hi = __shfl(static_cast<unsigned>(diag >> 32), j, 64);
+        rem |= (static_cast<unsigned long long>(hi) << 32) | lo;
+      }
+    }
+    // fold the kept rows into the words of later blocks
+    for (int w = blk + 1 + lane; w < nb; w += 64) {
+      unsigned long long acc = removed[w];
+      unsigned long long kb = keep_bits;
+      while (kb) {
+        const int j = __ffsll(static_cast<long long>(kb)) - 1;
+        kb &= kb - 1;
+        acc |= mask[(size_t)(blk * 64 + j) * nb + w];
+      }
+      removed[w] = acc;
+    }
+    __syncthreads();
+  }
+  if (lane == 0) *num_kept = count;
+}
+
+// rois[r] = (0, x1, y1, x2, y2) of the r-th kept box (proposal_layer.cpp:187-203).
+__global__ void proposal_gather_kernel(const float4* __restrict__ sorted_boxes,
+                                       const float* __restrict__ sorted_scores,
+                                       const int* __restrict__ kept,
+                                       const int* __restrict__ num_kept, float* __restrict__ rois,
+                                       float* __restrict__ roi_scores) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= *num_kept) return;
+  const float4 b = sorted_boxes[kept[r]];
+  rois[r * 5 + 0] = 0.f;
+  rois[r * 5 + 1] = b.x;
+  rois[r * 5 + 2] = b.y;
+  rois[r * 5 + 3] = b.z;
+  rois[r * 5 + 4] = b.w;
+  if (roi_scores) roi_scores[r] = sorted_scores[kept[r]];
+}
+
+__global__ void zero_ints_kernel(int* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+struct ProposalLayout {
+  size_t boxes, scores, k0, v0, k1, v1, korig, kb, vb, seg_lo, seg_hi, pref, posS, posB, mS, mB,
+      hole, dest, nseg, cls, sorted_boxes, sorted_scores, mask, kept, flags, total;
+};
+
+inline size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+
+ProposalLayout layout(int n, int pre, int post) {
+  ProposalLayout L;
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    const size_t at = off;
+    off += align256(bytes);
+    return at;
+  };
+  const int nb = ceil_div(pre, 64);
+  L.boxes = take(sizeof(float4) * n);
+  L.scores = take(sizeof(float) * n);
+  L.k0 = take(sizeof(uint32_t) * n);
+  L.v0 = take(sizeof(int) * n);
+  L.k1 = take(sizeof(uint32_t) * n);
+  L.v1 = take(sizeof(int) * n);
+  L.korig = take(sizeof(uint32_t) * n);
+  L.kb = take(sizeof(uint32_t) * n);
+  L.vb = take(sizeof(int) * n);
+  L.seg_lo = take(sizeof(int) * n);
+  L.seg_hi = take(sizeof(int) * n);
+  L.pref = take(sizeof(unsigned long long) * n);
+  L.posS = take(sizeof(int) * (n + 1));
+  L.posB = take(sizeof(int) * (n + 1));
+  L.mS = take(sizeof(int) * n);
+  L.mB = take(sizeof(int) * n);
+  L.hole = take(sizeof(int) * n);
+  L.dest = take(sizeof(int) * n);
+  L.nseg = take(sizeof(int) * 2 * n);
+  L.cls = take(n);
+  L.sorted_boxes = take(sizeof(float4) * pre);
+  L.sorted_scores = take(sizeof(float) * pre);
+  L.mask = take(sizeof(unsigned long long) * (size_t)pre * nb);
+  L.kept = take(sizeof(int) * post);
+  L.flags = take(sizeof(int) * 4);
+  L.total = off;
+  return L;
+}
+
+}  // namespace
+}  // namespace mchip
+
+using namespace mchip;
+
+extern "C" {
+
+int mcProposalWorkspaceSize(int num_proposals, int pre_nms_topn, int post_nms_topn,
+                            size_t* bytes) {
+  MC_REQUIRE(bytes && num_proposals > 0 && pre_nms_topn > 0 && post_nms_topn > 0,
+             "mcProposalWorkspaceSize: bad argument");
+  const int pre = pre_nms_topn < num_proposals ? pre_nms_topn : num_proposals;
+  *bytes = layout(num_proposals, pre, post_nms_topn).total;
+  return 0;
+}
+
+int mcProposal(const float* scores, const float* bbox, const float* im_info, const float* anchors,
+               int A, int H, int W, int feat_stride, float min_size, int pre_nms_topn,
+               int post_nms_topn, float nms_thresh, void* workspace, size_t workspace_bytes,
+               float* rois, float* roi_scores, int* num_rois, int* tie_flag, void* stream) {
+  MC_REQUIRE(scores && bbox && im_info && anchors && workspace && rois && num_rois,
+             "mcProposal: null argument");
+  MC_REQUIRE(A > 0 && H > 0 && W > 0 && pre_nms_topn > 0 && post_nms_topn > 0,
+             "mcProposal: bad extents");
+  const long n_long = (long)A * H * W;
+  MC_REQUIRE(n_long < (1L << 24), "mcProposal: too many proposals");
+  const int n = static_cast<int>(n_long);
+  const int pre = pre_nms_topn < n ? pre_nms_topn : n;
+  const ProposalLayout L = layout(n, pre, post_nms_topn);
+  MC_REQUIRE(workspace_bytes >= L.total, "mcProposal: workspace too small (%zu < %zu)",
+             workspace_bytes, L.total);
+  char* ws = static_cast<char*>(workspace);
+  float4* boxes = reinterpret_cast<float4*>(ws + L.boxes);
+  float* sc = reinterpret_cast<float*>(ws + L.scores);
+  uint32_t* k0 = reinterpret_cast<uint32_t*>(ws + L.k0);
+  int* v0 = reinterpret_cast<int*>(ws + L.v0);
+  uint32_t* k1 = reinterpret_cast<uint32_t*>(ws + L.k1);
+  int* v1 = reinterpret_cast<int*>(ws + L.v1);
+  uint32_t* korig = reinterpret_cast<uint32_t*>(ws + L.korig);
+  auto ints = [&](size_t off) { return reinterpret_cast<int*>(ws + off); };
+  float4* sboxes = reinterpret_cast<float4*>(ws + L.sorted_boxes);
+  float* sscores = reinterpret_cast<float*>(ws + L.sorted_scores);
+  unsigned long long* mask = reinterpret_cast<unsigned long long*>(ws + L.mask);
+  int* kept = reinterpret_cast<int*>(ws + L.kept);
+  int* flags = reinterpret_cast<int*>(ws + L.flags);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int nb = ceil_div(pre, 64);
+
+  zero_ints_kernel<<<1, 64, 0, st>>>(flags, 4);
+  MC_LAUNCH_CHECK();
+  // foreground scores are the second half of the score blob (proposal_layer.cpp:295)
+  proposal_decode_kernel<<<ceil_div(n, 256), 256, 0, st>>>(scores + n, bbox, anchors, im_info, A, H,
+                                                          W, feat_stride, min_size, boxes, k0,
+                                                          korig, v0, sc);
+  MC_LAUNCH_CHECK();
+  proposal_sort_kernel<<<1, kSortThreads, 0, st>>>(k0, v0, k1, v1, n, pre, flags);
+  MC_LAUNCH_CHECK();
+  // no-op unless equal scores reach into the first `pre` places
+  quicksort_replay_kernel<<<1, kQsThreads, 0, st>>>(
+      flags, korig, n, pre, k1, v1, reinterpret_cast<uint32_t*>(ws + L.kb), ints(L.vb),
+      ints(L.seg_lo), ints(L.seg_hi), reinterpret_cast<unsigned long long*>(ws + L.pref),
+      ints(L.posS), ints(L.posB), ints(L.mS), ints(L.mB), ints(L.hole), ints(L.dest), ints(L.nseg),
+      reinterpret_cast<unsigned char*>(ws + L.cls), v0);
+  MC_LAUNCH_CHECK();
+  proposal_order_gather_kernel<<<ceil_div(pre, 256), 256, 0, st>>>(v0, pre, boxes, sc, sboxes,
+                                                                   sscores);
+  MC_LAUNCH_CHECK();
+  nms_mask_kernel<<<dim3(nb, nb), 64, 0, st>>>(sboxes, pre, nms_thresh, nb, mask);
+  MC_LAUNCH_CHECK();
+  nms_scan_kernel<<<1, 64, sizeof(unsigned long long) * nb, st>>>(mask, pre, nb, post_nms_topn,
+                                                                   kept, num_rois);
+  MC_LAUNCH_CHECK();
+  proposal_gather_kernel<<<ceil_div(post_nms_topn, 256), 256, 0, st>>>(sboxes, sscores, kept,
+                                                                       num_rois, rois, roi_scores);
+  MC_LAUNCH_CHECK();
+  if (tie_flag) {
+    MC_HIP(hipMemcpyAsync(tie_flag, flags, sizeof(int), hipMemcpyDeviceToDevice, st));
+  }
+  return 0;
+}
+
+}  // extern "C"

@@ -54,6 +54,16 @@ LIB.mcNormalize.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_in
 LIB.mcConvTimingCollect.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(c_long),
                                     ctypes.POINTER(ctypes.c_double)]
 
+LIB.mcDetectionOutputWorkspaceSize.argtypes = [c_int, c_int, c_int, c_int, c_int,
+                                               ctypes.POINTER(ctypes.c_size_t)]
+LIB.mcDetectionOutputMaxRows.argtypes = [c_int] * 5
+LIB.mcDetectionOutput.argtypes = [c_void_p, c_void_p, c_void_p] + [c_int] * 8 + \
+    [c_float, c_float, c_float, c_int, c_void_p, ctypes.c_size_t, c_void_p, c_int, c_void_p, c_void_p]
+LIB.mcProposalWorkspaceSize.argtypes = [c_int, c_int, c_int, ctypes.POINTER(ctypes.c_size_t)]
+LIB.mcProposal.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                           c_float, c_int, c_int, c_float, c_void_p, ctypes.c_size_t, c_void_p,
+                           c_void_p, c_void_p, c_void_p, c_void_p]
+
 LIB.mcConvPlanCreate.argtypes = [ctypes.POINTER(ConvGeom), ctypes.POINTER(c_void_p)]
 LIB.mcConvPlanDestroy.argtypes = [c_void_p]
 LIB.mcConvPlanOutputShape.argtypes = [c_void_p, ctypes.POINTER(c_int), ctypes.POINTER(c_int)]

@@ -291,3 +291,160 @@ def softmax(x, axis=1):
     y = np.empty_like(x)
     _lib.orc_softmax(outer, x.shape[axis], inner, _fp(x), _fp(y))
     return y
+
+
+# ---- detection tail (mc_oracle_det.cc) -----------------------------------------
+
+_lib.orc_normalize.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, c_float_p, c_float_p,
+                               ctypes.c_int, ctypes.c_int, ctypes.c_float, c_float_p]
+_lib.orc_prior_box.argtypes = [ctypes.c_int] * 4 + [c_float_p, ctypes.c_int, c_float_p, ctypes.c_int,
+                                                    c_float_p, ctypes.c_int, c_float_p, ctypes.c_int,
+                                                    ctypes.c_int, ctypes.c_float, ctypes.c_float,
+                                                    ctypes.c_float, c_float_p]
+_lib.orc_generate_anchors.argtypes = [ctypes.c_int, c_float_p, ctypes.c_int, c_float_p, ctypes.c_int,
+                                      c_float_p]
+_lib.orc_generate_proposals.argtypes = [c_float_p, c_float_p, c_float_p, ctypes.c_int, ctypes.c_int,
+                                        ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_float,
+                                        ctypes.c_int, c_float_p]
+_lib.orc_sort_bbox.argtypes = [c_float_p, ctypes.c_int, ctypes.c_int]
+_lib.orc_nms_pixel.argtypes = [ctypes.c_int, c_float_p, ctypes.c_float, ctypes.c_int, c_int_p]
+_lib.orc_proposal.argtypes = [c_float_p, c_float_p, c_float_p, ctypes.c_int, ctypes.c_int,
+                              ctypes.c_int, c_float_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                              ctypes.c_int, ctypes.c_float, c_float_p, c_float_p, c_int_p, c_float_p]
+_lib.orc_detection_output.argtypes = [c_float_p, c_float_p, c_float_p] + [ctypes.c_int] * 8 + \
+    [ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_int, c_float_p, ctypes.c_int]
+
+
+def normalize(x, scale, across_spatial=True, channel_shared=True, eps=1e-10):
+    x, scale = _f32(x), _f32(scale).reshape(-1)
+    n, c = x.shape[0], x.shape[1]
+    y = np.empty_like(x)
+    _lib.orc_normalize(n, c, x.size // (n * c), _fp(x), _fp(scale), int(across_spatial),
+                       int(channel_shared), eps, _fp(y))
+    return y
+
+
+def _as_list(v):
+    if v is None:
+        return []
+    return list(v) if isinstance(v, (list, tuple)) else [v]
+
+
+def prior_box_aspect_ratios(param):
+    """The list PriorBoxLayer::LayerSetUp builds (prior_box_layer.cpp:21-37)."""
+    ars = [np.float32(1.0)]
+    flip = param.get("flip", True)
+    for ar in _as_list(param.get("aspect_ratio")):
+        ar = np.float32(ar)
+        if any(abs(float(ar) - float(a)) < 1e-6 for a in ars):
+            continue
+        ars.append(ar)
+        if flip:
+            ars.append(np.float32(1.0 / float(ar)))
+    return np.array(ars, np.float32)
+
+
+def prior_box(param, feat_shape, img_shape):
+    mins = _f32(_as_list(param["min_size"]))
+    maxs = _f32(_as_list(param.get("max_size")))
+    ars = prior_box_aspect_ratios(param)
+    var = _f32(_as_list(param.get("variance")) or [0.1])
+    lh, lw = feat_shape[2], feat_shape[3]
+    if "img_size" in param:
+        ih = iw = int(param["img_size"])
+    elif "img_h" in param:
+        ih, iw = int(param["img_h"]), int(param["img_w"])
+    else:
+        ih, iw = img_shape[2], img_shape[3]
+    if "step" in param:
+        sh = sw = float(param["step"])
+    else:
+        sh, sw = float(param.get("step_h", 0)), float(param.get("step_w", 0))
+    num_priors = len(ars) * len(mins) + len(maxs)
+    dim = lh * lw * num_priors * 4
+    out = np.empty((1, 2, dim), np.float32)
+    _lib.orc_prior_box(lh, lw, ih, iw, _fp(mins), len(mins), _fp(maxs) if len(maxs) else None,
+                       len(maxs), _fp(ars), len(ars), _fp(var), len(var), int(param.get("clip", False)),
+                       sh, sw, float(param.get("offset", 0.5)), _fp(out))
+    return out
+
+
+def generate_anchors(base_size=16, ratios=(0.5, 1, 2), scales=(8, 16, 32)):
+    r, s = _f32(ratios), _f32(scales)
+    out = np.empty((len(r) * len(s), 4), np.float32)
+    _lib.orc_generate_anchors(base_size, _fp(r), len(r), _fp(s), len(s), _fp(out))
+    return out
+
+
+def generate_proposals(fg_scores, bbox, anchors, im_h, im_w, min_bbox_size, feat_stride):
+    fg_scores, bbox, anchors = _f32(fg_scores), _f32(bbox), _f32(anchors)
+    A, (H, W) = anchors.shape[0], fg_scores.shape[-2:]
+    out = np.empty((A * H * W, 5), np.float32)
+    _lib.orc_generate_proposals(_fp(fg_scores), _fp(bbox), _fp(anchors), A, H, W, im_h, im_w,
+                                min_bbox_size, feat_stride, _fp(out))
+    return out
+
+
+def sort_bbox(rois, num_top):
+    rois = _f32(rois).copy()
+    _lib.orc_sort_bbox(_fp(rois), rois.shape[0], num_top)
+    return rois
+
+
+def nms_pixel(proposals, thr, max_rois):
+    proposals = _f32(proposals)
+    kept = np.empty(max_rois, np.int32)
+    n = _lib.orc_nms_pixel(proposals.shape[0], _fp(proposals), thr, max_rois,
+                           kept.ctypes.data_as(c_int_p))
+    return kept[:n].copy()
+
+
+def proposal(param, scores, bbox, im_info, ntop=1, details=False):
+    """ProposalLayer forward.  Returns [rois] or [rois, scores]; with details=True
+    also the kept indices (positions in the sorted table) and the sorted table."""
+    scores, bbox, im_info = _f32(scores), _f32(bbox), _f32(im_info).reshape(-1)
+    assert scores.shape[0] == 1, "Only support single scale."
+    ratios = _as_list(param.get("ratio")) or [0.5, 1, 2]
+    scales = _as_list(param.get("scale")) or [8, 16, 32]
+    anchors = generate_anchors(int(param.get("base_size", 16)), ratios, scales)
+    A, H, W = anchors.shape[0], scores.shape[2], scores.shape[3]
+    post = int(param.get("post_nms_topn", 300))
+    rois = np.empty((post, 5), np.float32)
+    rs = np.empty(post, np.float32)
+    kept = np.empty(post, np.int32)
+    table = np.empty((A * H * W, 5), np.float32)
+    r = _lib.orc_proposal(_fp(scores), _fp(bbox), _fp(im_info), A, H, W, _fp(anchors),
+                          int(param.get("feat_stride", 16)), int(param.get("min_size", 16)),
+                          int(param.get("pre_nms_topn", 6000)), post,
+                          float(param.get("nms_thresh", 0.7)), _fp(rois), _fp(rs),
+                          kept.ctypes.data_as(c_int_p), _fp(table))
+    tops = [rois[:r].copy()] + ([rs[:r].copy()] if ntop > 1 else [])
+    if details:
+        return tops, kept[:r].copy(), table
+    return tops
+
+
+_CODE = {"CORNER": 1, "CENTER_SIZE": 2, "CORNER_SIZE": 3}
+
+
+def detection_output(param, loc, conf, prior):
+    loc, conf, prior = _f32(loc), _f32(conf), _f32(prior)
+    num = loc.shape[0]
+    num_classes = int(param["num_classes"])
+    share = bool(param.get("share_location", True))
+    num_priors = prior.shape[2] // 4
+    nms = param.get("nms_param", {})
+    max_rows = max(num, num * num_priors * num_classes)
+    keep = int(param.get("keep_top_k", -1))
+    if keep > -1:
+        max_rows = max(num, min(max_rows, num * max(keep, num_classes * max(1, int(nms.get("top_k", num_priors))))))
+    out = np.empty((max_rows, 7), np.float32)
+    n = _lib.orc_detection_output(
+        _fp(loc), _fp(conf), _fp(prior), num, num_priors, num_classes, int(share),
+        int(param.get("background_label_id", 0)), _CODE[str(param.get("code_type", "CORNER"))],
+        int(param.get("variance_encoded_in_target", False)), keep,
+        float(param.get("confidence_threshold", -3.4028234663852886e38)),
+        float(nms.get("nms_threshold", 0.3)), float(nms.get("eta", 1.0)), int(nms.get("top_k", -1)),
+        _fp(out), max_rows)
+    assert n >= 0, "detection_output: row buffer too small"
+    return out[:n].copy()
