@@ -400,6 +400,12 @@ class BatchNormLayer : public Layer {
   bool IsChannelStage(int channels) const override {
     return use_global_stats_ && channels == channels_;
   }
+  // When it runs as its own pass, an in-place Scale/Bias and activation that
+  // follow ride along in that pass (the WGAN generator's BatchNorm with batch
+  // statistics -> Scale -> ReLU becomes statistics + one pass).
+  bool AcceptsEpilogue() const override { return true; }
+  int MaxAffineFollowers() const override { return 1; }
+  void SetEpilogue(const vector<Layer*>& followers) override { followers_ = followers; }
   uint64_t ChannelStageVersion() const override {
     return (BlobVersion(blobs_[0]) * 31 + BlobVersion(blobs_[1])) * 31 + BlobVersion(blobs_[2]);
   }
@@ -431,11 +437,15 @@ class BatchNormLayer : public Layer {
                                      cur_stream()));
       stats_version_ = ~0ull;
     }
-    mcChannelOp op = {mean_.gpu_data(), stdev_.gpu_data(), nullptr, nullptr, MC_ACT_NONE, 0.f};
+    mcChannelOp op = {nullptr, nullptr, nullptr, nullptr, MC_ACT_NONE, 0.f};
+    for (Layer* f : followers_) f->GetChannelStage(&op);  // fills mul / add / activation
+    op.sub = mean_.gpu_data();
+    op.div = stdev_.gpu_data();
     MC_CHECK(mcChannelTransform(bottom[0]->gpu_data(), top[0]->mutable_gpu_data(), num, channels_,
                                 spatial, &op, cur_stream()));
   }
 
+  vector<Layer*> followers_;
   bool use_global_stats_ = true;
   int channels_ = 0;
   float eps_ = 1e-5f;

@@ -195,12 +195,9 @@ void Net::PlanFusion() {
   fusion_dirty_ = false;
   layer_fused_.assign(layers_.size(), 0);
   for (size_t i = 0; i < layers_.size(); ++i) {
-    if (!layers_[i]->AcceptsEpilogue()) continue;
+    if (layer_fused_[i] || !layers_[i]->AcceptsEpilogue()) continue;
     vector<Layer*> followers;
-    const bool in_place = std::find(bottom_vecs_[i].begin(), bottom_vecs_[i].end(),
-                                    top_vecs_[i].empty() ? nullptr : top_vecs_[i][0]) !=
-                          bottom_vecs_[i].end();
-    if (top_vecs_[i].size() == 1 && !in_place && top_vecs_[i][0]->num_axes() >= 2) {
+    if (top_vecs_[i].size() == 1 && top_vecs_[i][0]->num_axes() >= 2) {
       Blob* t = top_vecs_[i][0];
       const int channels = t->shape(1);
       size_t j = i + 1;

@@ -198,3 +198,170 @@ def conv_flops(spec, inputs):
             for name in layer["top"]:
                 shapes[name] = b[0]
     return total
+
+
+def rpn_spec(seed=0, feat_shape=(1, 1024, 38, 63), im_info=(600.0, 1000.0, 1.0), std=0.01,
+             pre_nms_topn=6000, post_nms_topn=300, nms_thresh=0.7, mid=512):
+    """Config 4: region-proposal stage of a Faster R-CNN / R-FCN detector on a
+    stride-16 feature map: 3x3 conv + ReLU, 1x1 score and box heads for 9 anchors,
+    2-way softmax over (background, foreground), Proposal."""
+    n, c, h, w = feat_shape
+    A = 9
+    spec = [input_layer({"feat": feat_shape, "im_info": (1, 3)}),
+            conv_layer("rpn_conv/3x3", "feat", "rpn/output", c, mid, 3, pad=1, seed=seed, std=std),
+            relu_layer("rpn_relu/3x3", "rpn/output"),
+            conv_layer("rpn_cls_score", "rpn/output", "rpn_cls_score", mid, 2 * A, 1, seed=seed,
+                       std=std),
+            conv_layer("rpn_bbox_pred", "rpn/output", "rpn_bbox_pred", mid, 4 * A, 1, seed=seed,
+                       std=std),
+            {"name": "rpn_cls_score_reshape", "type": "Reshape", "bottom": ["rpn_cls_score"],
+             "top": ["rpn_cls_score_reshape"], "reshape_param": {"shape": {"dim": [0, 2, -1, 0]}}},
+            {"name": "rpn_cls_prob", "type": "Softmax", "bottom": ["rpn_cls_score_reshape"],
+             "top": ["rpn_cls_prob"]},
+            {"name": "rpn_cls_prob_reshape", "type": "Reshape", "bottom": ["rpn_cls_prob"],
+             "top": ["rpn_cls_prob_reshape"],
+             "reshape_param": {"shape": {"dim": [0, 2 * A, -1, 0]}}},
+            {"name": "proposal", "type": "Proposal",
+             "bottom": ["rpn_cls_prob_reshape", "rpn_bbox_pred", "im_info"], "top": ["rois"],
+             "proposal_param": {"feat_stride": 16, "base_size": 16, "min_size": 16,
+                                "ratio": [0.5, 1.0, 2.0], "scale": [8.0, 16.0, 32.0],
+                                "pre_nms_topn": pre_nms_topn, "post_nms_topn": post_nms_topn,
+                                "nms_thresh": nms_thresh}}]
+    x = np.random.default_rng(seed + 1).standard_normal(feat_shape).astype(np.float32)
+    return spec, {"feat": x, "im_info": np.array([im_info], np.float32)}
+
+
+def dcgan_spec(batch=128, seed=0, zdim=100, base=1024, use_global_stats=False, std=0.02):
+    """Config 5: DCGAN/WGAN generator: InnerProduct to 4x4xbase, three 4x4 stride-2
+    Deconvolutions halving the channels with BatchNorm + Scale + ReLU, a last one to
+    3 channels with TanH (64x64 output for base 1024)."""
+    spec = [input_layer({"z": (batch, zdim)})]
+    w = (_rng(seed, "fc", "w").standard_normal((base * 16, zdim)) * std).astype(np.float32)
+    spec.append({"name": "fc", "type": "InnerProduct", "bottom": ["z"], "top": ["fc"],
+                 "inner_product_param": {"num_output": base * 16},
+                 "blobs": [w, np.zeros(base * 16, np.float32)]})
+    spec.append({"name": "fc_reshape", "type": "Reshape", "bottom": ["fc"], "top": ["g0"],
+                 "reshape_param": {"shape": {"dim": [0, base, 4, 4]}}})
+    prev, cin = "g0", base
+    for i in range(1, 4):
+        cout = cin // 2
+        name = "gconv%d" % i
+        spec.append(conv_layer(name, prev, name, cin, cout, 4, stride=2, pad=1, bias=False,
+                               seed=seed, std=std, deconv=True))
+        bn = bn_layer("gbn%d" % i, name, cout, use_global_stats=use_global_stats,
+                      seed=(seed + 11) if use_global_stats else None)
+        if not use_global_stats:
+            bn["blobs"] = [np.zeros(cout, np.float32), np.zeros(cout, np.float32),
+                           np.zeros(1, np.float32)]
+        spec.append(bn)
+        spec.append(scale_layer("gbn%d_scale" % i, name, cout, seed=seed + 13))
+        spec.append(relu_layer("gact%d" % i, name))
+        prev, cin = name, cout
+    spec.append(conv_layer("gconv4", prev, "gconv4", cin, 3, 4, stride=2, pad=1, bias=False,
+                           seed=seed, std=std, deconv=True))
+    spec.append({"name": "gact4", "type": "TanH", "bottom": ["gconv4"], "top": ["gconv4"]})
+    z = np.random.default_rng(seed + 1).standard_normal((batch, zdim)).astype(np.float32)
+    return spec, {"z": z}
+
+
+SSD_SOURCES = [  # (source blob, channels, priors, min_size, max_size, aspect ratios, step)
+    ("conv4_3_norm", 512, 4, 30.0, 60.0, [2.0], 8),
+    ("fc7", 1024, 6, 60.0, 111.0, [2.0, 3.0], 16),
+    ("conv6_2", 512, 6, 111.0, 162.0, [2.0, 3.0], 32),
+    ("conv7_2", 256, 6, 162.0, 213.0, [2.0, 3.0], 64),
+    ("conv8_2", 256, 4, 213.0, 264.0, [2.0], 100),
+    ("conv9_2", 256, 4, 264.0, 315.0, [2.0], 300),
+]
+
+
+def ssd300_spec(batch=8, seed=0, num_classes=21, size=300, width=64):
+    """Config 3: SSD300 on VGG16 (atrous fc6, extra layers conv6-conv9, six multibox
+    heads with 4/6/6/6/4/4 priors, 8732 priors at 300x300), DetectionOutput with
+    NMS 0.45, top_k 400, keep_top_k 200.  `width` scales the channel counts for
+    small test nets (64 is the real model)."""
+    s = width / 64.0
+    ch = lambda c: max(4, int(round(c * s)))  # noqa: E731
+    spec = [input_layer({"data": (batch, 3, size, size)})]
+    prev, cin = "data", 3
+
+    def conv_relu(name, cout, k, stride=1, pad=0, dilation=1):
+        nonlocal prev, cin
+        spec.append(conv_layer(name, prev, name, cin, cout, k, stride, pad, dilation, seed=seed))
+        spec.append(relu_layer("relu" + name[4:] if name.startswith("conv") else name + "_relu",
+                               name))
+        prev, cin = name, cout
+
+    def pool(name, k, stride, pad=0):
+        nonlocal prev
+        p = {"pool": Enum("MAX"), "kernel_size": k, "stride": stride}
+        if pad:
+            p["pad"] = pad
+        spec.append({"name": name, "type": "Pooling", "bottom": [prev], "top": [name],
+                     "pooling_param": p})
+        prev = name
+
+    for blk, (n_conv, c) in enumerate([(2, 64), (2, 128), (3, 256), (3, 512), (3, 512)], 1):
+        for i in range(1, n_conv + 1):
+            conv_relu("conv%d_%d" % (blk, i), ch(c), 3, pad=1)
+        if blk < 5:
+            pool("pool%d" % blk, 2, 2)
+        else:
+            pool("pool5", 3, 1, 1)
+    conv_relu("fc6", ch(1024), 3, pad=6, dilation=6)
+    conv_relu("fc7", ch(1024), 1)
+    conv_relu("conv6_1", ch(256), 1)
+    conv_relu("conv6_2", ch(512), 3, stride=2, pad=1)
+    conv_relu("conv7_1", ch(128), 1)
+    conv_relu("conv7_2", ch(256), 3, stride=2, pad=1)
+    conv_relu("conv8_1", ch(128), 1)
+    conv_relu("conv8_2", ch(256), 3)
+    conv_relu("conv9_1", ch(128), 1)
+    conv_relu("conv9_2", ch(256), 3)
+    c43 = ch(512)
+    spec.append({"name": "conv4_3_norm", "type": "Normalize", "bottom": ["conv4_3"],
+                 "top": ["conv4_3_norm"],
+                 "norm_param": {"across_spatial": False, "channel_shared": False,
+                                "scale_filler": {"type": "constant", "value": 20.0}},
+                 "blobs": [np.full(c43, 20.0, np.float32)]})
+    locs, confs, priors = [], [], []
+    for src, c, npri, mn, mx, ars, step in SSD_SOURCES:
+        c = ch(c)
+        for kind, per in (("loc", 4), ("conf", num_classes)):
+            name = "%s_mbox_%s" % (src, kind)
+            spec.append(conv_layer(name, src, name, c, npri * per, 3, pad=1, seed=seed))
+            spec.append({"name": name + "_perm", "type": "Permute", "bottom": [name],
+                         "top": [name + "_perm"], "permute_param": {"order": [0, 2, 3, 1]}})
+            spec.append({"name": name + "_flat", "type": "Flatten", "bottom": [name + "_perm"],
+                         "top": [name + "_flat"], "flatten_param": {"axis": 1}})
+            (locs if kind == "loc" else confs).append(name + "_flat")
+        pname = "%s_mbox_priorbox" % src
+        spec.append({"name": pname, "type": "PriorBox", "bottom": [src, "data"], "top": [pname],
+                     "prior_box_param": {"min_size": mn, "max_size": mx, "aspect_ratio": ars,
+                                         "flip": True, "clip": False,
+                                         "variance": [0.1, 0.1, 0.2, 0.2], "step": float(step),
+                                         "offset": 0.5}})
+        priors.append(pname)
+    spec.append({"name": "mbox_loc", "type": "Concat", "bottom": locs, "top": ["mbox_loc"],
+                 "concat_param": {"axis": 1}})
+    spec.append({"name": "mbox_conf", "type": "Concat", "bottom": confs, "top": ["mbox_conf"],
+                 "concat_param": {"axis": 1}})
+    spec.append({"name": "mbox_priorbox", "type": "Concat", "bottom": priors,
+                 "top": ["mbox_priorbox"], "concat_param": {"axis": 2}})
+    spec.append({"name": "mbox_conf_reshape", "type": "Reshape", "bottom": ["mbox_conf"],
+                 "top": ["mbox_conf_reshape"],
+                 "reshape_param": {"shape": {"dim": [0, -1, num_classes]}}})
+    spec.append({"name": "mbox_conf_softmax", "type": "Softmax", "bottom": ["mbox_conf_reshape"],
+                 "top": ["mbox_conf_softmax"], "softmax_param": {"axis": 2}})
+    spec.append({"name": "mbox_conf_flatten", "type": "Flatten", "bottom": ["mbox_conf_softmax"],
+                 "top": ["mbox_conf_flatten"], "flatten_param": {"axis": 1}})
+    spec.append({"name": "detection_out", "type": "DetectionOutput",
+                 "bottom": ["mbox_loc", "mbox_conf_flatten", "mbox_priorbox"],
+                 "top": ["detection_out"],
+                 "detection_output_param": {
+                     "num_classes": num_classes, "share_location": True,
+                     "background_label_id": 0,
+                     "nms_param": {"nms_threshold": 0.45, "top_k": 400},
+                     "code_type": Enum("CENTER_SIZE"), "keep_top_k": 200,
+                     "confidence_threshold": 0.01}})
+    x = np.random.default_rng(seed + 1).uniform(-1, 1, (batch, 3, size, size)).astype(np.float32)
+    return spec, {"data": x}

@@ -186,3 +186,141 @@ def test_resnet50_b64_properties(gpu_mode):
     net.forward(data=x[17:18])
     p1 = net.get_blob("prob").data.copy()
     assert np.abs(p1[0] - p64[17]).max() < 1e-6
+
+
+def test_config4_rpn_proposal_full_size(gpu_mode):
+    """RPN head + Proposal at the benchmark size (1x1024x38x63, 21 546 anchors ->
+    top 6000 -> NMS 0.7 -> 300).  The dense part is compared within tolerance; the
+    tail is compared bit for bit on identical tail inputs (the blobs the device
+    produced), which is the only well-posed form of "same kept indices"."""
+    from minicaffe import zoo
+    oracle.use_openblas(True)
+    try:
+        spec, inputs = zoo.rpn_spec()
+        net = run_net(gpu_mode, spec, inputs, ["rpn_cls_prob_reshape", "rpn_bbox_pred"])
+        want = netrun.oracle_forward(spec[:-1], inputs)
+    finally:
+        oracle.use_openblas(False)
+    prob = net.get_blob("rpn_cls_prob_reshape").data.copy()
+    bbox = net.get_blob("rpn_bbox_pred").data.copy()
+    # two stacked contractions, the first with K = 9216: summation-order noise alone
+    # is above 1e-4 here, so the multi-layer tolerance applies
+    assert netrun.rel_err(prob, want["rpn_cls_prob_reshape"]) < 1e-3
+    assert netrun.rel_err(bbox, want["rpn_bbox_pred"]) < 1e-3
+    rois = net.get_blob("rois").data.copy()
+    (ref_rois,), kept, table = oracle.proposal(spec[-1]["proposal_param"], prob, bbox,
+                                               inputs["im_info"], 1, details=True)
+    assert rois.shape == ref_rois.shape and rois.shape[0] <= 300 and rois.shape[1] == 5
+    assert np.array_equal(rois, ref_rois)
+    # NMS invariants on the result itself: kept boxes are pairwise below the threshold
+    b = rois[:, 1:]
+    area = (b[:, 2] - b[:, 0] + 1) * (b[:, 3] - b[:, 1] + 1)
+    for i in range(min(50, len(b))):
+        xx1, yy1 = np.maximum(b[i, 0], b[:, 0]), np.maximum(b[i, 1], b[:, 1])
+        xx2, yy2 = np.minimum(b[i, 2], b[:, 2]), np.minimum(b[i, 3], b[:, 3])
+        inter = np.maximum(0, xx2 - xx1 + 1) * np.maximum(0, yy2 - yy1 + 1)
+        iou = inter / (area[i] + area - inter)
+        iou[i] = 0
+        assert iou.max() <= 0.7 + 1e-6
+
+
+def test_proposal_layer_with_score_ties_and_two_tops(gpu_mode):
+    """Quantised scores force ties inside the top-N prefix: the device must replay
+    the reference's quicksort order.  Also the optional second top (scores)."""
+    from minicaffe.craft import input_layer
+    rng = np.random.default_rng(5)
+    A, H, W = 9, 14, 17
+    spec = [input_layer({"prob": (1, 2 * A, H, W), "bbox": (1, 4 * A, H, W), "im_info": (1, 3)}),
+            {"name": "proposal", "type": "Proposal", "bottom": ["prob", "bbox", "im_info"],
+             "top": ["rois", "scores"],
+             "proposal_param": {"pre_nms_topn": 1500, "post_nms_topn": 80, "nms_thresh": 0.6,
+                                "min_size": 24}}]
+    prob = (np.round(rng.random((1, 2 * A, H, W)) * 40) / 40).astype(np.float32)
+    bbox = (rng.standard_normal((1, 4 * A, H, W)) * 0.4).astype(np.float32)
+    inputs = {"prob": prob, "bbox": bbox, "im_info": np.array([[H * 16, W * 16, 1.5]], np.float32)}
+    net = run_net(gpu_mode, spec, inputs)
+    ref = oracle.proposal(spec[1]["proposal_param"], prob, bbox, inputs["im_info"], 2)
+    assert np.array_equal(net.get_blob("rois").data, ref[0])
+    assert np.array_equal(net.get_blob("scores").data, ref[1])
+
+
+@pytest.mark.parametrize("use_global_stats", [False, True])
+def test_config5_dcgan_generator_full_size(gpu_mode, use_global_stats):
+    """DCGAN generator at batch 128: InnerProduct, Reshape, three stride-2
+    Deconvolutions with BatchNorm (batch statistics as in the reference's WGAN
+    graph, and stored statistics) + Scale + ReLU, Deconvolution + TanH."""
+    from minicaffe import zoo
+    oracle.use_openblas(True)
+    try:
+        spec, inputs = zoo.dcgan_spec(batch=128, use_global_stats=use_global_stats)
+        net = run_net(gpu_mode, spec, inputs, ["g0", "gconv1", "gconv3"])
+        want = netrun.oracle_forward(spec, inputs, keep={"g0", "gconv1", "gconv3", "gconv4"})
+    finally:
+        oracle.use_openblas(False)
+    for name in ("g0", "gconv1", "gconv3", "gconv4"):
+        got = net.get_blob(name).data
+        assert got.shape == want[name].shape
+        assert netrun.rel_err(got, want[name]) < 1e-3, name
+    out = net.get_blob("gconv4").data
+    assert out.shape == (128, 3, 64, 64) and np.abs(out).max() <= 1.0
+
+
+def _check_ssd_tail(net, spec):
+    """DetectionOutput rows of the device against the oracle run on the device's own
+    mbox_loc / softmaxed confidences / priors: must be identical."""
+    loc = net.get_blob("mbox_loc").data.copy()
+    conf = net.get_blob("mbox_conf_flatten").data.copy()
+    prior = net.get_blob("mbox_priorbox").data.copy()
+    want = oracle.detection_output(spec[-1]["detection_output_param"], loc, conf, prior)
+    got = net.get_blob("detection_out").data.copy()
+    assert got.shape == want.shape
+    assert np.array_equal(got, want)
+    return got
+
+
+def test_config3_ssd_small_width_every_stage(gpu_mode):
+    """The SSD300 graph (all 102 layers, 300x300 input, 8732 priors) at 1/4 width so
+    the CPU oracle can walk all of it: dilated fc6, Normalize, Permute / Flatten /
+    Concat, PriorBox, Reshape + Softmax(axis 2), DetectionOutput."""
+    from minicaffe import zoo
+    oracle.use_openblas(True)
+    try:
+        spec, inputs = zoo.ssd300_spec(batch=2, width=16)
+        marks = ["conv4_3_norm", "fc7", "conv9_2", "mbox_loc", "mbox_conf", "mbox_conf_flatten",
+                 "mbox_priorbox"]
+        net = run_net(gpu_mode, spec, inputs, marks)
+        want = netrun.oracle_forward(spec[:-1], inputs, keep=set(marks))
+    finally:
+        oracle.use_openblas(False)
+    assert np.array_equal(net.get_blob("mbox_priorbox").data, want["mbox_priorbox"])
+    assert want["mbox_priorbox"].shape == (1, 2, 8732 * 4)
+    for name in marks[:-1]:
+        assert netrun.rel_err(net.get_blob(name).data, want[name]) < 1e-3, name
+    rows = _check_ssd_tail(net, spec)
+    assert rows.shape[1] == 7 and rows.shape[0] <= 2 * 200
+
+
+def test_config3_ssd_full_size_b8(gpu_mode):
+    """Benchmark size (VGG16 widths, batch 8): the dense part is checked against the
+    oracle on the first image's source layers, the tail bit for bit on all 8 images."""
+    from minicaffe import zoo
+    spec, inputs = zoo.ssd300_spec(batch=8)
+    net = run_net(gpu_mode, spec, inputs, ["mbox_loc", "mbox_conf_flatten", "mbox_priorbox", "fc7"])
+    rows = _check_ssd_tail(net, spec)
+    assert set(np.unique(rows[:, 0]).astype(int)) <= set(range(8))
+    counts = np.bincount(rows[:, 0].astype(int), minlength=8)
+    assert counts.max() <= 200
+    # labels ascending within an image, scores descending within a label
+    for i in range(8):
+        r = rows[rows[:, 0] == i]
+        assert (np.diff(r[:, 1]) >= 0).all()
+        for lab in np.unique(r[:, 1]):
+            assert (np.diff(r[r[:, 1] == lab][:, 2]) <= 0).all()
+    fc7_gpu = net.get_blob("fc7").data[:1].copy()
+    oracle.use_openblas(True)
+    try:
+        idx = [i for i, l in enumerate(spec) if l["name"] == "fc7_relu"][0]
+        want = netrun.oracle_forward(spec[:idx + 1], {"data": inputs["data"][:1]}, keep={"fc7"})
+    finally:
+        oracle.use_openblas(False)
+    assert netrun.rel_err(fc7_gpu, want["fc7"]) < 1e-3
