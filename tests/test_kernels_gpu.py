@@ -236,3 +236,108 @@ def test_copy2d_and_fill(K):
     torch.cuda.synchronize()
     got = yd.cpu().numpy()
     assert np.array_equal(got[:, 10:43], x) and np.all(got[0, :5] == 2.5) and np.all(got[1:, :10] == 0)
+
+
+def test_normalize(K):
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((2, 12, 5, 7)).astype(np.float32)
+    for across, shared in ((0, 0), (0, 1), (1, 0), (1, 1)):
+        s = (rng.random(1 if shared else 12) + 0.5).astype(np.float32)
+        want = oracle.normalize(x, s, bool(across), bool(shared), 1e-10)
+        xd, sd, yd = dev(x), dev(s), torch.empty(x.shape, device="cuda")
+        K.check_mc(K.LIB.mcNormalize(fptr(xd), fptr(yd), 2, 12, 35, across, shared, ctypes.c_float(1e-10),
+                                     fptr(sd), None))
+        torch.cuda.synchronize()
+        assert np.abs(yd.cpu().numpy() - want).max() < 1e-6
+
+
+def run_proposal(K, scores, bbox, im_info, param):
+    anchors = oracle.generate_anchors()
+    A, H, W = 9, scores.shape[2], scores.shape[3]
+    pre, post = param["pre_nms_topn"], param["post_nms_topn"]
+    sz = ctypes.c_size_t()
+    K.check_mc(K.LIB.mcProposalWorkspaceSize(A * H * W, pre, post, ctypes.byref(sz)))
+    ws = torch.empty(sz.value, dtype=torch.uint8, device="cuda")
+    sd, bd, idv, ad = dev(scores), dev(bbox), dev(im_info), dev(anchors)
+    rois = torch.full((post, 5), float("nan"), device="cuda")
+    rs = torch.zeros(post, device="cuda")
+    cnt = torch.zeros(2, dtype=torch.int32, device="cuda")
+    K.check_mc(K.LIB.mcProposal(fptr(sd), fptr(bd), fptr(idv), fptr(ad), A, H, W, 16,
+                                ctypes.c_float(param.get("min_size", 16)), pre, post,
+                                ctypes.c_float(param["nms_thresh"]), fptr(ws), sz.value, fptr(rois),
+                                fptr(rs), ctypes.c_void_p(cnt.data_ptr()),
+                                ctypes.c_void_p(cnt.data_ptr() + 4), None))
+    torch.cuda.synchronize()
+    n, ties = int(cnt[0].item()), int(cnt[1].item())
+    return rois[:n].cpu().numpy(), rs[:n].cpu().numpy(), ties
+
+
+@pytest.mark.parametrize("hw,pre,post,thr,quant", [
+    ((38, 63), 6000, 300, 0.7, 0),       # config 4 size, tie-free
+    ((38, 63), 6000, 300, 0.7, 2000),    # ties inside the top 6000
+    ((38, 63), 300, 2000, 0.9, 0),       # fewer candidates than post_nms_topn
+    ((10, 12), 2000, 50, 0.5, 0),        # pre_nms_topn > proposals: zero-score ties
+    ((20, 20), 6000, 300, 0.7, 7),       # heavy ties
+    ((5, 4), 100, 300, 0.3, 0),
+])
+def test_proposal_bit_exact(K, hw, pre, post, thr, quant):
+    """Kept rois and scores equal the CPU path's bit for bit, with and without
+    score ties (ties replay the reference's quicksort on the device)."""
+    rng = np.random.default_rng(11)
+    A, (H, W) = 9, hw
+    n = A * H * W
+    scores = rng.random((1, 2 * A, H, W)).astype(np.float32)
+    scores[0, A:] = (rng.permutation(n).astype(np.float32) / n * 0.9 + 0.05).reshape(A, H, W)
+    if quant:
+        scores[0, A:] = np.round(scores[0, A:] * quant) / quant
+    bbox = (rng.standard_normal((1, 4 * A, H, W)) * 0.3).astype(np.float32)
+    im_info = np.array([H * 16, W * 16, 1.0], np.float32)
+    param = {"pre_nms_topn": pre, "post_nms_topn": post, "nms_thresh": thr}
+    want_rois, want_scores = oracle.proposal(param, scores, bbox, im_info, 2)
+    rois, rs, ties = run_proposal(K, scores, bbox, im_info, param)
+    assert np.array_equal(rois, want_rois)
+    assert np.array_equal(rs, want_scores)
+    if quant:
+        assert ties == 1
+
+
+@pytest.mark.parametrize("num,P,C,share,code,keep,thr,nms,eta,topk,sigma", [
+    (2, 64, 4, True, "CENTER_SIZE", 10, 0.01, 0.45, 1.0, 20, 2.0),
+    (8, 8732, 21, True, "CENTER_SIZE", 200, 0.01, 0.45, 1.0, 400, 2.0),   # config 3 tail, logits N(0, sigma=2)
+    (3, 500, 5, False, "CORNER", -1, None, 0.3, 1.0, None, 2.0),          # per-class boxes, no limits
+    (2, 300, 6, True, "CORNER_SIZE", 50, 0.05, 0.6, 0.9, 100, 2.0),       # adaptive threshold (eta < 1)
+    (2, 100, 3, True, "CENTER_SIZE", 10, 0.999999, 0.45, 1.0, 20, 2.0),   # nothing kept -> rows of -1
+    (1, 2000, 21, True, "CENTER_SIZE", 200, 0.01, 0.45, 1.0, 400, 0.5),
+])
+def test_detection_output_bit_exact(K, num, P, C, share, code, keep, thr, nms, eta, topk, sigma):
+    rng = np.random.default_rng(12)
+    lc = 1 if share else C
+    loc = (rng.standard_normal((num, P * lc * 4)) * 0.5).astype(np.float32)
+    conf = oracle.softmax((rng.standard_normal((num, P, C)) * sigma).astype(np.float32), 2).reshape(num, P * C)
+    c = rng.random((P, 2)) * 0.8 + 0.1
+    wh = rng.random((P, 2)) * 0.3 + 0.05
+    prior = np.concatenate([np.concatenate([c - wh / 2, c + wh / 2], 1).reshape(-1),
+                            np.tile([0.1, 0.1, 0.2, 0.2], P)]).reshape(1, 2, P * 4).astype(np.float32)
+    param = {"num_classes": C, "share_location": share, "background_label_id": 0, "code_type": code,
+             "keep_top_k": keep, "nms_param": {"nms_threshold": nms, "eta": eta}}
+    if thr is not None:
+        param["confidence_threshold"] = thr
+    if topk is not None:
+        param["nms_param"]["top_k"] = topk
+    want = oracle.detection_output(param, loc, conf, prior)
+    tk = -1 if topk is None else topk
+    sz = ctypes.c_size_t()
+    K.check_mc(K.LIB.mcDetectionOutputWorkspaceSize(num, P, C, int(share), tk, ctypes.byref(sz)))
+    max_rows = K.LIB.mcDetectionOutputMaxRows(num, P, C, tk, keep)
+    ws = torch.empty(sz.value, dtype=torch.uint8, device="cuda")
+    ld, cd, pd = dev(loc), dev(conf), dev(prior)
+    out = torch.full((max_rows, 7), float("nan"), device="cuda")
+    cnt = torch.zeros(1, dtype=torch.int32, device="cuda")
+    K.check_mc(K.LIB.mcDetectionOutput(
+        fptr(ld), fptr(cd), fptr(pd), num, P, C, int(share), 0, {"CORNER": 1, "CENTER_SIZE": 2, "CORNER_SIZE": 3}[code],
+        0, keep, ctypes.c_float(-3.4028234663852886e38 if thr is None else thr), ctypes.c_float(nms),
+        ctypes.c_float(eta), tk, fptr(ws), sz.value, fptr(out), max_rows, ctypes.c_void_p(cnt.data_ptr()), None))
+    torch.cuda.synchronize()
+    got = out[:int(cnt.item())].cpu().numpy()
+    assert got.shape == want.shape
+    assert np.array_equal(got, want)
