@@ -108,6 +108,12 @@ const char* mcConvPlanKernelName(const mcConvPlan* plan, int num);
  * -1 restores the automatic choice.  No counterpart in the reference. */
 int mcConvPlanForceConfig(mcConvPlan* plan, int config);
 
+/* Tuning/test knob: pin the number of K slices a launch is cut into (the
+ * slices' partial sums are added in slice order by a second kernel that also
+ * applies the epilogue); 0 restores the automatic choice, which slices only
+ * launches too small to fill the GPU.  No counterpart in the reference. */
+int mcConvPlanForceSplit(mcConvPlan* plan, int slices);
+
 
 /* Measurement hook (no counterpart in the reference): while enabled on the
  * calling thread, every contraction kernel launch is bracketed by two HIP events

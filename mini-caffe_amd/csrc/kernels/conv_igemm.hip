@@ -59,6 +59,8 @@ struct IgemmArgs {
   int y_nstride;      // Cout*Ho*Wo
   int out_sh, out_sw, out_oh, out_ow;  // top row = qh*out_sh + out_oh
   int MT, NT;         // tile counts
+  int kt_per_split;   // K tiles per blockIdx.z slice (split-K)
+  int split_stride;   // elements between the partial outputs of two slices
   int act;
   float slope;
 };
@@ -140,10 +142,15 @@ __global__ __launch_bounds__(256) void igemm_kernel(const IgemmArgs a) {
     }
   }
   const int KT = a.Kpad / BK;
+  // Split-K: slice z multiplies K tiles [kt_begin, kt_end) and writes its
+  // partial sums into its own copy of the top blob.
+  const int kt_begin = blockIdx.z * a.kt_per_split;
+  const int kt_end = min(KT, kt_begin + a.kt_per_split);
   // Packed filter: [g][K tile][m][16 k], so an A tile is one contiguous run.
   const float* __restrict__ wt_tile =
       a.wt + ((size_t)g * KT * a.Mpad + (size_t)mt * BM) * BK;
   const size_t wt_kt_stride = (size_t)a.Mpad * BK;
+  float* __restrict__ yout = a.y + (size_t)blockIdx.z * a.split_stride;
 
   float4 areg[A_VEC];
   float4 breg[B_Q];
@@ -228,20 +235,21 @@ __global__ __launch_bounds__(256) void igemm_kernel(const IgemmArgs a) {
   const int l32 = lane & 31;
   const int lhi = lane >> 5;
 
-  if (KT > 0) {
-    MC_LOAD_TILES(0);
+  if (kt_end > kt_begin) {
+    MC_LOAD_TILES(kt_begin);
     MC_STORE_TILES(0);
     __syncthreads();
-    for (int kt = 0; kt < KT - 1; ++kt) {
-      const int buf = kt & 1;
+    int buf = 0;
+    for (int kt = kt_begin; kt < kt_end - 1; ++kt) {
       MC_LOAD_TILES(kt + 1);
       __builtin_amdgcn_sched_barrier(0);  // keep the global loads ahead of the MFMA block
       MC_COMPUTE(buf);
       __builtin_amdgcn_sched_barrier(0);
       MC_STORE_TILES(buf ^ 1);
       __syncthreads();
+      buf ^= 1;
     }
-    MC_COMPUTE((KT - 1) & 1);
+    MC_COMPUTE(buf);
   }
 #undef MC_GATHER1
 #undef MC_LOAD_TILES
@@ -276,10 +284,62 @@ __global__ __launch_bounds__(256) void igemm_kernel(const IgemmArgs a) {
           if (has_shift) v += a.shift[c];
           const int yo = ybase + c * a.y_cstride;
           if (has_res) v += a.residual[yo];
-          a.y[yo] = apply_act(v, a.act, a.slope);
+          yout[yo] = apply_act(v, a.act, a.slope);
         }
       }
     }
+  }
+}
+
+// Split-K tail: y = act((sum over slices, in slice order) * scale[c] + shift[c]
+// + residual), c = (i / cstride) % C.  One thread per four consecutive elements.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(
+    const float* __restrict__ part, int slices, long slice_stride, long count,
+    float* __restrict__ y, const float* __restrict__ scale, const float* __restrict__ shift,
+    const float* __restrict__ residual, int cstride, int C, int act, float slope) {
+  const long i4 = (blockIdx.x * (long)blockDim.x + threadIdx.x) * 4;
+  if (i4 >= count) return;
+  float v[4];
+  if (i4 + 4 <= count) {
+    float4 s = *reinterpret_cast<const float4*>(part + i4);
+    for (int z = 1; z < slices; ++z) {
+      const float4 t = *reinterpret_cast<const float4*>(part + z * slice_stride + i4);
+      s.x += t.x;
+      s.y += t.y;
+      s.z += t.z;
+      s.w += t.w;
+    }
+    v[0] = s.x;
+    v[1] = s.y;
+    v[2] = s.z;
+    v[3] = s.w;
+  } else {
+    for (int e = 0; e < 4; ++e) {
+      v[e] = 0.f;
+      if (i4 + e < count) {
+        v[e] = part[i4 + e];
+        for (int z = 1; z < slices; ++z) v[e] += part[z * slice_stride + i4 + e];
+      }
+    }
+  }
+  const bool full = i4 + 4 <= count;
+  float4 res = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (residual && full) res = *reinterpret_cast<const float4*>(residual + i4);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const long i = i4 + e;
+    if (i >= count) break;
+    const int c = static_cast<int>((i / cstride) % C);
+    float r = v[e];
+    if (scale) r *= scale[c];
+    if (shift) r += shift[c];
+    if (residual) r += full ? f4at(res, e) : residual[i];
+    v[e] = apply_act(r, act, slope);
+  }
+  if (full) {
+    *reinterpret_cast<float4*>(y + i4) = make_float4(v[0], v[1], v[2], v[3]);
+  } else {
+    for (int e = 0; e < 4 && i4 + e < count; ++e) y[i4 + e] = v[e];
   }
 }
 
@@ -349,6 +409,7 @@ struct mcConvPlan {
   int Mpad = 0;
   int wm_stride = 0, wg_stride = 0;
   int forced_config = -1;
+  int forced_split = 0;  // 0 = choose, >= 1 = this many K slices
   std::vector<SubProblem> subs;
 };
 
@@ -380,6 +441,49 @@ int pick_config(const mcConvPlan* plan, long pixels) {
   }
   for (int i = 0; i < kNumConfigs; ++i)
     if (kConfigs[i].bm == bm && kConfigs[i].bn == bn) return i;
+  return 0;
+}
+
+// K slices for one launch.  A layer with few output tiles leaves most of the
+// 8 workgroup slots per CU empty, and a lone workgroup pays the full global
+// load latency on every K tile; slicing K brings the launch up to about one
+// full round of workgroups, each slice still long enough to amortise its
+// prologue and the extra pass that sums the slices.
+int pick_split(const mcConvPlan* plan, long blocks, int KT) {
+  if (plan->forced_split >= 1) return std::min(plan->forced_split, std::max(KT, 1));
+  if (plan->geom.transposed) return 1;
+  const long slots = 8L * kNumCu;
+  if (blocks * 2 > slots) return 1;
+  int s = static_cast<int>(slots / blocks);
+  s = std::min(s, KT / 8);
+  s = std::min(s, 8);
+  return std::max(s, 1);
+}
+
+// Partial sums of split-K launches: one grow-only buffer per (thread, stream);
+// launches on one stream are ordered, so consecutive layers can share it.
+struct Workspace {
+  float* ptr = nullptr;
+  size_t bytes = 0;
+};
+thread_local std::vector<std::pair<hipStream_t, Workspace>> g_workspaces;
+
+int get_workspace(hipStream_t st, size_t bytes, float** out) {
+  Workspace* ws = nullptr;
+  for (auto& e : g_workspaces)
+    if (e.first == st) ws = &e.second;
+  if (!ws) {
+    g_workspaces.emplace_back(st, Workspace());
+    ws = &g_workspaces.back().second;
+  }
+  if (ws->bytes < bytes) {
+    if (ws->ptr) MC_HIP(hipFree(ws->ptr));  // waits for the device
+    ws->ptr = nullptr;
+    ws->bytes = 0;
+    MC_HIP(hipMalloc(&ws->ptr, bytes));
+    ws->bytes = bytes;
+  }
+  *out = ws->ptr;
   return 0;
 }
 
@@ -578,6 +682,13 @@ int mcConvPlanForceConfig(mcConvPlan* plan, int config) {
   return 0;
 }
 
+int mcConvPlanForceSplit(mcConvPlan* plan, int slices) {
+  MC_REQUIRE(plan, "mcConvPlanForceSplit: null plan");
+  MC_REQUIRE(slices >= 0 && slices <= 64, "mcConvPlanForceSplit: slices out of range");
+  plan->forced_split = slices;
+  return 0;
+}
+
 int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* top,
                   const mcEpilogue* ep, void* stream) {
   MC_REQUIRE(plan && bottom && top, "mcConvForward: null argument");
@@ -629,7 +740,21 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
     a.slope = ep ? ep->negative_slope : 0.f;
     const long blocks = (long)a.MT * a.NT;
     MC_REQUIRE(blocks < (1L << 31), "mcConvForward: grid too large");
-    dim3 grid(static_cast<unsigned>(blocks), g.group, 1);
+    const int KT = s.Kpad / BK;
+    int slices = plan->subs.size() == 1 ? pick_split(plan, blocks * g.group, KT) : 1;
+    a.kt_per_split = ceil_div(std::max(KT, 1), slices);
+    slices = ceil_div(std::max(KT, 1), a.kt_per_split);  // no empty slice
+    a.split_stride = 0;
+    const long slice_stride = (out_count + 3) / 4 * 4;
+    if (slices > 1) {
+      float* ws = nullptr;
+      if (get_workspace(st, sizeof(float) * slice_stride * slices, &ws)) return -1;
+      a.y = ws;
+      a.split_stride = static_cast<int>(slice_stride);
+      a.scale = a.shift = a.residual = nullptr;
+      a.act = MC_ACT_NONE;
+    }
+    dim3 grid(static_cast<unsigned>(blocks), g.group, slices);
     TimedLaunch tl;
     if (g_timing) {
       MC_HIP(hipEventCreate(&tl.start));
@@ -640,6 +765,13 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
     }
     cfg.kernel<<<grid, 256, 0, st>>>(a);
     MC_LAUNCH_CHECK();
+    if (slices > 1) {
+      splitk_reduce_kernel<<<static_cast<unsigned>(ceil_div(out_count, 1024L)), 256, 0, st>>>(
+          a.y, slices, slice_stride, out_count, top, ep ? ep->scale : nullptr,
+          ep ? ep->shift : nullptr, ep ? ep->residual : nullptr, plan->Ho * plan->Wo,
+          g.channels_out, ep ? ep->activation : MC_ACT_NONE, ep ? ep->negative_slope : 0.f);
+      MC_LAUNCH_CHECK();
+    }
     if (g_timing) {
       MC_HIP(hipEventRecord(tl.stop, st));
       g_timed.push_back(tl);

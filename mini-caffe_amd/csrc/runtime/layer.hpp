@@ -90,6 +90,15 @@ class Layer {
   // How many non-activation stages it can absorb (an activation may follow them).
   virtual int MaxAffineFollowers() const { return 0; }
   virtual void SetEpilogue(const vector<Layer*>& followers) {}
+  // Residual folding.  A two-input sum with unit coefficients reports itself
+  // (and the activation it absorbed, if any) so that the layer producing one of
+  // its inputs can add the other in its own epilogue and the sum never runs.
+  virtual bool IsPlainSum() const { return false; }
+  virtual Layer* AbsorbedActivation() const { return nullptr; }
+  // True when the layer's epilogue can still take `+ residual` and an
+  // activation (its own followers end without an activation).
+  virtual bool AcceptsResidual() const { return false; }
+  virtual void SetResidual(Blob* residual, Layer* activation) {}
 
  protected:
   LayerParameter layer_param_;

@@ -77,6 +77,19 @@ class ContractionLayer : public Layer {
   void SetEpilogue(const vector<Layer*>& followers) override {
     followers_ = followers;
     fold_version_ = ~0ull;
+    residual_ = nullptr;
+    residual_act_ = nullptr;
+  }
+  bool AcceptsResidual() const override {
+    for (Layer* f : followers_) {
+      const string ty = f->type();
+      if (ty == "ReLU" || ty == "TanH" || ty == "Sigmoid") return false;
+    }
+    return true;
+  }
+  void SetResidual(Blob* residual, Layer* activation) override {
+    residual_ = residual;
+    residual_act_ = activation;
   }
 
  protected:
@@ -103,6 +116,15 @@ class ContractionLayer : public Layer {
       } else {
         ++n_affine;
         stages.push_back(op);
+      }
+    }
+    if (residual_) {
+      ep->residual = residual_->gpu_data();
+      if (residual_act_) {
+        mcChannelOp op = {nullptr, nullptr, nullptr, nullptr, MC_ACT_NONE, 0.f};
+        residual_act_->GetChannelStage(&op);
+        ep->activation = op.activation;
+        ep->negative_slope = op.negative_slope;
       }
     }
     if (n_affine == 0) {
@@ -136,6 +158,8 @@ class ContractionLayer : public Layer {
   mcConvPlan* plan_;
   uint64_t weights_version_ = ~0ull;
   vector<Layer*> followers_;
+  Blob* residual_ = nullptr;       // added after the per-channel stages
+  Layer* residual_act_ = nullptr;  // activation applied after the residual
   Blob fold_scale_, fold_shift_;
   uint64_t fold_version_ = ~0ull;
   int fold_channels_ = -1;
@@ -782,6 +806,10 @@ class EltwiseLayer : public Layer {
     CHECK(followers.size() <= 1) << "Eltwise can absorb a single activation";
     if (!followers.empty()) act_follower_ = followers[0];
   }
+  bool IsPlainSum() const override {
+    return op_ == MC_ELT_SUM && coeffs_.size() == 2 && coeffs_[0] == 1.f && coeffs_[1] == 1.f;
+  }
+  Layer* AbsorbedActivation() const override { return act_follower_; }
 
  protected:
   void Forward_gpu(const vector<Blob*>& bottom, const vector<Blob*>& top) override {

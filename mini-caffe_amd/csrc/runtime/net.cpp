@@ -68,6 +68,7 @@ void Net::Init(const NetParameter& param) {
   for (size_t layer_id = 0; layer_id < layer_names_.size(); ++layer_id)
     layer_names_index_[layer_names_[layer_id]] = static_cast<int>(layer_id);
   layer_fused_.assign(layers_.size(), 0);
+  residual_alias_.assign(layers_.size(), -1);
   PlaceMemory();
 }
 
@@ -137,6 +138,10 @@ void Net::AppendParam(const NetParameter& param, const int layer_id, const int p
 // calls, so the placement is recomputed only when they did.
 void Net::PlaceMemory() {
   this->Reshape();
+  if (fusion_dirty_) {
+    PlanFusion();  // decides which tops alias their producer's blob
+    placed_shapes_.clear();
+  }
   vector<vector<int> > shapes;
   shapes.reserve(blobs_.size());
   for (auto& b : blobs_) shapes.push_back(b->shape());
@@ -151,19 +156,31 @@ void Net::PlaceMemory() {
 
   typedef std::pair<size_t, Blob*> BlobPair;
   std::multimap<size_t, Blob*> pool;
+  // A blob that a folded sum's top aliases lives on under that top's name: it
+  // is handed back to the pool when the top dies, not when the blob does.
+  std::set<int> kept_alive;
+  for (int id : residual_alias_)
+    if (id >= 0) kept_alive.insert(id);
   for (size_t i = 0; i < layers_.size(); ++i) {
     vector<Blob*> temps = layers_[i]->GetTempBlobs();
     vector<Blob*>& bottoms = bottom_vecs_[i];
     vector<Blob*>& tops = top_vecs_[i];
     vector<BlobPair> to_place;
-    for (Blob* blob : temps) {
-      blob->ResetMemory();
-      to_place.push_back(std::make_pair(static_cast<size_t>(blob->count()), blob));
-    }
-    for (Blob* blob : tops) {
-      if (std::find(bottoms.begin(), bottoms.end(), blob) != bottoms.end()) continue;  // in place
-      blob->ResetMemory();
-      to_place.push_back(std::make_pair(static_cast<size_t>(blob->count()), blob));
+    if (residual_alias_[i] >= 0) {
+      // folded sum: no scratch, and the top is the producer's blob under a new name
+      temps.clear();
+      tops[0]->ResetMemory();
+      tops[0]->ShareData(*blobs_[residual_alias_[i]]);
+    } else {
+      for (Blob* blob : temps) {
+        blob->ResetMemory();
+        to_place.push_back(std::make_pair(static_cast<size_t>(blob->count()), blob));
+      }
+      for (Blob* blob : tops) {
+        if (std::find(bottoms.begin(), bottoms.end(), blob) != bottoms.end()) continue;  // in place
+        blob->ResetMemory();
+        to_place.push_back(std::make_pair(static_cast<size_t>(blob->count()), blob));
+      }
     }
     std::sort(to_place.begin(), to_place.end(),
               [](const BlobPair& x, const BlobPair& y) { return x.first > y.first; });
@@ -176,7 +193,8 @@ void Net::PlaceMemory() {
     }
     std::set<int> released;  // a blob listed twice as bottom is released once
     for (int blob_idx : bottom_id_vecs_[i]) {
-      if (blob_life_time_[blob_idx] <= static_cast<int>(i) && released.insert(blob_idx).second) {
+      if (blob_life_time_[blob_idx] <= static_cast<int>(i) && !kept_alive.count(blob_idx) &&
+          released.insert(blob_idx).second) {
         pool.insert(std::make_pair(static_cast<size_t>(blobs_[blob_idx]->capacity()),
                                    blobs_[blob_idx].get()));
       }
@@ -216,14 +234,59 @@ void Net::PlanFusion() {
     layers_[i]->SetEpilogue(followers);
     for (size_t k = 0; k < followers.size(); ++k) layer_fused_[i + 1 + k] = 1;
   }
+
+  // Residual sums (ResNet's  Eltwise(shortcut, branch) -> ReLU): when one input
+  // of a two-input unit-coefficient sum comes straight from a contraction that
+  // nothing else reads, and the other input is complete before that
+  // contraction runs, the contraction adds it (and applies the sum's
+  // activation) in its epilogue; the sum's top then aliases the contraction's
+  // top blob and the sum itself is skipped.
+  residual_alias_.assign(layers_.size(), -1);
+  for (size_t e = 0; e < layers_.size(); ++e) {
+    if (layer_fused_[e] || !layers_[e]->IsPlainSum()) continue;
+    if (bottom_vecs_[e].size() != 2 || top_vecs_[e].size() != 1) continue;
+    Blob* E = top_vecs_[e][0];
+    if (E == bottom_vecs_[e][0] || E == bottom_vecs_[e][1]) continue;
+    if (bottom_vecs_[e][0] == bottom_vecs_[e][1]) continue;
+    auto last_writer = [&](const Blob* b, int before) {
+      for (int j = before - 1; j >= 0; --j)
+        if (std::find(top_vecs_[j].begin(), top_vecs_[j].end(), b) != top_vecs_[j].end()) return j;
+      return -1;
+    };
+    // the input written last is the candidate; the other one is the residual
+    const int w0 = last_writer(bottom_vecs_[e][0], static_cast<int>(e));
+    const int w1 = last_writer(bottom_vecs_[e][1], static_cast<int>(e));
+    const int ti = w0 > w1 ? 0 : 1;
+    Blob* T = bottom_vecs_[e][ti];
+    Blob* R = bottom_vecs_[e][1 - ti];
+    const int t_id = bottom_id_vecs_[e][ti];
+    int c = std::max(w0, w1);
+    const int r_writer = std::min(w0, w1);
+    while (c >= 0 && layer_fused_[c]) --c;  // walk back over the folded in-place stages
+    if (c < 0 || r_writer >= c) continue;
+    if (!layers_[c]->AcceptsEpilogue() || !layers_[c]->AcceptsResidual()) continue;
+    if (top_vecs_[c].size() != 1 || top_vecs_[c][0] != T) continue;
+    if (blob_life_time_[t_id] != static_cast<int>(e)) continue;  // read later, or an output
+    bool exclusive = true;
+    for (size_t j = c + 1; j < e && exclusive; ++j) {
+      if (layer_fused_[j]) continue;
+      for (Blob* b : bottom_vecs_[j])
+        if (b == T) exclusive = false;
+      for (Blob* b : top_vecs_[j])
+        if (b == T || b == R) exclusive = false;
+    }
+    if (!exclusive || T->shape() != R->shape()) continue;
+    layers_[c]->SetResidual(R, layers_[e]->AbsorbedActivation());
+    layer_fused_[e] = 1;
+    residual_alias_[e] = t_id;
+  }
 }
 
 void Net::Forward(bool reshape) {
   CHECK(Context::mode() == GPU)
       << "Net::Forward: this library implements the HIP device path only; call "
       << "SetMode(GPU, device) on this thread first";
-  if (reshape) PlaceMemory();
-  if (fusion_dirty_) PlanFusion();
+  if (reshape || fusion_dirty_) PlaceMemory();
   Profiler* profiler = Profiler::Get();
   const bool profiling = profiler->enabled();
   for (size_t i = 0; i < layers_.size(); ++i) {
@@ -290,6 +353,7 @@ void Net::MarkOutputs(const std::vector<std::string>& outs) {
     blob_life_time_[it->second] = static_cast<int>(layers_.size());
   }
   placed_shapes_.clear();  // lifetimes changed: place again on the next Forward
+  fusion_dirty_ = true;    // and a blob that is now an output must keep its own values
 }
 
 const vector<int>& Net::top_ids(int i) const {
