@@ -82,8 +82,10 @@ __device__ __forceinline__ float apply_act(float v, int act, float slope) {
   }
 }
 
-template <int BM, int BN, int WM, int WN>
-__global__ __launch_bounds__(256) void igemm_kernel(const IgemmArgs a) {
+// OCC = wavefronts per SIMD the register allocation must leave room for.
+template <int BM, int BN, int WM, int WN, int OCC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC))) void igemm_kernel(
+    const IgemmArgs a) {
   static_assert(WM * WN == 4, "four wavefronts per workgroup");
   static_assert(BN >= 64 && 256 % BN == 0, "BN must be 64, 128 or 256");
   constexpr int TM = BM / WM / 32;
@@ -258,10 +260,16 @@ __global__ __launch_bounds__(256) void igemm_kernel(const IgemmArgs a) {
 
   // Epilogue.  Accumulator register r of lane l holds row 8*(r/4)+4*(l/32)+r%4,
   // column l%32 of its 32x32 block; a half-wave therefore stores 32 consecutive
-  // pixels of one output channel.
+  // pixels of one output channel.  Per-channel factors and residual values are
+  // fetched in batches whose loads all issue before the first use, so a block
+  // pays a few load latencies instead of one per value.
   const bool has_scale = a.scale != nullptr;
   const bool has_shift = a.shift != nullptr;
   const bool has_res = a.residual != nullptr;
+  // "no activation" is a leaky ReLU of slope 1, so one select covers both.
+  const bool relu_like = a.act == MC_ACT_NONE || a.act == MC_ACT_RELU;
+  const float slope = a.act == MC_ACT_NONE ? 1.f : a.slope;
+#define MC_ROW(r) (8 * ((r) / 4) + ((r) % 4))
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int p = nt * BN + wn0 + j * 32 + l32;
@@ -270,25 +278,71 @@ __global__ __launch_bounds__(256) void igemm_kernel(const IgemmArgs a) {
     const int rem = p - n * a.HqWq;
     const int qh = rem / a.Wq;
     const int qw = rem - qh * a.Wq;
-    const int ybase = n * a.y_nstride + (qh * a.out_sh + a.out_oh) * a.Wo +
-                      qw * a.out_sw + a.out_ow;
+    const int ybase =
+        n * a.y_nstride + (qh * a.out_sh + a.out_oh) * a.Wo + qw * a.out_sw + a.out_ow;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
+      const int mblock = mt * BM + wm0 + i * 32;  // wave-uniform
+      const int m0 = mblock + 4 * lhi;
+      if (mblock + 32 <= a.M) {
+        // All 32 rows are real channels: constant offsets from one base.
+        const unsigned c0 = g * a.M + m0;
+        const unsigned y0 = ybase + c0 * a.y_cstride;
+        const unsigned cs = a.y_cstride;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = mt * BM + wm0 + i * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
-        if (m < a.M) {
-          const int c = g * a.M + m;
-          float v = acc[i][j][r];
-          if (has_scale) v *= a.scale[c];
-          if (has_shift) v += a.shift[c];
-          const int yo = ybase + c * a.y_cstride;
-          if (has_res) v += a.residual[yo];
-          yout[yo] = apply_act(v, a.act, a.slope);
+        for (int half = 0; half < 2; ++half) {
+          if (has_scale | has_shift) {
+            float sc[8], sh[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+              sc[q] = 1.f;
+              sh[q] = 0.f;
+              if (has_scale) sc[q] = a.scale[c0 + MC_ROW(half * 8 + q)];
+              if (has_shift) sh[q] = a.shift[c0 + MC_ROW(half * 8 + q)];
+            }
+#pragma unroll
+            for (int q = 0; q < 8; ++q)
+              acc[i][j][half * 8 + q] = acc[i][j][half * 8 + q] * sc[q] + sh[q];
+          }
+          if (has_res) {
+            float rs[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) rs[q] = a.residual[y0 + MC_ROW(half * 8 + q) * cs];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) acc[i][j][half * 8 + q] += rs[q];
+          }
+          if (relu_like) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+              const float v = acc[i][j][half * 8 + q];
+              yout[y0 + MC_ROW(half * 8 + q) * cs] = v > 0.f ? v : v * slope;
+            }
+          } else {
+#pragma unroll
+            for (int q = 0; q < 8; ++q)
+              yout[y0 + MC_ROW(half * 8 + q) * cs] =
+                  apply_act(acc[i][j][half * 8 + q], a.act, a.slope);
+          }
+        }
+      } else {
+        // Block straddles the last channel: row by row, skipping rows >= M.
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + MC_ROW(r);
+          if (m < a.M) {
+            const int c = g * a.M + m;
+            float v = acc[i][j][r];
+            if (has_scale) v *= a.scale[c];
+            if (has_shift) v += a.shift[c];
+            const int yo = ybase + c * a.y_cstride;
+            if (has_res) v += a.residual[yo];
+            yout[yo] = relu_like ? (v > 0.f ? v : v * slope) : apply_act(v, a.act, a.slope);
+          }
         }
       }
     }
   }
+#undef MC_ROW
 }
 
 // Split-K tail: y = act((sum over slices, in slice order) * scale[c] + shift[c]
@@ -372,13 +426,13 @@ struct TileConfig {
 };
 
 const TileConfig kConfigs[] = {
-    {128, 128, "igemm_f32_128x128", igemm_kernel<128, 128, 2, 2>},
-    {128, 64, "igemm_f32_128x64", igemm_kernel<128, 64, 2, 2>},
-    {64, 128, "igemm_f32_64x128", igemm_kernel<64, 128, 2, 2>},
-    {64, 64, "igemm_f32_64x64", igemm_kernel<64, 64, 2, 2>},
-    {32, 128, "igemm_f32_32x128", igemm_kernel<32, 128, 1, 4>},
-    {32, 256, "igemm_f32_32x256", igemm_kernel<32, 256, 1, 4>},
-    {64, 256, "igemm_f32_64x256", igemm_kernel<64, 256, 1, 4>},
+    {128, 128, "igemm_f32_128x128", igemm_kernel<128, 128, 2, 2, 3>},
+    {128, 64, "igemm_f32_128x64", igemm_kernel<128, 64, 2, 2, 5>},
+    {64, 128, "igemm_f32_64x128", igemm_kernel<64, 128, 2, 2, 5>},
+    {64, 64, "igemm_f32_64x64", igemm_kernel<64, 64, 2, 2, 8>},
+    {32, 128, "igemm_f32_32x128", igemm_kernel<32, 128, 1, 4, 7>},
+    {32, 256, "igemm_f32_32x256", igemm_kernel<32, 256, 1, 4, 4>},
+    {64, 256, "igemm_f32_64x256", igemm_kernel<64, 256, 1, 4, 3>},
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 
