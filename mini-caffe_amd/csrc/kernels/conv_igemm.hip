@@ -36,12 +36,24 @@ constexpr int BK = 16;
 constexpr int LDK = BK + 4;  // LDS row pitch in floats
 
 typedef float acc16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+// Buffer descriptor word 3 for raw dword access on gfx9-family CDNA parts
+// (32-bit data format, no swizzle, offsets checked against num_records).
+constexpr int kBufferFlags = 0x00020000;
+// VGPR offset that is out of range for every buffer this file builds (all are
+// below 2 GiB) and still has room for the widest access without wrapping.
+constexpr unsigned kNoElement = 0x80000000u;
 
 struct IgemmArgs {
   const float* __restrict__ x;
   const float* __restrict__ wt;
   float* __restrict__ y;
-  const int4* __restrict__ ktab;  // [Kpad] {element offset, dh, dw, unused}
+  const int4* __restrict__ ktab;  // [Kpad] {byte offset, row-tap index, column-tap index, 0}
+  const int* __restrict__ tap_dh;  // bottom row offset of row-tap index b
+  const int* __restrict__ tap_dw;  // bottom column offset of column-tap index b
+  int n_dh, n_dw;
+  unsigned x_bytes, wt_bytes;      // extents for the buffer descriptors
+  int pix_shift;                   // bytes added to pixel origins (x points that far before the blob)
   const float* __restrict__ scale;
   const float* __restrict__ shift;
   const float* __restrict__ residual;
@@ -50,6 +62,8 @@ struct IgemmArgs {
   int H, W;           // bottom height / width
   int q_sh, q_sw;     // bottom origin of pixel (qh,qw): qh*q_sh + in_oh
   int in_oh, in_ow;
+  int K;              // rows of the gather before padding to a multiple of BK
+  int x_cstride;      // H*W
   int x_nstride;      // Cin*H*W
   int x_gstride;      // (Cin/g)*H*W
   int M;              // output channels per group
@@ -83,8 +97,11 @@ __device__ __forceinline__ float apply_act(float v, int act, float slope) {
 }
 
 // OCC = wavefronts per SIMD the register allocation must leave room for.
-template <int BM, int BN, int WM, int WN, int OCC>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC))) void igemm_kernel(
+// PW ("pointwise"): every row k of the gather is channel k of the bottom blob
+// at the thread's own pixel (1x1 kernel, no padding), so the K loop needs no
+// tap table and no bounds handling at all.
+template <int BM, int BN, int WM, int WN, int OCC, bool PW>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void igemm_kernel(
     const IgemmArgs a) {
   static_assert(WM * WN == 4, "four wavefronts per workgroup");
   static_assert(BN >= 64 && 256 % BN == 0, "BN must be 64, 128 or 256");
@@ -123,10 +140,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC))) void
     nt = logical / a.MT;
   }
 
+  // On this hardware ordinary vector ALU instructions and MFMA instructions of
+  // co-resident wavefronts do not overlap: every VALU cycle in the K loop is
+  // taken from the matrix pipe.  The loop therefore does its addressing on the
+  // scalar unit and in the memory instructions themselves:
+  //  * bottom and filter are read through buffer descriptors: scalar base,
+  //    scalar offset per K row / K tile, one fixed VGPR offset per thread, and
+  //    an out-of-range VGPR offset returns 0 without a branch or a select.
+  //    Both buffers are kept below 2 GiB and "no element" is offset bit 31.  The
+  //    bottom descriptor starts far enough before the blob that the sum of a
+  //    pixel origin and a tap offset is never negative, so a flagged offset lies
+  //    in [2^31, 2^32 - 16) and offset + access size cannot wrap around 2^32
+  //    (an access that carries into bit 32 would leave the checked range);
+  //  * per thread, bit b of row_bad / col_bad says that row (column) tap b
+  //    falls outside the image for this thread's pixel, so an element costs two
+  //    bit-field extracts, an add and two shift-ors (nothing at all when PW);
+  //  * the loop is unrolled over the two LDS buffers so every LDS address is
+  //    a base register plus an immediate.
+  const __amdgpu_buffer_rsrc_t xres =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.x), 0, a.x_bytes, kBufferFlags);
+  const __amdgpu_buffer_rsrc_t wres =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.wt), 0, a.wt_bytes, kBufferFlags);
+
   // The pixel this thread gathers for the B tile (fixed over the K loop).
   const int pj = tid % BN;
   const int prow = tid / BN;  // wave-uniform because BN >= 64
-  int hi0, wi0, xbase;
+  // byte offset of the pixel's origin from the descriptor base (never negative)
+  unsigned xvoff = PW ? kNoElement : 0u;
+  unsigned row_bad = 0xFFFFFFFFu, col_bad = 0xFFFFFFFFu;
   {
     const int p = nt * BN + pj;
     if (p < a.P) {
@@ -134,13 +175,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC))) void
       const int rem = p - n * a.HqWq;
       const int qh = rem / a.Wq;
       const int qw = rem - qh * a.Wq;
-      hi0 = qh * a.q_sh + a.in_oh;
-      wi0 = qw * a.q_sw + a.in_ow;
-      xbase = n * a.x_nstride + g * a.x_gstride + hi0 * a.W + wi0;
-    } else {
-      hi0 = -(1 << 24);  // fails every bounds test -> contributes zeros
-      wi0 = 0;
-      xbase = 0;
+      const int hi0 = qh * a.q_sh + a.in_oh;
+      const int wi0 = qw * a.q_sw + a.in_ow;
+      xvoff = static_cast<unsigned>(
+          ((n * a.x_nstride + g * a.x_gstride + hi0 * a.W + wi0) << 2) + a.pix_shift);
+      if constexpr (!PW) {
+        row_bad = 0x80000000u;  // bit 31: the tap of K padding rows, never valid
+        col_bad = 0u;
+        for (int b = 0; b < a.n_dh; ++b)
+          row_bad |= static_cast<unsigned>(static_cast<unsigned>(hi0 + a.tap_dh[b]) >=
+                                           static_cast<unsigned>(a.H))
+                     << b;
+        for (int b = 0; b < a.n_dw; ++b)
+          col_bad |= static_cast<unsigned>(static_cast<unsigned>(wi0 + a.tap_dw[b]) >=
+                                           static_cast<unsigned>(a.W))
+                     << b;
+      }
     }
   }
   const int KT = a.Kpad / BK;
@@ -148,44 +198,62 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC))) void
   // partial sums into its own copy of the top blob.
   const int kt_begin = blockIdx.z * a.kt_per_split;
   const int kt_end = min(KT, kt_begin + a.kt_per_split);
-  // Packed filter: [g][K tile][m][16 k], so an A tile is one contiguous run.
-  const float* __restrict__ wt_tile =
-      a.wt + ((size_t)g * KT * a.Mpad + (size_t)mt * BM) * BK;
-  const size_t wt_kt_stride = (size_t)a.Mpad * BK;
   float* __restrict__ yout = a.y + (size_t)blockIdx.z * a.split_stride;
+
+  // Packed filter: [g][K tile][m][16 k], so an A tile is one contiguous run:
+  // per-thread byte offset inside the tile, scalar byte offset of the tile.
+  unsigned avoff[A_VEC];
+#pragma unroll
+  for (int i = 0; i < A_VEC; ++i) {
+    const int f = tid + 256 * i;
+    avoff[i] = (A_F4 % 256 == 0 || f < A_F4) ? static_cast<unsigned>((mt * BM * BK + f * 4) * 4)
+                                              : kNoElement;
+  }
+  const unsigned wt_kt_bytes = static_cast<unsigned>(a.Mpad) * BK * 4;
+  const unsigned wt_g_bytes = static_cast<unsigned>(g) * KT * wt_kt_bytes;
+  const unsigned x_cbytes = static_cast<unsigned>(a.x_cstride) * 4;
+  const int kmax = a.K - 1;
 
   float4 areg[A_VEC];
   float4 breg[B_Q];
 
-  // Global -> registers for K tile kt.  Branch-free on purpose: tap entries are
-  // scalar loads, an out-of-image tap reads element 0 and is zeroed by a
-  // select, so all loads of a tile issue back to back.
+#define MC_LOADF(res, voff, soff) \
+  __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(res, voff, soff, 0))
 #define MC_GATHER1(dst, t)                                                                   \
   {                                                                                          \
-    const int hi = hi0 + (t).y;                                                              \
-    const int wi = wi0 + (t).z;                                                              \
-    const bool ok = (static_cast<unsigned>(hi) < static_cast<unsigned>(a.H)) &               \
-                    (static_cast<unsigned>(wi) < static_cast<unsigned>(a.W));                \
-    const int off = ok ? xbase + (t).x : 0;                                                  \
-    const float v = a.x[off];                                                                \
-    dst = ok ? v : 0.f;                                                                      \
+    const unsigned rb = __builtin_amdgcn_ubfe(row_bad, (t).y, 1);                            \
+    const unsigned cb = __builtin_amdgcn_ubfe(col_bad, (t).z, 1);                            \
+    /* a valid element's offset is below 2^31; bit 31 marks "no element" */                  \
+    const unsigned off = xvoff + static_cast<unsigned>((t).x);                               \
+    dst = MC_LOADF(xres, (cb << 31) | ((rb << 31) | off), 0);                                \
   }
 #define MC_LOAD_TILES(kt)                                                                    \
   {                                                                                          \
+    const unsigned a_soff = wt_g_bytes + static_cast<unsigned>(kt) * wt_kt_bytes;            \
     _Pragma("unroll") for (int i = 0; i < A_VEC; ++i) {                                      \
-      const int f = tid + 256 * i;                                                           \
-      if (A_F4 % 256 == 0 || f < A_F4)                                                       \
-        areg[i] = *reinterpret_cast<const float4*>(wt_tile + (kt)*wt_kt_stride + f * 4);     \
+      const u32x4 w4 = __builtin_amdgcn_raw_buffer_load_b128(wres, avoff[i], a_soff, 0);     \
+      areg[i] = __builtin_bit_cast(float4, w4);                                              \
     }                                                                                        \
     _Pragma("unroll") for (int i = 0; i < B_Q; ++i) {                                        \
       const int krow =                                                                       \
           __builtin_amdgcn_readfirstlane((kt)*BK + (i * ROWS_PER_PASS + prow) * 4);          \
-      const int4 t0 = a.ktab[krow], t1 = a.ktab[krow + 1], t2 = a.ktab[krow + 2],            \
-                 t3 = a.ktab[krow + 3];                                                      \
-      MC_GATHER1(breg[i].x, t0);                                                             \
-      MC_GATHER1(breg[i].y, t1);                                                             \
-      MC_GATHER1(breg[i].z, t2);                                                             \
-      MC_GATHER1(breg[i].w, t3);                                                             \
+      if constexpr (PW) {                                                                    \
+        /* padding rows re-read the last channel; their filter rows are zero */              \
+        breg[i].x = MC_LOADF(xres, xvoff, static_cast<unsigned>(min(krow, kmax)) * x_cbytes);\
+        breg[i].y =                                                                          \
+            MC_LOADF(xres, xvoff, static_cast<unsigned>(min(krow + 1, kmax)) * x_cbytes);    \
+        breg[i].z =                                                                          \
+            MC_LOADF(xres, xvoff, static_cast<unsigned>(min(krow + 2, kmax)) * x_cbytes);    \
+        breg[i].w =                                                                          \
+            MC_LOADF(xres, xvoff, static_cast<unsigned>(min(krow + 3, kmax)) * x_cbytes);    \
+      } else {                                                                               \
+        const int4 t0 = a.ktab[krow], t1 = a.ktab[krow + 1], t2 = a.ktab[krow + 2],          \
+                   t3 = a.ktab[krow + 3];                                                    \
+        MC_GATHER1(breg[i].x, t0);                                                           \
+        MC_GATHER1(breg[i].y, t1);                                                           \
+        MC_GATHER1(breg[i].z, t2);                                                           \
+        MC_GATHER1(breg[i].w, t3);                                                           \
+      }                                                                                      \
     }                                                                                        \
   }
 #define MC_STORE_TILES(buf)                                                                  \
@@ -238,21 +306,41 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC))) void
   const int lhi = lane >> 5;
 
   if (kt_end > kt_begin) {
+    // Tile kt_begin + t sits in LDS buffer t % 2; the loads of the next tile
+    // are in flight while the MFMA block of the current one runs.
+    const int nk = kt_end - kt_begin;
     MC_LOAD_TILES(kt_begin);
     MC_STORE_TILES(0);
     __syncthreads();
-    int buf = 0;
-    for (int kt = kt_begin; kt < kt_end - 1; ++kt) {
-      MC_LOAD_TILES(kt + 1);
+    int t = 0;
+    for (; t + 2 < nk; t += 2) {
+      MC_LOAD_TILES(kt_begin + t + 1);
       __builtin_amdgcn_sched_barrier(0);  // keep the global loads ahead of the MFMA block
-      MC_COMPUTE(buf);
+      MC_COMPUTE(0);
       __builtin_amdgcn_sched_barrier(0);
-      MC_STORE_TILES(buf ^ 1);
+      MC_STORE_TILES(1);
       __syncthreads();
-      buf ^= 1;
+      MC_LOAD_TILES(kt_begin + t + 2);
+      __builtin_amdgcn_sched_barrier(0);
+      MC_COMPUTE(1);
+      __builtin_amdgcn_sched_barrier(0);
+      MC_STORE_TILES(0);
+      __syncthreads();
     }
-    MC_COMPUTE(buf);
+    // one or two tiles left; tile t is in buffer 0
+    if (t + 1 < nk) {
+      MC_LOAD_TILES(kt_begin + t + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      MC_COMPUTE(0);
+      __builtin_amdgcn_sched_barrier(0);
+      MC_STORE_TILES(1);
+      __syncthreads();
+      MC_COMPUTE(1);
+    } else {
+      MC_COMPUTE(0);
+    }
   }
+#undef MC_LOADF
 #undef MC_GATHER1
 #undef MC_LOAD_TILES
 #undef MC_STORE_TILES
@@ -423,16 +511,24 @@ struct TileConfig {
   int bm, bn;
   const char* name;
   void (*kernel)(const IgemmArgs);
+  void (*kernel_pw)(const IgemmArgs);  // pointwise variant
 };
 
 const TileConfig kConfigs[] = {
-    {128, 128, "igemm_f32_128x128", igemm_kernel<128, 128, 2, 2, 3>},
-    {128, 64, "igemm_f32_128x64", igemm_kernel<128, 64, 2, 2, 5>},
-    {64, 128, "igemm_f32_64x128", igemm_kernel<64, 128, 2, 2, 5>},
-    {64, 64, "igemm_f32_64x64", igemm_kernel<64, 64, 2, 2, 8>},
-    {32, 128, "igemm_f32_32x128", igemm_kernel<32, 128, 1, 4, 7>},
-    {32, 256, "igemm_f32_32x256", igemm_kernel<32, 256, 1, 4, 4>},
-    {64, 256, "igemm_f32_64x256", igemm_kernel<64, 256, 1, 4, 3>},
+    {128, 128, "igemm_f32_128x128",
+     igemm_kernel<128, 128, 2, 2, 3, false>, igemm_kernel<128, 128, 2, 2, 3, true>},
+    {128, 64, "igemm_f32_128x64",
+     igemm_kernel<128, 64, 2, 2, 4, false>, igemm_kernel<128, 64, 2, 2, 4, true>},
+    {64, 128, "igemm_f32_64x128",
+     igemm_kernel<64, 128, 2, 2, 5, false>, igemm_kernel<64, 128, 2, 2, 5, true>},
+    {64, 64, "igemm_f32_64x64",
+     igemm_kernel<64, 64, 2, 2, 8, false>, igemm_kernel<64, 64, 2, 2, 8, true>},
+    {32, 128, "igemm_f32_32x128",
+     igemm_kernel<32, 128, 1, 4, 4, false>, igemm_kernel<32, 128, 1, 4, 4, true>},
+    {32, 256, "igemm_f32_32x256",
+     igemm_kernel<32, 256, 1, 4, 3, false>, igemm_kernel<32, 256, 1, 4, 3, true>},
+    {64, 256, "igemm_f32_64x256",
+     igemm_kernel<64, 256, 1, 4, 2, false>, igemm_kernel<64, 256, 1, 4, 2, true>},
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 
@@ -443,8 +539,15 @@ struct SubProblem {
   int Hq = 0, Wq = 0;
   int q_sh = 1, q_sw = 1, in_oh = 0, in_ow = 0;
   int out_sh = 1, out_sw = 1, out_oh = 0, out_ow = 0;
-  std::vector<int4> ktab;    // host copy
+  std::vector<int4> ktab;    // host copy: {byte offset, row-tap index, column-tap index, 0}
   std::vector<int> wk_off;   // host copy
+  std::vector<int> tap_dh, tap_dw;  // bottom offset of each row / column tap index
+  bool pointwise = false;    // every k is channel k at the pixel itself, always in range
+  // The bottom descriptor starts tap_shift + pix_shift bytes before the blob:
+  // tap offsets are stored plus tap_shift, pixel origins computed plus pix_shift,
+  // so both are non-negative.
+  int tap_shift = 0, pix_shift = 0;
+  int* tap_dev = nullptr;    // tap_dh followed by tap_dw
   int4* ktab_dev = nullptr;
   int* wk_off_dev = nullptr;
   float* wt_dev = nullptr;
@@ -464,6 +567,7 @@ struct mcConvPlan {
   int wm_stride = 0, wg_stride = 0;
   int forced_config = -1;
   int forced_split = 0;  // 0 = choose, >= 1 = this many K slices
+  bool force_general = false;  // use the tap-table gather even for pointwise geometry
   std::vector<SubProblem> subs;
 };
 
@@ -543,6 +647,8 @@ int get_workspace(hipStream_t st, size_t bytes, float** out) {
 
 int free_sub(SubProblem& s) {
   if (s.ktab_dev) (void)hipFree(s.ktab_dev);
+  if (s.tap_dev) (void)hipFree(s.tap_dev);
+  s.tap_dev = nullptr;
   if (s.wk_off_dev) (void)hipFree(s.wk_off_dev);
   if (s.wt_dev) (void)hipFree(s.wt_dev);
   s.ktab_dev = nullptr;
@@ -604,13 +710,16 @@ int mcConvPlanCreate(const mcConvGeom* gp, mcConvPlan** out) {
     s.q_sw = g.stride_w;
     s.in_oh = -g.pad_h;
     s.in_ow = -g.pad_w;
+    for (int i = 0; i < g.kernel_h; ++i) s.tap_dh.push_back(i * g.dilation_h);
+    for (int j = 0; j < g.kernel_w; ++j) s.tap_dw.push_back(j * g.dilation_w);
     for (int c = 0; c < plan->Cin_g; ++c)
       for (int i = 0; i < g.kernel_h; ++i)
         for (int j = 0; j < g.kernel_w; ++j) {
           const int dh = i * g.dilation_h, dw = j * g.dilation_w;
-          s.ktab.push_back(make_int4(c * HW + dh * g.width_in + dw, dh, dw, 0));
+          s.ktab.push_back(make_int4((c * HW + dh * g.width_in + dw) * 4, i, j, 0));
           s.wk_off.push_back((c * g.kernel_h + i) * g.kernel_w + j);
         }
+    s.pointwise = g.kernel_h == 1 && g.kernel_w == 1 && g.pad_h == 0 && g.pad_w == 0;
     plan->wm_stride = s.K;
     plan->wg_stride = plan->M * s.K;
     plan->subs.push_back(std::move(s));
@@ -647,10 +756,12 @@ int mcConvPlanCreate(const mcConvGeom* gp, mcConvPlan** out) {
         for (int c = 0; c < plan->Cin_g; ++c)
           for (size_t i = 0; i < tap_h.size(); ++i)
             for (size_t j = 0; j < tap_w.size(); ++j) {
-              s.ktab.push_back(
-                  make_int4(c * HW + off_h[i] * g.width_in + off_w[j], off_h[i], off_w[j], 0));
+              s.ktab.push_back(make_int4((c * HW + off_h[i] * g.width_in + off_w[j]) * 4,
+                                         static_cast<int>(i), static_cast<int>(j), 0));
               s.wk_off.push_back(c * plan->M * khkw + tap_h[i] * g.kernel_w + tap_w[j]);
             }
+        s.tap_dh = off_h;
+        s.tap_dw = off_w;
         s.K = static_cast<int>(s.ktab.size());
         plan->subs.push_back(std::move(s));
       }
@@ -658,22 +769,42 @@ int mcConvPlanCreate(const mcConvGeom* gp, mcConvPlan** out) {
 
   for (auto& s : plan->subs) {
     s.Kpad = ceil_div(s.K, BK) * BK;
-    // Padding rows multiply zero weights; give them a tap that fails the
-    // bounds test so nothing is fetched.
-    while (static_cast<int>(s.ktab.size()) < s.Kpad) s.ktab.push_back(make_int4(0, 1 << 20, 0, 0));
+    // Padding rows multiply zero weights; row-tap index 31 is out of the image
+    // for every pixel, so nothing is fetched for them.
+    while (static_cast<int>(s.ktab.size()) < s.Kpad) s.ktab.push_back(make_int4(0, 31, 0, 0));
+    int min_tap = 0;
+    for (const int4& t : s.ktab) min_tap = std::min(min_tap, t.x);
+    s.tap_shift = -min_tap;
+    for (int4& t : s.ktab) t.x += s.tap_shift;
+    s.pix_shift = std::max(0, -(s.in_oh * g.width_in + s.in_ow) * 4);
     if (s.Kpad == 0) continue;
-    hipError_t e = hipMalloc(&s.ktab_dev, sizeof(int4) * s.Kpad);
-    if (e == hipSuccess) e = hipMalloc(&s.wk_off_dev, sizeof(int) * s.K);
-    if (e == hipSuccess)
-      e = hipMalloc(&s.wt_dev, sizeof(float) * (size_t)g.group * s.Kpad * plan->Mpad);
-    if (e == hipSuccess)
-      e = hipMemcpy(s.ktab_dev, s.ktab.data(), sizeof(int4) * s.Kpad, hipMemcpyHostToDevice);
-    if (e == hipSuccess)
-      e = hipMemcpy(s.wk_off_dev, s.wk_off.data(), sizeof(int) * s.K, hipMemcpyHostToDevice);
-    if (e != hipSuccess) {
+    const size_t wt_bytes = sizeof(float) * (size_t)g.group * s.Kpad * plan->Mpad;
+    hipError_t e = hipSuccess;
+    const char* what = nullptr;
+    if (s.tap_dh.size() > 31 || s.tap_dw.size() > 31)
+      what = "kernels with more than 31 taps per dimension are not supported";
+    else if (wt_bytes >= (1ull << 31))
+      what = "packed filter exceeds 2 GiB";
+    if (!what) {
+      std::vector<int> taps(s.tap_dh);
+      taps.insert(taps.end(), s.tap_dw.begin(), s.tap_dw.end());
+      taps.push_back(0);  // never empty
+      e = hipMalloc(&s.ktab_dev, sizeof(int4) * s.Kpad);
+      if (e == hipSuccess) e = hipMalloc(&s.wk_off_dev, sizeof(int) * s.K);
+      if (e == hipSuccess) e = hipMalloc(&s.tap_dev, sizeof(int) * taps.size());
+      if (e == hipSuccess) e = hipMalloc(&s.wt_dev, wt_bytes);
+      if (e == hipSuccess)
+        e = hipMemcpy(s.ktab_dev, s.ktab.data(), sizeof(int4) * s.Kpad, hipMemcpyHostToDevice);
+      if (e == hipSuccess)
+        e = hipMemcpy(s.wk_off_dev, s.wk_off.data(), sizeof(int) * s.K, hipMemcpyHostToDevice);
+      if (e == hipSuccess)
+        e = hipMemcpy(s.tap_dev, taps.data(), sizeof(int) * taps.size(), hipMemcpyHostToDevice);
+    }
+    if (what || e != hipSuccess) {
       for (auto& t : plan->subs) free_sub(t);
       delete plan;
-      return fail("mcConvPlanCreate: device set-up failed: %s", hipGetErrorString(e));
+      return what ? fail("mcConvPlanCreate: %s", what)
+                  : fail("mcConvPlanCreate: device set-up failed: %s", hipGetErrorString(e));
     }
   }
   *out = plan;
@@ -731,6 +862,10 @@ int mcConvPlanSetWeights(mcConvPlan* plan, const float* weights, void* stream) {
 
 int mcConvPlanForceConfig(mcConvPlan* plan, int config) {
   MC_REQUIRE(plan, "mcConvPlanForceConfig: null plan");
+  // config + 100 pins the same tile with the tap-table gather (tests compare the
+  // pointwise fast path against it)
+  plan->force_general = config >= 100;
+  if (config >= 100) config -= 100;
   MC_REQUIRE(config >= -1 && config < kNumConfigs, "mcConvPlanForceConfig: no such configuration");
   plan->forced_config = config;
   return 0;
@@ -750,8 +885,9 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
   const mcConvGeom& g = plan->geom;
   const long in_count = (long)num * g.channels_in * g.height_in * g.width_in;
   const long out_count = (long)num * g.channels_out * plan->Ho * plan->Wo;
-  MC_REQUIRE(in_count < (1L << 31) && out_count < (1L << 31),
-             "mcConvForward: blob exceeds 2^31 elements");
+  // the bottom blob is addressed through a 31-bit byte offset
+  MC_REQUIRE(in_count < (1L << 29) && out_count < (1L << 31),
+             "mcConvForward: bottom blob exceeds 2^29 or top blob 2^31 elements");
   hipStream_t st = static_cast<hipStream_t>(stream);
   for (const auto& s : plan->subs) {
     const long pixels = (long)num * s.Hq * s.Wq;
@@ -759,10 +895,23 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
     MC_REQUIRE(pixels < (1L << 31), "mcConvForward: too many output pixels");
     const TileConfig& cfg = kConfigs[pick_config(plan, pixels)];
     IgemmArgs a;
-    a.x = bottom;
     a.wt = s.wt_dev;
     a.y = top;
     a.ktab = s.ktab_dev;
+    a.tap_dh = s.tap_dev;
+    a.tap_dw = s.tap_dev + s.tap_dh.size();
+    // a sub-problem without taps (K == 0) has no tables on the device
+    a.n_dh = s.tap_dev ? static_cast<int>(s.tap_dh.size()) : 0;
+    a.n_dw = s.tap_dev ? static_cast<int>(s.tap_dw.size()) : 0;
+    const long shift = (long)s.tap_shift + s.pix_shift;
+    MC_REQUIRE(in_count * 4 + 2 * shift + 64 < (1L << 31),
+               "mcConvForward: bottom blob too large for 31-bit byte offsets");
+    a.x = reinterpret_cast<const float*>(reinterpret_cast<const char*>(bottom) - shift);
+    a.x_bytes = static_cast<unsigned>(in_count * 4 + shift);
+    a.pix_shift = s.pix_shift;
+    a.wt_bytes = static_cast<unsigned>(sizeof(float) * (size_t)g.group * s.Kpad * plan->Mpad);
+    a.K = s.K;
+    a.x_cstride = g.height_in * g.width_in;
     a.scale = ep ? ep->scale : nullptr;
     a.shift = ep ? ep->shift : nullptr;
     a.residual = ep ? ep->residual : nullptr;
@@ -817,7 +966,8 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
       tl.name = cfg.name;
       MC_HIP(hipEventRecord(tl.start, st));
     }
-    cfg.kernel<<<grid, 256, 0, st>>>(a);
+    const bool pointwise = s.pointwise && !plan->force_general;
+    (pointwise ? cfg.kernel_pw : cfg.kernel)<<<grid, 256, 0, st>>>(a);
     MC_LAUNCH_CHECK();
     if (slices > 1) {
       splitk_reduce_kernel<<<static_cast<unsigned>(ceil_div(out_count, 1024L)), 256, 0, st>>>(
