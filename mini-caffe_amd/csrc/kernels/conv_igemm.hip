@@ -59,6 +59,9 @@ struct IgemmArgs {
   const float* __restrict__ residual;
   int P;              // pixels = num * Hq * Wq
   int Hq, Wq, HqWq;   // iteration grid of this sub-problem
+  unsigned div_hw_mul, div_hw_shift;  // p / HqWq  as multiply-high and shift (shift 32: divisor 1)
+  unsigned div_w_mul, div_w_shift;    // rem / Wq
+  unsigned y_bytes, c_bytes;          // top blob and per-channel vector extents (descriptors)
   int H, W;           // bottom height / width
   int q_sh, q_sw;     // bottom origin of pixel (qh,qw): qh*q_sh + in_oh
   int in_oh, in_ow;
@@ -81,6 +84,11 @@ struct IgemmArgs {
 
 __device__ __forceinline__ float f4at(const float4& v, int e) {
   return e == 0 ? v.x : (e == 1 ? v.y : (e == 2 ? v.z : v.w));
+}
+
+// n / d for the d the host prepared (mul, shift) for; shift == 32 means d == 1.
+__device__ __forceinline__ int fast_div(int n, unsigned mul, unsigned shift) {
+  return shift == 32 ? n : static_cast<int>(__umulhi(static_cast<unsigned>(n), mul) >> shift);
 }
 
 __device__ __forceinline__ float apply_act(float v, int act, float slope) {
@@ -171,9 +179,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
   {
     const int p = nt * BN + pj;
     if (p < a.P) {
-      const int n = p / a.HqWq;
+      const int n = fast_div(p, a.div_hw_mul, a.div_hw_shift);
       const int rem = p - n * a.HqWq;
-      const int qh = rem / a.Wq;
+      const int qh = fast_div(rem, a.div_w_mul, a.div_w_shift);
       const int qw = rem - qh * a.Wq;
       const int hi0 = qh * a.q_sh + a.in_oh;
       const int wi0 = qw * a.q_sw + a.in_ow;
@@ -348,23 +356,42 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 
   // Epilogue.  Accumulator register r of lane l holds row 8*(r/4)+4*(l/32)+r%4,
   // column l%32 of its 32x32 block; a half-wave therefore stores 32 consecutive
-  // pixels of one output channel.  Per-channel factors and residual values are
-  // fetched in batches whose loads all issue before the first use, so a block
-  // pays a few load latencies instead of one per value.
+  // pixels of one output channel.  Like the K loop it addresses through buffer
+  // descriptors: one VGPR offset per lane (bit 31 set for a column past the last
+  // pixel, which drops its stores), the row as a scalar offset.  Per-channel
+  // factors and residual values are fetched eight rows at a time, all loads of
+  // a batch issued before the first use.
   const bool has_scale = a.scale != nullptr;
   const bool has_shift = a.shift != nullptr;
   const bool has_res = a.residual != nullptr;
-  // "no activation" is a leaky ReLU of slope 1, so one select covers both.
-  const bool relu_like = a.act == MC_ACT_NONE || a.act == MC_ACT_RELU;
-  const float slope = a.act == MC_ACT_NONE ? 1.f : a.slope;
+  const __amdgpu_buffer_rsrc_t yres =
+      __builtin_amdgcn_make_buffer_rsrc(yout, 0, a.y_bytes, kBufferFlags);
+  const __amdgpu_buffer_rsrc_t rres = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(a.residual), 0, has_res ? a.y_bytes : 0, kBufferFlags);
+  const __amdgpu_buffer_rsrc_t sres = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(a.scale), 0, has_scale ? a.c_bytes : 0, kBufferFlags);
+  const __amdgpu_buffer_rsrc_t hres = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(a.shift), 0, has_shift ? a.c_bytes : 0, kBufferFlags);
+  // 0: none, 1: ReLU (max with 0), 2: leaky ReLU, 3: TanH / Sigmoid
+  const int act_mode = a.act == MC_ACT_NONE ? 0
+                       : a.act == MC_ACT_RELU ? (a.slope == 0.f ? 1 : 2)
+                                              : 3;
+  const unsigned cs4 = static_cast<unsigned>(a.y_cstride) * 4;
 #define MC_ROW(r) (8 * ((r) / 4) + ((r) % 4))
+#define MC_LOADF(res, voff, soff) \
+  __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(res, voff, soff, 0))
+#define MC_STORE_ROWS(EXPR)                                                                  \
+  _Pragma("unroll") for (int q = 0; q < 8; ++q) {                                            \
+    const float v = acc[i][j][half * 8 + q];                                                 \
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, (EXPR)), yres, y_voff,\
+                                          MC_ROW(half * 8 + q) * cs4, 0);                    \
+  }
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int p = nt * BN + wn0 + j * 32 + l32;
-    if (p >= a.P) continue;
-    const int n = p / a.HqWq;
+    const int n = fast_div(p, a.div_hw_mul, a.div_hw_shift);
     const int rem = p - n * a.HqWq;
-    const int qh = rem / a.Wq;
+    const int qh = fast_div(rem, a.div_w_mul, a.div_w_shift);
     const int qw = rem - qh * a.Wq;
     const int ybase =
         n * a.y_nstride + (qh * a.out_sh + a.out_oh) * a.Wo + qw * a.out_sw + a.out_ow;
@@ -373,10 +400,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
       const int mblock = mt * BM + wm0 + i * 32;  // wave-uniform
       const int m0 = mblock + 4 * lhi;
       if (mblock + 32 <= a.M) {
-        // All 32 rows are real channels: constant offsets from one base.
+        // All 32 rows are real channels.
         const unsigned c0 = g * a.M + m0;
-        const unsigned y0 = ybase + c0 * a.y_cstride;
-        const unsigned cs = a.y_cstride;
+        const unsigned c_voff = c0 * 4;
+        const unsigned y_voff =
+            p < a.P ? static_cast<unsigned>(ybase + c0 * a.y_cstride) * 4 : kNoElement;
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
           if (has_scale | has_shift) {
@@ -385,8 +413,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
             for (int q = 0; q < 8; ++q) {
               sc[q] = 1.f;
               sh[q] = 0.f;
-              if (has_scale) sc[q] = a.scale[c0 + MC_ROW(half * 8 + q)];
-              if (has_shift) sh[q] = a.shift[c0 + MC_ROW(half * 8 + q)];
+              if (has_scale) sc[q] = MC_LOADF(sres, c_voff, MC_ROW(half * 8 + q) * 4);
+              if (has_shift) sh[q] = MC_LOADF(hres, c_voff, MC_ROW(half * 8 + q) * 4);
             }
 #pragma unroll
             for (int q = 0; q < 8; ++q)
@@ -395,24 +423,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
           if (has_res) {
             float rs[8];
 #pragma unroll
-            for (int q = 0; q < 8; ++q) rs[q] = a.residual[y0 + MC_ROW(half * 8 + q) * cs];
+            for (int q = 0; q < 8; ++q) rs[q] = MC_LOADF(rres, y_voff, MC_ROW(half * 8 + q) * cs4);
 #pragma unroll
             for (int q = 0; q < 8; ++q) acc[i][j][half * 8 + q] += rs[q];
           }
-          if (relu_like) {
-#pragma unroll
-            for (int q = 0; q < 8; ++q) {
-              const float v = acc[i][j][half * 8 + q];
-              yout[y0 + MC_ROW(half * 8 + q) * cs] = v > 0.f ? v : v * slope;
-            }
+          if (act_mode == 0) {
+            MC_STORE_ROWS(v)
+          } else if (act_mode == 1) {
+            MC_STORE_ROWS(fmaxf(v, 0.f))
+          } else if (act_mode == 2) {
+            MC_STORE_ROWS(v > 0.f ? v : v * a.slope)
           } else {
-#pragma unroll
-            for (int q = 0; q < 8; ++q)
-              yout[y0 + MC_ROW(half * 8 + q) * cs] =
-                  apply_act(acc[i][j][half * 8 + q], a.act, a.slope);
+            MC_STORE_ROWS(apply_act(v, a.act, a.slope))
           }
         }
-      } else {
+      } else if (p < a.P) {
         // Block straddles the last channel: row by row, skipping rows >= M.
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -424,13 +449,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
             if (has_shift) v += a.shift[c];
             const int yo = ybase + c * a.y_cstride;
             if (has_res) v += a.residual[yo];
-            yout[yo] = relu_like ? (v > 0.f ? v : v * slope) : apply_act(v, a.act, a.slope);
+            yout[yo] = apply_act(v, a.act, a.slope);
           }
         }
       }
     }
   }
 #undef MC_ROW
+#undef MC_LOADF
+#undef MC_STORE_ROWS
 }
 
 // Split-K tail: y = act((sum over slices, in slice order) * scale[c] + shift[c]
@@ -655,6 +682,26 @@ int free_sub(SubProblem& s) {
   s.wk_off_dev = nullptr;
   s.wt_dev = nullptr;
   return 0;
+}
+
+// Multiplier and shift with  n / d == mulhi(n, mul) >> shift  for 0 <= n < n_max.
+// shift 32 stands for d == 1 (no 32-bit multiplier exists for it).
+void make_fast_div(unsigned d, unsigned long long n_max, unsigned* mul, unsigned* shift) {
+  *mul = 0;
+  *shift = 32;
+  if (d <= 1) return;
+  for (int s = 31; s >= 0; --s) {
+    const unsigned __int128 pow = (unsigned __int128)1 << (32 + s);
+    const unsigned __int128 m = (pow + d - 1) / d;
+    if (m >> 32) continue;
+    const unsigned __int128 err = m * d - pow;  // 0 <= err < d
+    if (err * n_max < pow) {
+      *mul = static_cast<unsigned>(m);
+      *shift = static_cast<unsigned>(s);
+      return;
+    }
+  }
+  // unreachable for n_max < 2^32: s = 0 gives err * n_max < d * 2^32 / d
 }
 
 // floor division for possibly negative numerators
@@ -886,8 +933,8 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
   const long in_count = (long)num * g.channels_in * g.height_in * g.width_in;
   const long out_count = (long)num * g.channels_out * plan->Ho * plan->Wo;
   // the bottom blob is addressed through a 31-bit byte offset
-  MC_REQUIRE(in_count < (1L << 29) && out_count < (1L << 31),
-             "mcConvForward: bottom blob exceeds 2^29 or top blob 2^31 elements");
+  MC_REQUIRE(in_count < (1L << 29) && out_count < (1L << 29),
+             "mcConvForward: blob exceeds 2^29 elements");
   hipStream_t st = static_cast<hipStream_t>(stream);
   for (const auto& s : plan->subs) {
     const long pixels = (long)num * s.Hq * s.Wq;
@@ -919,6 +966,11 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
     a.Hq = s.Hq;
     a.Wq = s.Wq;
     a.HqWq = s.Hq * s.Wq;
+    // columns up to the end of the last pixel tile are divided (and then ignored)
+    make_fast_div(a.HqWq, pixels + 512, &a.div_hw_mul, &a.div_hw_shift);
+    make_fast_div(a.Wq, (unsigned long long)a.HqWq + 1, &a.div_w_mul, &a.div_w_shift);
+    a.y_bytes = static_cast<unsigned>(out_count * 4);
+    a.c_bytes = static_cast<unsigned>(g.channels_out) * 4;
     a.H = g.height_in;
     a.W = g.width_in;
     a.q_sh = s.q_sh;
