@@ -35,6 +35,9 @@ def main():
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-batch", type=int, default=8)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="first run one plain 256 MiB device copy (mcCopy2D): under rocprofv3 --pmc "
+                         "its FETCH_SIZE / WRITE_SIZE reading calibrates the counters")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported "
@@ -48,6 +51,18 @@ def main():
     if not mc.check_gpu_available():
         sys.exit("bench.py: no HIP device visible")
     mc.set_runtime_mode(1, 0)
+
+    if args.copy_calibration:
+        import torch
+        from minicaffe import kernels  # noqa: F401  (declares the mc* prototypes: 64-bit pointers)
+        n = 64 << 20                      # floats: 256 MiB read, 256 MiB written
+        src = torch.ones(n, device="cuda")
+        dst = torch.empty(n, device="cuda")
+        for _ in range(2):
+            rc = LIB.mcCopy2D(ctypes.c_void_p(src.data_ptr()), n, ctypes.c_void_p(dst.data_ptr()), n, n, 1, None)
+            assert rc == 0, LIB.mcLastError()
+        torch.cuda.synchronize()
+        del src, dst
 
     spec, inputs = zoo.resnet50_spec(batch=args.batch, size=224, seed=0)
     flops = zoo.conv_flops(spec, inputs)

@@ -6,6 +6,7 @@ Net, Blob, set_mode helpers and the profiler, bound through ctypes to libcaffe.s
 from .base import LIB, LIB_PATH, MiniCaffeError, check_call  # noqa: F401
 from .blob import Blob  # noqa: F401
 from .net import Net  # noqa: F401
+from . import kernels  # noqa: F401  (declares the prototypes of the mc* kernel entry points)
 
 
 def check_gpu_available():

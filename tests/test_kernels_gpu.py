@@ -115,6 +115,97 @@ def test_conv_epilogue_matches_unfused_chain(K):
     assert netrun.rel_err(yd.cpu().numpy(), want) < 1e-4
 
 
+
+def _run_plan(K, plan, n, x, wt, out_shape, **ep):
+    xd, wd = dev(x), dev(wt)
+    keep = {k: dev(v) for k, v in ep.items() if isinstance(v, np.ndarray)}
+    args = {k: (keep[k].data_ptr() if k in keep else v) for k, v in ep.items()}
+    yd = torch.full(out_shape, float("nan"), device="cuda")
+    plan.set_weights(wd.data_ptr())
+    plan.forward(n, xd.data_ptr(), yd.data_ptr(), **args)
+    torch.cuda.synchronize()
+    return yd.cpu().numpy()
+
+
+@pytest.mark.parametrize("case", [
+    # cin, h, w, cout, stride, batch: 1x1 kernels without padding
+    (64, 14, 14, 256, 1, 3), (256, 14, 14, 128, 2, 2), (100, 1, 1, 1000, 1, 7), (40, 9, 7, 24, 1, 2),
+    (70, 5, 5, 64, 3, 2)])
+def test_conv_pointwise_path_equals_tap_table_path(K, case):
+    """A 1x1 unpadded convolution takes a K loop without tap table; pinned to the
+    general loop (configuration + 100) it must give the same bits: both add the
+    same products in the same order."""
+    cin, h, w, cout, s, n = case
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((n, cin, h, w)).astype(np.float32)
+    wt = (rng.standard_normal((cout, cin, 1, 1)) * 0.1).astype(np.float32)
+    b = rng.standard_normal(cout).astype(np.float32)
+    want = oracle.conv_forward(oracle.conv_geom(cin, h, w, cout, 1, s, 0), x, wt, b)
+    got = {}
+    for cfg in (3, 103):
+        plan = K.ConvPlan(K.conv_geom(cin, h, w, cout, 1, s, 0))
+        plan.force_config(cfg)
+        plan.force_split(1)
+        got[cfg] = _run_plan(K, plan, n, x, wt, want.shape, shift=b)
+    assert np.array_equal(got[3], got[103])
+    assert netrun.rel_err(got[3], want) < 1e-4
+
+
+@pytest.mark.parametrize("slices", [2, 3, 5, 64])
+@pytest.mark.parametrize("geom", [(96, 14, 14, 64, 3, 1, 1), (512, 7, 7, 96, 1, 1, 0), (20, 6, 5, 40, 3, 2, 1)])
+def test_conv_split_k_with_epilogue(K, geom, slices):
+    """K cut into slices whose partial sums a second kernel adds in slice order,
+    then scale, shift, residual and activation: against the oracle and against
+    the unsliced launch (slices beyond the K tile count are clamped)."""
+    cin, h, w, cout, k, s, p = geom
+    n = 2
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((n, cin, h, w)).astype(np.float32)
+    wt = (rng.standard_normal((cout, cin, k, k)) * 0.1).astype(np.float32)
+    sc = (rng.random(cout) + 0.5).astype(np.float32)
+    sh = rng.standard_normal(cout).astype(np.float32)
+    y = oracle.conv_forward(oracle.conv_geom(cin, h, w, cout, k, s, p), x, wt, None)
+    res = rng.standard_normal(y.shape).astype(np.float32)
+    want = oracle.relu(oracle.eltwise([oracle.scale(y, sc, sh), res], "SUM"), 0.0)
+    outs = []
+    for S in (1, slices):
+        plan = K.ConvPlan(K.conv_geom(cin, h, w, cout, k, s, p))
+        plan.force_split(S)
+        outs.append(_run_plan(K, plan, n, x, wt, want.shape, scale=sc, shift=sh, residual=res,
+                              activation=K.ACT_RELU, negative_slope=0.0))
+    assert netrun.rel_err(outs[0], want) < 1e-4
+    assert netrun.rel_err(outs[1], want) < 1e-4
+    assert netrun.rel_err(outs[1], outs[0]) < 1e-4   # summation order only
+
+
+@pytest.mark.parametrize("act,slope", [("none", 0.0), ("relu", 0.0), ("relu", 0.2), ("tanh", 0.0),
+                                       ("sigmoid", 0.0)])
+def test_conv_epilogue_activations_full_channel_blocks(K, act, slope):
+    """64 output channels: every 32-row block takes the batched epilogue path."""
+    rng = np.random.default_rng(5)
+    n, cin, cout, h = 2, 16, 64, 7
+    x = rng.standard_normal((n, cin, h, h)).astype(np.float32)
+    wt = (rng.standard_normal((cout, cin, 3, 3)) * 0.1).astype(np.float32)
+    b = rng.standard_normal(cout).astype(np.float32)
+    y = oracle.conv_forward(oracle.conv_geom(cin, h, h, cout, 3, 1, 1), x, wt, b)
+    want = {"none": lambda v: v, "relu": lambda v: oracle.relu(v, slope), "tanh": oracle.tanh,
+            "sigmoid": oracle.sigmoid}[act](y)
+    code = {"none": K.ACT_NONE, "relu": K.ACT_RELU, "tanh": K.ACT_TANH, "sigmoid": K.ACT_SIGMOID}[act]
+    plan = K.ConvPlan(K.conv_geom(cin, h, h, cout, 3, 1, 1))
+    got = _run_plan(K, plan, n, x, wt, want.shape, shift=b, activation=code, negative_slope=slope)
+    assert netrun.rel_err(got, want) < 1e-4
+
+
+def test_conv_limits_are_errors(K):
+    from minicaffe import MiniCaffeError
+    with pytest.raises(MiniCaffeError, match="31 taps"):
+        K.ConvPlan(K.conv_geom(1, 40, 40, 1, 33))
+    # a bottom blob of 2^29 elements or more cannot be addressed: refused before any launch
+    plan = K.ConvPlan(K.conv_geom(1024, 1024, 1024, 1, 1))
+    dummy = torch.zeros(16, device="cuda")
+    with pytest.raises(MiniCaffeError, match="2\\^29"):
+        plan.forward(1, dummy.data_ptr(), dummy.data_ptr())
+
 def test_conv_rejects_bad_geometry(K):
     from minicaffe import MiniCaffeError
     with pytest.raises(MiniCaffeError, match="multiples of group"):
