@@ -23,8 +23,8 @@ sys.path.insert(0, os.path.join(ROOT, "mini-caffe_amd"))
 FP32_MFMA_PEAK_TFLOPS = 157.3
 # HBM bytes per convolution launch (mean over the 53 launches of one forward),
 # from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in
-# profiles/igemm_resnet50_b64_pmc.txt; None until measured.
-CONV_TRAFFIC_BYTES_PER_LAUNCH = None
+# profiles/igemm_resnet50_b64_pmc_traffic.txt (algorithmic: 126.3e6).
+CONV_TRAFFIC_BYTES_PER_LAUNCH = 149.4e6
 
 
 def main():
