@@ -35,6 +35,9 @@ def main():
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-batch", type=int, default=8)
+    ap.add_argument("--configs-report", metavar="PATH",
+                    help="also time all five BASELINE configurations (whole forward, contraction "
+                         "launches, Proposal / DetectionOutput layers) and write a text table to PATH")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="first run one plain 256 MiB device copy (mcCopy2D): under rocprofv3 --pmc "
                          "its FETCH_SIZE / WRITE_SIZE reading calibrates the counters")
@@ -100,6 +103,9 @@ def main():
                 "kernel_ms_per_step": round(tot_ms.value / max(1, args.steps), 3),
                 "gflop_per_step": round(fl.value / max(1, args.steps) / 1e9, 1)}
 
+    if args.configs_report:
+        configs_report(args.configs_report, mc, craft, zoo, LIB)
+
     cpu = None
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(args.cpu_batch)
@@ -115,6 +121,62 @@ def main():
                       "api": "CaffeNetForward (Net::Forward(reshape=true))"},
            "roofline": roofline, "cpu_baseline": cpu}
     print(json.dumps(out))
+
+
+def configs_report(path, mc, craft, zoo, LIB):
+    """Whole-forward time, contraction TFLOP/s and detection-tail layer time of the five
+    BASELINE configurations on the GPU (synthetic inputs and weights from the zoo builders)."""
+    import tempfile
+    cases = [("C1 conv3x3+ReLU 1x64x56x56", zoo.c1_spec(seed=0), ()),
+             ("C2 ResNet-50 b64", zoo.resnet50_spec(batch=64, size=224, seed=0), ()),
+             ("C3 SSD300-VGG16 b8", zoo.ssd300_spec(batch=8, seed=0), ("detection_out",)),
+             ("C4 RPN+Proposal 1x1024x38x63", zoo.rpn_spec(seed=0), ("proposal",)),
+             ("C5 DCGAN generator b128", zoo.dcgan_spec(batch=128, seed=0), ())]
+    lines = ["%-30s %10s %10s %12s %10s %8s  %s" % ("configuration", "ms/forward", "GFLOP", "contr. ms",
+                                                    "TFLOP/s", "of peak", "tail layers (us, device time)")]
+    for name, (spec, inputs), tails in cases:
+        net = mc.Net.from_buffers(craft.to_prototxt(spec, "net"))
+        craft.load_weights(net, spec)
+        net.forward(**inputs)
+        reps = 20
+        for _ in range(3):
+            net.forward()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            net.forward()
+        ms = 1e3 * (time.perf_counter() - t0) / reps
+        LIB.mcConvTimingEnable(1)
+        for _ in range(reps):
+            net.forward()
+        tot_ms, launches, fl = ctypes.c_double(), ctypes.c_long(), ctypes.c_double()
+        LIB.mcConvTimingCollect(ctypes.byref(tot_ms), ctypes.byref(launches), ctypes.byref(fl))
+        LIB.mcConvTimingEnable(0)
+        tail_txt = ""
+        if tails:
+            # per-layer device time: the profiler synchronises the stream at every scope
+            mc.Profiler.enable()
+            for _ in range(reps):
+                net.forward()
+            mc.Profiler.disable()
+            with tempfile.NamedTemporaryFile(suffix=".json") as tf:
+                mc.Profiler.dump(tf.name)
+                events = json.load(open(tf.name))["traceEvents"]
+            begin, spans = {}, {}
+            for e in events:
+                if e["ph"] == "B":
+                    begin[e["name"]] = e["ts"]
+                elif e["name"] in begin:
+                    spans.setdefault(e["name"], []).append(e["ts"] - begin.pop(e["name"]))
+            tail_txt = ", ".join("%s %.0f (median of %d)" % (t, sorted(spans[t])[len(spans[t]) // 2],
+                                                             len(spans[t])) for t in tails if t in spans)
+        cms = tot_ms.value / reps
+        tf_s = fl.value / (tot_ms.value * 1e-3) / 1e12 if tot_ms.value else 0.0
+        lines.append("%-30s %10.3f %10.2f %12.3f %10.1f %7.1f%%  %s"
+                     % (name, ms, fl.value / reps / 1e9, cms, tf_s, 100 * tf_s / FP32_MFMA_PEAK_TFLOPS,
+                        tail_txt))
+        del net
+    with open(path, "w") as f:
+        f.write("\n".join(lines) + "\n")
 
 
 def cpu_baseline(batch):

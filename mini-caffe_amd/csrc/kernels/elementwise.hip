@@ -85,36 +85,71 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
-// Sum over a 256-thread workgroup; every thread gets the result.
-__device__ __forceinline__ float block_sum_256(float v, float* lds4) {
+// Sum over a workgroup of up to 1024 threads; every thread gets the result.
+__device__ __forceinline__ float block_sum(float v, float* lds16) {
   v = wave_sum(v);
   __syncthreads();
-  if ((threadIdx.x & 63) == 0) lds4[threadIdx.x >> 6] = v;
+  if ((threadIdx.x & 63) == 0) lds16[threadIdx.x >> 6] = v;
   __syncthreads();
-  return lds4[0] + lds4[1] + lds4[2] + lds4[3];
+  float t = 0.f;
+  for (int w = 0; w < static_cast<int>(blockDim.x >> 6); ++w) t += lds16[w];
+  return t;
 }
 
-__global__ __launch_bounds__(256) void bn_batch_stats_kernel(const float* __restrict__ x, int num,
-                                                             int C, int spatial, float eps,
-                                                             float* __restrict__ mean,
-                                                             float* __restrict__ stdev) {
-  __shared__ float red[4];
+// Batch statistics of one channel per workgroup (1024 threads): mean, then the
+// mean of squared deviations, as two passes over the channel's num x spatial
+// values (the second pass re-reads them from cache).  VEC = 4 walks each image's
+// plane with float4 loads; the (image, position) pair of a thread advances by a
+// fixed step, so the loops hold no division.
+template <int VEC>
+__global__ __launch_bounds__(1024) void bn_batch_stats_kernel(const float* __restrict__ x, int num,
+                                                              int C, int spatial, float eps,
+                                                              float* __restrict__ mean,
+                                                              float* __restrict__ stdev) {
+  __shared__ float red[16];
   const int c = blockIdx.x;
-  const long per_c = (long)num * spatial;
+  const int per_row = spatial / VEC;                    // vectors per image plane
+  const int step_n = blockDim.x / per_row, step_v = blockDim.x % per_row;
+  const int n0 = threadIdx.x / per_row, v0 = threadIdx.x % per_row;
   const float alpha = static_cast<float>(1. / (static_cast<double>(num) * spatial));
+  const long plane = spatial, image = (long)C * spatial;
+  const float* __restrict__ xc = x + c * plane;
   float s = 0.f;
-  for (long i = threadIdx.x; i < per_c; i += 256) {
-    const long n = i / spatial, sp = i - n * spatial;
-    s += x[(n * C + c) * spatial + sp];
+  for (int n = n0, v = v0; n < num;) {
+    const float* p = xc + n * image + v * VEC;
+    if (VEC == 4) {
+      const float4 t = *reinterpret_cast<const float4*>(p);
+      s += (t.x + t.y) + (t.z + t.w);
+    } else {
+      s += *p;
+    }
+    n += step_n;
+    v += step_v;
+    if (v >= per_row) {
+      v -= per_row;
+      ++n;
+    }
   }
-  const float m = alpha * block_sum_256(s, red);
+  const float m = alpha * block_sum(s, red);
   float q = 0.f;
-  for (long i = threadIdx.x; i < per_c; i += 256) {
-    const long n = i / spatial, sp = i - n * spatial;
-    const float d = x[(n * C + c) * spatial + sp] - m;
-    q += d * d;
+  for (int n = n0, v = v0; n < num;) {
+    const float* p = xc + n * image + v * VEC;
+    if (VEC == 4) {
+      const float4 t = *reinterpret_cast<const float4*>(p);
+      const float d0 = t.x - m, d1 = t.y - m, d2 = t.z - m, d3 = t.w - m;
+      q += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+    } else {
+      const float d = *p - m;
+      q += d * d;
+    }
+    n += step_n;
+    v += step_v;
+    if (v >= per_row) {
+      v -= per_row;
+      ++n;
+    }
   }
-  const float var = alpha * block_sum_256(q, red);
+  const float var = alpha * block_sum(q, red);
   if (threadIdx.x == 0) {
     mean[c] = m;
     stdev[c] = sqrtf(var + eps);
@@ -278,8 +313,15 @@ int mcBatchNormBatchStats(const float* x, int num, int channels, int spatial, fl
                           float* mean, float* stdev, void* stream) {
   MC_REQUIRE(x && mean && stdev, "mcBatchNormBatchStats: null argument");
   MC_REQUIRE(num > 0 && channels > 0 && spatial > 0, "mcBatchNormBatchStats: bad extents");
-  bn_batch_stats_kernel<<<channels, 256, 0, static_cast<hipStream_t>(stream)>>>(
-      x, num, channels, spatial, eps, mean, stdev);
+  const bool vec = spatial % 4 == 0 && aligned16(x);
+  const long per_c = (long)num * (vec ? spatial / 4 : spatial);
+  const int threads = per_c >= 1024 ? 1024 : 256;
+  if (vec)
+    bn_batch_stats_kernel<4><<<channels, threads, 0, static_cast<hipStream_t>(stream)>>>(
+        x, num, channels, spatial, eps, mean, stdev);
+  else
+    bn_batch_stats_kernel<1><<<channels, threads, 0, static_cast<hipStream_t>(stream)>>>(
+        x, num, channels, spatial, eps, mean, stdev);
   MC_LAUNCH_CHECK();
   return 0;
 }

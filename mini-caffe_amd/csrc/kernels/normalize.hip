@@ -5,26 +5,39 @@
 namespace mchip {
 namespace {
 
-// One thread per (image, pixel): neighbouring threads read neighbouring pixels
-// of each channel plane, so every pass over the channels is coalesced.
+// A workgroup takes 32 consecutive pixels of one image; its 8 groups of 32
+// threads each sum every eighth channel, so a half-wave reads 128 contiguous
+// bytes of a channel plane and a pixel's channels are covered by 8 threads
+// instead of one serial walk.  The 8 partial sums are added in a fixed order.
+constexpr int kNormPix = 32, kNormSlices = 8;
 __global__ __launch_bounds__(256) void normalize_pixel_kernel(
-    const float* __restrict__ x, float* __restrict__ y, long pixels, int C, int spatial,
+    const float* __restrict__ x, float* __restrict__ y, int C, int spatial, int tiles_per_image,
     int channel_shared, float eps, const float* __restrict__ scale) {
-  for (long i = blockIdx.x * 256L + threadIdx.x; i < pixels; i += gridDim.x * 256L) {
-    const long n = i / spatial, s = i - n * spatial;
-    const float* __restrict__ xp = x + n * C * spatial + s;
-    float* __restrict__ yp = y + n * C * spatial + s;
-    float acc = eps;
-    for (int c = 0; c < C; ++c) {
+  __shared__ float part[kNormSlices][kNormPix];
+  const int n = blockIdx.x / tiles_per_image;
+  const int tile = blockIdx.x - n * tiles_per_image;
+  const int px = threadIdx.x % kNormPix, sl = threadIdx.x / kNormPix;
+  const int s = tile * kNormPix + px;
+  const bool live = s < spatial;
+  const float* __restrict__ xp = x + (long)n * C * spatial + s;
+  float* __restrict__ yp = y + (long)n * C * spatial + s;
+  float acc = 0.f;
+  if (live)
+    for (int c = sl; c < C; c += kNormSlices) {
       const float v = xp[(long)c * spatial];
       acc += v * v;
     }
-    const float norm = sqrtf(acc);
-    for (int c = 0; c < C; ++c) {
+  part[sl][px] = acc;
+  __syncthreads();
+  float sum = eps;
+#pragma unroll
+  for (int k = 0; k < kNormSlices; ++k) sum += part[k][px];
+  const float norm = sqrtf(sum);
+  if (live)
+    for (int c = sl; c < C; c += kNormSlices) {
       const float v = xp[(long)c * spatial] / norm;
       yp[(long)c * spatial] = v * (channel_shared ? scale[0] : scale[c]);
     }
-  }
 }
 
 // One workgroup per image.
@@ -65,9 +78,10 @@ extern "C" int mcNormalize(const float* bottom, float* top, int num, int channel
     normalize_image_kernel<<<num, 256, 0, st>>>(bottom, top, channels, spatial, channel_shared,
                                                 eps, scale);
   } else {
-    const long pixels = (long)num * spatial;
-    normalize_pixel_kernel<<<ew_blocks(pixels, 256), 256, 0, st>>>(
-        bottom, top, pixels, channels, spatial, channel_shared, eps, scale);
+    const int tiles = ceil_div(spatial, kNormPix);
+    MC_REQUIRE((long)num * tiles < (1L << 31), "mcNormalize: too many pixels");
+    normalize_pixel_kernel<<<num * tiles, 256, 0, st>>>(bottom, top, channels, spatial, tiles,
+                                                        channel_shared, eps, scale);
   }
   MC_LAUNCH_CHECK();
   return 0;
