@@ -82,6 +82,14 @@ struct IgemmArgs {
   float slope;
 };
 
+// Up to four sub-problems (the output-parity classes of a Deconvolution) run
+// in one launch: blockIdx.z = sub-problem * slices + K slice.
+constexpr int kMaxSubs = 4;
+struct IgemmBatch {
+  IgemmArgs sub[kMaxSubs];
+  int slices;
+};
+
 __device__ __forceinline__ float f4at(const float4& v, int e) {
   return e == 0 ? v.x : (e == 1 ? v.y : (e == 2 ? v.z : v.w));
 }
@@ -110,8 +118,16 @@ __device__ __forceinline__ float apply_act(float v, int act, float slope) {
 // tap table and no bounds handling at all.
 template <int BM, int BN, int WM, int WN, int OCC, bool PW>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void igemm_kernel(
-    const IgemmArgs a) {
+    const IgemmBatch batch) {
   static_assert(WM * WN == 4, "four wavefronts per workgroup");
+  int sub_index = 0, kslice = blockIdx.z;
+  while (kslice >= batch.slices) {  // at most kMaxSubs - 1 rounds, on the scalar unit
+    kslice -= batch.slices;
+    ++sub_index;
+  }
+  const IgemmArgs& a = batch.sub[sub_index];
+  // sub-problems of one launch may differ in tile count: the grid is the largest
+  if (static_cast<int>(blockIdx.x) >= a.MT * a.NT) return;
   static_assert(BN >= 64 && 256 % BN == 0, "BN must be 64, 128 or 256");
   constexpr int TM = BM / WM / 32;
   constexpr int TN = BN / WN / 32;
@@ -204,9 +220,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
   const int KT = a.Kpad / BK;
   // Split-K: slice z multiplies K tiles [kt_begin, kt_end) and writes its
   // partial sums into its own copy of the top blob.
-  const int kt_begin = blockIdx.z * a.kt_per_split;
+  const int kt_begin = kslice * a.kt_per_split;
   const int kt_end = min(KT, kt_begin + a.kt_per_split);
-  float* __restrict__ yout = a.y + (size_t)blockIdx.z * a.split_stride;
+  float* __restrict__ yout = a.y + (size_t)kslice * a.split_stride;
 
   // Packed filter: [g][K tile][m][16 k], so an A tile is one contiguous run:
   // per-thread byte offset inside the tile, scalar byte offset of the tile.
@@ -537,8 +553,8 @@ __global__ void pack_weights_kernel(const float* __restrict__ w, float* __restri
 struct TileConfig {
   int bm, bn;
   const char* name;
-  void (*kernel)(const IgemmArgs);
-  void (*kernel_pw)(const IgemmArgs);  // pointwise variant
+  void (*kernel)(const IgemmBatch);
+  void (*kernel_pw)(const IgemmBatch);  // pointwise variant
 };
 
 const TileConfig kConfigs[] = {
@@ -636,7 +652,6 @@ int pick_config(const mcConvPlan* plan, long pixels) {
 // prologue and the extra pass that sums the slices.
 int pick_split(const mcConvPlan* plan, long blocks, int KT) {
   if (plan->forced_split >= 1) return std::min(plan->forced_split, std::max(KT, 1));
-  if (plan->geom.transposed) return 1;
   const long slots = 8L * kNumCu;
   if (blocks * 2 > slots) return 1;
   int s = static_cast<int>(slots / blocks);
@@ -936,102 +951,137 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
   MC_REQUIRE(in_count < (1L << 29) && out_count < (1L << 29),
              "mcConvForward: blob exceeds 2^29 elements");
   hipStream_t st = static_cast<hipStream_t>(stream);
+
+  // Sub-problems that have pixels at this batch size, their tile configuration
+  // (one for the whole plan: the largest sub-problem decides) and K slices.
+  std::vector<const SubProblem*> live;
+  long max_pixels = 0;
   for (const auto& s : plan->subs) {
     const long pixels = (long)num * s.Hq * s.Wq;
     if (pixels == 0) continue;
     MC_REQUIRE(pixels < (1L << 31), "mcConvForward: too many output pixels");
-    const TileConfig& cfg = kConfigs[pick_config(plan, pixels)];
-    IgemmArgs a;
-    a.wt = s.wt_dev;
-    a.y = top;
-    a.ktab = s.ktab_dev;
-    a.tap_dh = s.tap_dev;
-    a.tap_dw = s.tap_dev + s.tap_dh.size();
-    // a sub-problem without taps (K == 0) has no tables on the device
-    a.n_dh = s.tap_dev ? static_cast<int>(s.tap_dh.size()) : 0;
-    a.n_dw = s.tap_dev ? static_cast<int>(s.tap_dw.size()) : 0;
-    const long shift = (long)s.tap_shift + s.pix_shift;
-    MC_REQUIRE(in_count * 4 + 2 * shift + 64 < (1L << 31),
-               "mcConvForward: bottom blob too large for 31-bit byte offsets");
-    a.x = reinterpret_cast<const float*>(reinterpret_cast<const char*>(bottom) - shift);
-    a.x_bytes = static_cast<unsigned>(in_count * 4 + shift);
-    a.pix_shift = s.pix_shift;
-    a.wt_bytes = static_cast<unsigned>(sizeof(float) * (size_t)g.group * s.Kpad * plan->Mpad);
-    a.K = s.K;
-    a.x_cstride = g.height_in * g.width_in;
-    a.scale = ep ? ep->scale : nullptr;
-    a.shift = ep ? ep->shift : nullptr;
-    a.residual = ep ? ep->residual : nullptr;
-    a.P = static_cast<int>(pixels);
-    a.Hq = s.Hq;
-    a.Wq = s.Wq;
-    a.HqWq = s.Hq * s.Wq;
-    // columns up to the end of the last pixel tile are divided (and then ignored)
-    make_fast_div(a.HqWq, pixels + 512, &a.div_hw_mul, &a.div_hw_shift);
-    make_fast_div(a.Wq, (unsigned long long)a.HqWq + 1, &a.div_w_mul, &a.div_w_shift);
-    a.y_bytes = static_cast<unsigned>(out_count * 4);
-    a.c_bytes = static_cast<unsigned>(g.channels_out) * 4;
-    a.H = g.height_in;
-    a.W = g.width_in;
-    a.q_sh = s.q_sh;
-    a.q_sw = s.q_sw;
-    a.in_oh = s.in_oh;
-    a.in_ow = s.in_ow;
-    a.x_nstride = g.channels_in * g.height_in * g.width_in;
-    a.x_gstride = plan->Cin_g * g.height_in * g.width_in;
-    a.M = plan->M;
-    a.Mpad = plan->Mpad;
-    a.Kpad = s.Kpad;
-    a.Wo = plan->Wo;
-    a.y_cstride = plan->Ho * plan->Wo;
-    a.y_nstride = g.channels_out * plan->Ho * plan->Wo;
-    a.out_sh = s.out_sh;
-    a.out_sw = s.out_sw;
-    a.out_oh = s.out_oh;
-    a.out_ow = s.out_ow;
-    a.MT = ceil_div(plan->M, cfg.bm);
-    a.NT = ceil_div(pixels, cfg.bn);
-    a.act = ep ? ep->activation : MC_ACT_NONE;
-    a.slope = ep ? ep->negative_slope : 0.f;
-    const long blocks = (long)a.MT * a.NT;
-    MC_REQUIRE(blocks < (1L << 31), "mcConvForward: grid too large");
-    const int KT = s.Kpad / BK;
-    int slices = plan->subs.size() == 1 ? pick_split(plan, blocks * g.group, KT) : 1;
-    a.kt_per_split = ceil_div(std::max(KT, 1), slices);
-    slices = ceil_div(std::max(KT, 1), a.kt_per_split);  // no empty slice
-    a.split_stride = 0;
-    const long slice_stride = (out_count + 3) / 4 * 4;
-    if (slices > 1) {
-      float* ws = nullptr;
-      if (get_workspace(st, sizeof(float) * slice_stride * slices, &ws)) return -1;
-      a.y = ws;
-      a.split_stride = static_cast<int>(slice_stride);
-      a.scale = a.shift = a.residual = nullptr;
-      a.act = MC_ACT_NONE;
+    live.push_back(&s);
+    max_pixels = std::max(max_pixels, pixels);
+  }
+  if (live.empty()) return 0;
+  const TileConfig& cfg = kConfigs[pick_config(plan, max_pixels)];
+  const int MT = ceil_div(plan->M, cfg.bm);
+  long total_blocks = 0;
+  int min_kt = 1 << 30;
+  bool pointwise = !plan->force_general;
+  double flops = 0.;
+  for (const SubProblem* s : live) {
+    const long pixels = (long)num * s->Hq * s->Wq;
+    total_blocks += (long)MT * ceil_div(pixels, cfg.bn) * g.group;
+    if (s->Kpad > 0) min_kt = std::min(min_kt, s->Kpad / BK);
+    pointwise = pointwise && s->pointwise;
+    flops += 2.0 * pixels * plan->M * g.group * s->K;
+  }
+  if (min_kt == (1 << 30)) min_kt = 1;
+  // slices are chosen for the plan as a whole: all sub-problems of a launch run
+  // side by side, and one pass sums the slices of the whole top blob
+  const int slices = pick_split(plan, total_blocks, min_kt);
+  const long slice_stride = (out_count + 3) / 4 * 4;
+  float* ws = nullptr;
+  if (slices > 1 && get_workspace(st, sizeof(float) * slice_stride * slices, &ws)) return -1;
+
+  TimedLaunch tl;
+  if (g_timing) {
+    MC_HIP(hipEventCreate(&tl.start));
+    MC_HIP(hipEventCreate(&tl.stop));
+    tl.flops = flops;
+    tl.name = cfg.name;
+    MC_HIP(hipEventRecord(tl.start, st));
+  }
+  for (size_t first = 0; first < live.size(); first += kMaxSubs) {
+    const int nsub = static_cast<int>(std::min<size_t>(kMaxSubs, live.size() - first));
+    IgemmBatch batch;
+    std::memset(&batch, 0, sizeof(batch));
+    batch.slices = slices;
+    long max_blocks = 0;
+    for (int i = 0; i < nsub; ++i) {
+      const SubProblem& s = *live[first + i];
+      const long pixels = (long)num * s.Hq * s.Wq;
+      IgemmArgs& a = batch.sub[i];
+      a.wt = s.wt_dev;
+      a.y = top;
+      a.ktab = s.ktab_dev;
+      a.tap_dh = s.tap_dev;
+      a.tap_dw = s.tap_dev + s.tap_dh.size();
+      // a sub-problem without taps (K == 0) has no tables on the device
+      a.n_dh = s.tap_dev ? static_cast<int>(s.tap_dh.size()) : 0;
+      a.n_dw = s.tap_dev ? static_cast<int>(s.tap_dw.size()) : 0;
+      const long shift = (long)s.tap_shift + s.pix_shift;
+      MC_REQUIRE(in_count * 4 + 2 * shift + 64 < (1L << 31),
+                 "mcConvForward: bottom blob too large for 31-bit byte offsets");
+      a.x = reinterpret_cast<const float*>(reinterpret_cast<const char*>(bottom) - shift);
+      a.x_bytes = static_cast<unsigned>(in_count * 4 + shift);
+      a.pix_shift = s.pix_shift;
+      a.wt_bytes = static_cast<unsigned>(sizeof(float) * (size_t)g.group * s.Kpad * plan->Mpad);
+      a.K = s.K;
+      a.x_cstride = g.height_in * g.width_in;
+      a.scale = ep ? ep->scale : nullptr;
+      a.shift = ep ? ep->shift : nullptr;
+      a.residual = ep ? ep->residual : nullptr;
+      a.P = static_cast<int>(pixels);
+      a.Hq = s.Hq;
+      a.Wq = s.Wq;
+      a.HqWq = s.Hq * s.Wq;
+      // columns up to the end of the last pixel tile are divided (and then ignored)
+      make_fast_div(a.HqWq, pixels + 512, &a.div_hw_mul, &a.div_hw_shift);
+      make_fast_div(a.Wq, (unsigned long long)a.HqWq + 1, &a.div_w_mul, &a.div_w_shift);
+      a.y_bytes = static_cast<unsigned>(out_count * 4);
+      a.c_bytes = static_cast<unsigned>(g.channels_out) * 4;
+      a.H = g.height_in;
+      a.W = g.width_in;
+      a.q_sh = s.q_sh;
+      a.q_sw = s.q_sw;
+      a.in_oh = s.in_oh;
+      a.in_ow = s.in_ow;
+      a.x_nstride = g.channels_in * g.height_in * g.width_in;
+      a.x_gstride = plan->Cin_g * g.height_in * g.width_in;
+      a.M = plan->M;
+      a.Mpad = plan->Mpad;
+      a.Kpad = s.Kpad;
+      a.Wo = plan->Wo;
+      a.y_cstride = plan->Ho * plan->Wo;
+      a.y_nstride = g.channels_out * plan->Ho * plan->Wo;
+      a.out_sh = s.out_sh;
+      a.out_sw = s.out_sw;
+      a.out_oh = s.out_oh;
+      a.out_ow = s.out_ow;
+      a.MT = MT;
+      a.NT = ceil_div(pixels, cfg.bn);
+      a.act = ep ? ep->activation : MC_ACT_NONE;
+      a.slope = ep ? ep->negative_slope : 0.f;
+      const long blocks = (long)a.MT * a.NT;
+      MC_REQUIRE(blocks < (1L << 31), "mcConvForward: grid too large");
+      max_blocks = std::max(max_blocks, blocks);
+      // every slice gets the same number of K tiles; slices past the last tile
+      // of a short sub-problem write zeros
+      a.kt_per_split = ceil_div(std::max(s.Kpad / BK, 1), slices);
+      a.split_stride = 0;
+      if (slices > 1) {
+        a.y = ws;
+        a.split_stride = static_cast<int>(slice_stride);
+        a.scale = a.shift = a.residual = nullptr;
+        a.act = MC_ACT_NONE;
+      }
     }
-    dim3 grid(static_cast<unsigned>(blocks), g.group, slices);
-    TimedLaunch tl;
-    if (g_timing) {
-      MC_HIP(hipEventCreate(&tl.start));
-      MC_HIP(hipEventCreate(&tl.stop));
-      tl.flops = 2.0 * pixels * plan->M * g.group * s.K;
-      tl.name = cfg.name;
-      MC_HIP(hipEventRecord(tl.start, st));
-    }
-    const bool pointwise = s.pointwise && !plan->force_general;
-    (pointwise ? cfg.kernel_pw : cfg.kernel)<<<grid, 256, 0, st>>>(a);
+    dim3 grid(static_cast<unsigned>(max_blocks), g.group, nsub * slices);
+    (pointwise ? cfg.kernel_pw : cfg.kernel)<<<grid, 256, 0, st>>>(batch);
     MC_LAUNCH_CHECK();
-    if (slices > 1) {
-      splitk_reduce_kernel<<<static_cast<unsigned>(ceil_div(out_count, 1024L)), 256, 0, st>>>(
-          a.y, slices, slice_stride, out_count, top, ep ? ep->scale : nullptr,
-          ep ? ep->shift : nullptr, ep ? ep->residual : nullptr, plan->Ho * plan->Wo,
-          g.channels_out, ep ? ep->activation : MC_ACT_NONE, ep ? ep->negative_slope : 0.f);
-      MC_LAUNCH_CHECK();
-    }
-    if (g_timing) {
-      MC_HIP(hipEventRecord(tl.stop, st));
-      g_timed.push_back(tl);
-    }
+  }
+  if (slices > 1) {
+    splitk_reduce_kernel<<<static_cast<unsigned>(ceil_div(out_count, 1024L)), 256, 0, st>>>(
+        ws, slices, slice_stride, out_count, top, ep ? ep->scale : nullptr,
+        ep ? ep->shift : nullptr, ep ? ep->residual : nullptr, plan->Ho * plan->Wo,
+        g.channels_out, ep ? ep->activation : MC_ACT_NONE, ep ? ep->negative_slope : 0.f);
+    MC_LAUNCH_CHECK();
+  }
+  if (g_timing) {
+    MC_HIP(hipEventRecord(tl.stop, st));
+    g_timed.push_back(tl);
   }
   return 0;
 }
