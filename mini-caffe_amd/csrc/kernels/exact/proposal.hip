@@ -112,6 +112,7 @@ __global__ __launch_bounds__(256) void proposal_order_gather_kernel(
 // of the scores (smaller key = larger score).  One 1024-thread workgroup; runs
 // only when `flag` says ties reach into the first num_top places.
 constexpr int kQsThreads = 1024;
+constexpr int kQsLds = 7168;  // places the LDS phase can hold (21 bytes each)
 
 __global__ __launch_bounds__(kQsThreads) void quicksort_replay_kernel(
     const int* __restrict__ flag, const uint32_t* __restrict__ key_in, int n, int num_top,
@@ -122,27 +123,43 @@ __global__ __launch_bounds__(kQsThreads) void quicksort_replay_kernel(
     int* __restrict__ nseg, unsigned char* __restrict__ cls, int* __restrict__ order_out) {
   if (*flag == 0) return;
   __shared__ unsigned long long wave_tot[kQsThreads / 64];
+  __shared__ int range_lo, range_hi, next_lo, next_hi;
   const int tid = threadIdx.x;
   // Phases that only need "every element once" walk the array with a stride of
   // the workgroup size (coalesced, iterations independent so loads overlap);
-  // the prefix sum needs contiguous per-thread runs.
-  const int per = (n + kQsThreads - 1) / kQsThreads;
-  const int begin = min(tid * per, n), end = min(begin + per, n);
+  // the prefix sum needs contiguous per-thread runs.  A position whose segment
+  // is finished (or lies wholly beyond num_top) is final: its index is written
+  // to order_out then, and later levels only walk [range_lo, range_hi], the
+  // span of the segments still open, which shrinks to about num_top places
+  // after the first few levels.
   for (int p = tid; p < n; p += kQsThreads) {
     kA[p] = key_in[p];
     vA[p] = p;
     seg_lo[p] = 0;
     seg_hi[p] = n - 1;
   }
+  if (tid == 0) {
+    range_lo = 0;
+    range_hi = n - 1;
+  }
   __syncthreads();
   uint32_t* __restrict__ key = kA;
   int* __restrict__ val = vA;
   uint32_t* __restrict__ nkey = kB;
   int* __restrict__ nval = vB;
+  bool open_left = true;
   for (;;) {
+    const int r0 = range_lo, r1 = range_hi + 1;  // open span [r0, r1)
+    if (r1 - r0 <= kQsLds && n <= 65535) break;  // small enough to finish in LDS
+    const int per = (r1 - r0 + kQsThreads - 1) / kQsThreads;
+    const int begin = min(r0 + tid * per, r1), end = min(begin + per, r1);
+    if (tid == 0) {
+      next_lo = n;
+      next_hi = -1;
+    }
     // 1. classify against the segment's pivot: 1 = smaller score, 2 = larger score
-#pragma unroll 8
-    for (int p = tid; p < n; p += kQsThreads) {
+#pragma unroll 12
+    for (int p = r0 + tid; p < r1; p += kQsThreads) {
       const int lo = seg_lo[p];
       unsigned char f = 0;
       if (lo >= 0 && p != lo) {
@@ -157,7 +174,7 @@ __global__ __launch_bounds__(kQsThreads) void quicksort_replay_kernel(
       dest[p] = p;
     }
     __syncthreads();
-    // inclusive prefix counts over the whole array (smaller: low word, larger: high word)
+    // inclusive prefix counts over the open span (smaller: low word, larger: high word)
     unsigned long long local = 0;
     for (int p = begin; p < end; ++p) {
       const unsigned char f = cls[p];
@@ -185,8 +202,8 @@ __global__ __launch_bounds__(kQsThreads) void quicksort_replay_kernel(
     }
     __syncthreads();
     // 2. rank -> position tables
-#pragma unroll 8
-    for (int p = tid; p < n; p += kQsThreads) {
+#pragma unroll 12
+    for (int p = r0 + tid; p < r1; p += kQsThreads) {
       const unsigned char f = cls[p];
       if (f == 0) continue;
       const int lo = seg_lo[p];
@@ -200,8 +217,8 @@ __global__ __launch_bounds__(kQsThreads) void quicksort_replay_kernel(
     }
     __syncthreads();
     // 3. who moves where
-#pragma unroll 8
-    for (int p = tid; p < n; p += kQsThreads) {
+#pragma unroll 12
+    for (int p = r0 + tid; p < r1; p += kQsThreads) {
       const unsigned char f = cls[p];
       if (f == 0) continue;
       const int lo = seg_lo[p];
@@ -226,8 +243,8 @@ __global__ __launch_bounds__(kQsThreads) void quicksort_replay_kernel(
     }
     __syncthreads();
     // 4. pivots find the final hole; an all-equal segment is final as it stands
-#pragma unroll 8
-    for (int p = tid; p < n; p += kQsThreads) {
+#pragma unroll 12
+    for (int p = r0 + tid; p < r1; p += kQsThreads) {
       if (seg_lo[p] != p) continue;
       const bool all_equal = pref[seg_hi[p]] == pref[p];
       int h;
@@ -238,47 +255,269 @@ __global__ __launch_bounds__(kQsThreads) void quicksort_replay_kernel(
       dest[p] = h;
     }
     __syncthreads();
-    // 5. apply the moves, derive the next level's segments
-    int active = 0;
-#pragma unroll 8
-    for (int p = tid; p < n; p += kQsThreads) {
-      const int d = dest[p];
-      nkey[d] = key[p];
-      nval[d] = val[p];
+    // 5. apply the moves, derive the next level's segments; a place that stays
+    // open is carried to the other buffer, a place that closes is final
+    int my_lo = n, my_hi = -1;
+#pragma unroll 12
+    for (int p = r0 + tid; p < r1; p += kQsThreads) {
       const int lo = seg_lo[p];
+      if (lo < 0) {  // closed on an earlier level (inside the span, between open segments)
+        nseg[2 * p] = -1;
+        nseg[2 * p + 1] = -1;
+        continue;
+      }
+      const int d = dest[p];
+      const int hi = seg_hi[p];
+      const int h = hole[lo];
+      // the segment the element's NEW place d belongs to on the next level
       int nlo = -1, nhi = -1;
-      if (lo >= 0) {
-        const int hi = seg_hi[p];
-        const int h = hole[lo];
-        if (h >= 0) {
-          if (p < h) {
-            if (lo < h - 1) {
-              nlo = lo;
-              nhi = h - 1;
-            }
-          } else if (p > h) {
-            if (h + 1 < num_top && h + 1 < hi) {
-              nlo = h + 1;
-              nhi = hi;
-            }
+      if (h >= 0) {
+        if (d < h) {
+          if (lo < h - 1) {
+            nlo = lo;
+            nhi = h - 1;
+          }
+        } else if (d > h) {
+          if (h + 1 < num_top && h + 1 < hi) {
+            nlo = h + 1;
+            nhi = hi;
           }
         }
       }
-      nseg[2 * p] = nlo;
-      nseg[2 * p + 1] = nhi;
-      active |= nlo >= 0;
+      if (nlo >= 0) {
+        nkey[d] = key[p];
+        nval[d] = val[p];
+        my_lo = min(my_lo, nlo);
+        my_hi = max(my_hi, nhi);
+      } else if (d < num_top) {
+        order_out[d] = val[p];
+      }
+      nseg[2 * d] = nlo;
+      nseg[2 * d + 1] = nhi;
+    }
+    if (my_hi >= 0) {
+      atomicMin(&next_lo, my_lo);
+      atomicMax(&next_hi, my_hi);
     }
     __syncthreads();
-#pragma unroll 8
-    for (int p = tid; p < n; p += kQsThreads) {
+#pragma unroll 12
+    for (int p = r0 + tid; p < r1; p += kQsThreads) {
       seg_lo[p] = nseg[2 * p];
       seg_hi[p] = nseg[2 * p + 1];
     }
     uint32_t* tk = key; key = nkey; nkey = tk;
     int* tv = val; val = nval; nval = tv;
-    if (!__syncthreads_or(active)) break;
+    const int nh = next_hi, nl = next_lo;
+    __syncthreads();
+    if (nh < 0) {
+      open_left = false;
+      break;
+    }
+    if (tid == 0) {
+      range_lo = nl;
+      range_hi = nh;
+    }
+    __syncthreads();
   }
-  for (int p = tid; p < num_top; p += kQsThreads) order_out[p] = val[p];
+  if (!open_left) return;
+
+  // ---- the same levels with every per-place array in LDS -------------------
+  // Places are counted from `base`; 0xFFFF marks a closed place.  Per-pivot
+  // values live in otherwise unused slots: the counts of moved elements in
+  // slot 0 of the pivot's rank tables (ranks start at 1), the hole in the
+  // pivot's own dest, "all equal" as class 3 of the pivot.  Keys and indices
+  // are permuted in place: each thread reads its places, the workgroup
+  // synchronises, each thread writes them to their destinations.
+  __shared__ unsigned short s_lo[kQsLds], s_hi[kQsLds], s_posS[kQsLds], s_posB[kQsLds],
+      s_dest[kQsLds], s_val[kQsLds];
+  __shared__ unsigned char s_cls[kQsLds];
+  __shared__ uint32_t s_pref[kQsLds], s_key[kQsLds];
+  constexpr unsigned short kClosed = 0xFFFF;
+  constexpr int kPerThread = (kQsLds + kQsThreads - 1) / kQsThreads;
+  const int base = range_lo;
+  {
+    const int span = range_hi + 1 - base;
+    for (int q = tid; q < span; q += kQsThreads) {
+      const int lo = seg_lo[base + q];
+      s_lo[q] = lo < 0 ? kClosed : static_cast<unsigned short>(lo - base);
+      s_hi[q] = lo < 0 ? kClosed : static_cast<unsigned short>(seg_hi[base + q] - base);
+      s_key[q] = key[base + q];
+      s_val[q] = static_cast<unsigned short>(val[base + q]);
+    }
+  }
+  __syncthreads();
+  if (tid == 0) {
+    range_lo = 0;
+    range_hi = range_hi - base;
+  }
+  __syncthreads();
+  for (;;) {
+    const int r0 = range_lo, r1 = range_hi + 1;
+    const int per = (r1 - r0 + kQsThreads - 1) / kQsThreads;
+    const int begin = min(r0 + tid * per, r1), end = min(begin + per, r1);
+    if (tid == 0) {
+      next_lo = kQsLds;
+      next_hi = -1;
+    }
+    // 1. classify
+    for (int q = r0 + tid; q < r1; q += kQsThreads) {
+      const unsigned short lo = s_lo[q];
+      unsigned char f = 0;
+      if (lo != kClosed && q != lo) {
+        const uint32_t K = s_key[lo], k = s_key[q];
+        f = k > K ? 1 : (k < K ? 2 : 0);
+      }
+      if (lo == q) {
+        s_posS[q] = 0;  // moved smaller-score elements of this pivot's partition
+        s_posB[q] = 0;  // moved larger-score elements
+      }
+      s_cls[q] = f;
+      s_dest[q] = static_cast<unsigned short>(q);
+    }
+    __syncthreads();
+    // prefix counts: smaller in the low half, larger in the high half
+    uint32_t local = 0;
+    for (int q = begin; q < end; ++q) {
+      const unsigned char f = s_cls[q];
+      local += f == 1 ? 1u : (f == 2 ? (1u << 16) : 0u);
+    }
+    uint32_t inc = local;
+    {
+      const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const uint32_t up = __shfl_up(inc, o, 64);
+        if (lane >= o) inc += up;
+      }
+      if (lane == 63) wave_tot[wave] = inc;
+      __syncthreads();
+      uint32_t before = 0;
+      for (int w = 0; w < wave; ++w) before += static_cast<uint32_t>(wave_tot[w]);
+      inc = before + inc - local;
+    }
+    for (int q = begin; q < end; ++q) {
+      const unsigned char f = s_cls[q];
+      inc += f == 1 ? 1u : (f == 2 ? (1u << 16) : 0u);
+      s_pref[q] = inc;
+    }
+    __syncthreads();
+    // 2. rank -> place tables
+    for (int q = r0 + tid; q < r1; q += kQsThreads) {
+      const unsigned char f = s_cls[q];
+      if (f == 0) continue;
+      const int lo = s_lo[q];
+      const uint32_t b = s_pref[lo], mine = s_pref[q];
+      if (f == 1) {
+        s_posS[lo + static_cast<int>((mine & 0xffffu) - (b & 0xffffu))] = static_cast<unsigned short>(q);
+      } else {
+        const int nB = static_cast<int>((s_pref[s_hi[q]] >> 16) - (b >> 16));
+        s_posB[lo + nB - static_cast<int>((mine >> 16) - (b >> 16)) + 1] = static_cast<unsigned short>(q);
+      }
+    }
+    __syncthreads();
+    // 3. who moves where.  The moved counts go to slot 0 of the pivot's tables,
+    // which this pass never reads (ranks start at 1).
+    for (int q = r0 + tid; q < r1; q += kQsThreads) {
+      const unsigned char f = s_cls[q];
+      if (f == 0) continue;
+      const int lo = s_lo[q];
+      const uint32_t b = s_pref[lo], top = s_pref[s_hi[q]], mine = s_pref[q];
+      const int nS = static_cast<int>((top & 0xffffu) - (b & 0xffffu));
+      const int nB = static_cast<int>((top >> 16) - (b >> 16));
+      if (f == 1) {
+        const int i = static_cast<int>((mine & 0xffffu) - (b & 0xffffu));
+        if (i <= nB && q < s_posB[lo + i]) {
+          s_dest[q] = s_posB[lo + i];
+          const int nx = i + 1;
+          if (!(nx <= nS && nx <= nB && s_posS[lo + nx] < s_posB[lo + nx]))
+            s_posS[lo] = static_cast<unsigned short>(i);
+        }
+      } else {
+        const int i = nB - static_cast<int>((mine >> 16) - (b >> 16)) + 1;
+        if (i == 1 || (i - 1 <= nS && q > s_posS[lo + i - 1])) {
+          s_dest[q] = i == 1 ? static_cast<unsigned short>(lo) : s_posS[lo + i - 1];
+          const int nx = i + 1;
+          if (!(nx <= nB && nx - 1 <= nS && s_posB[lo + nx] > s_posS[lo + nx - 1]))
+            s_posB[lo] = static_cast<unsigned short>(i);
+        }
+      }
+    }
+    __syncthreads();
+    // 4. pivots find the final hole
+    for (int q = r0 + tid; q < r1; q += kQsThreads) {
+      if (s_lo[q] != q) continue;
+      const bool all_equal = s_pref[s_hi[q]] == s_pref[q];
+      const int mS_ = s_posS[q], mB_ = s_posB[q];
+      int h;
+      if (mB_ == 0) h = q;
+      else if (mB_ > mS_) h = s_posB[q + mB_];
+      else h = s_posS[q + mS_];
+      if (all_equal) s_cls[q] = 3;
+      s_dest[q] = static_cast<unsigned short>(h);
+    }
+    __syncthreads();
+    // 5. apply: read, synchronise, write
+    uint32_t rk[kPerThread];
+    unsigned short rv[kPerThread], rd[kPerThread], rlo[kPerThread], rhi[kPerThread];
+    int my_lo = kQsLds, my_hi = -1;
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j) {
+      const int q = r0 + tid + j * kQsThreads;
+      rd[j] = kClosed;  // nothing to write
+      if (q >= r1) continue;
+      const unsigned short lo = s_lo[q];
+      if (lo == kClosed) continue;
+      const int d = s_dest[q], hi = s_hi[q], h = s_dest[lo];
+      const bool all_equal = s_cls[lo] == 3;
+      int nlo = -1, nhi = -1;
+      if (!all_equal) {
+        if (d < h) {
+          if (lo < h - 1) {
+            nlo = lo;
+            nhi = h - 1;
+          }
+        } else if (d > h) {
+          if (base + h + 1 < num_top && h + 1 < hi) {
+            nlo = h + 1;
+            nhi = hi;
+          }
+        }
+      }
+      rk[j] = s_key[q];
+      rv[j] = s_val[q];
+      rd[j] = static_cast<unsigned short>(d);
+      rlo[j] = nlo < 0 ? kClosed : static_cast<unsigned short>(nlo);
+      rhi[j] = nlo < 0 ? kClosed : static_cast<unsigned short>(nhi);
+      if (nlo >= 0) {
+        my_lo = min(my_lo, nlo);
+        my_hi = max(my_hi, nhi);
+      }
+    }
+    if (my_hi >= 0) {
+      atomicMin(&next_lo, my_lo);
+      atomicMax(&next_hi, my_hi);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j) {
+      if (rd[j] == kClosed) continue;
+      const int d = rd[j];
+      s_key[d] = rk[j];
+      s_val[d] = rv[j];
+      s_lo[d] = rlo[j];
+      s_hi[d] = rhi[j];
+      if (rlo[j] == kClosed && base + d < num_top) order_out[base + d] = rv[j];
+    }
+    __syncthreads();
+    const int nh = next_hi, nl = next_lo;
+    __syncthreads();
+    if (nh < 0) break;
+    if (tid == 0) {
+      range_lo = nl;
+      range_hi = nh;
+    }
+    __syncthreads();
+  }
 }
 
 // mask[i][cb] bit j: box cb*64+j (> i) overlaps box i by more than thr, with
