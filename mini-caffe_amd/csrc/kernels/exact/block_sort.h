@@ -89,6 +89,63 @@ __device__ inline void block_sort_desc(uint32_t* k0, int* v0, uint32_t* k1, int*
   }
 }
 
+// The same sort with keys and values resident in LDS and sorted in place: per
+// pass every thread takes its contiguous run into registers, counts digits in
+// its private histogram column, the workgroup synchronises, and each thread
+// scatters its run back.  16-bit histogram entries and ranks: n < 65536.
+// MAXPER bounds the run length: n <= MAXPER * kSortThreads.  VT is the value
+// type (unsigned short halves the LDS footprint when values are indices < 65536).
+struct BlockSortLds16 {
+  unsigned short counts[16 * kSortThreads];
+  uint32_t wave_sum[kSortThreads / 64];
+};
+
+template <int MAXPER, typename VT>
+__device__ inline void block_sort_desc_lds(uint32_t* keys, VT* vals, int n, BlockSortLds16* lds) {
+  const int tid = threadIdx.x;
+  const int per = (n + kSortThreads - 1) / kSortThreads;
+  const int begin = min(tid * per, n), end = min(begin + per, n);
+  const int cnt = end - begin;
+  for (int shift = 0; shift < 32; shift += 4) {
+    uint32_t rk[MAXPER];
+    VT rv[MAXPER];
+#pragma unroll
+    for (int j = 0; j < MAXPER; ++j)
+      if (j < cnt) {
+        rk[j] = keys[begin + j];
+        rv[j] = vals[begin + j];
+      }
+#pragma unroll
+    for (int d = 0; d < 16; ++d) lds->counts[d * kSortThreads + tid] = 0;
+#pragma unroll
+    for (int j = 0; j < MAXPER; ++j)
+      if (j < cnt) lds->counts[((rk[j] >> shift) & 15u) * kSortThreads + tid]++;
+    __syncthreads();
+    // flattened [digit][thread] order == final rank order; thread t scans 16 entries
+    uint32_t local[16], sum = 0;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      local[j] = lds->counts[tid * 16 + j];
+      sum += local[j];
+    }
+    uint32_t run = block_exclusive_scan(sum, lds->wave_sum);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      lds->counts[tid * 16 + j] = static_cast<unsigned short>(run);
+      run += local[j];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < MAXPER; ++j)
+      if (j < cnt) {
+        const uint32_t pos = lds->counts[((rk[j] >> shift) & 15u) * kSortThreads + tid]++;
+        keys[pos] = rk[j];
+        vals[pos] = rv[j];
+      }
+    __syncthreads();
+  }
+}
+
 }  // namespace mchip
 
 #endif  // MCHIP_EXACT_BLOCK_SORT_H_

@@ -119,9 +119,46 @@ __device__ __forceinline__ float jaccard(const DBox& a, const DBox& b) {
 
 constexpr int kKeptLds = 512;  // kept boxes cached in LDS; further ones are read from memory
 
+// The greedy pass of ApplyNMSFast with its adaptive threshold, by one
+// wavefront: candidate r is prior cand_idx[r]; its box is cand_box[r] for
+// r < n_cached, else read from memory.
+template <typename IT>
+__device__ __forceinline__ void greedy_nms_wave(int lane, int ncand, int n_cached,
+                                                const IT* cand_idx, const DBox* cand_box,
+                                                const DBox* cls_boxes, DBox* kept_box, int* kept,
+                                                float nms_thr, float eta, int* kept_count_out) {
+  float adaptive = nms_thr;
+  int nkept = 0;
+  for (int r = 0; r < ncand; ++r) {
+    const int idx = static_cast<int>(cand_idx[r]);
+    const DBox b = r < n_cached ? cand_box[r] : cls_boxes[idx];
+    bool reject = false;
+    for (int base = 0; base < nkept && !reject; base += 64) {
+      const int k = base + lane;
+      bool over = false;
+      if (k < nkept) {
+        const DBox kb = k < kKeptLds ? kept_box[k] : cls_boxes[kept[k]];
+        over = !(jaccard(b, kb) <= adaptive);
+      }
+      reject = __any(over);
+    }
+    if (!reject) {
+      if (lane == 0) {
+        kept[nkept] = idx;
+        if (nkept < kKeptLds) kept_box[nkept] = b;
+      }
+      ++nkept;
+      if (eta < 1.f && adaptive > 0.5f) adaptive *= eta;
+      __builtin_amdgcn_wave_barrier();
+      __threadfence_block();
+    }
+  }
+  if (lane == 0) *kept_count_out = nkept;
+}
+
 // One workgroup per (image, class).  Candidates: scores above the confidence
 // threshold in (score desc, prior index asc) order, cut to top_k; then the
-// greedy pass of ApplyNMSFast with its adaptive threshold.
+// greedy pass.  This variant sorts through global scratch (any P).
 __global__ __launch_bounds__(kSortThreads) void det_class_nms_kernel(
     const float* __restrict__ conf, const DBox* __restrict__ boxes, int P, int C,
     int loc_classes, int background, float conf_thr, float nms_thr, float eta, int top_k,
@@ -158,38 +195,72 @@ __global__ __launch_bounds__(kSortThreads) void det_class_nms_kernel(
   block_sort_desc(k0, v0, k1, v1, P, &lds);
   int ncand = s_valid;
   if (top_k > -1 && top_k < ncand) ncand = top_k;
-
-  if (threadIdx.x >= 64) return;  // the greedy pass is one wavefront
-  const int lane = threadIdx.x;
   const DBox* cls_boxes = boxes + ((size_t)i * loc_classes + (loc_classes == 1 ? 0 : c)) * P;
-  int* kept = kept_idx + (size_t)seg * max_cand;
-  float adaptive = nms_thr;
-  int nkept = 0;
-  for (int r = 0; r < ncand; ++r) {
+  // The serial greedy pass would pay one dependent global load pair per
+  // candidate: the whole workgroup fetches the first candidates' indices and
+  // boxes into the (now free) histogram storage first.
+  constexpr int kCandLds = static_cast<int>(sizeof(lds.counts) / (sizeof(DBox) + sizeof(int)));
+  DBox* cand_box = reinterpret_cast<DBox*>(lds.counts);
+  int* cand_idx = reinterpret_cast<int*>(cand_box + kCandLds);
+  __syncthreads();
+  for (int r = threadIdx.x; r < min(ncand, kCandLds); r += kSortThreads) {
     const int idx = v0[r];
-    const DBox b = cls_boxes[idx];
-    bool reject = false;
-    for (int base = 0; base < nkept && !reject; base += 64) {
-      const int k = base + lane;
-      bool over = false;
-      if (k < nkept) {
-        const DBox kb = k < kKeptLds ? kept_box[k] : cls_boxes[kept[k]];
-        over = !(jaccard(b, kb) <= adaptive);
-      }
-      reject = __any(over);
-    }
-    if (!reject) {
-      if (lane == 0) {
-        kept[nkept] = idx;
-        if (nkept < kKeptLds) kept_box[nkept] = b;
-      }
-      ++nkept;
-      if (eta < 1.f && adaptive > 0.5f) adaptive *= eta;
-      __builtin_amdgcn_wave_barrier();
-      __threadfence_block();
-    }
+    cand_idx[r] = idx;
+    cand_box[r] = cls_boxes[idx];
   }
-  if (lane == 0) kept_count[seg] = nkept;
+  __syncthreads();
+  if (threadIdx.x >= 64) return;  // the greedy pass is one wavefront
+  // with more candidates than the cache holds, indices come from the sorted list in memory
+  greedy_nms_wave<int>(threadIdx.x, ncand, min(ncand, kCandLds), ncand <= kCandLds ? cand_idx : v0,
+                       cand_box, cls_boxes, kept_box, kept_idx + (size_t)seg * max_cand, nms_thr,
+                       eta, &kept_count[seg]);
+}
+
+// The same for P <= kDetLdsMax priors: scores are keyed straight into LDS and
+// sorted there (no global scratch traffic), the sorted prior indices double as
+// the candidate list.
+constexpr int kDetLdsPer = 24;
+constexpr int kDetLdsMax = kDetLdsPer * kSortThreads;  // 12288
+constexpr int kDetCandBoxes = 1024;
+__global__ __launch_bounds__(kSortThreads) void det_class_nms_lds_kernel(
+    const float* __restrict__ conf, const DBox* __restrict__ boxes, int P, int C,
+    int loc_classes, int background, float conf_thr, float nms_thr, float eta, int top_k,
+    int max_cand, int* __restrict__ kept_idx, int* __restrict__ kept_count) {
+  __shared__ BlockSortLds16 lds;
+  __shared__ uint32_t s_key[kDetLdsMax];
+  __shared__ unsigned short s_val[kDetLdsMax];
+  __shared__ DBox cand_box[kDetCandBoxes];
+  __shared__ DBox kept_box[kKeptLds];
+  __shared__ int s_valid;
+  const int c = blockIdx.x, i = blockIdx.y;
+  const int seg = i * C + c;
+  if (c == background) {
+    if (threadIdx.x == 0) kept_count[seg] = 0;
+    return;
+  }
+  if (threadIdx.x == 0) s_valid = 0;
+  __syncthreads();
+  int valid = 0;
+  for (int p = threadIdx.x; p < P; p += kSortThreads) {
+    const float s = conf[((size_t)i * P + p) * C + c];
+    const bool ok = s > conf_thr;
+    valid += ok;
+    s_key[p] = ok ? desc_key(s) : 0xffffffffu;  // below-threshold scores sort last
+    s_val[p] = static_cast<unsigned short>(p);
+  }
+  if (valid) atomicAdd(&s_valid, valid);
+  __syncthreads();
+  block_sort_desc_lds<kDetLdsPer, unsigned short>(s_key, s_val, P, &lds);
+  int ncand = s_valid;
+  if (top_k > -1 && top_k < ncand) ncand = top_k;
+  const DBox* cls_boxes = boxes + ((size_t)i * loc_classes + (loc_classes == 1 ? 0 : c)) * P;
+  const int n_cached = min(ncand, kDetCandBoxes);
+  for (int r = threadIdx.x; r < n_cached; r += kSortThreads) cand_box[r] = cls_boxes[s_val[r]];
+  __syncthreads();
+  if (threadIdx.x >= 64) return;  // the greedy pass is one wavefront
+  greedy_nms_wave<unsigned short>(threadIdx.x, ncand, n_cached, s_val, cand_box, cls_boxes, kept_box,
+                                  kept_idx + (size_t)seg * max_cand, nms_thr, eta,
+                                  &kept_count[seg]);
 }
 
 // One workgroup per image: applies keep_top_k over all classes and writes the
@@ -390,10 +461,15 @@ int mcDetectionOutput(const float* loc, const float* conf, const float* prior, i
                                                          code_type, variance_encoded_in_target,
                                                          boxes);
   MC_LAUNCH_CHECK();
-  det_class_nms_kernel<<<dim3(num_classes, num), kSortThreads, 0, st>>>(
-      conf, boxes, num_priors, num_classes, loc_classes, background_label, confidence_threshold,
-      nms_threshold, eta, top_k, max_cand, u32(L.k0), i32(L.v0), u32(L.k1), i32(L.v1),
-      i32(L.kept_idx), i32(L.kept_count));
+  if (num_priors <= kDetLdsMax)
+    det_class_nms_lds_kernel<<<dim3(num_classes, num), kSortThreads, 0, st>>>(
+        conf, boxes, num_priors, num_classes, loc_classes, background_label, confidence_threshold,
+        nms_threshold, eta, top_k, max_cand, i32(L.kept_idx), i32(L.kept_count));
+  else
+    det_class_nms_kernel<<<dim3(num_classes, num), kSortThreads, 0, st>>>(
+        conf, boxes, num_priors, num_classes, loc_classes, background_label, confidence_threshold,
+        nms_threshold, eta, top_k, max_cand, u32(L.k0), i32(L.v0), u32(L.k1), i32(L.v1),
+        i32(L.kept_idx), i32(L.kept_count));
   MC_LAUNCH_CHECK();
   det_select_kernel<<<num, kSortThreads, 0, st>>>(
       conf, boxes, num_priors, num_classes, loc_classes, keep_top_k, max_cand, i32(L.kept_idx),

@@ -86,6 +86,30 @@ __global__ __launch_bounds__(kSortThreads) void proposal_sort_kernel(
   if (ties) atomicOr(tie_flag, 1);
 }
 
+// The same for up to kSortLdsMax proposals, sorted inside LDS.
+constexpr int kSortLdsPer = 44;
+constexpr int kSortLdsMax = kSortLdsPer * kSortThreads;  // 22528
+__global__ __launch_bounds__(kSortThreads) void proposal_sort_lds_kernel(
+    uint32_t* k0, int* v0, int n, int pre, int* __restrict__ tie_flag) {
+  __shared__ BlockSortLds16 lds;
+  __shared__ uint32_t s_key[kSortLdsMax];
+  __shared__ unsigned short s_val[kSortLdsMax];
+  for (int i = threadIdx.x; i < n; i += kSortThreads) {
+    s_key[i] = k0[i];
+    s_val[i] = static_cast<unsigned short>(i);  // v0[i] == i on entry
+  }
+  __syncthreads();
+  block_sort_desc_lds<kSortLdsPer, unsigned short>(s_key, s_val, n, &lds);
+  for (int i = threadIdx.x; i < n; i += kSortThreads) {
+    k0[i] = s_key[i];
+    v0[i] = s_val[i];
+  }
+  int ties = 0;
+  for (int i = threadIdx.x; i < pre; i += kSortThreads)
+    if (i + 1 < n && s_key[i] == s_key[i + 1]) ties = 1;
+  if (ties) atomicOr(tie_flag, 1);
+}
+
 // Boxes and scores of the first `pre` proposals in their final order.
 __global__ __launch_bounds__(256) void proposal_order_gather_kernel(
     const int* __restrict__ order, int pre, const float4* __restrict__ boxes,
@@ -719,7 +743,10 @@ int mcProposal(const float* scores, const float* bbox, const float* im_info, con
                                                           W, feat_stride, min_size, boxes, k0,
                                                           korig, v0, sc);
   MC_LAUNCH_CHECK();
-  proposal_sort_kernel<<<1, kSortThreads, 0, st>>>(k0, v0, k1, v1, n, pre, flags);
+  if (n <= kSortLdsMax)
+    proposal_sort_lds_kernel<<<1, kSortThreads, 0, st>>>(k0, v0, n, pre, flags);
+  else
+    proposal_sort_kernel<<<1, kSortThreads, 0, st>>>(k0, v0, k1, v1, n, pre, flags);
   MC_LAUNCH_CHECK();
   // no-op unless equal scores reach into the first `pre` places
   quicksort_replay_kernel<<<1, kQsThreads, 0, st>>>(

@@ -370,6 +370,8 @@ def run_proposal(K, scores, bbox, im_info, param):
     ((10, 12), 2000, 50, 0.5, 0),        # pre_nms_topn > proposals: zero-score ties
     ((20, 20), 6000, 300, 0.7, 7),       # heavy ties
     ((5, 4), 100, 300, 0.3, 0),
+    ((50, 60), 6000, 300, 0.7, 0),       # 27000 proposals: sort through global scratch
+    ((50, 60), 6000, 300, 0.7, 5000),    # ... with ties: replay starts outside LDS
 ])
 def test_proposal_bit_exact(K, hw, pre, post, thr, quant):
     """Kept rois and scores equal the CPU path's bit for bit, with and without
@@ -399,6 +401,8 @@ def test_proposal_bit_exact(K, hw, pre, post, thr, quant):
     (2, 300, 6, True, "CORNER_SIZE", 50, 0.05, 0.6, 0.9, 100, 2.0),       # adaptive threshold (eta < 1)
     (2, 100, 3, True, "CENTER_SIZE", 10, 0.999999, 0.45, 1.0, 20, 2.0),   # nothing kept -> rows of -1
     (1, 2000, 21, True, "CENTER_SIZE", 200, 0.01, 0.45, 1.0, 400, 0.5),
+    (1, 13000, 3, True, "CENTER_SIZE", 100, 0.01, 0.45, 1.0, 1500, 2.0),   # sort through global scratch,
+                                                                           # more candidates than cached
 ])
 def test_detection_output_bit_exact(K, num, P, C, share, code, keep, thr, nms, eta, topk, sigma):
     rng = np.random.default_rng(12)
