@@ -61,6 +61,7 @@ struct IgemmArgs {
   int Hq, Wq, HqWq;   // iteration grid of this sub-problem
   unsigned div_hw_mul, div_hw_shift;  // p / HqWq  as multiply-high and shift (shift 32: divisor 1)
   unsigned div_w_mul, div_w_shift;    // rem / Wq
+  unsigned div_mt_mul, div_mt_shift;  // logical tile / MT
   unsigned y_bytes, c_bytes;          // top blob and per-channel vector extents (descriptors)
   int H, W;           // bottom height / width
   int q_sh, q_sw;     // bottom origin of pixel (qh,qw): qh*q_sh + in_oh
@@ -160,8 +161,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
     const int q = total / kNumXcd, r = total % kNumXcd;
     const int xcd = bid % kNumXcd, local = bid / kNumXcd;
     const int logical = xcd * q + (xcd < r ? xcd : r) + local;
-    mt = logical % a.MT;
-    nt = logical / a.MT;
+    nt = fast_div(logical, a.div_mt_mul, a.div_mt_shift);
+    mt = logical - nt * a.MT;
   }
 
   // On this hardware ordinary vector ALU instructions and MFMA instructions of
@@ -1052,6 +1053,7 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
       a.out_ow = s.out_ow;
       a.MT = MT;
       a.NT = ceil_div(pixels, cfg.bn);
+      make_fast_div(a.MT, (unsigned long long)a.MT * a.NT + 1, &a.div_mt_mul, &a.div_mt_shift);
       a.act = ep ? ep->activation : MC_ACT_NONE;
       a.slope = ep ? ep->negative_slope : 0.f;
       const long blocks = (long)a.MT * a.NT;
