@@ -127,14 +127,22 @@ def configs_report(path, mc, craft, zoo, LIB):
     """Whole-forward time, contraction TFLOP/s and detection-tail layer time of the five
     BASELINE configurations on the GPU (synthetic inputs and weights from the zoo builders)."""
     import tempfile
-    cases = [("C1 conv3x3+ReLU 1x64x56x56", zoo.c1_spec(seed=0), ()),
-             ("C2 ResNet-50 b64", zoo.resnet50_spec(batch=64, size=224, seed=0), ()),
-             ("C3 SSD300-VGG16 b8", zoo.ssd300_spec(batch=8, seed=0), ("detection_out",)),
-             ("C4 RPN+Proposal 1x1024x38x63", zoo.rpn_spec(seed=0), ("proposal",)),
-             ("C5 DCGAN generator b128", zoo.dcgan_spec(batch=128, seed=0), ())]
-    lines = ["%-30s %10s %10s %12s %10s %8s  %s" % ("configuration", "ms/forward", "GFLOP", "contr. ms",
-                                                    "TFLOP/s", "of peak", "tail layers (us, device time)")]
-    for name, (spec, inputs), tails in cases:
+    import oracle
+    from oracle import netrun
+    oracle.use_openblas(True)
+    # (name, GPU spec, tail layers, batch, CPU-sample spec at a reduced batch, its batch)
+    cases = [("C1 conv3x3+ReLU 1x64x56x56", zoo.c1_spec(seed=0), (), 1, zoo.c1_spec(seed=0), 1),
+             ("C2 ResNet-50 b64", zoo.resnet50_spec(batch=64, size=224, seed=0), (), 64,
+              zoo.resnet50_spec(batch=4, size=224, seed=0), 4),
+             ("C3 SSD300-VGG16 b8", zoo.ssd300_spec(batch=8, seed=0), ("detection_out",), 8,
+              zoo.ssd300_spec(batch=1, seed=0), 1),
+             ("C4 RPN+Proposal 1x1024x38x63", zoo.rpn_spec(seed=0), ("proposal",), 1, zoo.rpn_spec(seed=0), 1),
+             ("C5 DCGAN generator b128", zoo.dcgan_spec(batch=128, seed=0), (), 128,
+              zoo.dcgan_spec(batch=8, seed=0), 8)]
+    lines = ["%-30s %10s %10s %12s %10s %8s %12s %12s  %s"
+             % ("configuration", "ms/forward", "GFLOP", "contr. ms", "TFLOP/s", "of peak", "GPU img/s",
+                "CPU img/s", "tail layers (us, device time)")]
+    for name, (spec, inputs), tails, batch, (cspec, cinputs), cbatch in cases:
         net = mc.Net.from_buffers(craft.to_prototxt(spec, "net"))
         craft.load_weights(net, spec)
         net.forward(**inputs)
@@ -171,10 +179,18 @@ def configs_report(path, mc, craft, zoo, LIB):
                                                              len(spans[t])) for t in tails if t in spans)
         cms = tot_ms.value / reps
         tf_s = fl.value / (tot_ms.value * 1e-3) / 1e12 if tot_ms.value else 0.0
-        lines.append("%-30s %10.3f %10.2f %12.3f %10.1f %7.1f%%  %s"
+        # CPU path (oracle restatement of the reference, OpenBLAS sgemm, all host cores): one
+        # pass at the reduced batch
+        last = cspec[-1]["top"][0]
+        t0 = time.perf_counter()
+        netrun.oracle_forward(cspec, cinputs, keep={last})
+        cpu_rate = cbatch / (time.perf_counter() - t0)
+        lines.append("%-30s %10.3f %10.2f %12.3f %10.1f %7.1f%% %12.1f %12.2f  %s"
                      % (name, ms, fl.value / reps / 1e9, cms, tf_s, 100 * tf_s / FP32_MFMA_PEAK_TFLOPS,
-                        tail_txt))
+                        batch / (ms * 1e-3), cpu_rate, tail_txt))
         del net
+    lines.append("CPU column: one pass of the oracle (reference algorithm: per-image im2col + OpenBLAS sgemm, "
+                 "unfused layers) on %d host threads at batch 1/4/1/1/8." % oracle.openblas_threads())
     with open(path, "w") as f:
         f.write("\n".join(lines) + "\n")
 
