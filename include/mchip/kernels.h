@@ -279,6 +279,27 @@ int mcDetectionOutput(const float* loc, const float* conf, const float* prior, i
                       void* workspace, size_t workspace_bytes, float* out_rows, int max_rows,
                       int* num_rows, void* stream);
 
+/* ROIPoolingLayer::Forward (roi_pooling_layer.cpp:37-110; .cu:13-81): max pooling of
+ * bottom [num, channels, height, width] over num_rois regions, rois rows of
+ * [batch index, x1, y1, x2, y2] in image coordinates, top [num_rois, channels,
+ * pooled_h, pooled_w].  Region ends = round(coordinate * spatial_scale), bins from
+ * floor / ceil of multiples of the float bin size, clipped to the map; empty bin 0.
+ * A roi with a batch index outside [0, num) (a CHECK failure in the reference's CPU
+ * code) yields zeros and sets *bad_roi_flag (device int, may be NULL) to 1. */
+int mcROIPooling(const float* bottom, int num, int channels, int height, int width,
+                 const float* rois, int num_rois, int pooled_h, int pooled_w, float spatial_scale,
+                 float* top, int* bad_roi_flag, void* stream);
+
+/* PSROIPoolingLayer::Forward (psroi_pooling_layer.cpp:45-122; .cu:13-89): position-
+ * sensitive average pooling, bottom [num, output_dim*group_size^2, height, width],
+ * top [num_rois, output_dim, group_size, group_size]; bin (ph, pw) of output channel
+ * c averages input channel (c*group_size + ph)*group_size + pw.  Region corners are
+ * rounded before scaling, the end corner as round(x2 + 1) (the CPU code's form), the
+ * region is at least 0.1 wide; sums run row-major over the bin; empty bin 0. */
+int mcPSROIPooling(const float* bottom, int num, int output_dim, int group_size, int height,
+                   int width, const float* rois, int num_rois, float spatial_scale, float* top,
+                   int* bad_roi_flag, void* stream);
+
 /* Fill `count` floats with `value` (caffe_gpu_set, math_functions.cu:70-82). */
 int mcFill(float* dst, long count, float value, void* stream);
 

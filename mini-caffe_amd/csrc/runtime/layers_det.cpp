@@ -183,4 +183,94 @@ class DetectionOutputLayer : public Layer {
 };
 REGISTER_LAYER_CLASS(DetectionOutput);
 
+// ---------------------------------------------------------------------------
+// ROIPooling (reference src/layers/roi_pooling_layer.cpp:15-110; .cu:13-81) and
+// PSROIPooling (psroi_pooling_layer.cpp:18-122; .cu:13-89): the consumers of
+// Proposal's rois.  As in the reference the top keeps the row count the rois blob
+// had at Reshape time; Forward pools the rows the rois blob has then (Proposal
+// shrinks it to the kept count) and the remaining rows hold the reference's fill
+// value (-FLT_MAX for ROIPooling, 0 for PSROIPooling).
+// ---------------------------------------------------------------------------
+class RegionPoolingBase : public Layer {
+ public:
+  explicit RegionPoolingBase(const LayerParameter& param) : Layer(param) {}
+  int ExactNumBottomBlobs() const override { return 2; }
+  int ExactNumTopBlobs() const override { return 1; }
+
+ protected:
+  // rois rows to pool now, and the fill of the rows beyond them
+  int PrepareRows(const vector<Blob*>& bottom, const vector<Blob*>& top, float fill) {
+    CHECK_EQ(bottom[1]->count(1), 5) << "rois must be rows of [batch index, x1, y1, x2, y2]";
+    const int rows = std::min(bottom[1]->shape(0), top[0]->shape(0));
+    const long per_row = top[0]->count(1);
+    const long rest = (top[0]->shape(0) - rows) * per_row;
+    if (rest > 0)
+      MC_CHECK(mcFill(top[0]->mutable_gpu_data() + rows * per_row, rest, fill, cur_stream()));
+    return rows;
+  }
+  float spatial_scale_ = 1.f;
+};
+
+class ROIPoolingLayer : public RegionPoolingBase {
+ public:
+  explicit ROIPoolingLayer(const LayerParameter& param) : RegionPoolingBase(param) {}
+  const char* type() const override { return "ROIPooling"; }
+  void LayerSetUp(const vector<Blob*>& bottom, const vector<Blob*>& top) override {
+    const Message& p = layer_param_.sub("roi_pooling_param");
+    pooled_h_ = static_cast<int>(p.get_int("pooled_h", 0));
+    pooled_w_ = static_cast<int>(p.get_int("pooled_w", 0));
+    CHECK_GT(pooled_h_, 0) << "pooled_h must be > 0";
+    CHECK_GT(pooled_w_, 0) << "pooled_w must be > 0";
+    spatial_scale_ = static_cast<float>(p.get_float("spatial_scale", 1.));
+  }
+  void Reshape(const vector<Blob*>& bottom, const vector<Blob*>& top) override {
+    CHECK_EQ(bottom[0]->num_axes(), 4) << "ROIPooling bottom must be num x channels x height x width";
+    top[0]->Reshape(vector<int>{bottom[1]->shape(0), bottom[0]->shape(1), pooled_h_, pooled_w_});
+  }
+
+ protected:
+  void Forward_gpu(const vector<Blob*>& bottom, const vector<Blob*>& top) override {
+    const int rows = PrepareRows(bottom, top, -FLT_MAX);
+    MC_CHECK(mcROIPooling(bottom[0]->gpu_data(), bottom[0]->shape(0), bottom[0]->shape(1),
+                          bottom[0]->shape(2), bottom[0]->shape(3), bottom[1]->gpu_data(), rows,
+                          pooled_h_, pooled_w_, spatial_scale_,
+                          rows ? top[0]->mutable_gpu_data() : nullptr, nullptr, cur_stream()));
+  }
+  int pooled_h_ = 0, pooled_w_ = 0;
+};
+REGISTER_LAYER_CLASS(ROIPooling);
+
+class PSROIPoolingLayer : public RegionPoolingBase {
+ public:
+  explicit PSROIPoolingLayer(const LayerParameter& param) : RegionPoolingBase(param) {}
+  const char* type() const override { return "PSROIPooling"; }
+  void LayerSetUp(const vector<Blob*>& bottom, const vector<Blob*>& top) override {
+    const Message& p = layer_param_.sub("psroi_pooling_param");
+    CHECK(p.has("spatial_scale") && p.has("output_dim") && p.has("group_size"))
+        << "psroi_pooling_param needs spatial_scale, output_dim and group_size";
+    spatial_scale_ = static_cast<float>(p.get_float("spatial_scale", 1.));
+    output_dim_ = static_cast<int>(p.get_int("output_dim", 0));
+    group_size_ = static_cast<int>(p.get_int("group_size", 0));
+    CHECK_GT(output_dim_, 0) << "output_dim must be > 0";
+    CHECK_GT(group_size_, 0) << "group_size must be > 0";
+  }
+  void Reshape(const vector<Blob*>& bottom, const vector<Blob*>& top) override {
+    CHECK_EQ(bottom[0]->num_axes(), 4) << "PSROIPooling bottom must be num x channels x height x width";
+    CHECK_EQ(bottom[0]->shape(1), output_dim_ * group_size_ * group_size_)
+        << "input channel number does not match layer parameters";
+    top[0]->Reshape(vector<int>{bottom[1]->shape(0), output_dim_, group_size_, group_size_});
+  }
+
+ protected:
+  void Forward_gpu(const vector<Blob*>& bottom, const vector<Blob*>& top) override {
+    const int rows = PrepareRows(bottom, top, 0.f);
+    MC_CHECK(mcPSROIPooling(bottom[0]->gpu_data(), bottom[0]->shape(0), output_dim_, group_size_,
+                            bottom[0]->shape(2), bottom[0]->shape(3), bottom[1]->gpu_data(), rows,
+                            spatial_scale_, rows ? top[0]->mutable_gpu_data() : nullptr, nullptr,
+                            cur_stream()));
+  }
+  int output_dim_ = 0, group_size_ = 0;
+};
+REGISTER_LAYER_CLASS(PSROIPooling);
+
 }  // namespace caffe

@@ -315,6 +315,38 @@ _lib.orc_detection_output.argtypes = [c_float_p, c_float_p, c_float_p] + [ctypes
     [ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_int, c_float_p, ctypes.c_int]
 
 
+_lib.orc_roi_pooling.argtypes = [c_float_p] + [ctypes.c_int] * 4 + [c_float_p] + [ctypes.c_int] * 3 + \
+                                 [ctypes.c_float, c_float_p]
+_lib.orc_psroi_pooling.argtypes = [c_float_p] + [ctypes.c_int] * 5 + [c_float_p, ctypes.c_int,
+                                                                      ctypes.c_float, c_float_p]
+
+
+def roi_pooling(x, rois, pooled_h, pooled_w, spatial_scale):
+    """ROIPooling (roi_pooling_layer.cpp:37-110): x (N,C,H,W), rois (R,5) -> (R,C,ph,pw)."""
+    x, rois = _f32(x), _f32(rois).reshape(-1, 5)
+    n, c, h, w = x.shape
+    y = np.empty((rois.shape[0], c, pooled_h, pooled_w), np.float32)
+    rc = _lib.orc_roi_pooling(_fp(x), n, c, h, w, _fp(rois), rois.shape[0], pooled_h, pooled_w,
+                              spatial_scale, _fp(y))
+    if rc:
+        raise ValueError("roi batch index outside [0, %d)" % n)
+    return y
+
+
+def psroi_pooling(x, rois, output_dim, group_size, spatial_scale):
+    """PSROIPooling (psroi_pooling_layer.cpp:45-122): x (N, dim*g*g, H, W), rois (R,5) -> (R,dim,g,g)."""
+    x, rois = _f32(x), _f32(rois).reshape(-1, 5)
+    n, c, h, w = x.shape
+    if c != output_dim * group_size * group_size:
+        raise ValueError("input channel number does not match layer parameters")
+    y = np.empty((rois.shape[0], output_dim, group_size, group_size), np.float32)
+    rc = _lib.orc_psroi_pooling(_fp(x), n, output_dim, group_size, h, w, _fp(rois), rois.shape[0],
+                                spatial_scale, _fp(y))
+    if rc:
+        raise ValueError("roi batch index outside [0, %d)" % n)
+    return y
+
+
 def normalize(x, scale, across_spatial=True, channel_shared=True, eps=1e-10):
     x, scale = _f32(x), _f32(scale).reshape(-1)
     n, c = x.shape[0], x.shape[1]

@@ -1,6 +1,7 @@
 /*
  * mc_oracle_det.cc — CPU restatement of Mini-Caffe's detection tail
- * (Normalize, PriorBox, Proposal, DetectionOutput).
+ * (Normalize, PriorBox, Proposal, DetectionOutput) and of the two region
+ * pooling layers that consume Proposal's rois (ROIPooling, PSROIPooling).
  *
  * TEST INFRASTRUCTURE ONLY (see mc_oracle.c).  C++ rather than C because the
  * reference's orderings are those of std::stable_sort and std::sort; using the
@@ -25,6 +26,10 @@
  *   prior box          SSD300 prior count 8732 and closed-form centres / sizes
  *   detection output   brute-force greedy NMS per class in float64 on <= 64 priors
  *   normalize          closed form
+ *   roi / psroi pool   special cases that reduce to numpy routines: a roi over the
+ *                      whole map with 1x1 bins is the global max / mean, with one
+ *                      bin per cell the identity; integer-aligned rois are block
+ *                      max / block mean of a reshaped array; empty bins give 0
  */
 #include <algorithm>
 #include <cfloat>
@@ -486,6 +491,104 @@ int orc_detection_output(const float* loc, const float* conf, const float* prior
     }
   }
   return count;
+}
+
+/* ---- ROIPooling (src/layers/roi_pooling_layer.cpp:37-110) -------------------
+ * rois: R rows [batch index, x1, y1, x2, y2] in image coordinates.  Region ends
+ * are rounded after scaling; bins use floor / ceil of multiples of the float bin
+ * size, are shifted by the region start and clipped to the map; an empty bin
+ * yields 0, otherwise the maximum (initial value -FLT_MAX).  The reference
+ * CHECK-fails on a batch index outside [0, num); here such a roi returns -1. */
+int orc_roi_pooling(const float* bottom, int num, int channels, int height, int width,
+                    const float* rois, int num_rois, int pooled_h, int pooled_w,
+                    float spatial_scale, float* top) {
+  for (int n = 0; n < num_rois; ++n) {
+    const float* roi = rois + 5 * n;
+    const int batch = static_cast<int>(roi[0]);
+    if (batch < 0 || batch >= num) return -1;
+    const int roi_start_w = static_cast<int>(round(roi[1] * spatial_scale));
+    const int roi_start_h = static_cast<int>(round(roi[2] * spatial_scale));
+    const int roi_end_w = static_cast<int>(round(roi[3] * spatial_scale));
+    const int roi_end_h = static_cast<int>(round(roi[4] * spatial_scale));
+    const int roi_height = std::max(roi_end_h - roi_start_h + 1, 1);
+    const int roi_width = std::max(roi_end_w - roi_start_w + 1, 1);
+    const float bin_size_h = static_cast<float>(roi_height) / static_cast<float>(pooled_h);
+    const float bin_size_w = static_cast<float>(roi_width) / static_cast<float>(pooled_w);
+    for (int c = 0; c < channels; ++c) {
+      const float* plane = bottom + (static_cast<size_t>(batch) * channels + c) * height * width;
+      float* out = top + (static_cast<size_t>(n) * channels + c) * pooled_h * pooled_w;
+      for (int ph = 0; ph < pooled_h; ++ph) {
+        for (int pw = 0; pw < pooled_w; ++pw) {
+          int hstart = static_cast<int>(std::floor(static_cast<float>(ph) * bin_size_h));
+          int wstart = static_cast<int>(std::floor(static_cast<float>(pw) * bin_size_w));
+          int hend = static_cast<int>(std::ceil(static_cast<float>(ph + 1) * bin_size_h));
+          int wend = static_cast<int>(std::ceil(static_cast<float>(pw + 1) * bin_size_w));
+          hstart = std::min(std::max(hstart + roi_start_h, 0), height);
+          hend = std::min(std::max(hend + roi_start_h, 0), height);
+          wstart = std::min(std::max(wstart + roi_start_w, 0), width);
+          wend = std::min(std::max(wend + roi_start_w, 0), width);
+          const bool is_empty = (hend <= hstart) || (wend <= wstart);
+          float v = is_empty ? 0.f : -FLT_MAX;
+          for (int h = hstart; h < hend; ++h)
+            for (int w = wstart; w < wend; ++w) v = std::max(v, plane[h * width + w]);
+          out[ph * pooled_w + pw] = v;
+        }
+      }
+    }
+  }
+  return 0;
+}
+
+/* ---- PSROIPooling (src/layers/psroi_pooling_layer.cpp:45-122) ---------------
+ * Position-sensitive average pooling: output channel c, bin (ph, pw) averages
+ * input channel (c*group + ph)*group + pw over the bin.  Region corners are
+ * rounded BEFORE scaling (end corner: round(x2 + 1)), the region is at least
+ * 0.1 wide, bins use floor / ceil of float positions, clipped to the map; the
+ * sum runs row-major over the bin and is divided by the bin area; an empty bin
+ * yields 0. */
+int orc_psroi_pooling(const float* bottom, int num, int output_dim, int group_size, int height,
+                      int width, const float* rois, int num_rois, float spatial_scale,
+                      float* top) {
+  const int pooled_h = group_size, pooled_w = group_size;
+  const int channels = output_dim * group_size * group_size;
+  for (int n = 0; n < num_rois; ++n) {
+    const float* roi = rois + 5 * n;
+    const int batch = static_cast<int>(roi[0]);
+    if (batch < 0 || batch >= num) return -1;
+    const float roi_start_w = static_cast<float>(round(roi[1]) * spatial_scale);
+    const float roi_start_h = static_cast<float>(round(roi[2]) * spatial_scale);
+    const float roi_end_w = static_cast<float>(round(roi[3] + 1) * spatial_scale);
+    const float roi_end_h = static_cast<float>(round(roi[4] + 1) * spatial_scale);
+    const float roi_height = std::max(roi_end_h - roi_start_h, static_cast<float>(0.1));
+    const float roi_width = std::max(roi_end_w - roi_start_w, static_cast<float>(0.1));
+    const float bin_size_h = roi_height / static_cast<float>(pooled_h);
+    const float bin_size_w = roi_width / static_cast<float>(pooled_w);
+    const float* batch_data = bottom + static_cast<size_t>(batch) * channels * height * width;
+    for (int c = 0; c < output_dim; ++c) {
+      float* out = top + (static_cast<size_t>(n) * output_dim + c) * pooled_h * pooled_w;
+      for (int ph = 0; ph < pooled_h; ++ph) {
+        for (int pw = 0; pw < pooled_w; ++pw) {
+          int hstart = static_cast<int>(std::floor(static_cast<float>(ph) * bin_size_h + roi_start_h));
+          int wstart = static_cast<int>(std::floor(static_cast<float>(pw) * bin_size_w + roi_start_w));
+          int hend = static_cast<int>(std::ceil(static_cast<float>(ph + 1) * bin_size_h + roi_start_h));
+          int wend = static_cast<int>(std::ceil(static_cast<float>(pw + 1) * bin_size_w + roi_start_w));
+          hstart = std::min(std::max(hstart, 0), height);
+          hend = std::min(std::max(hend, 0), height);
+          wstart = std::min(std::max(wstart, 0), width);
+          wend = std::min(std::max(wend, 0), width);
+          const bool is_empty = (hend <= hstart) || (wend <= wstart);
+          const int fm_c = (c * group_size + ph) * group_size + pw;
+          const float* fm = batch_data + static_cast<size_t>(fm_c) * height * width;
+          float out_sum = 0;
+          for (int h = hstart; h < hend; ++h)
+            for (int w = wstart; w < wend; ++w) out_sum += fm[h * width + w];
+          const int bin_area = (hend - hstart) * (wend - wstart);
+          out[ph * pooled_w + pw] = is_empty ? 0.f : out_sum / static_cast<float>(bin_area);
+        }
+      }
+    }
+  }
+  return 0;
 }
 
 }  // extern "C"

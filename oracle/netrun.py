@@ -127,6 +127,14 @@ def run_layer(layer, bottoms):
     if t == "DetectionOutput":
         return [oracle.detection_output(layer["detection_output_param"], bottoms[0], bottoms[1],
                                         bottoms[2])]
+    if t == "ROIPooling":
+        p = layer["roi_pooling_param"]
+        return [oracle.roi_pooling(x, bottoms[1], p["pooled_h"], p["pooled_w"],
+                                   p.get("spatial_scale", 1.0))]
+    if t == "PSROIPooling":
+        p = layer["psroi_pooling_param"]
+        return [oracle.psroi_pooling(x, bottoms[1], p["output_dim"], p["group_size"],
+                                     p["spatial_scale"])]
     raise NotImplementedError(t)
 
 
@@ -135,6 +143,11 @@ def oracle_forward(spec, inputs, keep=None):
     Returns dict blob name -> final array (in-place layers overwrite).
     keep: optional set of blob names to retain (all are kept when None)."""
     blobs = {k: np.ascontiguousarray(v, dtype=np.float32) for k, v in inputs.items()}
+    # Proposal shrinks its tops to the kept count in Forward, after every layer's
+    # Reshape has run: a region pooling layer's top keeps the row count the rois had
+    # at Reshape time and fills the rows it does not pool
+    # (roi_pooling_layer.cpp:46 -FLT_MAX, psroi_pooling_layer.cpp:54 zero).
+    reshape_rows = {}
     for layer in spec:
         if layer["type"] == "Input":
             for name in layer["top"]:
@@ -142,6 +155,16 @@ def oracle_forward(spec, inputs, keep=None):
             continue
         bottoms = [blobs[b] for b in layer.get("bottom", [])]
         tops = run_layer(layer, bottoms)
+        if layer["type"] == "Proposal":
+            rows = bottoms[0].shape[0] * layer.get("proposal_param", {}).get("post_nms_topn", 300)
+            for name in layer["top"]:
+                reshape_rows[name] = rows
+        if layer["type"] in ("ROIPooling", "PSROIPooling"):
+            rows = reshape_rows.get(layer["bottom"][1], tops[0].shape[0])
+            if rows > tops[0].shape[0]:
+                fill = np.float32(-3.4028234663852886e38 if layer["type"] == "ROIPooling" else 0.0)
+                pad = np.full((rows - tops[0].shape[0],) + tops[0].shape[1:], fill, np.float32)
+                tops = [np.concatenate([tops[0], pad])]
         for name, arr in zip(layer["top"], tops):
             blobs[name] = np.ascontiguousarray(arr, dtype=np.float32)
     if keep is not None:

@@ -243,3 +243,26 @@ def test_reads_the_reference_wgan_prototxt():
     net = mc.Net.from_buffers(open(os.path.join(REF, "example", "models", "wgan", "g.prototxt")).read())
     shapes = {k: v.shape for k, v in net.blobs.items()}
     assert list(shapes.values())[-1][1:] == [3, 64, 64]
+
+
+def test_region_pooling_layers_setup_errors_and_shapes():
+    """ROIPooling / PSROIPooling construction (roi_pooling_layer.cpp:15-36,
+    psroi_pooling_layer.cpp:18-44): parameter checks and the top shape taken from the
+    rois blob's row count."""
+    from minicaffe import MiniCaffeError
+    base = [craft.input_layer({"feat": (1, 18, 6, 8), "rois": (7, 5)})]
+    ok = base + [{"name": "ps", "type": "PSROIPooling", "bottom": ["feat", "rois"], "top": ["ps"],
+                  "psroi_pooling_param": {"spatial_scale": 0.0625, "output_dim": 2, "group_size": 3}},
+                 {"name": "rp", "type": "ROIPooling", "bottom": ["feat", "rois"], "top": ["rp"],
+                  "roi_pooling_param": {"pooled_h": 2, "pooled_w": 4, "spatial_scale": 0.0625}}]
+    net = mc.Net.from_buffers(craft.to_prototxt(ok))
+    assert tuple(net.get_blob("ps").shape) == (7, 2, 3, 3)
+    assert tuple(net.get_blob("rp").shape) == (7, 18, 2, 4)
+    bad = base + [{"name": "ps", "type": "PSROIPooling", "bottom": ["feat", "rois"], "top": ["ps"],
+                   "psroi_pooling_param": {"spatial_scale": 0.0625, "output_dim": 4, "group_size": 3}}]
+    with pytest.raises(MiniCaffeError, match="input channel number does not match"):
+        mc.Net.from_buffers(craft.to_prototxt(bad))
+    bad = base + [{"name": "rp", "type": "ROIPooling", "bottom": ["feat", "rois"], "top": ["rp"],
+                   "roi_pooling_param": {"pooled_h": 0, "pooled_w": 4}}]
+    with pytest.raises(MiniCaffeError, match="pooled_h must be > 0"):
+        mc.Net.from_buffers(craft.to_prototxt(bad))

@@ -436,3 +436,60 @@ def test_detection_output_bit_exact(K, num, P, C, share, code, keep, thr, nms, e
     got = out[:int(cnt.item())].cpu().numpy()
     assert got.shape == want.shape
     assert np.array_equal(got, want)
+
+
+def _random_rois(rng, n_rois, num, img_h, img_w):
+    """Proposal-like rows [batch, x1, y1, x2, y2] in image coordinates, with some tiny,
+    some reaching past the image and some wholly outside."""
+    b = rng.integers(0, num, n_rois).astype(np.float32)
+    cx, cy = rng.random(n_rois) * img_w, rng.random(n_rois) * img_h
+    w, h = rng.random(n_rois) ** 2 * img_w, rng.random(n_rois) ** 2 * img_h
+    rois = np.stack([b, cx - w / 2, cy - h / 2, cx + w / 2, cy + h / 2], 1).astype(np.float32)
+    rois[0, 1:] = [0, 0, img_w - 1, img_h - 1]
+    rois[1, 1:] = [img_w + 5, img_h + 5, img_w + 40, img_h + 40]      # outside
+    rois[2, 1:] = [3.2, 4.7, 3.4, 4.9]                                # below one cell
+    rois[3, 1:] = [-30.5, -12.5, 20.5, 17.5]                          # negative corner, half-way values
+    return rois
+
+
+@pytest.mark.parametrize("shape,pooled,scale", [((2, 5, 38, 63), (6, 6), 0.0625), ((1, 3, 9, 7), (2, 3), 1.0),
+                                                ((3, 4, 20, 20), (7, 7), 0.125)])
+def test_roi_pooling_bit_exact(K, shape, pooled, scale):
+    rng = np.random.default_rng(20)
+    x = rng.standard_normal(shape).astype(np.float32)
+    rois = _random_rois(rng, 64, shape[0], shape[2] / scale, shape[3] / scale)
+    want = oracle.roi_pooling(x, rois, pooled[0], pooled[1], scale)
+    xd, rd = dev(x), dev(rois)
+    out = torch.full(want.shape, float("nan"), device="cuda")
+    K.check_mc(K.LIB.mcROIPooling(fptr(xd), *shape, fptr(rd), rois.shape[0], pooled[0], pooled[1],
+                                  ctypes.c_float(scale), fptr(out), None, None))
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("num,dim,g,hw,scale", [(1, 21, 7, (38, 63), 0.0625), (2, 8, 3, (20, 20), 0.125),
+                                                (1, 4, 1, (6, 6), 1.0)])
+def test_psroi_pooling_bit_exact(K, num, dim, g, hw, scale):
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((num, dim * g * g) + hw).astype(np.float32)
+    rois = _random_rois(rng, 64, num, hw[0] / scale, hw[1] / scale)
+    want = oracle.psroi_pooling(x, rois, dim, g, scale)
+    xd, rd = dev(x), dev(rois)
+    out = torch.full(want.shape, float("nan"), device="cuda")
+    flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+    K.check_mc(K.LIB.mcPSROIPooling(fptr(xd), num, dim, g, hw[0], hw[1], fptr(rd), rois.shape[0],
+                                    ctypes.c_float(scale), fptr(out), ctypes.c_void_p(flag.data_ptr()), None))
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), want)     # same expressions, same summation order
+    assert int(flag.item()) == 0
+    # a batch index outside the blob: zeros and the flag, where the reference's CPU code CHECK-fails
+    bad = rois[:4].copy()
+    bad[1, 0] = num
+    rd2 = dev(bad)
+    out2 = torch.full((4, dim, g, g), float("nan"), device="cuda")
+    K.check_mc(K.LIB.mcPSROIPooling(fptr(xd), num, dim, g, hw[0], hw[1], fptr(rd2), 4,
+                                    ctypes.c_float(scale), fptr(out2), ctypes.c_void_p(flag.data_ptr()), None))
+    torch.cuda.synchronize()
+    got = out2.cpu().numpy()
+    assert int(flag.item()) == 1 and np.array_equal(got[1], np.zeros((dim, g, g), np.float32))
+    assert np.array_equal(got[[0, 2, 3]], want[[0, 2, 3]])

@@ -324,3 +324,49 @@ def test_config3_ssd_full_size_b8(gpu_mode):
     finally:
         oracle.use_openblas(False)
     assert netrun.rel_err(fc7_gpu, want["fc7"]) < 1e-3
+
+
+def test_rfcn_second_stage_on_proposal_rois(gpu_mode):
+    """Config 4 continued into a detector head: the rois of Proposal feed a
+    position-sensitive pooling branch (R-FCN: 1x1 conv -> PSROIPooling -> global
+    average) and a ROIPooling branch.  Tops keep post_nms_topn rows with the
+    reference's fill in the rows past the kept count."""
+    import minicaffe as mc
+    from minicaffe import zoo
+    from minicaffe.craft import Enum
+    spec, inputs = zoo.rpn_spec(seed=3, feat_shape=(1, 64, 20, 30), im_info=(320.0, 480.0, 1.0), mid=32,
+                                post_nms_topn=50, nms_thresh=0.5)
+    dim, g = 5, 3
+    spec += [zoo.conv_layer("rfcn_cls", "feat", "rfcn_cls", 64, dim * g * g, 1, seed=4, std=0.05),
+             {"name": "psroipooled_cls_rois", "type": "PSROIPooling", "bottom": ["rfcn_cls", "rois"],
+              "top": ["psroipooled_cls_rois"],
+              "psroi_pooling_param": {"spatial_scale": 0.0625, "output_dim": dim, "group_size": g}},
+             {"name": "ave_cls_score_rois", "type": "Pooling", "bottom": ["psroipooled_cls_rois"],
+              "top": ["cls_score"], "pooling_param": {"pool": Enum("AVE"), "kernel_size": g, "stride": g}},
+             {"name": "roi_pool", "type": "ROIPooling", "bottom": ["feat", "rois"], "top": ["roi_pool"],
+              "roi_pooling_param": {"pooled_h": 4, "pooled_w": 4, "spatial_scale": 0.0625}}]
+    marks = ("rpn_cls_prob_reshape", "rpn_bbox_pred", "rfcn_cls", "rois", "psroipooled_cls_rois", "cls_score",
+             "roi_pool")
+    net = run_net(mc, spec, inputs, marks)
+    # the dense part within tolerance ...
+    dense = netrun.oracle_forward([l for l in spec if l["type"] not in ("Proposal", "PSROIPooling", "ROIPooling")
+                                   and l["name"] != "ave_cls_score_rois"], inputs)
+    for name in ("rpn_cls_prob_reshape", "rpn_bbox_pred", "rfcn_cls"):
+        assert netrun.rel_err(net.get_blob(name).data, dense[name]) < 1e-3
+    # ... the tail bit for bit on the blobs the device produced
+    tail_in = {name: net.get_blob(name).data.copy() for name in ("rpn_cls_prob_reshape", "rpn_bbox_pred", "rfcn_cls")}
+    tail_in.update(feat=inputs["feat"], im_info=inputs["im_info"])
+    tail = [{"name": "in", "type": "Input", "top": list(tail_in)}] + \
+           [l for l in spec if l["type"] in ("Proposal", "PSROIPooling", "ROIPooling") or l["name"] == "ave_cls_score_rois"]
+    want = netrun.oracle_forward(tail, tail_in)
+    rois = net.get_blob("rois").data
+    r = rois.shape[0]
+    assert np.array_equal(rois, want["rois"]) and 0 < r <= 50
+    ps = net.get_blob("psroipooled_cls_rois").data
+    assert ps.shape == (50, dim, g, g) == want["psroipooled_cls_rois"].shape
+    assert np.array_equal(ps, want["psroipooled_cls_rois"])        # same sums in the same order
+    if r < 50:
+        assert np.array_equal(ps[r:], np.zeros_like(ps[r:]))       # rows past the kept count
+    rp = net.get_blob("roi_pool").data
+    assert rp.shape == (50, 64, 4, 4) and np.array_equal(rp, want["roi_pool"])
+    assert netrun.rel_err(net.get_blob("cls_score").data, want["cls_score"]) < 1e-5

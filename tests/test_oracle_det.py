@@ -215,3 +215,57 @@ def test_normalize_closed_form():
     y = oracle.normalize(x, s[:1], across_spatial=True, channel_shared=True, eps=1e-10)
     want = x / np.sqrt((x.astype(np.float64) ** 2).sum(axis=(1, 2, 3), keepdims=True) + 1e-10) * s[0]
     assert np.abs(y - want).max() < 1e-6
+
+
+# ---- region pooling (roi_pooling_layer.cpp, psroi_pooling_layer.cpp) --------------------
+# Pinned through cases that reduce to numpy routines, chosen so that a wrong rounding
+# rule, a missing "+1", a transposed bin index or a wrong channel map fails one of them.
+
+def _blocks(a, bh, bw):
+    """(C, H, W) -> (C, H/bh, W/bw, bh*bw) blocks."""
+    c, h, w = a.shape
+    return a.reshape(c, h // bh, bh, w // bw, bw).transpose(0, 1, 3, 2, 4).reshape(c, h // bh, w // bw, -1)
+
+
+def test_roi_pooling_reduces_to_numpy_cases():
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((2, 3, 8, 12)).astype(np.float32)
+    whole = [[1, 0, 0, 11, 7]]                       # x1, y1, x2, y2 inclusive
+    assert np.array_equal(oracle.roi_pooling(x, whole, 1, 1, 1.0)[0, :, 0, 0], x[1].max(axis=(1, 2)))
+    assert np.array_equal(oracle.roi_pooling(x, whole, 8, 12, 1.0)[0], x[1])        # one bin per cell
+    assert np.array_equal(oracle.roi_pooling(x, whole, 4, 3, 1.0)[0], _blocks(x[1], 2, 4).max(-1))
+    # an aligned sub-region: rows 2..5, columns 4..9 (inclusive ends: the "+1" of the extent)
+    sub = oracle.roi_pooling(x, [[0, 4, 2, 9, 5]], 2, 3, 1.0)[0]
+    assert np.array_equal(sub, _blocks(x[0][:, 2:6, 4:10], 2, 2).max(-1))
+    # spatial_scale: image coordinates 16x the map's, rounded after scaling (40/16 = 2.5 -> 3)
+    scaled = oracle.roi_pooling(x, [[0, 40, 0, 191, 127]], 1, 1, 1 / 16.0)[0, :, 0, 0]
+    assert np.array_equal(scaled, x[0][:, 0:8, 3:12].max(axis=(1, 2)))
+    # a roi outside the map: every bin empty -> 0; a bad batch index is an error
+    assert np.array_equal(oracle.roi_pooling(x, [[0, 50, 50, 60, 60]], 2, 2, 1.0), np.zeros((1, 3, 2, 2)))
+    with pytest.raises(ValueError):
+        oracle.roi_pooling(x, [[2, 0, 0, 1, 1]], 1, 1, 1.0)
+
+
+def test_psroi_pooling_reduces_to_numpy_cases():
+    rng = np.random.default_rng(1)
+    dim, g = 3, 2
+    x = rng.standard_normal((2, dim * g * g, 8, 12)).astype(np.float32)
+    whole = [[1, 0, 0, 11, 7]]
+    got = oracle.psroi_pooling(x, whole, dim, g, 1.0)[0]
+    # bin (ph, pw) of output c = mean of the (ph, pw) block of input channel (c*g + ph)*g + pw
+    for c in range(dim):
+        for ph in range(g):
+            for pw in range(g):
+                blk = x[1, (c * g + ph) * g + pw, ph * 4:(ph + 1) * 4, pw * 6:(pw + 1) * 6]
+                assert abs(got[c, ph, pw] - blk.astype(np.float64).mean()) < 1e-6
+    # group_size 1: plain mean over the region, end corner x2 + 1 exclusive
+    x1 = rng.standard_normal((1, 4, 6, 6)).astype(np.float32)
+    got = oracle.psroi_pooling(x1, [[0, 1, 2, 4, 3]], 4, 1, 1.0)[0, :, 0, 0]
+    assert np.allclose(got, x1[0][:, 2:4, 1:5].astype(np.float64).mean(axis=(1, 2)), atol=1e-6)
+    # corners are rounded BEFORE scaling: x1 = 7.6 -> 8 -> 0.5 on a 1/16 map, i.e. bin start floor(0.5) = 0
+    got = oracle.psroi_pooling(x1, [[0, 7.6, 0, 31.4, 15.2]], 4, 1, 1 / 16.0)[0, :, 0, 0]
+    assert np.allclose(got, x1[0][:, 0:1, 0:2].astype(np.float64).mean(axis=(1, 2)), atol=1e-6)
+    # outside the map -> 0
+    assert np.array_equal(oracle.psroi_pooling(x1, [[0, 100, 100, 120, 120]], 4, 1, 1.0), np.zeros((1, 4, 1, 1)))
+    with pytest.raises(ValueError):
+        oracle.psroi_pooling(x1, [[0, 0, 0, 1, 1]], 3, 1, 1.0)      # channel count mismatch
