@@ -37,6 +37,7 @@ constexpr int LDK = BK + 4;  // LDS row pitch in floats
 
 typedef float acc16 __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+constexpr int kModeMasks = 0, kModeOneMask = 1, kModePointwise = 2;
 // Buffer descriptor word 3 for raw dword access on gfx9-family CDNA parts
 // (32-bit data format, no swizzle, offsets checked against num_records).
 constexpr int kBufferFlags = 0x00020000;
@@ -114,10 +115,17 @@ __device__ __forceinline__ float apply_act(float v, int act, float slope) {
 }
 
 // OCC = wavefronts per SIMD the register allocation must leave room for.
-// PW ("pointwise"): every row k of the gather is channel k of the bottom blob
+// MODE selects how the K loop finds and guards the elements it gathers:
+//   kModeMasks     tap table + one "outside the image" bit mask per tap row and
+//                  per tap column (any kernel up to 31 x 31 taps);
+//   kModeOneMask   tap table + one mask with a bit per (row, column) tap pair,
+//                  for kernels with at most 31 taps (3x3, 5x5): one extract
+//                  instead of two per element;
+//   kModePointwise no table and no mask, see below.
+// Pointwise: every row k of the gather is channel k of the bottom blob
 // at the thread's own pixel (1x1 kernel, no padding), so the K loop needs no
 // tap table and no bounds handling at all.
-template <int BM, int BN, int WM, int WN, int OCC, bool PW>
+template <int BM, int BN, int WM, int WN, int OCC, int MODE>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void igemm_kernel(
     const IgemmBatch batch) {
   static_assert(WM * WN == 4, "four wavefronts per workgroup");
@@ -191,6 +199,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
   const int pj = tid % BN;
   const int prow = tid / BN;  // wave-uniform because BN >= 64
   // byte offset of the pixel's origin from the descriptor base (never negative)
+  constexpr bool PW = MODE == kModePointwise;
   unsigned xvoff = PW ? kNoElement : 0u;
   unsigned row_bad = 0xFFFFFFFFu, col_bad = 0xFFFFFFFFu;
   {
@@ -215,6 +224,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
           col_bad |= static_cast<unsigned>(static_cast<unsigned>(wi0 + a.tap_dw[b]) >=
                                            static_cast<unsigned>(a.W))
                      << b;
+        if constexpr (MODE == kModeOneMask) {
+          // bit i*n_dw + j = row tap i or column tap j outside; the result replaces row_bad
+          const unsigned all_cols = (1u << a.n_dw) - 1u;
+          unsigned pair_bad = 0x80000000u;
+          for (int b = 0; b < a.n_dh; ++b)
+            pair_bad |= (((row_bad >> b) & 1u) ? all_cols : col_bad) << (b * a.n_dw);
+          row_bad = pair_bad;
+        }
       }
     }
   }
@@ -246,11 +263,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
   __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(res, voff, soff, 0))
 #define MC_GATHER1(dst, t)                                                                   \
   {                                                                                          \
-    const unsigned rb = __builtin_amdgcn_ubfe(row_bad, (t).y, 1);                            \
-    const unsigned cb = __builtin_amdgcn_ubfe(col_bad, (t).z, 1);                            \
-    /* a valid element's offset is below 2^31; bit 31 marks "no element" */                  \
-    const unsigned off = xvoff + static_cast<unsigned>((t).x);                               \
-    dst = MC_LOADF(xres, (cb << 31) | ((rb << 31) | off), 0);                                \
+    /* The tap's byte offset rides in the scalar offset of the load; the VGPR                \
+       offset is the pixel origin, with bit 31 set when the tap is outside the               \
+       image.  Origin + tap offset stays below 2^31, so a flagged sum cannot wrap            \
+       whether or not the hardware adds the scalar offset before its range check. */        \
+    if constexpr (MODE == kModeOneMask) {                                                    \
+      const unsigned pb = __builtin_amdgcn_ubfe(row_bad, (t).w, 1);                          \
+      dst = MC_LOADF(xres, (pb << 31) | xvoff, (t).x);                                       \
+    } else {                                                                                 \
+      const unsigned rb = __builtin_amdgcn_ubfe(row_bad, (t).y, 1);                          \
+      const unsigned cb = __builtin_amdgcn_ubfe(col_bad, (t).z, 1);                          \
+      dst = MC_LOADF(xres, (cb << 31) | ((rb << 31) | xvoff), (t).x);                        \
+    }                                                                                        \
   }
 #define MC_LOAD_TILES(kt)                                                                    \
   {                                                                                          \
@@ -554,25 +578,31 @@ __global__ void pack_weights_kernel(const float* __restrict__ w, float* __restri
 struct TileConfig {
   int bm, bn;
   const char* name;
-  void (*kernel)(const IgemmBatch);
-  void (*kernel_pw)(const IgemmBatch);  // pointwise variant
+  void (*kernel[3])(const IgemmBatch);  // indexed by kModeMasks / kModeOneMask / kModePointwise
 };
 
 const TileConfig kConfigs[] = {
     {128, 128, "igemm_f32_128x128",
-     igemm_kernel<128, 128, 2, 2, 3, false>, igemm_kernel<128, 128, 2, 2, 3, true>},
+     {igemm_kernel<128, 128, 2, 2, 3, kModeMasks>, igemm_kernel<128, 128, 2, 2, 3, kModeOneMask>,
+      igemm_kernel<128, 128, 2, 2, 3, kModePointwise>}},
     {128, 64, "igemm_f32_128x64",
-     igemm_kernel<128, 64, 2, 2, 4, false>, igemm_kernel<128, 64, 2, 2, 4, true>},
+     {igemm_kernel<128, 64, 2, 2, 4, kModeMasks>, igemm_kernel<128, 64, 2, 2, 4, kModeOneMask>,
+      igemm_kernel<128, 64, 2, 2, 4, kModePointwise>}},
     {64, 128, "igemm_f32_64x128",
-     igemm_kernel<64, 128, 2, 2, 5, false>, igemm_kernel<64, 128, 2, 2, 5, true>},
+     {igemm_kernel<64, 128, 2, 2, 5, kModeMasks>, igemm_kernel<64, 128, 2, 2, 5, kModeOneMask>,
+      igemm_kernel<64, 128, 2, 2, 5, kModePointwise>}},
     {64, 64, "igemm_f32_64x64",
-     igemm_kernel<64, 64, 2, 2, 8, false>, igemm_kernel<64, 64, 2, 2, 8, true>},
+     {igemm_kernel<64, 64, 2, 2, 8, kModeMasks>, igemm_kernel<64, 64, 2, 2, 8, kModeOneMask>,
+      igemm_kernel<64, 64, 2, 2, 8, kModePointwise>}},
     {32, 128, "igemm_f32_32x128",
-     igemm_kernel<32, 128, 1, 4, 4, false>, igemm_kernel<32, 128, 1, 4, 4, true>},
+     {igemm_kernel<32, 128, 1, 4, 4, kModeMasks>, igemm_kernel<32, 128, 1, 4, 4, kModeOneMask>,
+      igemm_kernel<32, 128, 1, 4, 4, kModePointwise>}},
     {32, 256, "igemm_f32_32x256",
-     igemm_kernel<32, 256, 1, 4, 3, false>, igemm_kernel<32, 256, 1, 4, 3, true>},
+     {igemm_kernel<32, 256, 1, 4, 3, kModeMasks>, igemm_kernel<32, 256, 1, 4, 3, kModeOneMask>,
+      igemm_kernel<32, 256, 1, 4, 3, kModePointwise>}},
     {64, 256, "igemm_f32_64x256",
-     igemm_kernel<64, 256, 1, 4, 2, false>, igemm_kernel<64, 256, 1, 4, 2, true>},
+     {igemm_kernel<64, 256, 1, 4, 2, kModeMasks>, igemm_kernel<64, 256, 1, 4, 2, kModeOneMask>,
+      igemm_kernel<64, 256, 1, 4, 2, kModePointwise>}},
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 
@@ -587,6 +617,7 @@ struct SubProblem {
   std::vector<int> wk_off;   // host copy
   std::vector<int> tap_dh, tap_dw;  // bottom offset of each row / column tap index
   bool pointwise = false;    // every k is channel k at the pixel itself, always in range
+  bool one_mask = false;     // at most 31 (row, column) tap pairs: one validity mask
   // The bottom descriptor starts tap_shift + pix_shift bytes before the blob:
   // tap offsets are stored plus tap_shift, pixel origins computed plus pix_shift,
   // so both are non-negative.
@@ -779,7 +810,7 @@ int mcConvPlanCreate(const mcConvGeom* gp, mcConvPlan** out) {
       for (int i = 0; i < g.kernel_h; ++i)
         for (int j = 0; j < g.kernel_w; ++j) {
           const int dh = i * g.dilation_h, dw = j * g.dilation_w;
-          s.ktab.push_back(make_int4((c * HW + dh * g.width_in + dw) * 4, i, j, 0));
+          s.ktab.push_back(make_int4((c * HW + dh * g.width_in + dw) * 4, i, j, i * g.kernel_w + j));
           s.wk_off.push_back((c * g.kernel_h + i) * g.kernel_w + j);
         }
     s.pointwise = g.kernel_h == 1 && g.kernel_w == 1 && g.pad_h == 0 && g.pad_w == 0;
@@ -820,7 +851,8 @@ int mcConvPlanCreate(const mcConvGeom* gp, mcConvPlan** out) {
           for (size_t i = 0; i < tap_h.size(); ++i)
             for (size_t j = 0; j < tap_w.size(); ++j) {
               s.ktab.push_back(make_int4((c * HW + off_h[i] * g.width_in + off_w[j]) * 4,
-                                         static_cast<int>(i), static_cast<int>(j), 0));
+                                         static_cast<int>(i), static_cast<int>(j),
+                                         static_cast<int>(i * tap_w.size() + j)));
               s.wk_off.push_back(c * plan->M * khkw + tap_h[i] * g.kernel_w + tap_w[j]);
             }
         s.tap_dh = off_h;
@@ -834,7 +866,7 @@ int mcConvPlanCreate(const mcConvGeom* gp, mcConvPlan** out) {
     s.Kpad = ceil_div(s.K, BK) * BK;
     // Padding rows multiply zero weights; row-tap index 31 is out of the image
     // for every pixel, so nothing is fetched for them.
-    while (static_cast<int>(s.ktab.size()) < s.Kpad) s.ktab.push_back(make_int4(0, 31, 0, 0));
+    while (static_cast<int>(s.ktab.size()) < s.Kpad) s.ktab.push_back(make_int4(0, 31, 0, 31));
     int min_tap = 0;
     for (const int4& t : s.ktab) min_tap = std::min(min_tap, t.x);
     s.tap_shift = -min_tap;
@@ -844,6 +876,7 @@ int mcConvPlanCreate(const mcConvGeom* gp, mcConvPlan** out) {
     const size_t wt_bytes = sizeof(float) * (size_t)g.group * s.Kpad * plan->Mpad;
     hipError_t e = hipSuccess;
     const char* what = nullptr;
+    s.one_mask = s.tap_dh.size() * s.tap_dw.size() <= 31;
     if (s.tap_dh.size() > 31 || s.tap_dw.size() > 31)
       what = "kernels with more than 31 taps per dimension are not supported";
     else if (wt_bytes >= (1ull << 31))
@@ -925,8 +958,8 @@ int mcConvPlanSetWeights(mcConvPlan* plan, const float* weights, void* stream) {
 
 int mcConvPlanForceConfig(mcConvPlan* plan, int config) {
   MC_REQUIRE(plan, "mcConvPlanForceConfig: null plan");
-  // config + 100 pins the same tile with the tap-table gather (tests compare the
-  // pointwise fast path against it)
+  // config + 100 pins the same tile with the two-mask tap-table gather (tests
+  // compare the pointwise and one-mask fast paths against it)
   plan->force_general = config >= 100;
   if (config >= 100) config -= 100;
   MC_REQUIRE(config >= -1 && config < kNumConfigs, "mcConvPlanForceConfig: no such configuration");
@@ -969,13 +1002,14 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
   const int MT = ceil_div(plan->M, cfg.bm);
   long total_blocks = 0;
   int min_kt = 1 << 30;
-  bool pointwise = !plan->force_general;
+  bool pointwise = !plan->force_general, one_mask = !plan->force_general;
   double flops = 0.;
   for (const SubProblem* s : live) {
     const long pixels = (long)num * s->Hq * s->Wq;
     total_blocks += (long)MT * ceil_div(pixels, cfg.bn) * g.group;
     if (s->Kpad > 0) min_kt = std::min(min_kt, s->Kpad / BK);
     pointwise = pointwise && s->pointwise;
+    one_mask = one_mask && s->one_mask;
     flops += 2.0 * pixels * plan->M * g.group * s->K;
   }
   if (min_kt == (1 << 30)) min_kt = 1;
@@ -1071,7 +1105,8 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
       }
     }
     dim3 grid(static_cast<unsigned>(max_blocks), g.group, nsub * slices);
-    (pointwise ? cfg.kernel_pw : cfg.kernel)<<<grid, 256, 0, st>>>(batch);
+    cfg.kernel[pointwise ? kModePointwise : (one_mask ? kModeOneMask : kModeMasks)]<<<grid, 256, 0, st>>>(
+        batch);
     MC_LAUNCH_CHECK();
   }
   if (slices > 1) {
