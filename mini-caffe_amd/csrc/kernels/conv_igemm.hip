@@ -119,8 +119,11 @@ __device__ __forceinline__ float apply_act(float v, int act, float slope) {
 //   kModeMasks     tap table + one "outside the image" bit mask per tap row and
 //                  per tap column (any kernel up to 31 x 31 taps);
 //   kModeOneMask   tap table + one mask with a bit per (row, column) tap pair,
-//                  for kernels with at most 31 taps (3x3, 5x5): one extract
-//                  instead of two per element;
+//                  for kernels with at most 31 taps (3x3, 5x5) and a channel
+//                  count that is a multiple of 4: the K rows are then ordered
+//                  (channel block of 4, tap, channel in block), so the four
+//                  rows a thread gathers per step share one tap and one
+//                  validity test;
 //   kModePointwise no table and no mask, see below.
 // Pointwise: every row k of the gather is channel k of the bottom blob
 // at the thread's own pixel (1x1 kernel, no padding), so the K loop needs no
@@ -267,14 +270,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
        offset is the pixel origin, with bit 31 set when the tap is outside the               \
        image.  Origin + tap offset stays below 2^31, so a flagged sum cannot wrap            \
        whether or not the hardware adds the scalar offset before its range check. */        \
-    if constexpr (MODE == kModeOneMask) {                                                    \
-      const unsigned pb = __builtin_amdgcn_ubfe(row_bad, (t).w, 1);                          \
-      dst = MC_LOADF(xres, (pb << 31) | xvoff, (t).x);                                       \
-    } else {                                                                                 \
-      const unsigned rb = __builtin_amdgcn_ubfe(row_bad, (t).y, 1);                          \
-      const unsigned cb = __builtin_amdgcn_ubfe(col_bad, (t).z, 1);                          \
-      dst = MC_LOADF(xres, (cb << 31) | ((rb << 31) | xvoff), (t).x);                        \
-    }                                                                                        \
+    const unsigned rb = __builtin_amdgcn_ubfe(row_bad, (t).y, 1);                            \
+    const unsigned cb = __builtin_amdgcn_ubfe(col_bad, (t).z, 1);                            \
+    dst = MC_LOADF(xres, (cb << 31) | ((rb << 31) | xvoff), (t).x);                          \
   }
 #define MC_LOAD_TILES(kt)                                                                    \
   {                                                                                          \
@@ -298,10 +296,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
       } else {                                                                               \
         const int4 t0 = a.ktab[krow], t1 = a.ktab[krow + 1], t2 = a.ktab[krow + 2],          \
                    t3 = a.ktab[krow + 3];                                                    \
-        MC_GATHER1(breg[i].x, t0);                                                           \
-        MC_GATHER1(breg[i].y, t1);                                                           \
-        MC_GATHER1(breg[i].z, t2);                                                           \
-        MC_GATHER1(breg[i].w, t3);                                                           \
+        if constexpr (MODE == kModeOneMask) {                                                \
+          /* rows krow .. krow+3: four channels at one tap */                                \
+          const unsigned pb = __builtin_amdgcn_ubfe(row_bad, t0.w, 1);                       \
+          const unsigned voff = (pb << 31) | xvoff;                                          \
+          breg[i].x = MC_LOADF(xres, voff, t0.x);                                            \
+          breg[i].y = MC_LOADF(xres, voff, t1.x);                                            \
+          breg[i].z = MC_LOADF(xres, voff, t2.x);                                            \
+          breg[i].w = MC_LOADF(xres, voff, t3.x);                                            \
+        } else {                                                                             \
+          MC_GATHER1(breg[i].x, t0);                                                         \
+          MC_GATHER1(breg[i].y, t1);                                                         \
+          MC_GATHER1(breg[i].z, t2);                                                         \
+          MC_GATHER1(breg[i].w, t3);                                                         \
+        }                                                                                    \
       }                                                                                      \
     }                                                                                        \
   }
@@ -876,7 +884,27 @@ int mcConvPlanCreate(const mcConvGeom* gp, mcConvPlan** out) {
     const size_t wt_bytes = sizeof(float) * (size_t)g.group * s.Kpad * plan->Mpad;
     hipError_t e = hipSuccess;
     const char* what = nullptr;
-    s.one_mask = s.tap_dh.size() * s.tap_dw.size() <= 31;
+    // Few taps and channels in fours: reorder the K rows from (channel, tap) to
+    // (channel block of 4, tap, channel in block).  Any order is a valid GEMM as
+    // long as filter packing (wk_off) follows it; this one gives a thread's four
+    // rows per step a common tap while the taps of a channel stay close in K, so
+    // their overlapping input lines are still re-read from L1.
+    const int pairs = static_cast<int>(s.tap_dh.size() * s.tap_dw.size());
+    s.one_mask = pairs >= 1 && pairs <= 31 && plan->Cin_g % 4 == 0 && s.K == plan->Cin_g * pairs;
+    if (s.one_mask) {
+      std::vector<int4> kt(s.K);
+      std::vector<int> wk(s.K);
+      int k = 0;
+      for (int cb = 0; cb < plan->Cin_g / 4; ++cb)
+        for (int t = 0; t < pairs; ++t)
+          for (int ci = 0; ci < 4; ++ci, ++k) {
+            const int old = (cb * 4 + ci) * pairs + t;
+            kt[k] = s.ktab[old];
+            wk[k] = s.wk_off[old];
+          }
+      std::copy(kt.begin(), kt.end(), s.ktab.begin());
+      s.wk_off = wk;
+    }
     if (s.tap_dh.size() > 31 || s.tap_dw.size() > 31)
       what = "kernels with more than 31 taps per dimension are not supported";
     else if (wt_bytes >= (1ull << 31))
