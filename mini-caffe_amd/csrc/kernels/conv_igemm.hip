@@ -128,7 +128,7 @@ __device__ __forceinline__ float apply_act(float v, int act, float slope) {
 // Pointwise: every row k of the gather is channel k of the bottom blob
 // at the thread's own pixel (1x1 kernel, no padding), so the K loop needs no
 // tap table and no bounds handling at all.
-template <int BM, int BN, int WM, int WN, int OCC, int MODE>
+template <int BM, int BN, int WM, int WN, int OCC, int MODE, int KS>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void igemm_kernel(
     const IgemmBatch batch) {
   static_assert(WM * WN == 4, "four wavefronts per workgroup");
@@ -154,8 +154,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
   // K runs fastest in LDS ([row][k], rows padded to LDK floats) so that one
   // ds_read_b128 hands a lane four K steps of its MFMA operand; the 80-byte row
   // pitch spreads eight consecutive rows over all 32 banks.
-  __shared__ __attribute__((aligned(16))) float As[2][BM][LDK];
-  __shared__ __attribute__((aligned(16))) float Bs[2][BN][LDK];
+  // KS 16-row K tiles form one stage (one barrier per stage).
+  __shared__ __attribute__((aligned(16))) float As[2][KS][BM][LDK];
+  __shared__ __attribute__((aligned(16))) float Bs[2][KS][BN][LDK];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -238,8 +239,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
       }
     }
   }
-  const int KT = a.Kpad / BK;
-  // Split-K: slice z multiplies K tiles [kt_begin, kt_end) and writes its
+  const int KT = a.Kpad / (BK * KS);  // stages
+  // Split-K: slice z multiplies K stages [kt_begin, kt_end) and writes its
   // partial sums into its own copy of the top blob.
   const int kt_begin = kslice * a.kt_per_split;
   const int kt_end = min(KT, kt_begin + a.kt_per_split);
@@ -255,12 +256,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
                                               : kNoElement;
   }
   const unsigned wt_kt_bytes = static_cast<unsigned>(a.Mpad) * BK * 4;
-  const unsigned wt_g_bytes = static_cast<unsigned>(g) * KT * wt_kt_bytes;
+  const unsigned wt_g_bytes = static_cast<unsigned>(g) * (a.Kpad / BK) * wt_kt_bytes;
   const unsigned x_cbytes = static_cast<unsigned>(a.x_cstride) * 4;
   const int kmax = a.K - 1;
 
-  float4 areg[A_VEC];
-  float4 breg[B_Q];
+  float4 areg[KS][A_VEC];
+  float4 breg[KS][B_Q];
 
 #define MC_LOADF(res, voff, soff) \
   __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(res, voff, soff, 0))
@@ -275,23 +276,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
     dst = MC_LOADF(xres, (cb << 31) | ((rb << 31) | xvoff), (t).x);                          \
   }
 #define MC_LOAD_TILES(kt)                                                                    \
-  {                                                                                          \
-    const unsigned a_soff = wt_g_bytes + static_cast<unsigned>(kt) * wt_kt_bytes;            \
+  _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
+    const int kt16 = (kt)*KS + ks;                                                           \
+    const unsigned a_soff = wt_g_bytes + static_cast<unsigned>(kt16) * wt_kt_bytes;          \
     _Pragma("unroll") for (int i = 0; i < A_VEC; ++i) {                                      \
       const u32x4 w4 = __builtin_amdgcn_raw_buffer_load_b128(wres, avoff[i], a_soff, 0);     \
-      areg[i] = __builtin_bit_cast(float4, w4);                                              \
+      areg[ks][i] = __builtin_bit_cast(float4, w4);                                          \
     }                                                                                        \
     _Pragma("unroll") for (int i = 0; i < B_Q; ++i) {                                        \
       const int krow =                                                                       \
-          __builtin_amdgcn_readfirstlane((kt)*BK + (i * ROWS_PER_PASS + prow) * 4);          \
+          __builtin_amdgcn_readfirstlane(kt16 * BK + (i * ROWS_PER_PASS + prow) * 4);        \
       if constexpr (PW) {                                                                    \
         /* padding rows re-read the last channel; their filter rows are zero */              \
-        breg[i].x = MC_LOADF(xres, xvoff, static_cast<unsigned>(min(krow, kmax)) * x_cbytes);\
-        breg[i].y =                                                                          \
+        breg[ks][i].x = MC_LOADF(xres, xvoff, static_cast<unsigned>(min(krow, kmax)) * x_cbytes);\
+        breg[ks][i].y =                                                                          \
             MC_LOADF(xres, xvoff, static_cast<unsigned>(min(krow + 1, kmax)) * x_cbytes);    \
-        breg[i].z =                                                                          \
+        breg[ks][i].z =                                                                          \
             MC_LOADF(xres, xvoff, static_cast<unsigned>(min(krow + 2, kmax)) * x_cbytes);    \
-        breg[i].w =                                                                          \
+        breg[ks][i].w =                                                                          \
             MC_LOADF(xres, xvoff, static_cast<unsigned>(min(krow + 3, kmax)) * x_cbytes);    \
       } else {                                                                               \
         const int4 t0 = a.ktab[krow], t1 = a.ktab[krow + 1], t2 = a.ktab[krow + 2],          \
@@ -300,41 +302,42 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
           /* rows krow .. krow+3: four channels at one tap */                                \
           const unsigned pb = __builtin_amdgcn_ubfe(row_bad, t0.w, 1);                       \
           const unsigned voff = (pb << 31) | xvoff;                                          \
-          breg[i].x = MC_LOADF(xres, voff, t0.x);                                            \
-          breg[i].y = MC_LOADF(xres, voff, t1.x);                                            \
-          breg[i].z = MC_LOADF(xres, voff, t2.x);                                            \
-          breg[i].w = MC_LOADF(xres, voff, t3.x);                                            \
+          breg[ks][i].x = MC_LOADF(xres, voff, t0.x);                                            \
+          breg[ks][i].y = MC_LOADF(xres, voff, t1.x);                                            \
+          breg[ks][i].z = MC_LOADF(xres, voff, t2.x);                                            \
+          breg[ks][i].w = MC_LOADF(xres, voff, t3.x);                                            \
         } else {                                                                             \
-          MC_GATHER1(breg[i].x, t0);                                                         \
-          MC_GATHER1(breg[i].y, t1);                                                         \
-          MC_GATHER1(breg[i].z, t2);                                                         \
-          MC_GATHER1(breg[i].w, t3);                                                         \
+          MC_GATHER1(breg[ks][i].x, t0);                                                         \
+          MC_GATHER1(breg[ks][i].y, t1);                                                         \
+          MC_GATHER1(breg[ks][i].z, t2);                                                         \
+          MC_GATHER1(breg[ks][i].w, t3);                                                         \
         }                                                                                    \
       }                                                                                      \
     }                                                                                        \
   }
 #define MC_STORE_TILES(buf)                                                                  \
-  {                                                                                          \
+  _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
     _Pragma("unroll") for (int i = 0; i < A_VEC; ++i) {                                      \
       const int f = tid + 256 * i;                                                           \
       if (A_F4 % 256 == 0 || f < A_F4)                                                       \
-        *reinterpret_cast<float4*>(&As[buf][f / QUADS][(f % QUADS) * 4]) = areg[i];          \
+        *reinterpret_cast<float4*>(&As[buf][ks][f / QUADS][(f % QUADS) * 4]) = areg[ks][i];  \
     }                                                                                        \
     _Pragma("unroll") for (int i = 0; i < B_Q; ++i) {                                        \
-      *reinterpret_cast<float4*>(&Bs[buf][pj][(i * ROWS_PER_PASS + prow) * 4]) = breg[i];    \
+      *reinterpret_cast<float4*>(&Bs[buf][ks][pj][(i * ROWS_PER_PASS + prow) * 4]) =         \
+          breg[ks][i];                                                                       \
     }                                                                                        \
   }
   // One MFMA K step multiplies k-pairs; which two physical k rows form a pair
   // is free as long as A and B agree, so half-wave 0 takes k = 8h+e and
   // half-wave 1 takes k = 8h+4+e for step (h, e): four steps per b128 read.
 #define MC_COMPUTE(buf)                                                                      \
-  {                                                                                          \
+  _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
     float4 av[TM][2], bv[TN][2];                                                             \
     _Pragma("unroll") for (int h = 0; h < 2; ++h) {                                          \
-      _Pragma("unroll") for (int i = 0; i < TM; ++i) av[i][h] =                              \
-          *reinterpret_cast<const float4*>(&As[buf][wm0 + i * 32 + l32][h * 8 + lhi * 4]);   \
-      _Pragma("unroll") for (int j = 0; j < TN; ++j) bv[j][h] =                              \
-          *reinterpret_cast<const float4*>(&Bs[buf][wn0 + j * 32 + l32][h * 8 + lhi * 4]);   \
+      _Pragma("unroll") for (int i = 0; i < TM; ++i) av[i][h] = *reinterpret_cast<           \
+          const float4*>(&As[buf][ks][wm0 + i * 32 + l32][h * 8 + lhi * 4]);                 \
+      _Pragma("unroll") for (int j = 0; j < TN; ++j) bv[j][h] = *reinterpret_cast<           \
+          const float4*>(&Bs[buf][ks][wn0 + j * 32 + l32][h * 8 + lhi * 4]);                 \
     }                                                                                        \
     _Pragma("unroll") for (int h = 0; h < 2; ++h) {                                          \
       _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                        \
@@ -585,32 +588,36 @@ __global__ void pack_weights_kernel(const float* __restrict__ w, float* __restri
 
 struct TileConfig {
   int bm, bn;
+  int ks;  // 16-row K tiles per stage
   const char* name;
   void (*kernel[3])(const IgemmBatch);  // indexed by kModeMasks / kModeOneMask / kModePointwise
 };
 
 const TileConfig kConfigs[] = {
-    {128, 128, "igemm_f32_128x128",
-     {igemm_kernel<128, 128, 2, 2, 3, kModeMasks>, igemm_kernel<128, 128, 2, 2, 3, kModeOneMask>,
-      igemm_kernel<128, 128, 2, 2, 3, kModePointwise>}},
-    {128, 64, "igemm_f32_128x64",
-     {igemm_kernel<128, 64, 2, 2, 4, kModeMasks>, igemm_kernel<128, 64, 2, 2, 4, kModeOneMask>,
-      igemm_kernel<128, 64, 2, 2, 4, kModePointwise>}},
-    {64, 128, "igemm_f32_64x128",
-     {igemm_kernel<64, 128, 2, 2, 5, kModeMasks>, igemm_kernel<64, 128, 2, 2, 5, kModeOneMask>,
-      igemm_kernel<64, 128, 2, 2, 5, kModePointwise>}},
-    {64, 64, "igemm_f32_64x64",
-     {igemm_kernel<64, 64, 2, 2, 8, kModeMasks>, igemm_kernel<64, 64, 2, 2, 8, kModeOneMask>,
-      igemm_kernel<64, 64, 2, 2, 8, kModePointwise>}},
-    {32, 128, "igemm_f32_32x128",
-     {igemm_kernel<32, 128, 1, 4, 4, kModeMasks>, igemm_kernel<32, 128, 1, 4, 4, kModeOneMask>,
-      igemm_kernel<32, 128, 1, 4, 4, kModePointwise>}},
-    {32, 256, "igemm_f32_32x256",
-     {igemm_kernel<32, 256, 1, 4, 3, kModeMasks>, igemm_kernel<32, 256, 1, 4, 3, kModeOneMask>,
-      igemm_kernel<32, 256, 1, 4, 3, kModePointwise>}},
-    {64, 256, "igemm_f32_64x256",
-     {igemm_kernel<64, 256, 1, 4, 2, kModeMasks>, igemm_kernel<64, 256, 1, 4, 2, kModeOneMask>,
-      igemm_kernel<64, 256, 1, 4, 2, kModePointwise>}},
+    {128, 128, 1, "igemm_f32_128x128",
+     {igemm_kernel<128, 128, 2, 2, 3, kModeMasks, 1>, igemm_kernel<128, 128, 2, 2, 3, kModeOneMask, 1>,
+      igemm_kernel<128, 128, 2, 2, 3, kModePointwise, 1>}},
+    {128, 64, 1, "igemm_f32_128x64",
+     {igemm_kernel<128, 64, 2, 2, 4, kModeMasks, 1>, igemm_kernel<128, 64, 2, 2, 4, kModeOneMask, 1>,
+      igemm_kernel<128, 64, 2, 2, 4, kModePointwise, 1>}},
+    {64, 128, 1, "igemm_f32_64x128",
+     {igemm_kernel<64, 128, 2, 2, 5, kModeMasks, 1>, igemm_kernel<64, 128, 2, 2, 5, kModeOneMask, 1>,
+      igemm_kernel<64, 128, 2, 2, 5, kModePointwise, 1>}},
+    {64, 64, 1, "igemm_f32_64x64",
+     {igemm_kernel<64, 64, 2, 2, 8, kModeMasks, 1>, igemm_kernel<64, 64, 2, 2, 8, kModeOneMask, 1>,
+      igemm_kernel<64, 64, 2, 2, 8, kModePointwise, 1>}},
+    {32, 128, 1, "igemm_f32_32x128",
+     {igemm_kernel<32, 128, 1, 4, 4, kModeMasks, 1>, igemm_kernel<32, 128, 1, 4, 4, kModeOneMask, 1>,
+      igemm_kernel<32, 128, 1, 4, 4, kModePointwise, 1>}},
+    {32, 256, 1, "igemm_f32_32x256",
+     {igemm_kernel<32, 256, 1, 4, 3, kModeMasks, 1>, igemm_kernel<32, 256, 1, 4, 3, kModeOneMask, 1>,
+      igemm_kernel<32, 256, 1, 4, 3, kModePointwise, 1>}},
+    {64, 256, 1, "igemm_f32_64x256",
+     {igemm_kernel<64, 256, 1, 4, 2, kModeMasks, 1>, igemm_kernel<64, 256, 1, 4, 2, kModeOneMask, 1>,
+      igemm_kernel<64, 256, 1, 4, 2, kModePointwise, 1>}},
+    {64, 64, 2, "igemm_f32_64x64x32",
+     {igemm_kernel<64, 64, 2, 2, 4, kModeMasks, 2>, igemm_kernel<64, 64, 2, 2, 4, kModeOneMask, 2>,
+      igemm_kernel<64, 64, 2, 2, 4, kModePointwise, 2>}},
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 
@@ -871,7 +878,7 @@ int mcConvPlanCreate(const mcConvGeom* gp, mcConvPlan** out) {
   }
 
   for (auto& s : plan->subs) {
-    s.Kpad = ceil_div(s.K, BK) * BK;
+    s.Kpad = ceil_div(s.K, 2 * BK) * 2 * BK;  // whole stages for every configuration
     // Padding rows multiply zero weights; row-tap index 31 is out of the image
     // for every pixel, so nothing is fetched for them.
     while (static_cast<int>(s.ktab.size()) < s.Kpad) s.ktab.push_back(make_int4(0, 31, 0, 31));
@@ -1035,7 +1042,7 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
   for (const SubProblem* s : live) {
     const long pixels = (long)num * s->Hq * s->Wq;
     total_blocks += (long)MT * ceil_div(pixels, cfg.bn) * g.group;
-    if (s->Kpad > 0) min_kt = std::min(min_kt, s->Kpad / BK);
+    if (s->Kpad > 0) min_kt = std::min(min_kt, s->Kpad / (BK * cfg.ks));
     pointwise = pointwise && s->pointwise;
     one_mask = one_mask && s->one_mask;
     flops += 2.0 * pixels * plan->M * g.group * s->K;
@@ -1123,7 +1130,7 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
       max_blocks = std::max(max_blocks, blocks);
       // every slice gets the same number of K tiles; slices past the last tile
       // of a short sub-problem write zeros
-      a.kt_per_split = ceil_div(std::max(s.Kpad / BK, 1), slices);
+      a.kt_per_split = ceil_div(std::max(s.Kpad / (BK * cfg.ks), 1), slices);
       a.split_stride = 0;
       if (slices > 1) {
         a.y = ws;
