@@ -1,0 +1,163 @@
+// Direct depthwise convolution (group == input channels): each output channel
+// reads one input channel through kh*kw taps, 2*kh*kw FLOP per 4-byte output, so
+// the layer is bound by HBM, not by the matrix pipe, and gains nothing from the
+// implicit-GEMM kernel (whose tiles would hold one useful row).  It replaces the
+// reference's per-group im2col + sgemm for such layers
+// (base_conv_layer.cpp:254-271 with group == channels) and corresponds to its
+// ConvolutionDepthwise kernel (conv_dw_layer.cu:8-72): taps are accumulated in
+// (kh, kw) order.
+//
+// One thread per output element, neighbouring threads along the output row, so
+// loads and stores are coalesced and the kh*kw overlapping reads of neighbouring
+// outputs are served by L1/L2.  A workgroup covers 256 consecutive outputs of the
+// flattened [num*Cout][Ho*Wo] array; the per-channel filter is read with plain
+// loads (same address across most of a wavefront).
+#include "conv_internal.h"
+#include "mc_common.h"
+#include "mchip/kernels.h"
+
+namespace mchip {
+namespace {
+
+__device__ __forceinline__ float dw_act(float v, int act, float slope) {
+  switch (act) {
+    case MC_ACT_RELU:
+      return v > 0.f ? v : v * slope;
+    case MC_ACT_TANH:
+      return static_cast<float>(tanh(static_cast<double>(v)));
+    case MC_ACT_SIGMOID:
+      return static_cast<float>(1. / (1. + exp(-static_cast<double>(v))));
+    default:
+      return v;
+  }
+}
+
+// KH/KW > 0: compile-time taps (fully unrolled); 0: run-time extents.
+template <int KH, int KW>
+__global__ __launch_bounds__(256) void depthwise_kernel(const DepthwiseArgs a, long count) {
+  const int kh_n = KH ? KH : a.kh, kw_n = KW ? KW : a.kw;
+  const int plane = a.Ho * a.Wo;
+  for (long i = blockIdx.x * 256L + threadIdx.x; i < count; i += gridDim.x * 256L) {
+    const unsigned iu = static_cast<unsigned>(i);    // count < 2^31: 32-bit divisions
+    const unsigned row = iu / static_cast<unsigned>(a.Wo);
+    const int wo = static_cast<int>(iu - row * a.Wo);
+    const unsigned nc = iu / static_cast<unsigned>(plane);  // n * Cout + oc
+    const int ho = static_cast<int>(row - nc * a.Ho);
+    const unsigned cout = static_cast<unsigned>(a.C * a.mult);
+    const long n = nc / cout;
+    const int oc = static_cast<int>(nc - static_cast<unsigned>(n) * cout);
+    const int c = oc / a.mult;
+    const float* __restrict__ xp = a.x + (n * a.C + c) * a.H * a.W;
+    const float* __restrict__ wp = a.w + static_cast<long>(oc) * kh_n * kw_n;
+    const int hi0 = ho * a.sh - a.ph, wi0 = wo * a.sw - a.pw;
+    float acc = 0.f;
+#pragma unroll
+    for (int r = 0; r < kh_n; ++r) {
+      const int hi = hi0 + r * a.dh;
+      const bool row_ok = static_cast<unsigned>(hi) < static_cast<unsigned>(a.H);
+#pragma unroll
+      for (int s = 0; s < kw_n; ++s) {
+        const int wi = wi0 + s * a.dw;
+        const bool ok = row_ok && static_cast<unsigned>(wi) < static_cast<unsigned>(a.W);
+        const float v = ok ? xp[hi * a.W + wi] : 0.f;
+        acc += wp[r * kw_n + s] * v;
+      }
+    }
+    if (a.scale) acc *= a.scale[oc];
+    if (a.shift) acc += a.shift[oc];
+    if (a.residual) acc += a.residual[i];
+    a.y[i] = dw_act(acc, a.act, a.slope);
+  }
+}
+
+// Undilated kernels with stride SH down the column: a thread makes four
+// vertically neighbouring outputs (same column, rows 4*q .. 4*q+3) from
+// 3*SH + KH input rows, so overlapping taps are read once per thread instead of
+// once per output and the index arithmetic is shared; neighbouring threads sit on
+// neighbouring columns, so every load and store stays coalesced.
+template <int KH, int KW, int SH>
+__global__ __launch_bounds__(256) void depthwise4_kernel(const DepthwiseArgs a, long groups,
+                                                         int ho_groups) {
+  constexpr int L = 3 * SH + KH;
+  for (long gi = blockIdx.x * 256L + threadIdx.x; gi < groups; gi += gridDim.x * 256L) {
+    const unsigned gu = static_cast<unsigned>(gi);   // groups < 2^31
+    const unsigned row = gu / static_cast<unsigned>(a.Wo);        // (n*Cout + oc)*ho_groups + q
+    const int wo = static_cast<int>(gu - row * a.Wo);
+    const unsigned nc = row / static_cast<unsigned>(ho_groups);
+    const int ho0 = static_cast<int>(row - nc * ho_groups) * 4;
+    const unsigned cout = static_cast<unsigned>(a.C * a.mult);
+    const unsigned n = nc / cout;
+    const int oc = static_cast<int>(nc - n * cout);
+    const int c = oc / a.mult;
+    const float* __restrict__ xp = a.x + (static_cast<long>(n) * a.C + c) * a.H * a.W;
+    const float* __restrict__ wp = a.w + static_cast<long>(oc) * KH * KW;
+    const int hi0 = ho0 * SH - a.ph, wi0 = wo * a.sw - a.pw;
+    float wv[KH][KW];
+#pragma unroll
+    for (int r = 0; r < KH; ++r)
+#pragma unroll
+      for (int s = 0; s < KW; ++s) wv[r][s] = wp[r * KW + s];
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < L; ++t) {
+      const int hi = hi0 + t;
+      const bool row_ok = static_cast<unsigned>(hi) < static_cast<unsigned>(a.H);
+      float v[KW];
+#pragma unroll
+      for (int s = 0; s < KW; ++s) {
+        const int wi = wi0 + s;
+        const bool ok = row_ok && static_cast<unsigned>(wi) < static_cast<unsigned>(a.W);
+        v[s] = ok ? xp[hi * a.W + wi] : 0.f;
+      }
+      // input row t is tap row t - o*SH of output o
+#pragma unroll
+      for (int o = 0; o < 4; ++o) {
+        const int r = t - o * SH;
+        if (r >= 0 && r < KH) {
+#pragma unroll
+          for (int s = 0; s < KW; ++s) acc[o] += wv[r][s] * v[s];
+        }
+      }
+    }
+    const float sc = a.scale ? a.scale[oc] : 1.f, sf = a.shift ? a.shift[oc] : 0.f;
+#pragma unroll
+    for (int o = 0; o < 4; ++o) {
+      if (ho0 + o >= a.Ho) break;
+      const long out = (static_cast<long>(nc) * a.Ho + ho0 + o) * a.Wo + wo;
+      float val = acc[o];
+      if (a.scale) val *= sc;
+      if (a.shift) val += sf;
+      if (a.residual) val += a.residual[out];
+      a.y[out] = dw_act(val, a.act, a.slope);
+    }
+  }
+}
+
+}  // namespace
+
+int depthwise_forward(const DepthwiseArgs& a, hipStream_t stream) {
+  const long count = static_cast<long>(a.num) * a.C * a.mult * a.Ho * a.Wo;
+  if (count == 0) return 0;
+  if (a.kh == 3 && a.kw == 3 && a.dh == 1 && a.dw == 1 && (a.sh == 1 || a.sh == 2)) {
+    const int ho_groups = ceil_div(a.Ho, 4);
+    const long groups = static_cast<long>(a.num) * a.C * a.mult * ho_groups * a.Wo;
+    const unsigned gb = ew_blocks(groups, 256);
+    if (a.sh == 1)
+      depthwise4_kernel<3, 3, 1><<<gb, 256, 0, stream>>>(a, groups, ho_groups);
+    else
+      depthwise4_kernel<3, 3, 2><<<gb, 256, 0, stream>>>(a, groups, ho_groups);
+    MC_LAUNCH_CHECK();
+    return 0;
+  }
+  const unsigned blocks = ew_blocks(count, 256);
+  if (a.kh == 3 && a.kw == 3)
+    depthwise_kernel<3, 3><<<blocks, 256, 0, stream>>>(a, count);
+  else if (a.kh == 5 && a.kw == 5)
+    depthwise_kernel<5, 5><<<blocks, 256, 0, stream>>>(a, count);
+  else
+    depthwise_kernel<0, 0><<<blocks, 256, 0, stream>>>(a, count);
+  MC_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace mchip

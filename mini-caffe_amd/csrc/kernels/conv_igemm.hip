@@ -22,6 +22,7 @@
 // 32x32 accumulators fed by v_mfma_f32_32x32x2_f32.  Filters are repacked once
 // into K-major, zero-padded [g][Kpad][Mpad] so that A-tile loads are aligned
 // float4 rows and need no predicates.
+#include "conv_internal.h"
 #include "mc_common.h"
 #include "mchip/kernels.h"
 
@@ -658,6 +659,9 @@ struct mcConvPlan {
   int forced_config = -1;
   int forced_split = 0;  // 0 = choose, >= 1 = this many K slices
   bool force_general = false;  // use the tap-table gather even for pointwise geometry
+  // group == input channels: a direct kernel reads the layer's own filter layout
+  bool depthwise = false;
+  float* dw_weights = nullptr;  // copy of the [Cout, 1, kh, kw] filter blob
   std::vector<SubProblem> subs;
 };
 
@@ -806,6 +810,17 @@ int mcConvPlanCreate(const mcConvGeom* gp, mcConvPlan** out) {
   }
   plan->M = g.channels_out / g.group;
   plan->Cin_g = g.channels_in / g.group;
+  if (!g.transposed && g.group > 1 && g.group == g.channels_in) {
+    plan->depthwise = true;
+    const hipError_t e =
+        hipMalloc(&plan->dw_weights, sizeof(float) * (size_t)g.channels_out * g.kernel_h * g.kernel_w);
+    if (e != hipSuccess) {
+      delete plan;
+      return fail("mcConvPlanCreate: device set-up failed: %s", hipGetErrorString(e));
+    }
+    *out = plan;
+    return 0;
+  }
   plan->Mpad = ceil_div(plan->M, 128) * 128;
   const int HW = g.height_in * g.width_in;
   const int khkw = g.kernel_h * g.kernel_w;
@@ -965,6 +980,7 @@ int mcInnerProductPlanCreate(int K, int N, int transpose, mcConvPlan** out) {
 
 int mcConvPlanDestroy(mcConvPlan* plan) {
   if (!plan) return 0;
+  if (plan->dw_weights) (void)hipFree(plan->dw_weights);
   for (auto& s : plan->subs) free_sub(s);
   delete plan;
   return 0;
@@ -980,6 +996,13 @@ int mcConvPlanOutputShape(const mcConvPlan* plan, int* ho, int* wo) {
 int mcConvPlanSetWeights(mcConvPlan* plan, const float* weights, void* stream) {
   MC_REQUIRE(plan && weights, "mcConvPlanSetWeights: null argument");
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (plan->depthwise) {
+    const mcConvGeom& g = plan->geom;
+    MC_HIP(hipMemcpyAsync(plan->dw_weights, weights,
+                          sizeof(float) * (size_t)g.channels_out * g.kernel_h * g.kernel_w,
+                          hipMemcpyDeviceToDevice, st));
+    return 0;
+  }
   for (auto& s : plan->subs) {
     if (s.Kpad == 0) continue;
     const long total = (long)plan->geom.group * s.Kpad * plan->Mpad;
@@ -1020,6 +1043,28 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
   MC_REQUIRE(in_count < (1L << 29) && out_count < (1L << 29),
              "mcConvForward: blob exceeds 2^29 elements");
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (plan->depthwise) {
+    DepthwiseArgs d = {bottom, plan->dw_weights, top, ep ? ep->scale : nullptr,
+                       ep ? ep->shift : nullptr, ep ? ep->residual : nullptr, num,
+                       g.channels_in, plan->M, g.height_in, g.width_in, plan->Ho, plan->Wo,
+                       g.kernel_h, g.kernel_w, g.stride_h, g.stride_w, g.pad_h, g.pad_w,
+                       g.dilation_h, g.dilation_w, ep ? ep->activation : MC_ACT_NONE,
+                       ep ? ep->negative_slope : 0.f};
+    TimedLaunch tl;
+    if (g_timing) {
+      MC_HIP(hipEventCreate(&tl.start));
+      MC_HIP(hipEventCreate(&tl.stop));
+      tl.flops = mcConvPlanFlops(plan, num);
+      tl.name = "depthwise_f32";
+      MC_HIP(hipEventRecord(tl.start, st));
+    }
+    if (depthwise_forward(d, st)) return -1;
+    if (g_timing) {
+      MC_HIP(hipEventRecord(tl.stop, st));
+      g_timed.push_back(tl);
+    }
+    return 0;
+  }
 
   // Sub-problems that have pixels at this batch size, their tile configuration
   // (one for the whole plan: the largest sub-problem decides) and K slices.
@@ -1191,6 +1236,7 @@ double mcConvPlanFlops(const mcConvPlan* plan, int num) {
 }
 
 const char* mcConvPlanKernelName(const mcConvPlan* plan, int num) {
+  if (plan && plan->depthwise) return "depthwise_f32";
   if (!plan || plan->subs.empty()) return "";
   const auto& s = plan->subs[0];
   return kConfigs[pick_config(plan, (long)num * s.Hq * s.Wq)].name;

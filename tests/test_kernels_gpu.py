@@ -52,6 +52,10 @@ CONV_CASES = [
     (8, 6, 6, 12, 2, 3, 0, 1, 1, True, 2),          # kernel < stride: tapless output classes
     (8, 6, 6, 12, 5, 2, 2, 1, 2, True, 2),          # grouped deconv
     (8, 6, 6, 12, 3, 2, 1, 2, 1, True, 2),          # dilated deconv
+    (32, 28, 28, 32, 3, 1, 1, 1, 32, False, 3),     # depthwise 3x3 (MobileNet): direct kernel
+    (32, 29, 27, 32, 3, 2, 1, 1, 32, False, 2),     # depthwise, stride 2, odd extents
+    (16, 12, 12, 32, 5, 1, 2, 1, 16, False, 2),     # depthwise 5x5 with channel multiplier 2
+    (16, 12, 12, 16, 3, 1, 2, 2, 16, False, 2),     # depthwise, dilated
 ]
 
 
@@ -193,6 +197,25 @@ def test_conv_epilogue_activations_full_channel_blocks(K, act, slope):
     code = {"none": K.ACT_NONE, "relu": K.ACT_RELU, "tanh": K.ACT_TANH, "sigmoid": K.ACT_SIGMOID}[act]
     plan = K.ConvPlan(K.conv_geom(cin, h, h, cout, 3, 1, 1))
     got = _run_plan(K, plan, n, x, wt, want.shape, shift=b, activation=code, negative_slope=slope)
+    assert netrun.rel_err(got, want) < 1e-4
+
+
+def test_depthwise_with_epilogue(K):
+    """group == channels takes the direct kernel; scale, shift, residual and ReLU as for the
+    implicit-GEMM path."""
+    rng = np.random.default_rng(6)
+    n, c, h = 3, 48, 19
+    x = rng.standard_normal((n, c, h, h)).astype(np.float32)
+    wt = (rng.standard_normal((c, 1, 3, 3)) * 0.3).astype(np.float32)
+    sc = (rng.random(c) + 0.5).astype(np.float32)
+    sh = rng.standard_normal(c).astype(np.float32)
+    y = oracle.conv_forward(oracle.conv_geom(c, h, h, c, 3, 1, 1, 1, c), x, wt, None)
+    res = rng.standard_normal(y.shape).astype(np.float32)
+    want = oracle.relu(oracle.eltwise([oracle.scale(y, sc, sh), res], "SUM"), 0.1)
+    plan = K.ConvPlan(K.conv_geom(c, h, h, c, 3, 1, 1, 1, c))
+    assert plan.kernel_name(n) == "depthwise_f32"
+    got = _run_plan(K, plan, n, x, wt, want.shape, scale=sc, shift=sh, residual=res,
+                    activation=K.ACT_RELU, negative_slope=0.1)
     assert netrun.rel_err(got, want) < 1e-4
 
 
