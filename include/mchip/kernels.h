@@ -300,6 +300,86 @@ int mcPSROIPooling(const float* bottom, int num, int output_dim, int group_size,
                    int width, const float* rois, int num_rois, float spatial_scale, float* top,
                    int* bad_roi_flag, void* stream);
 
+/* ---- further layers of the model zoo ------------------------------------------ */
+
+/* Elementwise functions with up to three scalar parameters; bottom == top allowed.
+ *   MC_UNARY_POWER      (p1 + p0*x)^p2           power_layer.cpp:17-40, .cu:8-29
+ *   MC_UNARY_EXP        p1 * exp(p0*x)           exp_layer.cpp:31-45  (p0 = log(base)*scale,
+ *                                                p1 = base^shift, both folded by the caller)
+ *   MC_UNARY_LOG        p2 * log(p1 + p0*x)      log_layer.cpp:35-54  (p2 = 1/log(base))
+ *   MC_UNARY_ABS        |x|                      absval_layer.cpp:8-13
+ *   MC_UNARY_BNLL       log(1 + exp(x))          bnll_layer.cpp:8-18
+ *   MC_UNARY_ELU        max(x,0)+p0*(exp(min(x,0))-1)   elu_layer.cpp:8-18
+ *   MC_UNARY_THRESHOLD  x > p0 ? 1 : 0           threshold_layer.cpp:13-21 */
+enum mcUnaryOp {
+  MC_UNARY_POWER = 0,
+  MC_UNARY_EXP = 1,
+  MC_UNARY_LOG = 2,
+  MC_UNARY_ABS = 3,
+  MC_UNARY_BNLL = 4,
+  MC_UNARY_ELU = 5,
+  MC_UNARY_THRESHOLD = 6
+};
+int mcUnary(int op, const float* bottom, float* top, long count, float p0, float p1, float p2,
+            void* stream);
+
+/* PReLULayer::Forward (prelu_layer.cpp:50-84; .cu:9-33): max(x,0) + slope[c]*min(x,0)
+ * with c the index on the `channels` axis of a [outer, channels, inner] view, or 0
+ * when channel_shared.  bottom == top allowed. */
+int mcPReLU(const float* bottom, float* top, int outer, int channels, int inner,
+            const float* slope, int channel_shared, void* stream);
+
+/* LRNLayer::CrossChannelForward (lrn_layer.cpp:112-155; .cu:9-94):
+ * top = bottom * (k + alpha/local_size * sum of squares over local_size neighbouring
+ * channels)^-beta, the window centred on the channel and clipped to the blob. */
+int mcLRNAcrossChannels(const float* bottom, float* top, int num, int channels, int height,
+                        int width, int local_size, float alpha, float beta, float k,
+                        void* stream);
+
+/* LRNLayer::WithinChannelForward (lrn_layer.cpp:20-66,157-164: Split -> Power(2) ->
+ * average Pooling(local_size, pad (local_size-1)/2) -> Power(1 + alpha*., -beta) ->
+ * Eltwise PROD) as one pass over `planes` maps of height x width. */
+int mcLRNWithinChannel(const float* bottom, float* top, long planes, int height, int width,
+                       int local_size, float alpha, float beta, void* stream);
+
+/* ArgMaxLayer::Forward_cpu (argmax_layer.cpp:56-93; the reference has no device
+ * version): the top_k largest of the `dim` values of every line of a
+ * [outer, dim, inner] view, in the order of std::greater on (value, index) pairs —
+ * among equal values the larger index comes first.  Indices are stored as floats.
+ *   MC_ARGMAX_INDEX             top[outer, top_k, inner] = index
+ *   MC_ARGMAX_VALUE             top[outer, top_k, inner] = value
+ *   MC_ARGMAX_INDEX_THEN_VALUE  top[outer, 2, top_k] = indices then values (inner == 1) */
+enum mcArgMaxLayout { MC_ARGMAX_INDEX = 0, MC_ARGMAX_VALUE = 1, MC_ARGMAX_INDEX_THEN_VALUE = 2 };
+int mcArgMax(const float* bottom, float* top, long outer, int dim, int inner, int top_k,
+             int layout, void* stream);
+
+/* ReductionLayer::Forward (reduction_layer.cpp:38-72; .cu:8-40): top[i] = coeff *
+ * reduce(bottom[i, 0:dim]); MEAN divides by dim.  Values as in ReductionParameter. */
+enum mcReduceOp { MC_REDUCE_SUM = 1, MC_REDUCE_ASUM = 2, MC_REDUCE_SUMSQ = 3, MC_REDUCE_MEAN = 4 };
+int mcReduction(int op, const float* bottom, float* top, int num, int dim, float coeff,
+                void* stream);
+
+/* MVNLayer::Forward (mvn_layer.cpp:36-75; .cu:8-49): per row of a [num, dim] view,
+ * x - mean, divided by sqrt(mean((x-mean)^2)) + eps when normalize_variance. */
+int mcMVN(const float* bottom, float* top, int num, int dim, int normalize_variance, float eps,
+          void* stream);
+
+/* top[r, :] = table[(int)rows[r], :] (+ bias).  EmbedLayer::Forward
+ * (embed_layer.cpp:62-79; .cu:9-35) with the row numbers held as floats, and the
+ * row copy of FilterLayer::Forward (filter_layer.cpp:61-75).  A row number outside
+ * [0, table_rows) (a DCHECK in the reference) yields NaN. */
+int mcGatherRows(const float* table, int table_rows, int row_len, const float* rows, long num_rows,
+                 const float* bias, float* top, void* stream);
+
+/* CropLayer::Forward (crop_layer.cpp:61-107; .cu:11-80): top = the box of shape
+ * top_shape at `offsets` inside bottom; up to MC_MAX_AXES axes. */
+#define MC_MAX_AXES 8
+int mcCrop(const float* bottom, float* top, int num_axes, const int* bottom_shape,
+           const int* top_shape, const int* offsets, void* stream);
+
+/* TileLayer::Forward (tile_layer.cpp:24-35; .cu:9-29): [outer, inner] -> [outer, tiles, inner]. */
+int mcTile(const float* bottom, float* top, long outer, int inner, int tiles, void* stream);
+
 /* Fill `count` floats with `value` (caffe_gpu_set, math_functions.cu:70-82). */
 int mcFill(float* dst, long count, float value, void* stream);
 

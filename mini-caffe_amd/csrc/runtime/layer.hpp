@@ -189,6 +189,32 @@ class LayerRegisterer {
   }                                                                         \
   REGISTER_LAYER_CREATOR(type, Creator_##type##Layer)
 
+// Every filler type fills with FillerParameter.value (default 0), as in the
+// reference (src/filler.hpp:28-71).
+inline void FillConstant(const Message& filler, Blob* blob, double default_value = 0.) {
+  const string type = filler.get_string("type", "constant");
+  static const char* kKnown[] = {"constant", "gaussian", "positive_unitball", "uniform",
+                                 "xavier",   "msra",     "bilinear"};
+  bool known = false;
+  for (const char* k : kKnown) known = known || type == k;
+  CHECK(known) << "Unknown filler name: " << type;
+  const real_t value = static_cast<real_t>(filler.get_float("value", default_value));
+  real_t* data = blob->mutable_cpu_data();
+  for (int i = 0; i < blob->count(); ++i) data[i] = value;
+}
+
+// Changes whenever the blob's memory may have been written.
+inline uint64_t BlobVersion(const shared_ptr<Blob>& b) {
+  return b && b->data() ? b->data()->version() : 0;
+}
+
+// Device-to-device copy of a whole blob on the calling thread's stream.
+inline void DeviceCopy(const Blob& src, Blob* dst) {
+  if (src.count() == 0) return;
+  MC_CHECK(mcCopy2D(src.gpu_data(), src.count(), dst->mutable_gpu_data(), src.count(),
+                    src.count(), 1, Context::Get().stream()));
+}
+
 // Stream of the calling thread, as the void* the kernel ABI takes.
 inline void* cur_stream() { return Context::Get().stream(); }
 

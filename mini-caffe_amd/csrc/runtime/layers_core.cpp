@@ -11,26 +11,6 @@
 
 namespace caffe {
 
-namespace {
-
-// Every filler type fills with FillerParameter.value (default 0), as in the
-// reference (src/filler.hpp:28-71).
-void FillConstant(const Message& filler, Blob* blob) {
-  const string type = filler.get_string("type", "constant");
-  static const char* kKnown[] = {"constant", "gaussian", "positive_unitball", "uniform",
-                                 "xavier",   "msra",     "bilinear"};
-  bool known = false;
-  for (const char* k : kKnown) known = known || type == k;
-  CHECK(known) << "Unknown filler name: " << type;
-  const real_t value = static_cast<real_t>(filler.get_float("value", 0.));
-  real_t* data = blob->mutable_cpu_data();
-  for (int i = 0; i < blob->count(); ++i) data[i] = value;
-}
-
-uint64_t BlobVersion(const shared_ptr<Blob>& b) { return b && b->data() ? b->data()->version() : 0; }
-
-}  // namespace
-
 // ---------------------------------------------------------------------------
 // Input (reference src/layers/input_layer.cpp:7-21)
 // ---------------------------------------------------------------------------
@@ -218,9 +198,15 @@ class BaseConvolutionLayer : public ContractionLayer {
       geom_.dilation_w = n == 0 ? 1 : static_cast<int>(p.get_int("dilation", 1, n == 1 ? 0 : 1));
     }
     geom_.channels_in = bottom[0]->shape(1);
-    geom_.channels_out = static_cast<int>(p.get_int("num_output", 0));
-    CHECK_GT(geom_.channels_out, 0);
-    geom_.group = static_cast<int>(p.get_int("group", 1));
+    if (depthwise()) {
+      // One filter per input channel whatever num_output and group say.
+      geom_.channels_out = geom_.channels_in;
+      geom_.group = geom_.channels_in;
+    } else {
+      geom_.channels_out = static_cast<int>(p.get_int("num_output", 0));
+      CHECK_GT(geom_.channels_out, 0);
+      geom_.group = static_cast<int>(p.get_int("group", 1));
+    }
     CHECK_EQ(geom_.channels_in % geom_.group, 0);
     CHECK_EQ(geom_.channels_out % geom_.group, 0) << "Number of output should be multiples of group.";
     geom_.transposed = transposed() ? 1 : 0;
@@ -281,6 +267,7 @@ class BaseConvolutionLayer : public ContractionLayer {
 
  protected:
   virtual bool transposed() const = 0;
+  virtual bool depthwise() const { return false; }
 
   void Forward_gpu(const vector<Blob*>& bottom, const vector<Blob*>& top) override {
     if (!plan_ || plan_h_ != geom_.height_in || plan_w_ != geom_.width_in) {
@@ -324,6 +311,20 @@ class DeconvolutionLayer : public BaseConvolutionLayer {
   bool transposed() const override { return true; }
 };
 REGISTER_LAYER_CLASS(Deconvolution);
+
+// ConvolutionDepthwise (reference src/layers/conv_dw_layer.cpp:9-158; .cu:9-72):
+// reads convolution_param, filter blob [channels, 1, kernel_h, kernel_w], output
+// channels = input channels.  Runs on the convolution plan's depthwise kernel.
+class ConvolutionDepthwiseLayer : public BaseConvolutionLayer {
+ public:
+  explicit ConvolutionDepthwiseLayer(const LayerParameter& param) : BaseConvolutionLayer(param) {}
+  const char* type() const override { return "ConvolutionDepthwise"; }
+
+ protected:
+  bool transposed() const override { return false; }
+  bool depthwise() const override { return true; }
+};
+REGISTER_LAYER_CLASS(ConvolutionDepthwise);
 
 // ---------------------------------------------------------------------------
 // InnerProduct (reference src/layers/inner_product_layer.cpp:9-99; .cu:9-31)
@@ -477,6 +478,76 @@ class BatchNormLayer : public Layer {
   uint64_t stats_version_ = ~0ull;
 };
 REGISTER_LAYER_CLASS(BatchNorm);
+
+// ---------------------------------------------------------------------------
+// BN (reference src/layers/bn_layer.cpp:14-147; .cu:9-80): the frozen, fused form
+// top = (x - blobs[2][c]) * blobs[3][c] * blobs[0][c] + blobs[1][c]; blobs[3]
+// holds the multiplier itself (the reference never takes a root of it).
+// ---------------------------------------------------------------------------
+class BNLayer : public Layer {
+ public:
+  explicit BNLayer(const LayerParameter& param) : Layer(param) {}
+  const char* type() const override { return "BN"; }
+  int ExactNumBottomBlobs() const override { return 1; }
+  int ExactNumTopBlobs() const override { return 1; }
+
+  void LayerSetUp(const vector<Blob*>& bottom, const vector<Blob*>& top) override {
+    const Message& p = layer_param_.sub("bn_param");
+    CHECK_GE(bottom[0]->num_axes(), 2) << "BN needs a channel axis";
+    channels_ = bottom[0]->shape(1);
+    if (blobs_.empty()) {
+      blobs_.resize(4);
+      for (auto& b : blobs_) b.reset(new Blob(vector<int>{1, channels_}));
+      FillConstant(p.sub("slope_filler"), blobs_[0].get());
+      FillConstant(p.sub("bias_filler"), blobs_[1].get());
+      Message zero, one;
+      one.set("value", "1");
+      FillConstant(zero, blobs_[2].get());
+      FillConstant(one, blobs_[3].get());
+    } else {
+      CHECK_EQ(blobs_.size(), 4u) << "BN takes 4 parameter blobs (slope, bias, mean, multiplier)";
+      for (auto& b : blobs_) CHECK_EQ(b->count(), channels_) << "BN parameter size mismatch";
+    }
+  }
+  void Reshape(const vector<Blob*>& bottom, const vector<Blob*>& top) override {
+    CHECK_EQ(bottom[0]->shape(1), channels_);
+    top[0]->ReshapeLike(*bottom[0]);
+    scale_.Reshape(vector<int>{channels_});
+  }
+
+  bool IsChannelStage(int channels) const override { return channels == channels_; }
+  uint64_t ChannelStageVersion() const override {
+    uint64_t v = 0;
+    for (auto& b : blobs_) v = v * 31 + BlobVersion(b);
+    return v;
+  }
+  void GetChannelStage(mcChannelOp* op) override {
+    const uint64_t v = ChannelStageVersion();
+    if (v != scale_version_) {
+      const float* both[2] = {blobs_[3]->gpu_data(), blobs_[0]->gpu_data()};
+      MC_CHECK(mcEltwise(MC_ELT_PROD, 2, both, nullptr, channels_, scale_.mutable_gpu_data(),
+                         MC_ACT_NONE, 0.f, cur_stream()));
+      scale_version_ = v;
+    }
+    op->sub = blobs_[2]->gpu_data();
+    op->mul = scale_.gpu_data();
+    op->add = blobs_[1]->gpu_data();
+  }
+
+ protected:
+  void Forward_gpu(const vector<Blob*>& bottom, const vector<Blob*>& top) override {
+    if (bottom[0]->count() == 0) return;
+    mcChannelOp op = {nullptr, nullptr, nullptr, nullptr, MC_ACT_NONE, 0.f};
+    GetChannelStage(&op);
+    const int num = bottom[0]->shape(0);
+    MC_CHECK(mcChannelTransform(bottom[0]->gpu_data(), top[0]->mutable_gpu_data(), num, channels_,
+                                bottom[0]->count() / (num * channels_), &op, cur_stream()));
+  }
+  int channels_ = 0;
+  Blob scale_;
+  uint64_t scale_version_ = ~0ull;
+};
+REGISTER_LAYER_CLASS(BN);
 
 // ---------------------------------------------------------------------------
 // Scale and Bias (reference src/layers/scale_layer.cpp:10-119, .cu:9-47;

@@ -7,14 +7,6 @@
 
 namespace caffe {
 
-namespace {
-void DeviceCopy(const Blob& src, Blob* dst) {
-  if (src.count() == 0) return;
-  MC_CHECK(mcCopy2D(src.gpu_data(), src.count(), dst->mutable_gpu_data(), src.count(),
-                    src.count(), 1, cur_stream()));
-}
-}  // namespace
-
 // ---------------------------------------------------------------------------
 // Concat (reference src/layers/concat_layer.cpp:8-70; .cu:8-46)
 // ---------------------------------------------------------------------------

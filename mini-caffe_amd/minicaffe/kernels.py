@@ -63,6 +63,19 @@ LIB.mcROIPooling.argtypes = [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_i
                              c_float, c_void_p, c_void_p, c_void_p]
 LIB.mcPSROIPooling.argtypes = [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float,
                                c_void_p, c_void_p, c_void_p]
+LIB.mcUnary.argtypes = [c_int, c_void_p, c_void_p, c_long, c_float, c_float, c_float, c_void_p]
+LIB.mcPReLU.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p]
+LIB.mcLRNAcrossChannels.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
+                                    c_float, c_float, c_void_p]
+LIB.mcLRNWithinChannel.argtypes = [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_float, c_float,
+                                   c_void_p]
+LIB.mcArgMax.argtypes = [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p]
+LIB.mcReduction.argtypes = [c_int, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p]
+LIB.mcMVN.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p]
+LIB.mcGatherRows.argtypes = [c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p]
+LIB.mcCrop.argtypes = [c_void_p, c_void_p, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int),
+                       ctypes.POINTER(c_int), c_void_p]
+LIB.mcTile.argtypes = [c_void_p, c_void_p, c_long, c_int, c_int, c_void_p]
 LIB.mcProposalWorkspaceSize.argtypes = [c_int, c_int, c_int, ctypes.POINTER(ctypes.c_size_t)]
 LIB.mcProposal.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                            c_float, c_int, c_int, c_float, c_void_p, ctypes.c_size_t, c_void_p,

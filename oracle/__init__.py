@@ -480,3 +480,202 @@ def detection_output(param, loc, conf, prior):
         _fp(out), max_rows)
     assert n >= 0, "detection_output: row buffer too small"
     return out[:n].copy()
+
+
+# ---- less common layers (mc_oracle_zoo.c) ------------------------------------------
+
+_I, _F, _Z = ctypes.c_int, ctypes.c_float, ctypes.c_size_t
+_lib.orc_bn.argtypes = [_I, _I, _I] + [c_float_p] * 6
+_lib.orc_conv_dw.argtypes = [_I] * 12 + [c_float_p] * 4
+_lib.orc_power.argtypes = [_Z, c_float_p, _F, _F, _F, c_float_p]
+_lib.orc_exp_layer.argtypes = [_Z, c_float_p, _F, _F, _F, c_float_p]
+_lib.orc_log_layer.argtypes = [_Z, c_float_p, _F, _F, _F, c_float_p]
+_lib.orc_absval.argtypes = [_Z, c_float_p, c_float_p]
+_lib.orc_bnll.argtypes = [_Z, c_float_p, c_float_p]
+_lib.orc_elu.argtypes = [_Z, c_float_p, _F, c_float_p]
+_lib.orc_threshold.argtypes = [_Z, c_float_p, _F, c_float_p]
+_lib.orc_prelu.argtypes = [_I, _I, _I, c_float_p, c_float_p, _I, c_float_p]
+_lib.orc_lrn_across.argtypes = [_I] * 5 + [_F] * 3 + [c_float_p, c_float_p]
+_lib.orc_argmax.argtypes = [_I] * 5 + [c_float_p, c_float_p]
+_lib.orc_reduction.argtypes = [_I, _I, _I, _F, c_float_p, c_float_p]
+_lib.orc_mvn.argtypes = [_I, _I, _I, _F, c_float_p, c_float_p]
+_lib.orc_embed.argtypes = [_I, _I] + [c_float_p] * 4
+_lib.orc_shuffle_channel.argtypes = [_I] * 4 + [c_float_p, c_float_p]
+
+
+def _two(v):
+    return (v, v) if np.isscalar(v) else tuple(v)
+
+
+def bn(x, slope, bias, mean, mult):
+    """BN layer (bn_layer.cpp:77-147): (x - mean) * mult * slope + bias per channel."""
+    x = _f32(x)
+    num, ch = x.shape[0], x.shape[1]
+    y = np.empty_like(x)
+    s, b, m, v = (_f32(a).reshape(-1) for a in (slope, bias, mean, mult))
+    _lib.orc_bn(num, ch, x.size // (num * ch), _fp(x), _fp(s), _fp(b), _fp(m), _fp(v), _fp(y))
+    return y
+
+
+def conv_dw(x, w, bias=None, stride=1, pad=0, dilation=1):
+    """ConvolutionDepthwise (conv_dw_layer.cpp:105-158): x (N,C,H,W), w (C,1,kh,kw)."""
+    x, w = _f32(x), _f32(w)
+    n, c, h, wd = x.shape
+    kh, kw = w.shape[2], w.shape[3]
+    (sh, sw), (ph, pw), (dh, dw) = _two(stride), _two(pad), _two(dilation)
+    ho = (h + 2 * ph - (dh * (kh - 1) + 1)) // sh + 1
+    wo = (wd + 2 * pw - (dw * (kw - 1) + 1)) // sw + 1
+    y = np.empty((n, c, ho, wo), np.float32)
+    b = _f32(bias) if bias is not None else None
+    _lib.orc_conv_dw(n, c, h, wd, kh, kw, sh, sw, ph, pw, dh, dw, _fp(x), _fp(w),
+                     _fp(b) if b is not None else None, _fp(y))
+    return y
+
+
+def power(x, power=1.0, scale=1.0, shift=0.0):
+    x = _f32(x)
+    y = np.empty_like(x)
+    _lib.orc_power(x.size, _fp(x), scale, shift, power, _fp(y))
+    return y
+
+
+def exp_layer(x, base=-1.0, scale=1.0, shift=0.0):
+    x = _f32(x)
+    y = np.empty_like(x)
+    _lib.orc_exp_layer(x.size, _fp(x), base, scale, shift, _fp(y))
+    return y
+
+
+def log_layer(x, base=-1.0, scale=1.0, shift=0.0):
+    x = _f32(x)
+    y = np.empty_like(x)
+    _lib.orc_log_layer(x.size, _fp(x), base, scale, shift, _fp(y))
+    return y
+
+
+def absval(x):
+    x = _f32(x)
+    y = np.empty_like(x)
+    _lib.orc_absval(x.size, _fp(x), _fp(y))
+    return y
+
+
+def bnll(x):
+    x = _f32(x)
+    y = np.empty_like(x)
+    _lib.orc_bnll(x.size, _fp(x), _fp(y))
+    return y
+
+
+def elu(x, alpha=1.0):
+    x = _f32(x)
+    y = np.empty_like(x)
+    _lib.orc_elu(x.size, _fp(x), alpha, _fp(y))
+    return y
+
+
+def threshold(x, threshold=0.0):
+    x = _f32(x)
+    y = np.empty_like(x)
+    _lib.orc_threshold(x.size, _fp(x), threshold, _fp(y))
+    return y
+
+
+def prelu(x, slope, channel_shared=False):
+    x, slope = _f32(x), _f32(slope).reshape(-1)
+    y = np.empty_like(x)
+    num, ch = x.shape[0], x.shape[1]
+    _lib.orc_prelu(num, ch, x.size // max(1, num * ch), _fp(x), _fp(slope), int(channel_shared),
+                   _fp(y))
+    return y
+
+
+def lrn(x, local_size=5, alpha=1.0, beta=0.75, k=1.0, norm_region="ACROSS_CHANNELS"):
+    """LRN (lrn_layer.cpp:112-164).  The within-channel region is the reference's own
+    chain: Power(2) -> average Pooling -> Power(1 + alpha*., -beta) -> Eltwise PROD."""
+    x = _f32(x)
+    if str(norm_region) == "ACROSS_CHANNELS":
+        n, c, h, w = x.shape
+        y = np.empty_like(x)
+        _lib.orc_lrn_across(n, c, h, w, local_size, alpha, beta, k, _fp(x), _fp(y))
+        return y
+    pre_pad = (local_size - 1) // 2
+    sq = power(x, power=2.0)
+    pooled = pooling(sq, "AVE", (local_size, local_size), (1, 1), (pre_pad, pre_pad))
+    denom = power(pooled, power=-beta, scale=alpha, shift=1.0)
+    return eltwise([x, denom], "PROD")
+
+
+def argmax(x, top_k=1, out_max_val=False, axis=None):
+    """ArgMax (argmax_layer.cpp:36-93)."""
+    x = _f32(x)
+    if axis is not None:
+        axis = axis % x.ndim
+        dim = x.shape[axis]
+        dist = int(np.prod(x.shape[axis + 1:]))
+        shape = list(x.shape)
+        shape[axis] = top_k
+        layout = 1 if out_max_val else 0
+    else:
+        dim = int(np.prod(x.shape[1:]))
+        dist = 1
+        shape = [1] * max(3, x.ndim)
+        shape[0], shape[2] = x.shape[0], top_k
+        if out_max_val:
+            shape[1] = 2
+        layout = 2 if out_max_val else 0
+    y = np.empty(shape, np.float32)
+    _lib.orc_argmax(x.size, dim, dist, top_k, layout, _fp(x), _fp(y))
+    return y
+
+
+def reduction(x, operation="SUM", axis=0, coeff=1.0):
+    x = _f32(x)
+    axis = axis % x.ndim if x.ndim else 0
+    num = int(np.prod(x.shape[:axis]))
+    y = np.empty(x.shape[:axis], np.float32)
+    _lib.orc_reduction({"SUM": 1, "ASUM": 2, "SUMSQ": 3, "MEAN": 4}[str(operation)], num,
+                       x.size // max(1, num), coeff, _fp(x), _fp(y))
+    return y
+
+
+def mvn(x, normalize_variance=True, across_channels=False, eps=1e-9):
+    x = _f32(x)
+    x4 = x.reshape(x.shape + (1,) * (4 - x.ndim))
+    num = x4.shape[0] if across_channels else x4.shape[0] * x4.shape[1]
+    y = np.empty_like(x4)
+    _lib.orc_mvn(num, x4.size // num, int(normalize_variance), eps, _fp(x4), _fp(y))
+    return y
+
+
+def embed(x, weight, bias=None):
+    x, weight = _f32(x), _f32(weight)
+    b = _f32(bias) if bias is not None else None
+    n_out = weight.shape[1]
+    y = np.empty(x.shape + (n_out,), np.float32)
+    _lib.orc_embed(x.size, n_out, _fp(x), _fp(weight), _fp(b) if b is not None else None, _fp(y))
+    return y
+
+
+def shuffle_channel(x, group):
+    x = _f32(x)
+    y = np.empty_like(x)
+    n, c = x.shape[0], x.shape[1]
+    _lib.orc_shuffle_channel(n, c, x.size // (n * c), group, _fp(x), _fp(y))
+    return y
+
+
+def spp(x, pyramid_height, pool="MAX"):
+    """SPP (spp_layer.cpp:16-199): per level 2^l bins per side through the Pooling layer's
+    own arithmetic, flattened and concatenated on axis 1."""
+    x = _f32(x)
+    h, w = x.shape[2], x.shape[3]
+    outs = []
+    for level in range(pyramid_height):
+        bins = 2 ** level
+        kh, kw = -(-h // bins), -(-w // bins)
+        ph, pw = (kh * bins - h + 1) // 2, (kw * bins - w + 1) // 2
+        outs.append(pooling(x, str(pool), (kh, kw), (kh, kw), (ph, pw)))
+    if pyramid_height == 1:
+        return outs[0]
+    return np.ascontiguousarray(np.concatenate([o.reshape(o.shape[0], -1) for o in outs], axis=1))

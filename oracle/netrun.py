@@ -135,6 +135,80 @@ def run_layer(layer, bottoms):
         p = layer["psroi_pooling_param"]
         return [oracle.psroi_pooling(x, bottoms[1], p["output_dim"], p["group_size"],
                                      p["spatial_scale"])]
+    if t == "ConvolutionDepthwise":
+        p = layer["convolution_param"]
+        blobs = layer["blobs"]
+        return [oracle.conv_dw(x, blobs[0], blobs[1] if p.get("bias_term", True) else None,
+                               _pair(p, "stride", "stride_h", "stride_w", 1),
+                               _pair(p, "pad", "pad_h", "pad_w", 0), _pair(p, "dilation", "_", "_", 1))]
+    if t == "BN":
+        b = layer["blobs"]
+        return [oracle.bn(x, b[0], b[1], b[2], b[3])]
+    if t == "Dropout":
+        return [x.copy()]
+    if t == "Power":
+        p = layer.get("power_param", {})
+        return [oracle.power(x, p.get("power", 1.0), p.get("scale", 1.0), p.get("shift", 0.0))]
+    if t == "Exp":
+        p = layer.get("exp_param", {})
+        return [oracle.exp_layer(x, p.get("base", -1.0), p.get("scale", 1.0), p.get("shift", 0.0))]
+    if t == "Log":
+        p = layer.get("log_param", {})
+        return [oracle.log_layer(x, p.get("base", -1.0), p.get("scale", 1.0), p.get("shift", 0.0))]
+    if t == "AbsVal":
+        return [oracle.absval(x)]
+    if t == "BNLL":
+        return [oracle.bnll(x)]
+    if t == "ELU":
+        return [oracle.elu(x, layer.get("elu_param", {}).get("alpha", 1.0))]
+    if t == "Threshold":
+        return [oracle.threshold(x, layer.get("threshold_param", {}).get("threshold", 0.0))]
+    if t == "PReLU":
+        shared = layer.get("prelu_param", {}).get("channel_shared", False)
+        return [oracle.prelu(x, layer["blobs"][0], shared)]
+    if t == "LRN":
+        p = layer.get("lrn_param", {})
+        return [oracle.lrn(x, p.get("local_size", 5), p.get("alpha", 1.0), p.get("beta", 0.75),
+                           p.get("k", 1.0), p.get("norm_region", "ACROSS_CHANNELS"))]
+    if t == "ArgMax":
+        p = layer.get("argmax_param", {})
+        return [oracle.argmax(x, p.get("top_k", 1), p.get("out_max_val", False), p.get("axis"))]
+    if t == "Reduction":
+        p = layer.get("reduction_param", {})
+        return [oracle.reduction(x, p.get("operation", "SUM"), p.get("axis", 0), p.get("coeff", 1.0))]
+    if t == "MVN":
+        p = layer.get("mvn_param", {})
+        return [oracle.mvn(x, p.get("normalize_variance", True), p.get("across_channels", False),
+                           p.get("eps", 1e-9))]
+    if t == "Embed":
+        p = layer["embed_param"]
+        b = layer["blobs"]
+        return [oracle.embed(x, b[0], b[1] if p.get("bias_term", True) else None)]
+    if t == "Crop":
+        # crop_layer.cpp:29-107: axes from `axis` on take bottom[1]'s extent at the offset
+        p = layer.get("crop_param", {})
+        axis = _canon(p.get("axis", 2), x.ndim)
+        offs = p.get("offset", [])
+        offs = list(offs) if isinstance(offs, (list, tuple)) else [offs]
+        index = [slice(None)] * x.ndim
+        for i in range(axis, x.ndim):
+            o = 0 if not offs else (offs[0] if len(offs) == 1 else offs[i - axis])
+            index[i] = slice(o, o + bottoms[1].shape[i])
+        return [np.ascontiguousarray(x[tuple(index)])]
+    if t == "Tile":
+        # tile_layer.cpp:24-35
+        p = layer["tile_param"]
+        axis = _canon(p.get("axis", 1), x.ndim)
+        reps = [1] * x.ndim
+        reps[axis] = p["tiles"]
+        return [np.ascontiguousarray(np.tile(x, reps))]
+    if t == "ShuffleChannel":
+        return [oracle.shuffle_channel(x, layer.get("shuffle_channel_param", {}).get("group", 1))]
+    if t == "SPP":
+        p = layer["spp_param"]
+        return [oracle.spp(x, p["pyramid_height"], p.get("pool", "MAX"))]
+    if t == "Parameter":
+        return [layer["blobs"][0].copy()]
     raise NotImplementedError(t)
 
 

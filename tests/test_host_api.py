@@ -266,3 +266,88 @@ def test_region_pooling_layers_setup_errors_and_shapes():
                    "roi_pooling_param": {"pooled_h": 0, "pooled_w": 4}}]
     with pytest.raises(MiniCaffeError, match="pooled_h must be > 0"):
         mc.Net.from_buffers(craft.to_prototxt(bad))
+
+
+# Every type string the reference registers (REGISTER_LAYER_CLASS / _CREATOR in
+# src/layers/*.cpp).
+REFERENCE_LAYER_TYPES = """AbsVal ArgMax BN BNLL BatchNorm Bias Concat Convolution ConvolutionDepthwise
+Crop Deconvolution DetectionOutput Dropout ELU Eltwise Embed Exp Filter Flatten InnerProduct Input LRN
+Log MVN Normalize PReLU PSROIPooling Parameter Permute Pooling Power PriorBox Proposal ROIPooling ReLU
+Reduction Reshape SPP Scale ShuffleChannel Sigmoid Slice Softmax Split TanH Threshold Tile""".split()
+
+
+def test_registry_holds_every_reference_layer_type():
+    msg = err(lambda: mc.Net.from_buffers('layer { name: "x" type: "NoSuchLayer" top: "x" }'))
+    assert "Unknown layer type: NoSuchLayer" in msg
+    known = msg.split("known types:")[1].strip(" )").split(", ")
+    assert sorted(known) == sorted(REFERENCE_LAYER_TYPES)
+
+
+def test_zoo_layers_shapes_params_and_setup_errors():
+    E = craft.Enum
+    base = [craft.input_layer({"d": (2, 6, 8, 8), "small": (2, 6, 4, 5), "idx": (3, 4), "sel": (2,)})]
+
+    def one(ltype, bottoms, tops, **params):
+        return base + [dict({"name": "l", "type": ltype, "bottom": bottoms, "top": tops}, **params)]
+
+    def shape_of(spec, top="t"):
+        net = mc.Net.from_buffers(craft.to_prototxt(spec))   # must outlive the blob view
+        return tuple(net.get_blob(top).shape)
+
+    for ltype in ("Dropout", "Power", "Exp", "Log", "AbsVal", "BNLL", "ELU", "Threshold", "PReLU",
+                  "LRN", "MVN", "ShuffleChannel", "BN"):
+        assert shape_of(one(ltype, ["d"], ["t"])) == (2, 6, 8, 8), ltype
+    # parameter blobs: PReLU slope (default filler 0.25), BN's four, Embed, ConvolutionDepthwise
+    net = mc.Net.from_buffers(craft.to_prototxt(one("PReLU", ["d"], ["t"])))
+    assert [(n, b.shape) for n, b in net.param_list] == [("l_0", [6])]
+    assert np.all(net.param_list[0][1].data == 0.25)
+    net = mc.Net.from_buffers(craft.to_prototxt(
+        one("PReLU", ["d"], ["t"], prelu_param={"channel_shared": True, "filler": {"value": 0.1}})))
+    assert net.param_list[0][1].shape == [] and np.allclose(net.param_list[0][1].data, 0.1)
+    net = mc.Net.from_buffers(craft.to_prototxt(one("BN", ["d"], ["t"])))
+    assert [b.shape for _, b in net.param_list] == [[1, 6]] * 4
+    assert [float(b.data.ravel()[0]) for _, b in net.param_list] == [0.0, 0.0, 0.0, 1.0]
+    net = mc.Net.from_buffers(craft.to_prototxt(
+        one("ConvolutionDepthwise", ["d"], ["t"],
+            convolution_param={"num_output": 99, "kernel_size": 3, "stride": 2, "pad": 1})))
+    assert tuple(net.get_blob("t").shape) == (2, 6, 4, 4)
+    assert [b.shape for _, b in net.param_list] == [[6, 1, 3, 3], [6]]
+    net = mc.Net.from_buffers(craft.to_prototxt(
+        one("Embed", ["idx"], ["t"], embed_param={"num_output": 5, "input_dim": 9})))
+    assert tuple(net.get_blob("t").shape) == (3, 4, 5)
+    assert [b.shape for _, b in net.param_list] == [[9, 5], [5]]
+    # shapes
+    assert shape_of(one("ArgMax", ["d"], ["t"])) == (2, 1, 1, 1)
+    assert shape_of(one("ArgMax", ["d"], ["t"], argmax_param={"top_k": 3, "out_max_val": True})) == (2, 2, 3, 1)
+    assert shape_of(one("ArgMax", ["d"], ["t"], argmax_param={"top_k": 2, "axis": 1})) == (2, 2, 8, 8)
+    assert shape_of(one("Reduction", ["d"], ["t"], reduction_param={"axis": 2})) == (2, 6)
+    assert shape_of(one("Reduction", ["d"], ["t"])) == ()
+    assert shape_of(one("Crop", ["d", "small"], ["t"], crop_param={"offset": [2, 1]})) == (2, 6, 4, 5)
+    assert shape_of(one("Crop", ["d", "small"], ["t"], crop_param={"axis": 1, "offset": 0})) == (2, 6, 4, 5)
+    assert shape_of(one("Tile", ["d"], ["t"], tile_param={"tiles": 3})) == (2, 18, 8, 8)
+    assert shape_of(one("Tile", ["d"], ["t"], tile_param={"tiles": 2, "axis": -1})) == (2, 6, 8, 16)
+    assert shape_of(one("SPP", ["d"], ["t"], spp_param={"pyramid_height": 3})) == (2, 6 * 21)
+    assert shape_of(one("SPP", ["d"], ["t"], spp_param={"pyramid_height": 1, "pool": E("AVE")})) == (2, 6, 1, 1)
+    # Net::Init reshapes twice (SetUp, then PlaceMemory): the second time the all-zero
+    # selector keeps no item, as in the reference (net.cpp:52,72,149).
+    assert shape_of(one("Filter", ["d", "sel"], ["t"])) == (0, 6, 8, 8)
+    par = base + [{"name": "p", "type": "Parameter", "top": ["t"], "parameter_param": {"shape": {"dim": [3, 2]}}}]
+    net = mc.Net.from_buffers(craft.to_prototxt(par))
+    assert tuple(net.get_blob("t").shape) == (3, 2) and net.param_list[0][1].shape == [3, 2]
+    # set-up errors carry the reference's messages
+    bad = lambda *a, **k: err(lambda: mc.Net.from_buffers(craft.to_prototxt(one(*a, **k))))
+    assert "odd values for local_size" in bad("LRN", ["d"], ["t"], lrn_param={"local_size": 4})
+    assert "base must be strictly positive" in bad("Exp", ["d"], ["t"], exp_param={"base": -2.0})
+    assert "base must be strictly positive" in bad("Log", ["d"], ["t"], log_param={"base": 0.0})
+    assert "top_k must be less than or equal" in bad("ArgMax", ["d"], ["t"], argmax_param={"top_k": 7, "axis": 1})
+    assert "top k must not be less than 1" in bad("ArgMax", ["d"], ["t"], argmax_param={"top_k": 0})
+    assert "Number of tiles must be specified" in bad("Tile", ["d"], ["t"])
+    assert "out-of-bounds" in bad("Crop", ["d", "small"], ["t"], crop_param={"offset": 5})
+    assert "number of offset values" in bad("Crop", ["d", "small"], ["t"], crop_param={"offset": [1, 1, 1]})
+    assert "group must be greater than 0" in bad("ShuffleChannel", ["d"], ["t"], shuffle_channel_param={"group": 0})
+    assert "Wrong group size" in bad("ShuffleChannel", ["d"], ["t"], shuffle_channel_param={"group": 4})
+    assert "input_dim must be positive" in bad("Embed", ["idx"], ["t"], embed_param={"num_output": 5})
+    assert "shape mismatch" in err(lambda: mc.Net.from_buffers(
+        craft.to_prototxt(one("PReLU", ["d"], ["t"])), wire.net("m", [wire.layer("l", "PReLU", [np.zeros(5, np.float32)])])))
+    assert "Selector blob dimensions must be singletons" in bad("Filter", ["d", "idx"], ["t"])
+    assert "Unknown reduction op" in bad("Reduction", ["d"], ["t"], reduction_param={"operation": E("PRODUCT")})

@@ -516,3 +516,197 @@ def test_psroi_pooling_bit_exact(K, num, dim, g, hw, scale):
     got = out2.cpu().numpy()
     assert int(flag.item()) == 1 and np.array_equal(got[1], np.zeros((dim, g, g), np.float32))
     assert np.array_equal(got[[0, 2, 3]], want[[0, 2, 3]])
+
+
+# ---- less common layers ------------------------------------------------------------
+
+def close(got, want, tol=1e-5):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    return np.abs(got - want).max() <= tol * max(1.0, np.abs(want).max())
+
+
+UNARY = {"POWER": 0, "EXP": 1, "LOG": 2, "ABS": 3, "BNLL": 4, "ELU": 5, "THRESHOLD": 6}
+
+
+def run_unary(K, op, x, p0=0.0, p1=0.0, p2=0.0, offset=0):
+    xd = dev(x.reshape(-1))
+    yd = torch.full((x.size + offset,), float("nan"), device="cuda")
+    K.check_mc(K.LIB.mcUnary(UNARY[op], fptr(xd), ctypes.c_void_p(yd.data_ptr() + 4 * offset), x.size,
+                             p0, p1, p2, None))
+    torch.cuda.synchronize()
+    return yd[offset:].cpu().numpy().reshape(x.shape)
+
+
+@pytest.mark.parametrize("n", [1, 3, 1021, 4096, 100003])
+def test_unary_functions(K, n):
+    rng = np.random.default_rng(n)
+    x = (rng.standard_normal(n) * 3).astype(np.float32)
+    pos = (rng.random(n) * 4 + 0.05).astype(np.float32)
+    assert close(run_unary(K, "POWER", pos, 2.0, 1.0, 0.5), oracle.power(pos, 0.5, 2.0, 1.0))
+    assert close(run_unary(K, "POWER", pos, 1e-2, 1.0, -0.75), oracle.power(pos, -0.75, 1e-2, 1.0))
+    assert close(run_unary(K, "POWER", x, 1.0, 0.0, 2.0), oracle.power(x, 2.0), 1e-6)
+    assert np.array_equal(run_unary(K, "POWER", x, 1.0, 0.0, 1.0), x)
+    assert close(run_unary(K, "EXP", x, 1.0, 1.0), oracle.exp_layer(x))
+    assert close(run_unary(K, "EXP", x, np.float32(np.log(np.float32(2.0))) * np.float32(0.5), 8.0),
+                 oracle.exp_layer(x, 2.0, 0.5, 3.0))
+    assert close(run_unary(K, "LOG", pos, 1.0, 0.0, 1.0), oracle.log_layer(pos))
+    assert close(run_unary(K, "LOG", pos, 2.0, 1.0, 1.0 / np.log(np.float32(10.0))),
+                 oracle.log_layer(pos, 10.0, 2.0, 1.0))
+    assert np.array_equal(run_unary(K, "ABS", x), oracle.absval(x))
+    big = np.concatenate([x, np.array([90.0, -90.0, 0.0], np.float32)])
+    assert close(run_unary(K, "BNLL", big), oracle.bnll(big), 1e-6)
+    assert close(run_unary(K, "ELU", x, 1.5), oracle.elu(x, 1.5), 1e-6)
+    assert np.array_equal(run_unary(K, "THRESHOLD", x, 0.25), oracle.threshold(x, 0.25))
+    # a destination that is not 16-byte aligned takes the scalar walk
+    assert np.array_equal(run_unary(K, "ABS", x, offset=1), oracle.absval(x))
+
+
+def test_unary_in_place_and_bad_op(K):
+    x = np.random.default_rng(0).standard_normal(777).astype(np.float32)
+    xd = dev(x)
+    K.check_mc(K.LIB.mcUnary(UNARY["ABS"], fptr(xd), fptr(xd), x.size, 0.0, 0.0, 0.0, None))
+    assert np.array_equal(xd.cpu().numpy(), np.abs(x))
+    assert K.LIB.mcUnary(42, fptr(xd), fptr(xd), x.size, 0.0, 0.0, 0.0, None) != 0
+
+
+@pytest.mark.parametrize("shape,shared", [((2, 5, 7, 3), False), ((3, 4), False), ((2, 6, 9, 9), True)])
+def test_prelu(K, shape, shared):
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal(shape).astype(np.float32)
+    slope = rng.standard_normal(1 if shared else shape[1]).astype(np.float32)
+    xd, sd = dev(x), dev(slope)
+    yd = torch.empty_like(xd)
+    inner = int(np.prod(shape[2:]))
+    K.check_mc(K.LIB.mcPReLU(fptr(xd), fptr(yd), shape[0], shape[1], inner, fptr(sd), int(shared), None))
+    assert np.array_equal(yd.cpu().numpy(), oracle.prelu(x, slope, shared))
+
+
+@pytest.mark.parametrize("case", [(2, 96, 27, 27, 5), (1, 7, 3, 5, 3), (2, 40, 6, 6, 9), (1, 3, 4, 4, 1),
+                                  (1, 2, 5, 5, 7)])
+def test_lrn_across_channels(K, case):
+    n, c, h, w, size = case
+    x = (np.random.default_rng(2).standard_normal((n, c, h, w)) * 4).astype(np.float32)
+    xd = dev(x)
+    yd = torch.full_like(xd, float("nan"))
+    K.check_mc(K.LIB.mcLRNAcrossChannels(fptr(xd), fptr(yd), n, c, h, w, size, 1e-2, 0.75, 2.0, None))
+    assert close(yd.cpu().numpy(), oracle.lrn(x, size, 1e-2, 0.75, 2.0), 1e-5)
+    assert K.LIB.mcLRNAcrossChannels(fptr(xd), fptr(yd), n, c, h, w, 4, 1e-2, 0.75, 2.0, None) != 0
+
+
+@pytest.mark.parametrize("case", [(6, 13, 11, 3), (2, 5, 5, 5), (3, 2, 9, 7)])
+def test_lrn_within_channel(K, case):
+    planes, h, w, size = case
+    x = (np.random.default_rng(3).standard_normal((1, planes, h, w)) * 3).astype(np.float32)
+    xd = dev(x)
+    yd = torch.full_like(xd, float("nan"))
+    K.check_mc(K.LIB.mcLRNWithinChannel(fptr(xd), fptr(yd), planes, h, w, size, 0.5, 0.75, None))
+    assert close(yd.cpu().numpy(), oracle.lrn(x, size, 0.5, 0.75, norm_region="WITHIN_CHANNEL"), 1e-5)
+
+
+ARGMAX_CASES = [
+    # shape, top_k, out_max_val, axis
+    ((4, 1000), 1, False, None),
+    ((4, 1000), 5, True, None),
+    ((2, 21, 30, 40), 1, False, 1),       # segmentation argmax: many short lines
+    ((2, 21, 30, 40), 3, True, 1),
+    ((3, 7, 300), 4, False, 2),           # long lines, inner == 1
+    ((2, 3000, 4), 2, False, 1),          # long strided lines: one workgroup each
+    ((2, 5, 6), 30, True, None),          # top_k = whole flattened instance
+    ((70, 33), 33, False, 1),
+]
+
+
+@pytest.mark.parametrize("shape,top_k,omv,axis", ARGMAX_CASES)
+@pytest.mark.parametrize("ties", [False, True])
+def test_argmax_indices_bit_exact(K, shape, top_k, omv, axis, ties):
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal(shape).astype(np.float32)
+    if ties:
+        x = np.round(x * 2) / 2            # few distinct values: order among equals matters
+    want = oracle.argmax(x, top_k, omv, axis)
+    xd = dev(x)
+    yd = torch.full(want.shape, float("nan"), device="cuda")
+    if axis is None:
+        outer, dim, inner, layout = shape[0], int(np.prod(shape[1:])), 1, 2 if omv else 0
+    else:
+        outer, dim, inner = int(np.prod(shape[:axis])), shape[axis], int(np.prod(shape[axis + 1:]))
+        layout = 1 if omv else 0
+    K.check_mc(K.LIB.mcArgMax(fptr(xd), fptr(yd), outer, dim, inner, top_k, layout, None))
+    assert np.array_equal(yd.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("num,dim", [(1, 100000), (7, 300), (2048, 9), (5, 1), (3000, 64)])
+def test_reduction(K, num, dim):
+    x = np.random.default_rng(5).standard_normal((num, dim)).astype(np.float32)
+    xd = dev(x)
+    for op, name in ((1, "SUM"), (2, "ASUM"), (3, "SUMSQ"), (4, "MEAN")):
+        yd = torch.full((num,), float("nan"), device="cuda")
+        K.check_mc(K.LIB.mcReduction(op, fptr(xd), fptr(yd), num, dim, 0.5, None))
+        want = oracle.reduction(x, name, 1, 0.5)
+        scale = np.abs(x).sum(axis=1).max() * (0.5 / dim if name == "MEAN" else 0.5)
+        got = yd.cpu().numpy()
+        if dim <= 300:
+            assert np.abs(got - want).max() <= 1e-5 * max(scale, 1e-6), name
+        # Long rows: the oracle adds in index order in fp32, as plain loops do, and drifts;
+        # both are held against the float64 sum, the device's tree sum being the closer.
+        x64 = x.astype(np.float64)
+        exact = 0.5 * {"SUM": x64.sum(1), "ASUM": np.abs(x64).sum(1), "SUMSQ": (x64 ** 2).sum(1),
+                       "MEAN": x64.mean(1)}[name]
+        if name == "SUMSQ":
+            scale = (x64 ** 2).sum(1).max() * 0.5
+        assert np.abs(got - exact).max() <= 1e-5 * max(scale, 1e-6), name
+        assert np.abs(got - exact).max() <= np.abs(want - exact).max() + 1e-6 * max(scale, 1e-6), name
+    assert K.LIB.mcReduction(9, fptr(xd), fptr(xd), num, dim, 1.0, None) != 0
+
+
+@pytest.mark.parametrize("num,dim,norm", [(6, 35, True), (2, 5000, True), (6, 35, False), (3, 1, True)])
+def test_mvn(K, num, dim, norm):
+    x = (np.random.default_rng(6).standard_normal((num, dim, 1, 1)) * 2 + 3).astype(np.float32)
+    xd = dev(x)
+    yd = torch.full_like(xd, float("nan"))
+    K.check_mc(K.LIB.mcMVN(fptr(xd), fptr(yd), num, dim, int(norm), 0.1, None))
+    want = oracle.mvn(x.reshape(1, num, dim, 1), norm, False, 0.1).reshape(x.shape)
+    assert close(yd.cpu().numpy(), want, 1e-5)
+
+
+def test_gather_rows_embed_and_out_of_range(K):
+    rng = np.random.default_rng(7)
+    w = rng.standard_normal((50, 33)).astype(np.float32)
+    b = rng.standard_normal(33).astype(np.float32)
+    idx = rng.integers(0, 50, 200).astype(np.float32)
+    wd, bd, idd = dev(w), dev(b), dev(idx)
+    yd = torch.full((200, 33), float("nan"), device="cuda")
+    K.check_mc(K.LIB.mcGatherRows(fptr(wd), 50, 33, fptr(idd), 200, fptr(bd), fptr(yd), None))
+    assert np.array_equal(yd.cpu().numpy(), oracle.embed(idx, w, b))
+    K.check_mc(K.LIB.mcGatherRows(fptr(wd), 50, 33, fptr(idd), 200, None, fptr(yd), None))
+    assert np.array_equal(yd.cpu().numpy(), w[idx.astype(int)])
+    bad = dev(np.array([3, 50, -1, 0], np.float32))
+    K.check_mc(K.LIB.mcGatherRows(fptr(wd), 50, 33, fptr(bad), 4, None, fptr(yd), None))
+    got = yd[:4].cpu().numpy()
+    assert np.array_equal(got[[0, 3]], w[[3, 0]]) and np.isnan(got[[1, 2]]).all()
+
+
+def test_crop_and_tile_bit_exact(K):
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((2, 5, 9, 11)).astype(np.float32)
+    xd = dev(x)
+    arr = lambda v: (ctypes.c_int * len(v))(*v)
+    for top, off in [((2, 5, 4, 6), (0, 0, 3, 2)), ((1, 2, 9, 11), (1, 3, 0, 0)), ((2, 5, 9, 11), (0, 0, 0, 0)),
+                     ((2, 5, 1, 1), (0, 0, 8, 10))]:
+        yd = torch.full(top, float("nan"), device="cuda")
+        K.check_mc(K.LIB.mcCrop(fptr(xd), fptr(yd), 4, arr(x.shape), arr(top), arr(off), None))
+        want = x[tuple(slice(o, o + t) for o, t in zip(off, top))]
+        assert np.array_equal(yd.cpu().numpy(), want)
+    yd = torch.empty((2, 5, 4, 6), device="cuda")
+    assert K.LIB.mcCrop(fptr(xd), fptr(yd), 4, arr(x.shape), arr((2, 5, 4, 6)), arr((0, 0, 6, 0)), None) != 0
+    assert "out-of-bounds" in K.LIB.mcLastError().decode()
+    for axis, tiles in [(1, 3), (0, 2), (3, 4)]:
+        shape = list(x.shape)
+        shape[axis] *= tiles
+        yd = torch.full(shape, float("nan"), device="cuda")
+        K.check_mc(K.LIB.mcTile(fptr(xd), fptr(yd), int(np.prod(x.shape[:axis])),
+                                int(np.prod(x.shape[axis:])), tiles, None))
+        reps = [1] * 4
+        reps[axis] = tiles
+        assert np.array_equal(yd.cpu().numpy(), np.tile(x, reps))

@@ -370,3 +370,107 @@ def test_rfcn_second_stage_on_proposal_rois(gpu_mode):
     rp = net.get_blob("roi_pool").data
     assert rp.shape == (50, 64, 4, 4) and np.array_equal(rp, want["roi_pool"])
     assert netrun.rel_err(net.get_blob("cls_score").data, want["cls_score"]) < 1e-5
+
+
+def test_zoo_layers_in_a_net(gpu_mode):
+    """The less common layer types wired into one graph, every top compared with the
+    CPU oracle walking the same layers: a MobileNet-style block (ConvolutionDepthwise
+    -> BN -> PReLU, the BN folded into the convolution's epilogue), AlexNet-style
+    LRN + Dropout, and the rest of the registry as side branches."""
+    from minicaffe.craft import Enum, input_layer
+    rng = np.random.default_rng(11)
+    f = lambda *s: rng.standard_normal(s).astype(np.float32)
+    C = 8
+    spec = [
+        input_layer({"data": (2, C, 12, 10), "ref": (2, C, 7, 6), "words": (2, 5)}),
+        {"name": "dw", "type": "ConvolutionDepthwise", "bottom": ["data"], "top": ["dw"],
+         "convolution_param": {"num_output": C, "kernel_size": 3, "pad": 1, "bias_term": False},
+         "blobs": [f(C, 1, 3, 3) * 0.3]},
+        {"name": "dw_bn", "type": "BN", "bottom": ["dw"], "top": ["dw"],
+         "blobs": [f(1, C), f(1, C), f(1, C) * 0.1, (rng.random((1, C)) + 0.5).astype(np.float32)]},
+        {"name": "dw_prelu", "type": "PReLU", "bottom": ["dw"], "top": ["dw"], "blobs": [f(C) * 0.3]},
+        {"name": "pw", "type": "Convolution", "bottom": ["dw"], "top": ["pw"],
+         "convolution_param": {"num_output": 12, "kernel_size": 1}, "blobs": [f(12, C, 1, 1) * 0.3, f(12)]},
+        {"name": "pw_elu", "type": "ELU", "bottom": ["pw"], "top": ["pw"], "elu_param": {"alpha": 0.7}},
+        {"name": "shuf", "type": "ShuffleChannel", "bottom": ["pw"], "top": ["shuf"],
+         "shuffle_channel_param": {"group": 3}},
+        {"name": "lrn", "type": "LRN", "bottom": ["shuf"], "top": ["lrn"],
+         "lrn_param": {"local_size": 5, "alpha": 1e-2, "beta": 0.75, "k": 2.0}},
+        {"name": "drop", "type": "Dropout", "bottom": ["lrn"], "top": ["lrn"], "dropout_param": {"dropout_ratio": 0.5}},
+        {"name": "lrn_w", "type": "LRN", "bottom": ["lrn"], "top": ["lrn_w"],
+         "lrn_param": {"local_size": 3, "alpha": 0.5, "norm_region": Enum("WITHIN_CHANNEL")}},
+        {"name": "bn_alone", "type": "BN", "bottom": ["lrn_w"], "top": ["bn_alone"],
+         "blobs": [f(1, 12), f(1, 12), f(1, 12) * 0.1, (rng.random((1, 12)) + 0.5).astype(np.float32)]},
+        {"name": "crop", "type": "Crop", "bottom": ["bn_alone", "ref"], "top": ["crop"],
+         "crop_param": {"axis": 2, "offset": [3, 2]}},
+        {"name": "mvn", "type": "MVN", "bottom": ["crop"], "top": ["mvn"], "mvn_param": {"eps": 1e-3}},
+        {"name": "abs", "type": "AbsVal", "bottom": ["mvn"], "top": ["abs"]},
+        {"name": "pow", "type": "Power", "bottom": ["abs"], "top": ["pow"],
+         "power_param": {"power": 0.5, "scale": 2.0, "shift": 0.25}},
+        {"name": "log", "type": "Log", "bottom": ["pow"], "top": ["log"], "log_param": {"base": 2.0, "shift": 1.0}},
+        {"name": "exp", "type": "Exp", "bottom": ["log"], "top": ["exp"], "exp_param": {"scale": -0.5}},
+        {"name": "bnll", "type": "BNLL", "bottom": ["mvn"], "top": ["bnll"]},
+        {"name": "thr", "type": "Threshold", "bottom": ["mvn"], "top": ["thr"],
+         "threshold_param": {"threshold": 0.1}},
+        {"name": "tile", "type": "Tile", "bottom": ["exp"], "top": ["tile"], "tile_param": {"axis": 1, "tiles": 2}},
+        {"name": "spp", "type": "SPP", "bottom": ["data"], "top": ["spp"], "spp_param": {"pyramid_height": 2}},
+        {"name": "red", "type": "Reduction", "bottom": ["spp"], "top": ["red"],
+         "reduction_param": {"operation": Enum("SUMSQ"), "axis": 1, "coeff": 0.1}},
+        {"name": "am", "type": "ArgMax", "bottom": ["bnll"], "top": ["am"], "argmax_param": {"axis": 1, "top_k": 2}},
+        {"name": "am_flat", "type": "ArgMax", "bottom": ["spp"], "top": ["am_flat"],
+         "argmax_param": {"top_k": 3, "out_max_val": True}},
+        {"name": "emb", "type": "Embed", "bottom": ["words"], "top": ["emb"],
+         "embed_param": {"num_output": 4, "input_dim": 9}, "blobs": [f(9, 4), f(4)]},
+        {"name": "par", "type": "Parameter", "top": ["par"], "parameter_param": {"shape": {"dim": [2, 3]}},
+         "blobs": [f(2, 3)]},
+    ]
+    inputs = {"data": f(2, C, 12, 10), "ref": np.zeros((2, C, 7, 6), np.float32),
+              "words": rng.integers(0, 9, (2, 5)).astype(np.float32)}
+    marks = ["dw", "pw", "shuf", "lrn", "lrn_w", "bn_alone", "crop", "mvn", "abs", "pow", "log", "exp",
+             "bnll", "thr", "tile", "spp", "red", "am", "am_flat", "emb", "par"]
+    net = run_net(gpu_mode, spec, inputs, marks)
+    # device-produced inputs for the index-valued tops, so that "same indices" is well posed
+    bnll_dev = net.get_blob("bnll").data.copy()
+    spp_dev = net.get_blob("spp").data.copy()
+    want = netrun.oracle_forward(spec, inputs)
+    for name in marks:
+        got = net.get_blob(name).data
+        assert tuple(got.shape) == want[name].shape, name
+        if name in ("am", "am_flat", "thr"):
+            continue
+        # MVN subtracts a mean several times the spread it keeps: from there on the
+        # deep-net tolerance applies
+        deep = name in ("mvn", "abs", "pow", "log", "exp", "bnll", "tile")
+        assert netrun.rel_err(got, want[name]) < (1e-3 if deep else 1e-4), name
+    assert np.array_equal(net.get_blob("am").data, oracle.argmax(bnll_dev, 2, False, 1))
+    assert np.array_equal(net.get_blob("am_flat").data, oracle.argmax(spp_dev, 3, True))
+    assert np.array_equal(net.get_blob("thr").data, oracle.threshold(net.get_blob("mvn").data, 0.1))
+    assert np.array_equal(net.get_blob("spp").data, want["spp"])      # max pooling moves values
+    assert np.array_equal(net.get_blob("emb").data, want["emb"])
+    assert np.array_equal(net.get_blob("par").data, spec[-1]["blobs"][0])
+    # a second forward with another batch size re-plans every layer
+    x3 = f(3, C, 12, 10)
+    in3 = {"data": x3, "ref": np.zeros((3, C, 7, 6), np.float32),
+           "words": rng.integers(0, 9, (3, 5)).astype(np.float32)}
+    net.forward(**in3)
+    want3 = netrun.oracle_forward(spec, in3)
+    for name in ("tile", "red", "bn_alone", "emb"):
+        assert netrun.rel_err(net.get_blob(name).data, want3[name]) < 1e-4, name
+
+
+def test_filter_layer_selects_items_at_reshape(gpu_mode):
+    """Filter reads its selector when the net is reshaped (filter_layer.cpp:19-59): the
+    selector is an input written before Forward(reshape=True), as a caller of the
+    reference has to do."""
+    from minicaffe.craft import input_layer
+    rng = np.random.default_rng(12)
+    spec = [input_layer({"a": (5, 3, 4), "b": (5, 2), "sel": (5,)}),
+            {"name": "flt", "type": "Filter", "bottom": ["a", "b", "sel"], "top": ["fa", "fb"]}]
+    a, b = rng.standard_normal((5, 3, 4)).astype(np.float32), rng.standard_normal((5, 2)).astype(np.float32)
+    sel = np.array([0, 1, 0, 2, 1], np.float32)
+    net = run_net(gpu_mode, spec, {"a": a, "b": b, "sel": sel})
+    keep = sel != 0
+    assert np.array_equal(net.get_blob("fa").data, a[keep])
+    assert np.array_equal(net.get_blob("fb").data, b[keep])
+    net.forward(a=a, b=b, sel=np.zeros(5, np.float32))
+    assert tuple(net.get_blob("fa").shape) == (0, 3, 4)
