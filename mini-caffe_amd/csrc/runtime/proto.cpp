@@ -538,10 +538,84 @@ void ReadNetParamsFromBinaryFileOrDie(const std::string& file, NetParameter* par
   ParseBinaryNet(reinterpret_cast<const uint8_t*>(bytes.data()), bytes.size(), param);
 }
 
+namespace {
+
+// V1LayerParameter.LayerType -> type string (reference src/util/upgrade_proto.cpp:215-265;
+// enum values from caffe.proto's V1LayerParameter).  A text file names the enum
+// by identifier; the number is accepted as well.
+struct V1Type {
+  const char* ident;
+  int number;
+  const char* type;
+};
+const V1Type kV1Types[] = {
+    {"NONE", 0, ""},
+    {"ABSVAL", 35, "AbsVal"},
+    {"BNLL", 2, "BNLL"},
+    {"CONCAT", 3, "Concat"},
+    {"CONVOLUTION", 4, "Convolution"},
+    {"DECONVOLUTION", 39, "Deconvolution"},
+    {"DROPOUT", 6, "Dropout"},
+    {"ELTWISE", 25, "Eltwise"},
+    {"EXP", 38, "Exp"},
+    {"FLATTEN", 8, "Flatten"},
+    {"INNER_PRODUCT", 14, "InnerProduct"},
+    {"LRN", 15, "LRN"},
+    {"MVN", 34, "MVN"},
+    {"POOLING", 17, "Pooling"},
+    {"POWER", 26, "Power"},
+    {"RELU", 18, "ReLU"},
+    {"SIGMOID", 19, "Sigmoid"},
+    {"SOFTMAX", 20, "Softmax"},
+    {"SPLIT", 22, "Split"},
+    {"SLICE", 33, "Slice"},
+    {"TANH", 23, "TanH"},
+    {"THRESHOLD", 31, "Threshold"},
+};
+
+// The fields of a V1 layer that UpgradeV1LayerParameter carries over and that
+// matter to a forward pass (reference src/util/upgrade_proto.cpp:86-213); the
+// learning-rate, weight-decay, loss-weight and parameter-sharing fields have no
+// reader in this library and are dropped.
+const char* const kV1Carried[] = {
+    "bottom", "top", "name", "include", "exclude", "blobs", "concat_param", "convolution_param",
+    "dropout_param", "eltwise_param", "exp_param", "inner_product_param", "lrn_param", "mvn_param",
+    "pooling_param", "power_param", "relu_param", "sigmoid_param", "softmax_param", "slice_param",
+    "tanh_param", "threshold_param"};
+
+void UpgradeV1Net(const std::string& source, NetParameter* param) {
+  CHECK(!param->has("layer"))
+      << source << ": Refusing to upgrade inconsistent NetParameter input; the definition "
+      << "includes both 'layer' and 'layers' fields. The current format defines 'layer' fields "
+      << "with string type like layer { type: 'Layer' ... } and not layers { type: LAYER ... }. "
+      << "Manually switch the definition to 'layer' format to continue.";
+  for (auto& f : param->fields()) {
+    if (f.name != "layers" || !f.msg) continue;
+    const Message& v1 = *f.msg;
+    auto layer = std::make_shared<Message>();
+    for (const auto& g : v1.fields()) {
+      bool carried = false;
+      for (const char* k : kV1Carried) carried = carried || g.name == k;
+      if (carried) layer->fields().push_back(g);
+    }
+    if (v1.has("type")) {
+      const Message::Field* t = v1.find("type");
+      const char* mapped = nullptr;
+      for (const V1Type& e : kV1Types)
+        if (t->text == e.ident || t->text == std::to_string(e.number)) mapped = e.type;
+      CHECK(mapped && !t->quoted)
+          << source << ": Unknown V1LayerParameter layer type: " << t->text;
+      layer->add("type", mapped, true);
+    }
+    f.name = "layer";
+    f.msg = layer;
+  }
+}
+
+}  // namespace
+
 void UpgradeNetAsNeeded(const std::string& source, NetParameter* param) {
-  CHECK(!param->has("layers"))
-      << source << ": V1 'layers' definitions are not supported; upgrade the file with "
-      << "Caffe's upgrade_net_proto_text first";
+  if (param->has("layers")) UpgradeV1Net(source, param);
   if (!param->has("input")) return;
   // `input: "data"` + (`input_shape {dim..}` | 4 x `input_dim`) -> Input layer.
   const int n_in = param->count("input");

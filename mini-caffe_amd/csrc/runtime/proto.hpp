@@ -73,9 +73,10 @@ void ParseBinaryNet(const uint8_t* data, size_t len, Message* out);
 void ReadNetParamsFromTextFileOrDie(const std::string& file, NetParameter* param);
 void ReadNetParamsFromBinaryFileOrDie(const std::string& file, NetParameter* param);
 
-// Folds legacy top-level `input:` / `input_shape` / `input_dim` declarations
-// into a leading Input layer (reference src/util/upgrade_proto.cpp:267-305) and
-// rejects V1 `layers` definitions with a clear message.
+// Rewrites V1 `layers { type: CONVOLUTION ... }` definitions as `layer` messages
+// (reference src/util/upgrade_proto.cpp:60-265) and folds legacy top-level
+// `input:` / `input_shape` / `input_dim` declarations into a leading Input layer
+// (reference src/util/upgrade_proto.cpp:267-305).
 void UpgradeNetAsNeeded(const std::string& source, NetParameter* param);
 
 // Serialises a NetParameter holding name / layer{name,type,blobs} to wire format.

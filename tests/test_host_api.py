@@ -351,3 +351,41 @@ def test_zoo_layers_shapes_params_and_setup_errors():
         craft.to_prototxt(one("PReLU", ["d"], ["t"])), wire.net("m", [wire.layer("l", "PReLU", [np.zeros(5, np.float32)])])))
     assert "Selector blob dimensions must be singletons" in bad("Filter", ["d", "idx"], ["t"])
     assert "Unknown reduction op" in bad("Reduction", ["d"], ["t"], reduction_param={"operation": E("PRODUCT")})
+
+
+V1_NET = """
+name: "v1"
+input: "data"
+input_dim: 2 input_dim: 3 input_dim: 12 input_dim: 10
+layers { name: "conv1" type: CONVOLUTION bottom: "data" top: "conv1"
+         blobs_lr: 1 blobs_lr: 2 weight_decay: 1 weight_decay: 0
+         convolution_param { num_output: 8 kernel_h: 3 kernel_w: 2 stride_h: 2 stride_w: 1 pad_h: 1 pad_w: 0 } }
+layers { name: "relu" type: RELU bottom: "conv1" top: "conv1" }
+layers { name: "norm" type: LRN bottom: "conv1" top: "norm" lrn_param { local_size: 3 alpha: 0.1 } }
+layers { name: "pool" type: POOLING bottom: "norm" top: "pool" pooling_param { pool: AVE kernel_size: 2 stride: 2 } }
+layers { name: "drop" type: DROPOUT bottom: "pool" top: "pool" dropout_param { dropout_ratio: 0.3 } }
+layers { name: "ip" type: INNER_PRODUCT bottom: "pool" top: "ip" inner_product_param { num_output: 5 bias_term: false } }
+layers { name: "prob" type: 20 bottom: "ip" top: "prob" }
+"""
+
+
+def test_v1_layers_definition_is_upgraded():
+    """V1 `layers { type: ENUM }` prototxt and caffemodel (upgrade_proto.cpp:60-265)."""
+    net = mc.Net.from_buffers(V1_NET)
+    shapes = {k: v.shape for k, v in net.blobs.items()}
+    assert shapes == {"data": [2, 3, 12, 10], "conv1": [2, 8, 6, 9], "norm": [2, 8, 6, 9],
+                      "pool": [2, 8, 3, 5], "ip": [2, 5], "prob": [2, 5]}
+    assert [n for n, _ in net.param_list] == ["conv1_0", "conv1_1", "ip_0"]
+    rng = np.random.default_rng(0)
+    w = rng.standard_normal((8, 3, 3, 2)).astype(np.float32)
+    b = rng.standard_normal(8).astype(np.float32)
+    ipw = rng.standard_normal((5, 120)).astype(np.float32)
+    model = wire.net("m", [], v1_layers=[wire.v1_layer("conv1", 4, [w, b], legacy=True),
+                                         wire.v1_layer("ip", 14, [ipw], legacy=True)])
+    net = mc.Net.from_buffers(V1_NET, model)
+    params = dict(net.param_list)
+    assert np.array_equal(params["conv1_0"].data, w) and np.array_equal(params["ip_0"].data, ipw)
+    assert "Unknown V1LayerParameter layer type: ARGMAX" in err(
+        lambda: mc.Net.from_buffers(V1_NET.replace("type: RELU", "type: ARGMAX")))
+    assert "both 'layer' and 'layers'" in err(
+        lambda: mc.Net.from_buffers(V1_NET + 'layer { name: "x" type: "ReLU" bottom: "ip" top: "ip" }'))

@@ -52,8 +52,18 @@ def layer(name, type_, blobs, **kw):
     return out
 
 
-def net(name, layers):
+def v1_layer(name, type_number, blobs, **kw):
+    """V1LayerParameter: name = 4, type (enum) = 5, blobs = 6, blobs_lr = 7."""
+    out = ld(4, name.encode()) + key(5, 0) + varint(type_number)
+    for b in blobs:
+        out += ld(6, blob(b, **kw)) + key(7, 5) + struct.pack("<f", 1.0)
+    return out
+
+
+def net(name, layers, v1_layers=()):
     out = ld(1, name.encode())
+    for l in v1_layers:
+        out += ld(2, l)
     for l in layers:
         out += ld(100, l)
     return out
