@@ -125,7 +125,7 @@ def main():
 
 def configs_report(path, mc, craft, zoo, LIB):
     """Whole-forward time, contraction TFLOP/s and detection-tail layer time of the five
-    BASELINE configurations on the GPU (synthetic inputs and weights from the zoo builders)."""
+    BASELINE configurations (plus MobileNet-SSD) on the GPU (synthetic inputs and weights from the zoo builders)."""
     import tempfile
     import oracle
     from oracle import netrun
@@ -138,7 +138,10 @@ def configs_report(path, mc, craft, zoo, LIB):
               zoo.ssd300_spec(batch=1, seed=0), 1),
              ("C4 RPN+Proposal 1x1024x38x63", zoo.rpn_spec(seed=0), ("proposal",), 1, zoo.rpn_spec(seed=0), 1),
              ("C5 DCGAN generator b128", zoo.dcgan_spec(batch=128, seed=0), (), 128,
-              zoo.dcgan_spec(batch=8, seed=0), 8)]
+              zoo.dcgan_spec(batch=8, seed=0), 8),
+             # not a BASELINE configuration: the depthwise-separable graph of the reference's ssd example
+             ("+  MobileNet-SSD b32", zoo.mobilenet_ssd_spec(batch=32, seed=0), ("detection_out",), 32,
+              zoo.mobilenet_ssd_spec(batch=2, seed=0), 2)]
     lines = ["%-30s %10s %10s %12s %10s %8s %12s %12s  %s"
              % ("configuration", "ms/forward", "GFLOP", "contr. ms", "TFLOP/s", "of peak", "GPU img/s",
                 "CPU img/s", "tail layers (us, device time)")]
@@ -190,7 +193,7 @@ def configs_report(path, mc, craft, zoo, LIB):
                         batch / (ms * 1e-3), cpu_rate, tail_txt))
         del net
     lines.append("CPU column: one pass of the oracle (reference algorithm: per-image im2col + OpenBLAS sgemm, "
-                 "unfused layers) on %d host threads at batch 1/4/1/1/8." % oracle.openblas_threads())
+                 "unfused layers) on %d host threads at batch 1/4/1/1/8/2." % oracle.openblas_threads())
     with open(path, "w") as f:
         f.write("\n".join(lines) + "\n")
 

@@ -274,6 +274,59 @@ SSD_SOURCES = [  # (source blob, channels, priors, min_size, max_size, aspect ra
 ]
 
 
+def _multibox_tail(spec, sources, num_classes, seed, head_kernel, nms_top_k, keep_top_k,
+                   confidence_threshold):
+    """Appends the SSD heads (loc / conf convolutions -> Permute -> Flatten, PriorBox per
+    source), their concatenations, the class softmax and DetectionOutput.
+    sources: (blob, channels, priors per cell, min_size, max_size or None, aspect ratios,
+    step or None)."""
+    locs, confs, priors = [], [], []
+    for src, c, npri, mn, mx, ars, step in sources:
+        for kind, per in (("loc", 4), ("conf", num_classes)):
+            name = "%s_mbox_%s" % (src, kind)
+            spec.append(conv_layer(name, src, name, c, npri * per, head_kernel,
+                                   pad=head_kernel // 2, seed=seed))
+            spec.append({"name": name + "_perm", "type": "Permute", "bottom": [name],
+                         "top": [name + "_perm"], "permute_param": {"order": [0, 2, 3, 1]}})
+            spec.append({"name": name + "_flat", "type": "Flatten", "bottom": [name + "_perm"],
+                         "top": [name + "_flat"], "flatten_param": {"axis": 1}})
+            (locs if kind == "loc" else confs).append(name + "_flat")
+        pname = "%s_mbox_priorbox" % src
+        pb = {"min_size": mn}
+        if mx is not None:
+            pb["max_size"] = mx
+        pb.update({"aspect_ratio": ars, "flip": True, "clip": False,
+                   "variance": [0.1, 0.1, 0.2, 0.2]})
+        if step is not None:
+            pb["step"] = float(step)
+        pb["offset"] = 0.5
+        spec.append({"name": pname, "type": "PriorBox", "bottom": [src, "data"], "top": [pname],
+                     "prior_box_param": pb})
+        priors.append(pname)
+    spec.append({"name": "mbox_loc", "type": "Concat", "bottom": locs, "top": ["mbox_loc"],
+                 "concat_param": {"axis": 1}})
+    spec.append({"name": "mbox_conf", "type": "Concat", "bottom": confs, "top": ["mbox_conf"],
+                 "concat_param": {"axis": 1}})
+    spec.append({"name": "mbox_priorbox", "type": "Concat", "bottom": priors,
+                 "top": ["mbox_priorbox"], "concat_param": {"axis": 2}})
+    spec.append({"name": "mbox_conf_reshape", "type": "Reshape", "bottom": ["mbox_conf"],
+                 "top": ["mbox_conf_reshape"],
+                 "reshape_param": {"shape": {"dim": [0, -1, num_classes]}}})
+    spec.append({"name": "mbox_conf_softmax", "type": "Softmax", "bottom": ["mbox_conf_reshape"],
+                 "top": ["mbox_conf_softmax"], "softmax_param": {"axis": 2}})
+    spec.append({"name": "mbox_conf_flatten", "type": "Flatten", "bottom": ["mbox_conf_softmax"],
+                 "top": ["mbox_conf_flatten"], "flatten_param": {"axis": 1}})
+    spec.append({"name": "detection_out", "type": "DetectionOutput",
+                 "bottom": ["mbox_loc", "mbox_conf_flatten", "mbox_priorbox"],
+                 "top": ["detection_out"],
+                 "detection_output_param": {
+                     "num_classes": num_classes, "share_location": True,
+                     "background_label_id": 0,
+                     "nms_param": {"nms_threshold": 0.45, "top_k": nms_top_k},
+                     "code_type": Enum("CENTER_SIZE"), "keep_top_k": keep_top_k,
+                     "confidence_threshold": confidence_threshold}})
+
+
 def ssd300_spec(batch=8, seed=0, num_classes=21, size=300, width=64):
     """Config 3: SSD300 on VGG16 (atrous fc6, extra layers conv6-conv9, six multibox
     heads with 4/6/6/6/4/4 priors, 8732 priors at 300x300), DetectionOutput with
@@ -323,45 +376,59 @@ def ssd300_spec(batch=8, seed=0, num_classes=21, size=300, width=64):
                  "norm_param": {"across_spatial": False, "channel_shared": False,
                                 "scale_filler": {"type": "constant", "value": 20.0}},
                  "blobs": [np.full(c43, 20.0, np.float32)]})
-    locs, confs, priors = [], [], []
-    for src, c, npri, mn, mx, ars, step in SSD_SOURCES:
-        c = ch(c)
-        for kind, per in (("loc", 4), ("conf", num_classes)):
-            name = "%s_mbox_%s" % (src, kind)
-            spec.append(conv_layer(name, src, name, c, npri * per, 3, pad=1, seed=seed))
-            spec.append({"name": name + "_perm", "type": "Permute", "bottom": [name],
-                         "top": [name + "_perm"], "permute_param": {"order": [0, 2, 3, 1]}})
-            spec.append({"name": name + "_flat", "type": "Flatten", "bottom": [name + "_perm"],
-                         "top": [name + "_flat"], "flatten_param": {"axis": 1}})
-            (locs if kind == "loc" else confs).append(name + "_flat")
-        pname = "%s_mbox_priorbox" % src
-        spec.append({"name": pname, "type": "PriorBox", "bottom": [src, "data"], "top": [pname],
-                     "prior_box_param": {"min_size": mn, "max_size": mx, "aspect_ratio": ars,
-                                         "flip": True, "clip": False,
-                                         "variance": [0.1, 0.1, 0.2, 0.2], "step": float(step),
-                                         "offset": 0.5}})
-        priors.append(pname)
-    spec.append({"name": "mbox_loc", "type": "Concat", "bottom": locs, "top": ["mbox_loc"],
-                 "concat_param": {"axis": 1}})
-    spec.append({"name": "mbox_conf", "type": "Concat", "bottom": confs, "top": ["mbox_conf"],
-                 "concat_param": {"axis": 1}})
-    spec.append({"name": "mbox_priorbox", "type": "Concat", "bottom": priors,
-                 "top": ["mbox_priorbox"], "concat_param": {"axis": 2}})
-    spec.append({"name": "mbox_conf_reshape", "type": "Reshape", "bottom": ["mbox_conf"],
-                 "top": ["mbox_conf_reshape"],
-                 "reshape_param": {"shape": {"dim": [0, -1, num_classes]}}})
-    spec.append({"name": "mbox_conf_softmax", "type": "Softmax", "bottom": ["mbox_conf_reshape"],
-                 "top": ["mbox_conf_softmax"], "softmax_param": {"axis": 2}})
-    spec.append({"name": "mbox_conf_flatten", "type": "Flatten", "bottom": ["mbox_conf_softmax"],
-                 "top": ["mbox_conf_flatten"], "flatten_param": {"axis": 1}})
-    spec.append({"name": "detection_out", "type": "DetectionOutput",
-                 "bottom": ["mbox_loc", "mbox_conf_flatten", "mbox_priorbox"],
-                 "top": ["detection_out"],
-                 "detection_output_param": {
-                     "num_classes": num_classes, "share_location": True,
-                     "background_label_id": 0,
-                     "nms_param": {"nms_threshold": 0.45, "top_k": 400},
-                     "code_type": Enum("CENTER_SIZE"), "keep_top_k": 200,
-                     "confidence_threshold": 0.01}})
+    _multibox_tail(spec, [(src, ch(c), npri, mn, mx, ars, step)
+                          for src, c, npri, mn, mx, ars, step in SSD_SOURCES],
+                   num_classes, seed, head_kernel=3, nms_top_k=400, keep_top_k=200,
+                   confidence_threshold=0.01)
+    x = np.random.default_rng(seed + 1).uniform(-1, 1, (batch, 3, size, size)).astype(np.float32)
+    return spec, {"data": x}
+
+
+
+# MobileNet-SSD sources: blob, channels, priors per cell, min_size, max_size, aspect ratios.
+MOBILENET_SSD_SOURCES = [
+    ("conv11", 512, 3, 60.0, None, [2.0]),
+    ("conv13", 1024, 6, 105.0, 150.0, [2.0, 3.0]),
+    ("conv14_2", 512, 6, 150.0, 195.0, [2.0, 3.0]),
+    ("conv15_2", 256, 6, 195.0, 240.0, [2.0, 3.0]),
+    ("conv16_2", 256, 6, 240.0, 285.0, [2.0, 3.0]),
+    ("conv17_2", 128, 6, 285.0, 300.0, [2.0, 3.0]),
+]
+
+
+def mobilenet_ssd_spec(batch=1, seed=0, num_classes=21, size=300, width=1.0, depthwise_type=False):
+    """MobileNet-v1 SSD in its deploy form (batch norm merged into the convolutions), the
+    graph of the reference's ssd example (example/models/ssd/MobileNetSSD_deploy.prototxt):
+    conv0, 13 depthwise-separable blocks (`Convolution` with group == channels, then 1x1),
+    four extra stride-2 stages, six 1x1 multibox heads, 1917 priors at 300x300,
+    DetectionOutput with NMS 0.45, top_k 100, keep_top_k 100, confidence 0.25.
+    depthwise_type=True declares the depthwise layers as `ConvolutionDepthwise` instead."""
+    ch = lambda c: max(8, int(round(c * width)))  # noqa: E731
+    spec = [input_layer({"data": (batch, 3, size, size)})]
+
+    def conv_relu(name, bottom, cin, cout, k, stride=1, group=1):
+        layer = conv_layer(name, bottom, name, cin, cout, k, stride, k // 2, group=group, seed=seed)
+        if group != 1 and depthwise_type:
+            layer["type"] = "ConvolutionDepthwise"
+            del layer["convolution_param"]["group"]
+        spec.append(layer)
+        spec.append(relu_layer(name + "/relu", name))
+
+    conv_relu("conv0", "data", 3, ch(32), 3, 2)
+    prev, cin = "conv0", ch(32)
+    for i, (cout, stride) in enumerate([(64, 1), (128, 2), (128, 1), (256, 2), (256, 1), (512, 2),
+                                        (512, 1), (512, 1), (512, 1), (512, 1), (512, 1),
+                                        (1024, 2), (1024, 1)], 1):
+        conv_relu("conv%d/dw" % i, prev, cin, cin, 3, stride, group=cin)
+        conv_relu("conv%d" % i, "conv%d/dw" % i, cin, ch(cout), 1)
+        prev, cin = "conv%d" % i, ch(cout)
+    for i, (mid, cout) in enumerate([(256, 512), (128, 256), (128, 256), (64, 128)], 14):
+        conv_relu("conv%d_1" % i, prev, cin, ch(mid), 1)
+        conv_relu("conv%d_2" % i, "conv%d_1" % i, ch(mid), ch(cout), 3, 2)
+        prev, cin = "conv%d_2" % i, ch(cout)
+    _multibox_tail(spec, [(src, ch(c), npri, mn, mx, ars, None)
+                          for src, c, npri, mn, mx, ars in MOBILENET_SSD_SOURCES],
+                   num_classes, seed, head_kernel=1, nms_top_k=100, keep_top_k=100,
+                   confidence_threshold=0.25)
     x = np.random.default_rng(seed + 1).uniform(-1, 1, (batch, 3, size, size)).astype(np.float32)
     return spec, {"data": x}

@@ -389,3 +389,20 @@ def test_v1_layers_definition_is_upgraded():
         lambda: mc.Net.from_buffers(V1_NET.replace("type: RELU", "type: ARGMAX")))
     assert "both 'layer' and 'layers'" in err(
         lambda: mc.Net.from_buffers(V1_NET + 'layer { name: "x" type: "ReLU" bottom: "ip" top: "ip" }'))
+
+
+@needs_ref
+def test_mobilenet_ssd_builder_matches_the_reference_prototxt():
+    """zoo.mobilenet_ssd_spec builds the graph of example/models/ssd/MobileNetSSD_deploy.prototxt:
+    same blobs, shapes and parameter blobs, 1917 priors."""
+    spec, _ = zoo.mobilenet_ssd_spec()
+    mine = mc.Net.from_buffers(craft.to_prototxt(spec))
+    ref = mc.Net.from_buffers(open(os.path.join(REF, "example", "models", "ssd",
+                                                "MobileNetSSD_deploy.prototxt")).read())
+    assert {k: v.shape for k, v in mine.blobs.items()} == {k: v.shape for k, v in ref.blobs.items()}
+    assert [(n, b.shape) for n, b in mine.param_list] == [(n, b.shape) for n, b in ref.param_list]
+    assert mine.get_blob("mbox_priorbox").shape == [1, 2, 1917 * 4]
+    # the ConvolutionDepthwise spelling of the same graph has the same blobs and parameters
+    spec_dw, _ = zoo.mobilenet_ssd_spec(depthwise_type=True)
+    dw = mc.Net.from_buffers(craft.to_prototxt(spec_dw))
+    assert [(n, b.shape) for n, b in dw.param_list] == [(n, b.shape) for n, b in ref.param_list]

@@ -474,3 +474,29 @@ def test_filter_layer_selects_items_at_reshape(gpu_mode):
     assert np.array_equal(net.get_blob("fb").data, b[keep])
     net.forward(a=a, b=b, sel=np.zeros(5, np.float32))
     assert tuple(net.get_blob("fa").shape) == (0, 3, 4)
+
+
+@pytest.mark.parametrize("depthwise_type", [False, True])
+def test_mobilenet_ssd_full_size(gpu_mode, depthwise_type):
+    """MobileNet-SSD at its real size (300x300, 47 convolutions of which 13 depthwise,
+    1917 priors), the graph of the reference's ssd example with seeded weights: the
+    dense part against the oracle, the DetectionOutput rows bit for bit on the device's
+    own tail inputs.  The confidence heads are sharpened so that detections pass the
+    0.25 threshold.  Both spellings of the depthwise layers give the same numbers."""
+    from minicaffe import zoo
+    spec, inputs = zoo.mobilenet_ssd_spec(batch=2, depthwise_type=depthwise_type)
+    for layer in spec:
+        if layer["name"].endswith("_mbox_conf"):
+            layer["blobs"][0] = layer["blobs"][0] * 6
+    marks = ["conv1/dw", "conv6", "conv13", "conv17_2", "mbox_loc", "mbox_conf_flatten", "mbox_priorbox"]
+    net = run_net(gpu_mode, spec, inputs, marks)
+    oracle.use_openblas(True)
+    try:
+        want = netrun.oracle_forward(spec[:-1], inputs, keep=set(marks))
+    finally:
+        oracle.use_openblas(False)
+    assert np.array_equal(net.get_blob("mbox_priorbox").data, want["mbox_priorbox"])
+    for name in marks[:-1]:
+        assert netrun.rel_err(net.get_blob(name).data, want[name]) < 1e-3, name
+    rows = _check_ssd_tail(net, spec)
+    assert rows.shape == (200, 7) and (rows[:, 2] >= 0.25).all()
