@@ -500,3 +500,74 @@ def test_mobilenet_ssd_full_size(gpu_mode, depthwise_type):
         assert netrun.rel_err(net.get_blob(name).data, want[name]) < 1e-3, name
     rows = _check_ssd_tail(net, spec)
     assert rows.shape == (200, 7) and (rows[:, 2] >= 0.25).all()
+
+
+def test_ssh_context_module_upsample_crop_and_two_top_proposal(gpu_mode):
+    """The motif of the reference's ssh example (example/models/ssh/test_ssh.prototxt):
+    1x1 reduction of the stride-16 map, bilinear 2x upsampling by a Deconvolution with
+    group == channels, Crop to the stride-8 map, Eltwise SUM, 3x3 convolutions, 2-anchor
+    score / box heads, Reshape -> Softmax -> Reshape, and a Proposal with two tops
+    (boxes and their scores).  Dense blobs within tolerance; the Proposal tops bit for
+    bit on the device's own score / box blobs."""
+    from minicaffe import zoo
+    from minicaffe.craft import Enum, input_layer
+    C, R, A = 24, 16, 2
+    h8, w8 = 37, 50                      # stride-8 map; the stride-16 map is 19 x 25
+    h16, w16 = (h8 + 1) // 2, (w8 + 1) // 2
+    # bilinear upsampling filter (factor 2, kernel 4), one per channel
+    f = np.array([0.25, 0.75, 0.75, 0.25], np.float32)
+    up = np.tile(np.outer(f, f).reshape(1, 1, 4, 4), (R, 1, 1, 1))
+    spec = [input_layer({"conv4_3": (1, C, h8, w8), "conv5_3": (1, C, h16, w16), "im_info": (1, 3)}),
+            zoo.conv_layer("conv5_128", "conv5_3", "conv5_128", C, R, 1, seed=1),
+            zoo.relu_layer("conv5_128_relu", "conv5_128"),
+            {"name": "conv5_128_up", "type": "Deconvolution", "bottom": ["conv5_128"], "top": ["conv5_128_up"],
+             "convolution_param": {"kernel_size": 4, "stride": 2, "num_output": R, "group": R, "pad": 1,
+                                   "bias_term": False}, "blobs": [up]},
+            zoo.conv_layer("conv4_128", "conv4_3", "conv4_128", C, R, 1, seed=2),
+            zoo.relu_layer("conv4_128_relu", "conv4_128"),
+            {"name": "conv5_128_crop", "type": "Crop", "bottom": ["conv5_128_up", "conv4_128"],
+             "top": ["conv5_128_crop"], "crop_param": {"axis": 2, "offset": 0}},
+            {"name": "conv4_fuse", "type": "Eltwise", "bottom": ["conv5_128_crop", "conv4_128"],
+             "top": ["conv4_fuse"], "eltwise_param": {"operation": Enum("SUM")}},
+            zoo.conv_layer("conv4_fuse_final", "conv4_fuse", "conv4_fuse_final", R, R, 3, pad=1, seed=3),
+            zoo.relu_layer("conv4_fuse_final_relu", "conv4_fuse_final"),
+            zoo.conv_layer("m1@ssh_3x3", "conv4_fuse_final", "m1@ssh_3x3_output", R, R, 3, pad=1, seed=4),
+            zoo.conv_layer("m1@ssh_dimred", "conv4_fuse_final", "m1@ssh_dimred_output", R, R // 2, 3, pad=1, seed=5),
+            zoo.relu_layer("m1@ssh_dimred_relu", "m1@ssh_dimred_output"),
+            zoo.conv_layer("m1@ssh_5x5", "m1@ssh_dimred_output", "m1@ssh_5x5_output", R // 2, R // 2, 3, pad=1, seed=6),
+            {"name": "m1@ssh_output", "type": "Concat", "bottom": ["m1@ssh_3x3_output", "m1@ssh_5x5_output"],
+             "top": ["m1@ssh_output"], "concat_param": {"axis": 1}},
+            zoo.relu_layer("m1@ssh_output_relu", "m1@ssh_output"),
+            zoo.conv_layer("m1@ssh_cls_score", "m1@ssh_output", "m1@ssh_cls_score_output", R + R // 2, 2 * A, 1,
+                           seed=7, std=0.3),
+            zoo.conv_layer("m1@ssh_bbox_pred", "m1@ssh_output", "m1@ssh_bbox_pred_output", R + R // 2, 4 * A, 1,
+                           seed=8, std=0.02),
+            {"name": "m1@ssh_cls_reshape", "type": "Reshape", "bottom": ["m1@ssh_cls_score_output"],
+             "top": ["m1@ssh_cls_score_reshape_output"], "reshape_param": {"shape": {"dim": [0, 2, -1, 0]}}},
+            {"name": "m1@ssh_cls_prob", "type": "Softmax", "bottom": ["m1@ssh_cls_score_reshape_output"],
+             "top": ["m1@ssh_cls_prob_output"]},
+            {"name": "m1@ssh_cls_prob_reshape", "type": "Reshape", "bottom": ["m1@ssh_cls_prob_output"],
+             "top": ["m1@ssh_cls_prob_reshape_output"], "reshape_param": {"shape": {"dim": [0, 2 * A, -1, 0]}}},
+            {"name": "m1@ssh_proposal", "type": "Proposal",
+             "bottom": ["m1@ssh_cls_prob_reshape_output", "m1@ssh_bbox_pred_output", "im_info"],
+             "top": ["m1@ssh_boxes", "m1@ssh_cls_prob"],
+             "proposal_param": {"feat_stride": 8, "scale": [1.0, 2.0], "ratio": [1.0], "min_size": 4,
+                                "nms_thresh": 0.3}}]
+    rng = np.random.default_rng(21)
+    inputs = {"conv4_3": rng.standard_normal((1, C, h8, w8)).astype(np.float32),
+              "conv5_3": rng.standard_normal((1, C, h16, w16)).astype(np.float32),
+              "im_info": np.array([[h8 * 8.0, w8 * 8.0, 1.0]], np.float32)}
+    marks = ["conv5_128_up", "conv5_128_crop", "conv4_fuse", "m1@ssh_output",
+             "m1@ssh_cls_prob_reshape_output", "m1@ssh_bbox_pred_output"]
+    net = run_net(gpu_mode, spec, inputs, marks)
+    want = netrun.oracle_forward(spec[:-1], inputs)
+    assert want["conv5_128_up"].shape == (1, R, 2 * h16, 2 * w16) and want["conv5_128_crop"].shape == (1, R, h8, w8)
+    for name in marks:
+        assert netrun.rel_err(net.get_blob(name).data, want[name]) < 1e-3, name
+    scores = net.get_blob("m1@ssh_cls_prob_reshape_output").data.copy()
+    boxes = net.get_blob("m1@ssh_bbox_pred_output").data.copy()
+    rois, probs = oracle.proposal(spec[-1]["proposal_param"], scores, boxes, inputs["im_info"], 2)
+    n = rois.shape[0]
+    assert 10 < n <= 300
+    assert np.array_equal(net.get_blob("m1@ssh_boxes").data[:n], rois)
+    assert np.array_equal(net.get_blob("m1@ssh_cls_prob").data.reshape(-1)[:n], probs)
