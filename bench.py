@@ -38,6 +38,10 @@ def main():
     ap.add_argument("--configs-report", metavar="PATH",
                     help="also time all five BASELINE configurations (whole forward, contraction "
                          "launches, Proposal / DetectionOutput layers) and write a text table to PATH")
+    ap.add_argument("--layer-scaling", metavar="PATH",
+                    help="also time representative ResNet-50 convolutions alone at batch 16..512 "
+                         "(how far a single launch is from the kernel's steady state) and write a "
+                         "text table to PATH")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="first run one plain 256 MiB device copy (mcCopy2D): under rocprofv3 --pmc "
                          "its FETCH_SIZE / WRITE_SIZE reading calibrates the counters")
@@ -105,6 +109,8 @@ def main():
 
     if args.configs_report:
         configs_report(args.configs_report, mc, craft, zoo, LIB)
+    if args.layer_scaling:
+        layer_scaling(args.layer_scaling)
 
     cpu = None
     if not args.no_cpu_baseline:
@@ -194,6 +200,49 @@ def configs_report(path, mc, craft, zoo, LIB):
         del net
     lines.append("CPU column: one pass of the oracle (reference algorithm: per-image im2col + OpenBLAS sgemm, "
                  "unfused layers) on %d host threads at batch 1/4/1/1/8/2." % oracle.openblas_threads())
+    with open(path, "w") as f:
+        f.write("\n".join(lines) + "\n")
+
+
+def layer_scaling(path):
+    """One convolution launch (ReLU epilogue) at growing batch sizes: time per launch and
+    TFLOP/s, through the kernel-level C ABI on torch-owned device memory."""
+    import torch
+    from minicaffe import kernels as K
+    # cin, height = width, cout, kernel, stride, pad: shapes of ResNet-50 stages 2-5
+    shapes = [(64, 56, 64, 3, 1, 1), (64, 56, 256, 1, 1, 0), (256, 56, 64, 1, 1, 0), (128, 28, 128, 3, 1, 1),
+              (256, 14, 256, 3, 1, 1), (1024, 14, 256, 1, 1, 0), (256, 14, 1024, 1, 1, 0),
+              (512, 7, 512, 3, 1, 1), (2048, 7, 512, 1, 1, 0)]
+    batches = (16, 32, 64, 128, 256, 512)
+    lines = ["%-22s" % "convolution" + "".join("%16s" % ("batch %d" % n) for n in batches)]
+    stream = torch.cuda.current_stream().cuda_stream
+    for cin, h, cout, k, s, p in shapes:
+        cells = []
+        for n in batches:
+            if n * max(cin, cout) * h * h > 2 ** 28:
+                cells.append("%16s" % "-")
+                continue
+            plan = K.ConvPlan(K.conv_geom(cin, h, h, cout, k, s, p))
+            ho, wo = plan.output_shape()
+            x = torch.randn(n, cin, h, h, device="cuda")
+            w = torch.randn(cout, cin, k, k, device="cuda") * 0.05
+            y = torch.empty(n, cout, ho, wo, device="cuda")
+            plan.set_weights(w.data_ptr())
+            for _ in range(3):
+                plan.forward(n, x.data_ptr(), y.data_ptr(), activation=K.ACT_RELU, stream=stream)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            reps = 10
+            e0.record()
+            for _ in range(reps):
+                plan.forward(n, x.data_ptr(), y.data_ptr(), activation=K.ACT_RELU, stream=stream)
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / reps
+            cells.append("%8.0f us %4.0f" % (ms * 1e3, plan.flops(n) / ms / 1e9))
+            del x, y, w, plan
+        lines.append("%-22s" % ("%d->%d %dx%d @%d" % (cin, cout, k, k, h)) + "".join(cells))
+    lines.append("cells: time per launch (10 back-to-back launches between two events) and TFLOP/s")
     with open(path, "w") as f:
         f.write("\n".join(lines) + "\n")
 
