@@ -184,8 +184,10 @@ def configs_report(path, mc, craft, zoo, LIB):
                     begin[e["name"]] = e["ts"]
                 elif e["name"] in begin:
                     spans.setdefault(e["name"], []).append(e["ts"] - begin.pop(e["name"]))
-            tail_txt = ", ".join("%s %.0f (median of %d)" % (t, sorted(spans[t])[len(spans[t]) // 2],
-                                                             len(spans[t])) for t in tails if t in spans)
+            # the profiler keeps the scopes of earlier configurations: the last `reps` are this net's
+            last = {t: spans[t][-reps:] for t in tails if t in spans}
+            tail_txt = ", ".join("%s %.0f (median of %d)" % (t, sorted(v)[len(v) // 2], len(v))
+                                 for t, v in last.items())
         cms = tot_ms.value / reps
         tf_s = fl.value / (tot_ms.value * 1e-3) / 1e12 if tot_ms.value else 0.0
         # CPU path (oracle restatement of the reference, OpenBLAS sgemm, all host cores): one

@@ -216,6 +216,50 @@ __global__ __launch_bounds__(kSortThreads) void det_class_nms_kernel(
                        eta, &kept_count[seg]);
 }
 
+// The greedy pass for a constant threshold (eta == 1) as a bit matrix and a scan.
+// All threads of the workgroup fill row k of `mask` with one bit per later
+// candidate r > k: set when candidate r would be rejected against a kept k, the
+// same expression the greedy pass evaluates (the overlap is symmetric in its two
+// boxes bit for bit).  Then one wavefront walks the candidates in order: lane w
+// holds word w of the "rejected" set; a candidate whose bit is clear is kept and
+// its row is OR-ed into the set.  `words` = ceil(ncand / 64) <= 64.
+template <typename IT>
+__device__ __forceinline__ void greedy_nms_mask(int ncand, const IT* cand_idx, const DBox* cand_box,
+                                                unsigned long long* mask, int* kept, float nms_thr,
+                                                int* kept_count_out) {
+  const int words = (ncand + 63) >> 6;
+  for (int item = threadIdx.x; item < ncand * words; item += kSortThreads) {
+    const int k = item / words, w = item - k * words;
+    unsigned long long bits = 0;
+    if (64 * w + 63 > k) {
+      const DBox kb = cand_box[k];
+      const int r0 = max(64 * w, k + 1), r1 = min(64 * w + 64, ncand);
+      for (int r = r0; r < r1; ++r)
+        bits |= static_cast<unsigned long long>(!(jaccard(cand_box[r], kb) <= nms_thr)) << (r & 63);
+    }
+    mask[item] = bits;
+  }
+  __syncthreads();
+  if (threadIdx.x >= 64) return;
+  const int lane = threadIdx.x;
+  unsigned rej_lo = 0, rej_hi = 0;  // word `lane` of the rejected set
+  int nkept = 0;
+  for (int r = 0; r < ncand; ++r) {
+    // the row is fetched before the decision so that its latency overlaps the test
+    const unsigned long long row = lane < words ? mask[r * words + lane] : 0ull;
+    const int w = r >> 6;
+    const unsigned half = (r & 32) ? __builtin_amdgcn_readlane(rej_hi, w)
+                                   : __builtin_amdgcn_readlane(rej_lo, w);
+    if (!((half >> (r & 31)) & 1u)) {
+      if (lane == 0) kept[nkept] = static_cast<int>(cand_idx[r]);
+      ++nkept;
+      rej_lo |= static_cast<unsigned>(row);
+      rej_hi |= static_cast<unsigned>(row >> 32);
+    }
+  }
+  if (lane == 0) *kept_count_out = nkept;
+}
+
 // The same for P <= kDetLdsMax priors: scores are keyed straight into LDS and
 // sorted there (no global scratch traffic), the sorted prior indices double as
 // the candidate list.
@@ -227,7 +271,7 @@ __global__ __launch_bounds__(kSortThreads) void det_class_nms_lds_kernel(
     int loc_classes, int background, float conf_thr, float nms_thr, float eta, int top_k,
     int max_cand, int* __restrict__ kept_idx, int* __restrict__ kept_count) {
   __shared__ BlockSortLds16 lds;
-  __shared__ uint32_t s_key[kDetLdsMax];
+  __shared__ __attribute__((aligned(8))) uint32_t s_key[kDetLdsMax];
   __shared__ unsigned short s_val[kDetLdsMax];
   __shared__ DBox cand_box[kDetCandBoxes];
   __shared__ DBox kept_box[kKeptLds];
@@ -257,6 +301,15 @@ __global__ __launch_bounds__(kSortThreads) void det_class_nms_lds_kernel(
   const int n_cached = min(ncand, kDetCandBoxes);
   for (int r = threadIdx.x; r < n_cached; r += kSortThreads) cand_box[r] = cls_boxes[s_val[r]];
   __syncthreads();
+  // constant threshold and a bit matrix that fits the (now free) key storage:
+  // overlaps in parallel, then a scan; otherwise the greedy pass of one wavefront
+  if (eta >= 1.f && ncand <= kDetCandBoxes &&
+      ncand * ((ncand + 63) >> 6) <= static_cast<int>(sizeof(s_key) / sizeof(unsigned long long))) {
+    greedy_nms_mask<unsigned short>(ncand, s_val, cand_box,
+                                    reinterpret_cast<unsigned long long*>(s_key),
+                                    kept_idx + (size_t)seg * max_cand, nms_thr, &kept_count[seg]);
+    return;
+  }
   if (threadIdx.x >= 64) return;  // the greedy pass is one wavefront
   greedy_nms_wave<unsigned short>(threadIdx.x, ncand, n_cached, s_val, cand_box, cls_boxes, kept_box,
                                   kept_idx + (size_t)seg * max_cand, nms_thr, eta,

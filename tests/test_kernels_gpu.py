@@ -426,6 +426,13 @@ def test_proposal_bit_exact(K, hw, pre, post, thr, quant):
     (1, 2000, 21, True, "CENTER_SIZE", 200, 0.01, 0.45, 1.0, 400, 0.5),
     (1, 13000, 3, True, "CENTER_SIZE", 100, 0.01, 0.45, 1.0, 1500, 2.0),   # sort through global scratch,
                                                                            # more candidates than cached
+    # candidate counts around the limits of the bit-matrix form of the greedy pass (constant threshold)
+    (2, 3000, 3, True, "CENTER_SIZE", -1, 0.001, 0.45, 1.0, 576, 1.0),     # largest matrix that fits
+    (2, 3000, 3, True, "CENTER_SIZE", -1, 0.001, 0.45, 1.0, 577, 1.0),     # one more: one-wavefront pass
+    (2, 3000, 3, True, "CENTER_SIZE", -1, 0.001, 0.3, 1.0, 64, 1.0),       # exactly one word
+    (2, 3000, 3, True, "CENTER_SIZE", -1, 0.001, 0.3, 1.0, 65, 1.0),
+    (2, 3000, 4, False, "CORNER", -1, 0.001, 0.7, 1.0, 1, 1.0),            # a single candidate per class
+    (1, 400, 2, True, "CENTER_SIZE", -1, None, 0.05, 1.0, None, 1.0),      # low threshold: long reject chains
 ])
 def test_detection_output_bit_exact(K, num, P, C, share, code, keep, thr, nms, eta, topk, sigma):
     rng = np.random.default_rng(12)
