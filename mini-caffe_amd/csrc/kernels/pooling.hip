@@ -53,6 +53,57 @@ __global__ __launch_bounds__(256) void pool_kernel(const PoolArgs a) {
   }
 }
 
+// Max pooling with a compile-time window and stride, padding 0 or more, for the
+// shapes the model zoo uses (3x3/2 ResNet stem, 2x2/2 VGG, 3x3/1 SSD pool5): one
+// thread makes two vertically adjacent outputs of a column, so the rows the two
+// windows share are read once, all loads are issued before the first compare, and
+// there is no loop-carried address arithmetic.  Neighbouring threads take
+// neighbouring output columns.
+template <int KH, int KW, int SH, int SW>
+__global__ __launch_bounds__(256) void max_pool_fixed_kernel(const PoolArgs a, int row_pairs,
+                                                             long count) {
+  constexpr int ROWS = SH + KH;  // input rows under two vertically adjacent windows
+  const long i = blockIdx.x * 256L + threadIdx.x;
+  if (i >= count) return;
+  const int ow = static_cast<int>(i % a.Wo);
+  const long t = i / a.Wo;
+  const int op = static_cast<int>(t % row_pairs);
+  const long plane = t / row_pairs;
+  const int oh = 2 * op;
+  const float* __restrict__ xp = a.x + plane * a.H * a.W;
+  const int h0 = oh * SH - a.ph, w0 = ow * SW - a.pw;
+  float v[ROWS][KW];
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) {
+    const int h = h0 + r;
+    const bool hok = h >= 0 && h < a.H;
+#pragma unroll
+    for (int c = 0; c < KW; ++c) {
+      const int w = w0 + c;
+      v[r][c] = (hok && w >= 0 && w < a.W) ? xp[h * a.W + w] : -FLT_MAX;
+    }
+  }
+  float m0 = -FLT_MAX, m1 = -FLT_MAX;
+#pragma unroll
+  for (int r = 0; r < KH; ++r)
+#pragma unroll
+    for (int c = 0; c < KW; ++c) {
+      m0 = fmaxf(m0, v[r][c]);
+      m1 = fmaxf(m1, v[r + SH][c]);
+    }
+  float* __restrict__ yp = a.y + (plane * a.Ho + oh) * a.Wo + ow;
+  yp[0] = m0;
+  if (oh + 1 < a.Ho) yp[a.Wo] = m1;
+}
+
+template <int KH, int KW, int SH, int SW>
+void launch_max_pool_fixed(const PoolArgs& a, long planes, hipStream_t st) {
+  const int row_pairs = (a.Ho + 1) / 2;
+  const long count = planes * row_pairs * a.Wo;
+  max_pool_fixed_kernel<KH, KW, SH, SW>
+      <<<ceil_div(count, 256), 256, 0, st>>>(a, row_pairs, count);
+}
+
 // One wavefront per plane; 4 planes per 256-thread workgroup.
 template <int METHOD>
 __global__ __launch_bounds__(256) void global_pool_kernel(const float* __restrict__ x,
@@ -134,6 +185,19 @@ int mcPooling(int method, const float* bottom, float* top, int planes, int H, in
   a.sw = sw;
   a.ph = ph;
   a.pw = pw;
+  if (method == MC_POOL_MAX && a.total < (1L << 31)) {
+    // every window holds at least one element (the output shape guarantees it), so
+    // the padding value never reaches the output
+    bool done = true;
+    if (kh == 3 && kw == 3 && sh == 2 && sw == 2) launch_max_pool_fixed<3, 3, 2, 2>(a, planes, st);
+    else if (kh == 2 && kw == 2 && sh == 2 && sw == 2) launch_max_pool_fixed<2, 2, 2, 2>(a, planes, st);
+    else if (kh == 3 && kw == 3 && sh == 1 && sw == 1) launch_max_pool_fixed<3, 3, 1, 1>(a, planes, st);
+    else done = false;
+    if (done) {
+      MC_LAUNCH_CHECK();
+      return 0;
+    }
+  }
   const int blocks = ew_blocks(a.total, 256);
   if (method == MC_POOL_MAX) pool_kernel<MC_POOL_MAX><<<blocks, 256, 0, st>>>(a);
   else pool_kernel<MC_POOL_AVE><<<blocks, 256, 0, st>>>(a);

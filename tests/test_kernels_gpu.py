@@ -281,7 +281,10 @@ def test_batch_norm_batch_stats(K):
 
 @pytest.mark.parametrize("method", ["MAX", "AVE"])
 @pytest.mark.parametrize("hw,k,s,p", [((112, 112), 3, 2, 0), ((75, 75), 2, 2, 0), ((19, 19), 3, 1, 1),
-                                      ((7, 7), 7, 1, 0), ((6, 6), 2, 2, 1), ((9, 13), 3, 3, 1)])
+                                      ((7, 7), 7, 1, 0), ((6, 6), 2, 2, 1), ((9, 13), 3, 3, 1),
+                                      # fixed-window max kernels: odd output heights, padding, 1-wide maps
+                                      ((10, 7), 2, 2, 0), ((13, 9), 3, 2, 0), ((5, 9), 3, 2, 1), ((6, 1), 3, 1, 1),
+                                      ((3, 3), 3, 2, 0), ((300, 300), 2, 2, 0)])
 def test_pooling(K, method, hw, k, s, p):
     x = np.random.default_rng(5).standard_normal((2, 5) + hw).astype(np.float32)
     want = oracle.pooling(x, method, (k, k), (s, s), (p, p))
