@@ -108,6 +108,44 @@ def test_reshape_and_batch_invariance(gpu_mode):
     assert netrun.rel_err(net.get_blob("prob").data, want) < 1e-3
 
 
+def test_three_threads_each_with_their_own_net(gpu_mode):
+    """The reference's concurrency smoke test (tests/run_net.cpp:238-246): every
+    thread selects the device itself, builds and runs its own net and clears its
+    own memory pool.  Here each thread's result is also checked against the oracle."""
+    import threading
+    from minicaffe import zoo
+    oracle.use_openblas(False)
+    jobs = []
+    for t in range(3):
+        spec, inputs = zoo.resnet50_spec(batch=2 + t, size=48 + 16 * t, stages=(1, 1, 1, 1), width=8,
+                                         num_classes=7, bn_seed=10 + t, seed=20 + t)
+        jobs.append((spec, inputs, netrun.oracle_forward(spec, inputs)["prob"]))
+    got, errors = [None] * 3, []
+
+    def work(t):
+        try:
+            gpu_mode.set_runtime_mode(1, 0)
+            spec, inputs, _ = jobs[t]
+            net = run_net(gpu_mode, spec, inputs)
+            for _ in range(3):
+                net.forward()
+            got[t] = net.get_blob("prob").data.copy()
+            del net                      # a net is destroyed on the thread that ran it
+            gpu_mode.memory_pool_clear()
+        except Exception as e:           # noqa: BLE001 - reported by the main thread
+            errors.append((t, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(3)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=100)
+    assert not errors, errors
+    for t in range(3):
+        assert got[t] is not None and got[t].shape == jobs[t][2].shape
+        assert netrun.rel_err(got[t], jobs[t][2]) < 1e-3, t
+
+
 def test_unfused_layers_standalone(gpu_mode):
     """BatchNorm / Scale / Bias / ReLU / TanH / Sigmoid / Eltwise that do NOT follow a
     contraction run as their own kernels; Split, Slice, Concat, Flatten, Reshape,
