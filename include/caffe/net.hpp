@@ -87,8 +87,9 @@ class CAFFE_API Net {
   vector<vector<int> > top_id_vecs_;
   // layers whose work was folded into an earlier layer's kernel
   vector<char> layer_fused_;
-  // for a sum folded into the layer that produces one of its inputs: the blob
-  // id whose memory the sum's top aliases, else -1 (indexed by layer)
+  // for a sum folded into the layer that produces one of its inputs, and for a
+  // skipped view (Flatten, Reshape): the blob id whose memory the layer's top
+  // aliases, else -1 (indexed by layer)
   vector<int> residual_alias_;
   // shapes of all blobs at the last PlaceMemory
   vector<vector<int> > placed_shapes_;

@@ -707,7 +707,9 @@ int pick_split(const mcConvPlan* plan, long blocks, int KT) {
   if (blocks * 2 > slots) return 1;
   int s = static_cast<int>(slots / blocks);
   s = std::min(s, KT / 8);
-  s = std::min(s, 8);
+  // A launch of a few dozen workgroups (detection heads on small maps) is pure
+  // latency: its time is the number of K tiles per slice, so it takes finer slices.
+  s = std::min(s, blocks * 10 <= kNumCu ? 24 : 8);
   return std::max(s, 1);
 }
 

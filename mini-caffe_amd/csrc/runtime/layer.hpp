@@ -99,6 +99,10 @@ class Layer {
   // activation (its own followers end without an activation).
   virtual bool AcceptsResidual() const { return false; }
   virtual void SetResidual(Blob* residual, Layer* activation) {}
+  // True when the top holds the bottom's values in the same order under another
+  // shape (Flatten, Reshape).  When nothing reads the bottom afterwards Net lets
+  // the top take over the bottom's memory and skips the layer's copy.
+  virtual bool IsView() const { return false; }
 
  protected:
   LayerParameter layer_param_;

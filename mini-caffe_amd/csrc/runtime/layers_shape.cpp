@@ -162,6 +162,7 @@ class FlattenLayer : public Layer {
  public:
   explicit FlattenLayer(const LayerParameter& param) : Layer(param) {}
   const char* type() const override { return "Flatten"; }
+  bool IsView() const override { return true; }
   int ExactNumBottomBlobs() const override { return 1; }
   int ExactNumTopBlobs() const override { return 1; }
   void Reshape(const vector<Blob*>& bottom, const vector<Blob*>& top) override {
@@ -187,6 +188,7 @@ class ReshapeLayer : public Layer {
  public:
   explicit ReshapeLayer(const LayerParameter& param) : Layer(param) {}
   const char* type() const override { return "Reshape"; }
+  bool IsView() const override { return true; }
   int ExactNumBottomBlobs() const override { return 1; }
   int ExactNumTopBlobs() const override { return 1; }
   void LayerSetUp(const vector<Blob*>& bottom, const vector<Blob*>& top) override {

@@ -156,8 +156,9 @@ void Net::PlaceMemory() {
 
   typedef std::pair<size_t, Blob*> BlobPair;
   std::multimap<size_t, Blob*> pool;
-  // A blob that a folded sum's top aliases lives on under that top's name: it
-  // is handed back to the pool when the top dies, not when the blob does.
+  // A blob that the top of a folded sum or of a view aliases lives on under that
+  // top's name: it is handed back to the pool when the top dies, not when the
+  // blob does.
   std::set<int> kept_alive;
   for (int id : residual_alias_)
     if (id >= 0) kept_alive.insert(id);
@@ -167,7 +168,7 @@ void Net::PlaceMemory() {
     vector<Blob*>& tops = top_vecs_[i];
     vector<BlobPair> to_place;
     if (residual_alias_[i] >= 0) {
-      // folded sum: no scratch, and the top is the producer's blob under a new name
+      // folded sum or view: no scratch, and the top is the aliased blob under a new name
       temps.clear();
       tops[0]->ResetMemory();
       tops[0]->ShareData(*blobs_[residual_alias_[i]]);
@@ -279,6 +280,20 @@ void Net::PlanFusion() {
     layers_[c]->SetResidual(R, layers_[e]->AbsorbedActivation());
     layer_fused_[e] = 1;
     residual_alias_[e] = t_id;
+  }
+
+  // Views (Flatten, Reshape; the reference copies, src/layers/flatten_layer.cpp:34-39,
+  // reshape_layer.cpp:98-103): when the view is the last reader of its bottom and
+  // the bottom is neither a net input nor a marked output, the top takes over the
+  // bottom's memory and the copy is skipped.
+  for (size_t v = 0; v < layers_.size(); ++v) {
+    if (layer_fused_[v] || !layers_[v]->IsView()) continue;
+    if (bottom_vecs_[v].size() != 1 || top_vecs_[v].size() != 1) continue;
+    if (bottom_vecs_[v][0] == top_vecs_[v][0]) continue;
+    const int b_id = bottom_id_vecs_[v][0];
+    if (blob_life_time_[b_id] != static_cast<int>(v)) continue;
+    layer_fused_[v] = 1;
+    residual_alias_[v] = b_id;
   }
 }
 

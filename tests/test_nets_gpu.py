@@ -146,6 +146,48 @@ def test_three_threads_each_with_their_own_net(gpu_mode):
         assert netrun.rel_err(got[t], jobs[t][2]) < 1e-3, t
 
 
+def test_flatten_and_reshape_as_views(gpu_mode):
+    """Flatten and Reshape take over their bottom's memory when they are its last
+    reader; a bottom that is read again, is a net input or is a marked output is
+    copied.  All variants give the reference's values, on repeated passes and
+    across a reshape of the input."""
+    from minicaffe.craft import input_layer
+    rng = np.random.default_rng(5)
+    f = lambda *s: rng.standard_normal(s).astype(np.float32)
+    spec = [
+        input_layer({"data": (2, 3, 6, 5)}),
+        {"name": "in_flat", "type": "Flatten", "bottom": ["data"], "top": ["in_flat"]},          # input: copied
+        {"name": "conv", "type": "Convolution", "bottom": ["data"], "top": ["conv"],
+         "convolution_param": {"num_output": 4, "kernel_size": 3, "pad": 1}, "blobs": [f(4, 3, 3, 3) * 0.3, f(4)]},
+        {"name": "perm", "type": "Permute", "bottom": ["conv"], "top": ["perm"], "permute_param": {"order": [0, 2, 3, 1]}},
+        {"name": "flat", "type": "Flatten", "bottom": ["perm"], "top": ["flat"]},                  # view
+        {"name": "resh", "type": "Reshape", "bottom": ["flat"], "top": ["resh"],
+         "reshape_param": {"shape": {"dim": [0, -1, 4]}}},                                         # view of a view
+        {"name": "sm", "type": "Softmax", "bottom": ["resh"], "top": ["sm"], "softmax_param": {"axis": 2}},
+        {"name": "sm_flat", "type": "Flatten", "bottom": ["sm"], "top": ["sm_flat"]},              # view
+        {"name": "relu", "type": "ReLU", "bottom": ["sm_flat"], "top": ["sm_flat"]},               # in place on a view
+        {"name": "conv_flat", "type": "Flatten", "bottom": ["conv"], "top": ["conv_flat"]},        # conv read again below
+        {"name": "pool", "type": "Pooling", "bottom": ["conv"], "top": ["pool"],
+         "pooling_param": {"kernel_size": 2, "stride": 2}},
+        {"name": "pool_flat", "type": "Flatten", "bottom": ["pool"], "top": ["pool_flat"]},        # pool is marked
+        {"name": "cat", "type": "Concat", "bottom": ["in_flat", "sm_flat", "conv_flat", "pool_flat"], "top": ["cat"]},
+    ]
+    x = f(2, 3, 6, 5)
+    net = run_net(gpu_mode, spec, {"data": x}, ["pool", "resh"])
+    want = netrun.oracle_forward(spec, {"data": x})
+    for _ in range(2):
+        assert netrun.rel_err(net.get_blob("cat").data, want["cat"]) < 1e-5
+        assert netrun.rel_err(net.get_blob("pool").data, want["pool"]) < 1e-5
+        assert netrun.rel_err(net.get_blob("resh").data, want["resh"]) < 1e-5
+        net.forward()
+    x3 = f(3, 3, 9, 4)
+    net.forward(data=x3)
+    want = netrun.oracle_forward(spec, {"data": x3})
+    assert net.get_blob("cat").data.shape == want["cat"].shape
+    assert netrun.rel_err(net.get_blob("cat").data, want["cat"]) < 1e-5
+    assert netrun.rel_err(net.get_blob("resh").data, want["resh"]) < 1e-5
+
+
 def test_unfused_layers_standalone(gpu_mode):
     """BatchNorm / Scale / Bias / ReLU / TanH / Sigmoid / Eltwise that do NOT follow a
     contraction run as their own kernels; Split, Slice, Concat, Flatten, Reshape,
