@@ -574,51 +574,137 @@ __global__ __launch_bounds__(64) void nms_mask_kernel(const float4* __restrict__
   mask[(size_t)i * nb + cb] = bits;
 }
 
-// One wavefront walks the boxes in score order.  Lane l owns words l, l+64, ...
-// of the running "removed" bitmap.  Per block of 64 boxes: the block's removed
-// word and the 64 diagonal mask words are brought into lanes, the 64 greedy
-// decisions are taken with wave broadcasts (no memory in the loop), then the
-// rows of the boxes that were kept are OR-ed into the bitmap.
-__global__ __launch_bounds__(64) void nms_scan_kernel(const unsigned long long* __restrict__ mask,
-                                                      int n, int nb, int max_keep,
-                                                      int* __restrict__ kept,
-                                                      int* __restrict__ num_kept) {
+// Greedy scan over the boxes in score order, one workgroup.  The decisions are a
+// dependent chain, so nothing on that chain may wait for global memory:
+//   * the boxes are taken in super-blocks of kScanBlocks * 64; the part of the
+//     mask that relates the boxes of one super-block to each other (64 bytes per
+//     box) is staged in LDS; the next super-block's part is fetched into
+//     registers while this one is decided and stored once the decisions are done;
+//   * wavefront 0 decides: per block of 64 boxes the running "removed" word and
+//     the candidates live in scalar registers, so only the boxes that are kept
+//     cost an iteration (a lane read of their diagonal word); the rows of kept
+//     boxes are folded into the later words of the same super-block from LDS;
+//   * after a super-block the whole workgroup folds the rows of its kept boxes
+//     into the removed words of all later super-blocks (independent loads, one
+//     latency per super-block instead of one per block).
+// Words left of the diagonal are never written by nms_mask_kernel and never used.
+constexpr int kScanThreads = 512;
+constexpr int kScanBlocks = 8;                    // blocks of 64 boxes per super-block
+constexpr int kScanRows = kScanBlocks * 64;       // boxes per super-block
+constexpr int kScanLoads = kScanRows * kScanBlocks / kScanThreads;  // staged words per thread
+
+__device__ inline unsigned long long wave_uniform(unsigned long long v) {
+  const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v));
+  const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v >> 32));
+  return (static_cast<unsigned long long>(hi) << 32) | lo;
+}
+
+__global__ __launch_bounds__(kScanThreads) void nms_scan_kernel(
+    const unsigned long long* __restrict__ mask, int n, int nb, int max_keep,
+    int* __restrict__ kept, int* __restrict__ num_kept) {
   extern __shared__ unsigned long long removed[];  // nb words
-  const int lane = threadIdx.x;
-  for (int w = lane; w < nb; w += 64) removed[w] = 0;
+  __shared__ unsigned long long sub[kScanRows * kScanBlocks];
+  __shared__ int sb_kept[kScanRows];
+  __shared__ int s_count, s_ns;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const bool decider = tid < 64;
+  // word `c` of the super-block's row `r`, 0 outside the mask
+  auto fetch = [&](int base_blk, int idx) -> unsigned long long {
+    const int r = idx / kScanBlocks, c = idx % kScanBlocks;
+    const long row = static_cast<long>(base_blk) * 64 + r;
+    const int col = base_blk + c;
+    return (row < n && col < nb) ? mask[row * nb + col] : 0ull;
+  };
+  for (int w = tid; w < nb; w += kScanThreads) removed[w] = 0;
+#pragma unroll
+  for (int k = 0; k < kScanLoads; ++k) sub[tid + k * kScanThreads] = fetch(0, tid + k * kScanThreads);
+  if (tid == 0) {
+    s_count = 0;
+    s_ns = 0;
+  }
   __syncthreads();
-  int count = 0;
-  for (int blk = 0; blk < nb && count < max_keep; ++blk) {
-    const int i = blk * 64 + lane;
-    unsigned long long diag = i < n ? mask[(size_t)i * nb + blk] : 0ull;
-    unsigned long long rem = removed[blk];
-    const int bn = min(64, n - blk * 64);
-    unsigned long long keep_bits = 0;
-    for (int j = 0; j < bn && count < max_keep; ++j) {
-      if (!((rem >> j) & 1ull)) {
-        keep_bits |= 1ull << j;
-        if (lane == 0) kept[count] = blk * 64 + j;
-        ++count;
-        // broadcast row j's diagonal word
-        const unsigned lo = __shfl(static_cast<unsigned>(diag), j, 64);
-        const unsigned hi = __shfl(static_cast<unsigned>(diag >> 32), j, 64);
-        rem |= (static_cast<unsigned long long>(hi) << 32) | lo;
-      }
+  for (int base_blk = 0; base_blk < nb; base_blk += kScanBlocks) {
+    // next super-block's part of the mask, in flight while this one is decided
+    unsigned long long ahead[kScanLoads];
+    const bool more = base_blk + kScanBlocks < nb;
+    if (more) {
+#pragma unroll
+      for (int k = 0; k < kScanLoads; ++k)
+        ahead[k] = fetch(base_blk + kScanBlocks, tid + k * kScanThreads);
     }
-    // fold the kept rows into the words of later blocks
-    for (int w = blk + 1 + lane; w < nb; w += 64) {
-      unsigned long long acc = removed[w];
-      unsigned long long kb = keep_bits;
-      while (kb) {
-        const int j = __ffsll(static_cast<long long>(kb)) - 1;
-        kb &= kb - 1;
-        acc |= mask[(size_t)(blk * 64 + j) * nb + w];
+    if (decider) {
+      int count = __builtin_amdgcn_readfirstlane(s_count);
+      int ns = 0;
+      const unsigned long long* sm = sub;
+      for (int b = 0; b < kScanBlocks && base_blk + b < nb && count < max_keep; ++b) {
+        const int blk = base_blk + b;
+        const unsigned long long diag = sm[(b * 64 + lane) * kScanBlocks + b];
+        unsigned long long rem = wave_uniform(removed[blk]);
+        const int bn = min(64, n - blk * 64);
+        const unsigned long long valid = bn >= 64 ? ~0ull : ((1ull << bn) - 1ull);
+        unsigned long long avail = ~rem & valid;
+        unsigned long long keep_bits = 0;
+        while (avail != 0 && count < max_keep) {
+          const int j = __builtin_ctzll(avail);
+          keep_bits |= 1ull << j;
+          if (lane == 0) {
+            kept[count] = blk * 64 + j;
+            sb_kept[ns] = blk * 64 + j;
+          }
+          ++count;
+          ++ns;
+          const unsigned lo = __builtin_amdgcn_readlane(static_cast<unsigned>(diag), j);
+          const unsigned hi = __builtin_amdgcn_readlane(static_cast<unsigned>(diag >> 32), j);
+          rem |= (static_cast<unsigned long long>(hi) << 32) | lo;
+          avail = ~rem & valid & ~(((1ull << j) << 1) - 1ull);  // candidates after j
+        }
+        // rows kept in this block -> later words of the same super-block
+        const int wl = b + 1 + lane;
+        if (wl < kScanBlocks && base_blk + wl < nb) {
+          unsigned long long acc = 0, kb = keep_bits;
+          while (kb) {
+            const int j = __builtin_ctzll(kb);
+            kb &= kb - 1;
+            acc |= sm[(b * 64 + j) * kScanBlocks + wl];
+          }
+          if (acc) removed[base_blk + wl] |= acc;
+        }
+        __builtin_amdgcn_wave_barrier();
       }
-      removed[w] = acc;
+      if (lane == 0) {
+        s_count = count;
+        s_ns = ns;
+      }
     }
     __syncthreads();
+    const int ns = s_ns;
+    if (s_count >= max_keep || !more) break;
+    // rows kept in this super-block -> words of all later super-blocks
+    const int first = base_blk + kScanBlocks, far = nb - first;
+    const int total = ns * far;
+    for (int p0 = tid; p0 < total; p0 += 4 * kScanThreads) {
+      unsigned long long v[4];
+      int w[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int p = p0 + u * kScanThreads;
+        v[u] = 0;
+        w[u] = first;
+        if (p < total) {
+          const int k = p / far;
+          w[u] = first + (p - k * far);
+          v[u] = mask[static_cast<long>(sb_kept[k]) * nb + w[u]];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (v[u]) atomicOr(&removed[w[u]], v[u]);
+    }
+#pragma unroll
+    for (int k = 0; k < kScanLoads; ++k) sub[tid + k * kScanThreads] = ahead[k];
+    __syncthreads();
   }
-  if (lane == 0) *num_kept = count;
+  if (tid == 0) *num_kept = s_count;
 }
 
 // rois[r] = (0, x1, y1, x2, y2) of the r-th kept box (proposal_layer.cpp:187-203).
@@ -760,8 +846,8 @@ int mcProposal(const float* scores, const float* bbox, const float* im_info, con
   MC_LAUNCH_CHECK();
   nms_mask_kernel<<<dim3(nb, nb), 64, 0, st>>>(sboxes, pre, nms_thresh, nb, mask);
   MC_LAUNCH_CHECK();
-  nms_scan_kernel<<<1, 64, sizeof(unsigned long long) * nb, st>>>(mask, pre, nb, post_nms_topn,
-                                                                   kept, num_rois);
+  nms_scan_kernel<<<1, kScanThreads, sizeof(unsigned long long) * nb, st>>>(
+      mask, pre, nb, post_nms_topn, kept, num_rois);
   MC_LAUNCH_CHECK();
   proposal_gather_kernel<<<ceil_div(post_nms_topn, 256), 256, 0, st>>>(sboxes, sscores, kept,
                                                                        num_rois, rois, roi_scores);
