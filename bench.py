@@ -21,6 +21,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "mini-caffe_amd"))
 
 FP32_MFMA_PEAK_TFLOPS = 157.3
+HBM_PEAK_GBS = 8000.0
 # HBM bytes per convolution launch (mean over the 53 launches of one forward),
 # from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in
 # profiles/igemm_resnet50_b64_pmc_traffic.txt (algorithmic: 126.3e6).
@@ -42,6 +43,11 @@ def main():
                     help="also time representative ResNet-50 convolutions alone at batch 16..512 "
                          "(how far a single launch is from the kernel's steady state) and write a "
                          "text table to PATH")
+    ap.add_argument("--bandwidth-report", metavar="PATH",
+                    help="also time the HBM-bound kernels (pooling, eltwise, channel transform, "
+                         "softmax, permute, normalize, LRN, copies, depthwise convolution) alone at "
+                         "the shapes of the configurations and write GB/s against the 8 TB/s "
+                         "roofline to PATH")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="first run one plain 256 MiB device copy (mcCopy2D): under rocprofv3 --pmc "
                          "its FETCH_SIZE / WRITE_SIZE reading calibrates the counters")
@@ -111,6 +117,8 @@ def main():
         configs_report(args.configs_report, mc, craft, zoo, LIB)
     if args.layer_scaling:
         layer_scaling(args.layer_scaling)
+    if args.bandwidth_report:
+        bandwidth_report(args.bandwidth_report)
 
     cpu = None
     if not args.no_cpu_baseline:
@@ -247,6 +255,101 @@ def layer_scaling(path):
     lines.append("cells: time per launch (10 back-to-back launches between two events) and TFLOP/s")
     with open(path, "w") as f:
         f.write("\n".join(lines) + "\n")
+
+
+def bandwidth_report(path):
+    """The kernels whose bound is HBM, one launch at a time through the kernel-level C ABI
+    on torch-owned device memory: 20 warm-up launches, 100 launches timed one by one with
+    HIP events on the launch stream, median; algorithmic bytes = 4 * (elements read +
+    elements written), parameters left out."""
+    import statistics
+    import torch
+    from minicaffe import kernels as K
+    from minicaffe.base import LIB
+    stream = torch.cuda.current_stream().cuda_stream
+    P = ctypes.c_void_p
+    ints = lambda v: (ctypes.c_int * len(v))(*v)
+    dev = lambda *shape: torch.randn(*shape, device="cuda")
+    rows = []
+
+    def timed(name, nbytes, launch):
+        for _ in range(20):
+            rc = launch()
+            assert rc in (0, None), LIB.mcLastError()
+        torch.cuda.synchronize()
+        spans = []
+        for _ in range(100):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            launch()
+            e1.record()
+            spans.append((e0, e1))
+        torch.cuda.synchronize()
+        us = statistics.median(a.elapsed_time(b) for a, b in spans) * 1e3
+        gbs = nbytes / us / 1e3
+        rows.append("%-58s %9.1f MB %9.1f us %9.0f GB/s %6.1f %%" % (name, nbytes / 1e6, us, gbs, gbs / HBM_PEAK_GBS * 100))
+
+    def pool(name, method, planes, h, w, k, s_, pad):
+        ho, wo = ctypes.c_int(), ctypes.c_int()
+        LIB.mcPoolingOutputShape(h, w, k, k, s_, s_, pad, pad, ctypes.byref(ho), ctypes.byref(wo))
+        x, y = dev(planes, h, w), dev(planes, ho.value, wo.value)
+        timed(name, 4 * (x.numel() + y.numel()),
+              lambda: LIB.mcPooling(method, P(x.data_ptr()), P(y.data_ptr()), planes, h, w, k, k, s_, s_, pad, pad, P(stream)))
+
+    pool("Pooling MAX 3x3/2, 64x64x112x112 (ResNet-50 stem)", 0, 64 * 64, 112, 112, 3, 2, 0)
+    pool("Pooling MAX 2x2/2, 8x64x300x300 (SSD300 pool1)", 0, 8 * 64, 300, 300, 2, 2, 0)
+    pool("Pooling MAX 3x3/1 pad 1, 8x512x19x19 (SSD300 pool5)", 0, 8 * 512, 19, 19, 3, 1, 1)
+    pool("Pooling AVE 7x7 global, 64x2048x7x7 (ResNet-50 pool5)", 1, 64 * 2048, 7, 7, 7, 1, 0)
+
+    n, c, sp = 64, 256, 56 * 56
+    a, b, y = dev(n, c, sp), dev(n, c, sp), dev(n, c, sp)
+    bottoms = (ctypes.c_void_p * 2)(a.data_ptr(), b.data_ptr())
+    coeffs = (ctypes.c_float * 2)(1.0, 1.0)
+    timed("Eltwise SUM + ReLU, 2 x 64x256x56x56 (residual, unfused)", 4 * 3 * a.numel(),
+          lambda: LIB.mcEltwise(1, 2, bottoms, coeffs, a.numel(), P(y.data_ptr()), 1, 0.0, P(stream)))
+    mul, add = dev(c), dev(c)
+    op = K.ChannelOp(None, None, mul.data_ptr(), add.data_ptr(), 1, 0.0)
+    timed("channel transform x*g+b, ReLU, 64x256x56x56 (BN/Scale/ReLU)", 4 * 2 * a.numel(),
+          lambda: LIB.mcChannelTransform(P(a.data_ptr()), P(y.data_ptr()), n, c, sp, ctypes.byref(op), P(stream)))
+    timed("Unary ELU, 64x256x56x56", 4 * 2 * a.numel(),
+          lambda: LIB.mcUnary(5, P(a.data_ptr()), P(y.data_ptr()), a.numel(), 1.0, 0.0, 0.0, P(stream)))
+    timed("copy (Concat / Slice / Split), 64x256x56x56", 4 * 2 * a.numel(),
+          lambda: LIB.mcCopy2D(P(a.data_ptr()), a.numel(), P(y.data_ptr()), a.numel(), a.numel(), 1, P(stream)))
+    shape, order = ints([n, c, 56, 56]), ints([0, 2, 3, 1])
+    timed("Permute (0,2,3,1), 64x256x56x56", 4 * 2 * a.numel(),
+          lambda: LIB.mcPermute(P(a.data_ptr()), P(y.data_ptr()), 4, shape, order, P(stream)))
+    del a, b, y
+
+    x, y = dev(8, 84, 38, 38), dev(8, 84, 38, 38)
+    shape2 = ints([8, 84, 38, 38])
+    timed("Permute (0,2,3,1), 8x84x38x38 (SSD300 conv4_3 conf head)", 4 * 2 * x.numel(),
+          lambda: LIB.mcPermute(P(x.data_ptr()), P(y.data_ptr()), 4, shape2, order, P(stream)))
+    x, y = dev(8 * 8732, 21), dev(8 * 8732, 21)
+    timed("Softmax over 21 classes, 8x8732 rows (SSD300 mbox_conf)", 4 * 2 * x.numel(),
+          lambda: LIB.mcSoftmax(P(x.data_ptr()), P(y.data_ptr()), 8 * 8732, 21, 1, P(stream)))
+    x, y = dev(64, 1000), dev(64, 1000)
+    timed("Softmax over 1000 classes, 64 rows (ResNet-50 prob)", 4 * 2 * x.numel(),
+          lambda: LIB.mcSoftmax(P(x.data_ptr()), P(y.data_ptr()), 64, 1000, 1, P(stream)))
+    x, y, sc = dev(8, 512, 38 * 38), dev(8, 512, 38 * 38), dev(512)
+    timed("Normalize across channels, 8x512x38x38 (SSD300 conv4_3_norm)", 4 * 2 * x.numel(),
+          lambda: LIB.mcNormalize(P(x.data_ptr()), P(y.data_ptr()), 8, 512, 38 * 38, 0, 0, 1e-10, P(sc.data_ptr()), P(stream)))
+    x, y = dev(64, 96, 55, 55), dev(64, 96, 55, 55)
+    timed("LRN across 5 channels, 64x96x55x55 (AlexNet norm1)", 4 * 2 * x.numel(),
+          lambda: LIB.mcLRNAcrossChannels(P(x.data_ptr()), P(y.data_ptr()), 64, 96, 55, 55, 5, 1e-4, 0.75, 1.0, P(stream)))
+    for cin, h, s_ in ((512, 19, 1), (256, 38, 2), (64, 150, 1)):
+        plan = K.ConvPlan(K.conv_geom(cin, h, h, cin, 3, s_, 1, group=cin))
+        ho, wo = plan.output_shape()
+        x, w, y = dev(32, cin, h, h), dev(cin, 1, 3, 3), dev(32, cin, ho, wo)
+        plan.set_weights(w.data_ptr())
+        timed("depthwise 3x3/%d + ReLU, 32x%dx%dx%d (MobileNet)" % (s_, cin, h, h), 4 * (x.numel() + y.numel()),
+              lambda: plan.forward(32, x.data_ptr(), y.data_ptr(), activation=K.ACT_RELU, stream=stream))
+        del plan
+    head = ["%-58s %12s %12s %14s %8s" % ("kernel, shape", "alg. bytes", "median", "achieved", "of 8 TB/s")]
+    tail = ["20 warm-up + 100 launches timed one by one with HIP events, median.  Buffers smaller than the 256 MB",
+            "last-level cache can be served from it on repeated launches (as they are inside a net, where the",
+            "producer has just written them), so small shapes may read above what HBM alone would give."]
+    with open(path, "w") as f:
+        f.write("\n".join(head + rows + tail) + "\n")
 
 
 def cpu_baseline(batch):

@@ -22,11 +22,15 @@ __global__ __launch_bounds__(256) void normalize_pixel_kernel(
   const float* __restrict__ xp = x + (long)n * C * spatial + s;
   float* __restrict__ yp = y + (long)n * C * spatial + s;
   float acc = 0.f;
-  if (live)
+  if (live) {
+    // batches of 8 independent loads: the launch is small, so memory latency
+    // has to be covered inside a thread
+#pragma unroll 8
     for (int c = sl; c < C; c += kNormSlices) {
       const float v = xp[(long)c * spatial];
       acc += v * v;
     }
+  }
   part[sl][px] = acc;
   __syncthreads();
   float sum = eps;
@@ -34,6 +38,7 @@ __global__ __launch_bounds__(256) void normalize_pixel_kernel(
   for (int k = 0; k < kNormSlices; ++k) sum += part[k][px];
   const float norm = sqrtf(sum);
   if (live)
+#pragma unroll 8
     for (int c = sl; c < C; c += kNormSlices) {
       const float v = xp[(long)c * spatial] / norm;
       yp[(long)c * spatial] = v * (channel_shared ? scale[0] : scale[c]);

@@ -319,7 +319,10 @@ def test_eltwise(K, op, coeffs, count):
 
 
 @pytest.mark.parametrize("shape,axis", [((64, 1000), 1), ((8, 873, 21), 2), ((1, 2, 342, 63), 1),
-                                        ((3, 5, 7), 1), ((4, 1500), 1)])
+                                        ((3, 5, 7), 1), ((4, 1500), 1),
+                                        # rows that share a wavefront: every group width, ragged last wavefront
+                                        ((7, 1), 1), ((13, 2), 1), ((67, 4), 1), ((9, 5), 1), ((131, 16), 1),
+                                        ((5, 17), 1), ((3, 33), 1), ((6, 64), 1), ((6, 65), 1)])
 def test_softmax(K, shape, axis):
     x = (np.random.default_rng(7).standard_normal(shape) * 3).astype(np.float32)
     want = oracle.softmax(x, axis)
