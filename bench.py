@@ -43,6 +43,10 @@ def main():
                     help="also time representative ResNet-50 convolutions alone at batch 16..512 "
                          "(how far a single launch is from the kernel's steady state) and write a "
                          "text table to PATH")
+    ap.add_argument("--layer-roofline", metavar="PATH",
+                    help="also time the 20 distinct ResNet-50 convolutions alone at the bench batch "
+                         "and write, per layer, FLOPs, algorithmic bytes, the roofline that binds "
+                         "(fp32 MFMA or HBM) and the fraction reached to PATH")
     ap.add_argument("--bandwidth-report", metavar="PATH",
                     help="also time the HBM-bound kernels (pooling, eltwise, channel transform, "
                          "softmax, permute, normalize, LRN, copies, depthwise convolution) alone at "
@@ -117,6 +121,8 @@ def main():
         configs_report(args.configs_report, mc, craft, zoo, LIB)
     if args.layer_scaling:
         layer_scaling(args.layer_scaling)
+    if args.layer_roofline:
+        layer_roofline(args.layer_roofline, args.batch)
     if args.bandwidth_report:
         bandwidth_report(args.bandwidth_report)
 
@@ -253,6 +259,58 @@ def layer_scaling(path):
             del x, y, w, plan
         lines.append("%-22s" % ("%d->%d %dx%d @%d" % (cin, cout, k, k, h)) + "".join(cells))
     lines.append("cells: time per launch (10 back-to-back launches between two events) and TFLOP/s")
+    with open(path, "w") as f:
+        f.write("\n".join(lines) + "\n")
+
+
+def layer_roofline(path, batch):
+    """Every distinct convolution of ResNet-50 v1 alone (ReLU epilogue, no residual), one
+    launch at a time through the kernel-level C ABI: which roofline binds it and how close
+    the launch comes.  Bytes = bottom + top + filter, each once."""
+    import torch
+    from minicaffe import kernels as K
+    # cin, height = width, cout, kernel, stride, pad, number of layers of this shape
+    shapes = [(3, 224, 64, 7, 2, 3, 1), (64, 56, 256, 1, 1, 0, 4), (64, 56, 64, 1, 1, 0, 1), (64, 56, 64, 3, 1, 1, 3),
+              (256, 56, 64, 1, 1, 0, 2), (256, 56, 512, 1, 2, 0, 1), (256, 56, 128, 1, 2, 0, 1), (128, 28, 128, 3, 1, 1, 4),
+              (128, 28, 512, 1, 1, 0, 4), (512, 28, 128, 1, 1, 0, 3), (512, 28, 1024, 1, 2, 0, 1), (512, 28, 256, 1, 2, 0, 1),
+              (256, 14, 256, 3, 1, 1, 6), (256, 14, 1024, 1, 1, 0, 6), (1024, 14, 256, 1, 1, 0, 5),
+              (1024, 14, 2048, 1, 2, 0, 1), (1024, 14, 512, 1, 2, 0, 1), (512, 7, 512, 3, 1, 1, 3),
+              (512, 7, 2048, 1, 1, 0, 3), (2048, 7, 512, 1, 1, 0, 2)]
+    stream = torch.cuda.current_stream().cuda_stream
+    lines = ["%-24s %3s %8s %9s %8s %6s %9s %9s %9s %7s" % ("convolution (batch %d)" % batch, "x", "GFLOP", "MB", "FLOP/B",
+                                                           "bound", "roof us", "meas. us", "TFLOP/s", "of roof")]
+    sum_roof = sum_meas = 0.0
+    for cin, h, cout, k, s_, p_, cnt in shapes:
+        plan = K.ConvPlan(K.conv_geom(cin, h, h, cout, k, s_, p_))
+        ho, wo = plan.output_shape()
+        x = torch.randn(batch, cin, h, h, device="cuda")
+        w = torch.randn(cout, cin, k, k, device="cuda") * 0.05
+        y = torch.empty(batch, cout, ho, wo, device="cuda")
+        plan.set_weights(w.data_ptr())
+        for _ in range(5):
+            plan.forward(batch, x.data_ptr(), y.data_ptr(), activation=K.ACT_RELU, stream=stream)
+        torch.cuda.synchronize()
+        reps = 20
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            plan.forward(batch, x.data_ptr(), y.data_ptr(), activation=K.ACT_RELU, stream=stream)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / reps * 1e3
+        fl = plan.flops(batch)
+        nbytes = 4.0 * (x.numel() + y.numel() + w.numel())
+        t_mfma, t_hbm = fl / (FP32_MFMA_PEAK_TFLOPS * 1e6), nbytes / (HBM_PEAK_GBS * 1e3)
+        roof = max(t_mfma, t_hbm)
+        sum_roof += roof * cnt
+        sum_meas += us * cnt
+        lines.append("%-24s %3d %8.2f %9.1f %8.1f %6s %9.1f %9.1f %9.1f %6.1f%%" % (
+            "%d->%d %dx%d/%d @%d" % (cin, cout, k, k, s_, h), cnt, fl / 1e9, nbytes / 1e6, fl / nbytes,
+            "mfma" if t_mfma >= t_hbm else "hbm", roof, us, fl / us / 1e6, 100 * roof / us))
+        del x, y, w, plan
+    lines.append("all 53 convolutions: roofline %.0f us, measured %.0f us = %.1f%% of the per-layer roofline"
+                 % (sum_roof, sum_meas, 100 * sum_roof / sum_meas))
+    lines.append("roof us = max(FLOP / 157.3 TFLOP/s, bytes / 8 TB/s); 20 back-to-back launches between two events.")
     with open(path, "w") as f:
         f.write("\n".join(lines) + "\n")
 
