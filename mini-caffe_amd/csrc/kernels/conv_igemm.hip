@@ -565,6 +565,103 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(
   }
 }
 
+// Convolutions with at most kThinM output channels per group (the image-producing
+// last layer of a generator, a one-channel score map): a 32-row MFMA tile would
+// multiply mostly padding, and the layer is bound by reading its bottom blob
+// anyway.  One thread per output pixel walks the K rows of the same gather
+// (same tap table, same packed filter, read through scalar loads) and keeps the
+// kThinM sums in registers; neighbouring threads read neighbouring addresses.
+constexpr int kThinM = 4;
+__global__ __launch_bounds__(256) void thin_conv_kernel(const IgemmBatch batch, int pointwise) {
+  const IgemmArgs& a = batch.sub[blockIdx.z];
+  const int p = blockIdx.x * 256 + threadIdx.x;
+  const int g = blockIdx.y;
+  // the gather of igemm_kernel's kModeMasks: pixel origin in the VGPR offset of a
+  // buffer load, tap offset in its scalar offset, bit 31 for "outside the image"
+  const __amdgpu_buffer_rsrc_t xres =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.x), 0, a.x_bytes, kBufferFlags);
+  unsigned xvoff = kNoElement;
+  unsigned row_bad = 0xFFFFFFFFu, col_bad = 0xFFFFFFFFu;
+  int n = 0, qh = 0, qw = 0;
+  if (p < a.P) {
+    n = fast_div(p, a.div_hw_mul, a.div_hw_shift);
+    const int rem = p - n * a.HqWq;
+    qh = fast_div(rem, a.div_w_mul, a.div_w_shift);
+    qw = rem - qh * a.Wq;
+    const int hi0 = qh * a.q_sh + a.in_oh;
+    const int wi0 = qw * a.q_sw + a.in_ow;
+    xvoff = static_cast<unsigned>(
+        ((n * a.x_nstride + g * a.x_gstride + hi0 * a.W + wi0) << 2) + a.pix_shift);
+    row_bad = 0x80000000u;
+    col_bad = 0u;
+    for (int b = 0; b < a.n_dh; ++b)
+      row_bad |= static_cast<unsigned>(static_cast<unsigned>(hi0 + a.tap_dh[b]) >=
+                                       static_cast<unsigned>(a.H))
+                 << b;
+    for (int b = 0; b < a.n_dw; ++b)
+      col_bad |= static_cast<unsigned>(static_cast<unsigned>(wi0 + a.tap_dw[b]) >=
+                                       static_cast<unsigned>(a.W))
+                 << b;
+  }
+  const float* __restrict__ wg = a.wt + static_cast<size_t>(g) * a.Kpad * a.Mpad;
+  float acc[kThinM];
+#pragma unroll
+  for (int m = 0; m < kThinM; ++m) acc[m] = 0.f;
+#define MC_LOADF(res, voff, soff) \
+  __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(res, voff, soff, 0))
+  // K in tiles of 16 over the padded extent (padding rows have zero filters and,
+  // with a tap table, the never-valid tap): per tile the 4 x 16 filter values and
+  // the 16 table entries are contiguous, so they arrive in a few wide scalar loads.
+  const int kmax = a.K - 1;
+  const unsigned x_cbytes = static_cast<unsigned>(a.x_cstride) * 4;
+  auto gather16 = [&](int k0, float (&v)[BK]) {
+    if (pointwise) {
+#pragma unroll
+      for (int j = 0; j < BK; ++j)
+        v[j] = MC_LOADF(xres, xvoff, static_cast<unsigned>(min(k0 + j, kmax)) * x_cbytes);
+    } else {
+      const int4* __restrict__ tk = a.ktab + k0;
+#pragma unroll
+      for (int j = 0; j < BK; ++j) {
+        const int4 t = tk[j];
+        const unsigned rb = __builtin_amdgcn_ubfe(row_bad, t.y, 1);
+        const unsigned cb = __builtin_amdgcn_ubfe(col_bad, t.z, 1);
+        v[j] = MC_LOADF(xres, (cb << 31) | ((rb << 31) | xvoff), t.x);
+      }
+    }
+  };
+  // one K tile of 16 rows per step; the loads of the next tile are issued before
+  // this one is multiplied
+  float v[BK], ahead[BK];
+  if (a.Kpad > 0) gather16(0, v);
+  for (int k0 = 0; k0 < a.Kpad; k0 += BK) {
+    const float* __restrict__ wk = wg + (k0 >> 4) * (a.Mpad * BK);
+    if (k0 + BK < a.Kpad) gather16(k0 + BK, ahead);
+#pragma unroll
+    for (int j = 0; j < BK; ++j) {
+#pragma unroll
+      for (int m = 0; m < kThinM; ++m) acc[m] += wk[m * BK + j] * v[j];
+    }
+#pragma unroll
+    for (int j = 0; j < BK; ++j) v[j] = ahead[j];
+  }
+#undef MC_LOADF
+  if (p >= a.P) return;
+  const long ybase = static_cast<long>(n) * a.y_nstride +
+                     static_cast<long>(qh * a.out_sh + a.out_oh) * a.Wo + qw * a.out_sw + a.out_ow;
+#pragma unroll
+  for (int m = 0; m < kThinM; ++m) {
+    if (m >= a.M) break;
+    const int c = g * a.M + m;
+    const long idx = ybase + static_cast<long>(c) * a.y_cstride;
+    float v = acc[m];
+    if (a.scale) v *= a.scale[c];
+    if (a.shift) v += a.shift[c];
+    if (a.residual) v += a.residual[idx];
+    a.y[idx] = apply_act(v, a.act, a.slope);
+  }
+}
+
 // Packed filter wt[g][kt][m][kl] = w[g*wg_stride + wk_off[k] + m*wm_stride] with
 // k = kt*16 + kl, zero where k >= K or m >= M.
 __global__ void pack_weights_kernel(const float* __restrict__ w, float* __restrict__ wt,
@@ -701,6 +798,14 @@ int pick_config(const mcConvPlan* plan, long pixels) {
 // load latency on every K tile; slicing K brings the launch up to about one
 // full round of workgroups, each slice still long enough to amortise its
 // prologue and the extra pass that sums the slices.
+// A handful of output channels over many pixels goes to the per-pixel kernel.
+bool use_thin(const mcConvPlan* plan, int num) {
+  long total_pixels = 0;
+  for (const auto& s : plan->subs) total_pixels += (long)num * s.Hq * s.Wq;
+  return plan->M <= kThinM && plan->forced_config < 0 && plan->forced_split == 0 &&
+         total_pixels * plan->geom.group >= 65536;
+}
+
 int pick_split(const mcConvPlan* plan, long blocks, int KT) {
   if (plan->forced_split >= 1) return std::min(plan->forced_split, std::max(KT, 1));
   const long slots = 8L * kNumCu;
@@ -1095,9 +1200,10 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
     flops += 2.0 * pixels * plan->M * g.group * s->K;
   }
   if (min_kt == (1 << 30)) min_kt = 1;
+  const bool thin = use_thin(plan, num);
   // slices are chosen for the plan as a whole: all sub-problems of a launch run
   // side by side, and one pass sums the slices of the whole top blob
-  const int slices = pick_split(plan, total_blocks, min_kt);
+  const int slices = thin ? 1 : pick_split(plan, total_blocks, min_kt);
   const long slice_stride = (out_count + 3) / 4 * 4;
   float* ws = nullptr;
   if (slices > 1 && get_workspace(st, sizeof(float) * slice_stride * slices, &ws)) return -1;
@@ -1107,7 +1213,7 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
     MC_HIP(hipEventCreate(&tl.start));
     MC_HIP(hipEventCreate(&tl.stop));
     tl.flops = flops;
-    tl.name = cfg.name;
+    tl.name = thin ? "thin_f32" : cfg.name;
     MC_HIP(hipEventRecord(tl.start, st));
   }
   for (size_t first = 0; first < live.size(); first += kMaxSubs) {
@@ -1186,9 +1292,16 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
         a.act = MC_ACT_NONE;
       }
     }
-    dim3 grid(static_cast<unsigned>(max_blocks), g.group, nsub * slices);
-    cfg.kernel[pointwise ? kModePointwise : (one_mask ? kModeOneMask : kModeMasks)]<<<grid, 256, 0, st>>>(
-        batch);
+    if (thin) {
+      long most = 0;
+      for (int i = 0; i < nsub; ++i) most = std::max<long>(most, batch.sub[i].P);
+      dim3 grid(static_cast<unsigned>(ceil_div(most, 256L)), g.group, nsub);
+      thin_conv_kernel<<<grid, 256, 0, st>>>(batch, pointwise ? 1 : 0);
+    } else {
+      dim3 grid(static_cast<unsigned>(max_blocks), g.group, nsub * slices);
+      cfg.kernel[pointwise ? kModePointwise : (one_mask ? kModeOneMask : kModeMasks)]<<<grid, 256, 0, st>>>(
+          batch);
+    }
     MC_LAUNCH_CHECK();
   }
   if (slices > 1) {
@@ -1240,6 +1353,7 @@ double mcConvPlanFlops(const mcConvPlan* plan, int num) {
 const char* mcConvPlanKernelName(const mcConvPlan* plan, int num) {
   if (plan && plan->depthwise) return "depthwise_f32";
   if (!plan || plan->subs.empty()) return "";
+  if (use_thin(plan, num)) return "thin_f32";
   const auto& s = plan->subs[0];
   return kConfigs[pick_config(plan, (long)num * s.Hq * s.Wq)].name;
 }

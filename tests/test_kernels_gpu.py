@@ -34,6 +34,8 @@ def fptr(t):
     return ctypes.c_void_p(t.data_ptr())
 
 
+K_ACT_NONE, K_ACT_TANH = 0, 2
+
 CONV_CASES = [
     # cin, h, w, cout, k, s, p, d, g, transposed, batch
     (64, 56, 56, 64, 3, 1, 1, 1, 1, False, 1),      # config 1
@@ -79,6 +81,55 @@ def test_conv_forward(K, case, cfg):
     plan.forward(n, xd.data_ptr(), yd.data_ptr(), shift=bd.data_ptr())
     torch.cuda.synchronize()
     assert netrun.rel_err(yd.cpu().numpy(), want) < 1e-4
+
+
+THIN_CASES = [
+    (8, 96, 90, 3, 3, 1, 1, 1, 1, False, 8),        # 3x3 to 3 channels (one validity mask per tap pair)
+    (16, 96, 90, 1, 1, 1, 0, 1, 1, False, 8),       # 1x1 score map: pointwise path
+    (8, 40, 44, 3, 4, 2, 1, 1, 1, True, 10),        # generator's last layer: deconv 4x4/2 to RGB, 4 output classes
+    (8, 64, 64, 8, 3, 2, 1, 1, 2, False, 33),       # two groups of 4 outputs, stride 2
+    (3, 200, 180, 4, 7, 2, 3, 1, 1, False, 8),      # 7x7/2 from 3 channels (row and column masks)
+    (4, 90, 100, 2, 3, 1, 2, 2, 1, False, 8),       # dilated
+]
+
+
+@pytest.mark.parametrize("case", THIN_CASES)
+@pytest.mark.parametrize("act", [K_ACT_NONE, K_ACT_TANH])
+def test_conv_few_output_channels(K, case, act):
+    """At most 4 output channels per group over many pixels: the per-pixel kernel,
+    with the whole epilogue, against the oracle's convolution + the same tail."""
+    cin, h, w, cout, k, s, p, d, g, tr, n = case
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((n, cin, h, w)).astype(np.float32)
+    wshape = (cin, cout // g, k, k) if tr else (cout, cin // g, k, k)
+    wt = (rng.standard_normal(wshape) * 0.2).astype(np.float32)
+    sc = (rng.random(cout) + 0.5).astype(np.float32)
+    sh = rng.standard_normal(cout).astype(np.float32)
+    y = oracle.conv_forward(oracle.conv_geom(cin, h, w, cout, k, s, p, d, g, tr), x, wt, None)
+    res = rng.standard_normal(y.shape).astype(np.float32)
+    want = y * sc[None, :, None, None] + sh[None, :, None, None] + res
+    if act == K_ACT_TANH:
+        want = np.tanh(want.astype(np.float64)).astype(np.float32)
+    plan = K.ConvPlan(K.conv_geom(cin, h, w, cout, k, s, p, d, g, tr))
+    assert plan.kernel_name(n) == "thin_f32"
+    xd, wd, scd, shd, rd = dev(x), dev(wt), dev(sc), dev(sh), dev(res)
+    yd = torch.full(want.shape, float("nan"), device="cuda")
+    plan.set_weights(wd.data_ptr())
+    plan.forward(n, xd.data_ptr(), yd.data_ptr(), scale=scd.data_ptr(), shift=shd.data_ptr(),
+                 residual=rd.data_ptr(), activation=act)
+    torch.cuda.synchronize()
+    got = yd.cpu().numpy()
+    # tanh outputs near 0 carry the absolute error of sums of magnitude ~10: absolute bound there
+    close = (lambda a, b: np.abs(a - b).max() < 1e-5) if act == K_ACT_TANH else \
+        (lambda a, b: netrun.rel_err(a, b) < 1e-4)
+    assert close(got, want)
+    # the matrix-core kernel on the same problem agrees
+    plan.force_config(4)
+    y2 = torch.full(want.shape, float("nan"), device="cuda")
+    plan.forward(n, xd.data_ptr(), y2.data_ptr(), scale=scd.data_ptr(), shift=shd.data_ptr(),
+                 residual=rd.data_ptr(), activation=act)
+    torch.cuda.synchronize()
+    assert close(y2.cpu().numpy(), got)
 
 
 def test_conv_epilogue_matches_unfused_chain(K):
