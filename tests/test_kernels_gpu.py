@@ -452,6 +452,13 @@ def run_proposal(K, scores, bbox, im_info, param):
     ((5, 4), 100, 300, 0.3, 0),
     ((50, 60), 6000, 300, 0.7, 0),       # 27000 proposals: sort through global scratch
     ((50, 60), 6000, 300, 0.7, 5000),    # ... with ties: replay starts outside LDS
+    # the greedy scan's super-blocks of 512 boxes
+    ((50, 60), 12000, 1000, 0.7, 0),     # 188 mask words per row: more words than lanes
+    ((38, 63), 513, 600, 0.1, 0),        # one box into the second super-block, heavy suppression
+    ((38, 63), 512, 600, 0.95, 0),       # exactly one super-block, almost everything kept
+    ((38, 63), 6000, 37, 0.7, 0),        # post_nms_topn reached inside the first block
+    ((38, 63), 6000, 5000, 0.3, 0),      # every super-block walked, post_nms_topn never reached
+    ((38, 63), 6000, 700, 0.8, 0),       # post_nms_topn reached in a later super-block
 ])
 def test_proposal_bit_exact(K, hw, pre, post, thr, quant):
     """Kept rois and scores equal the CPU path's bit for bit, with and without
