@@ -294,8 +294,33 @@ __global__ __launch_bounds__(kSortThreads) void det_class_nms_lds_kernel(
   }
   if (valid) atomicAdd(&s_valid, valid);
   __syncthreads();
-  block_sort_desc_lds<kDetLdsPer, unsigned short>(s_key, s_val, P, &lds);
-  int ncand = s_valid;
+  // Only scores above the threshold can become candidates: squeeze them to the
+  // front in prior order (a stable sort of the survivors alone gives the order the
+  // sort of all priors would give them) and sort just those.
+  const int nvalid = s_valid;
+  if (nvalid < P) {
+    const int per = (P + kSortThreads - 1) / kSortThreads;
+    const int begin = min(static_cast<int>(threadIdx.x) * per, P), end = min(begin + per, P);
+    uint32_t rk[kDetLdsPer];
+    uint32_t mine = 0;
+#pragma unroll
+    for (int j = 0; j < kDetLdsPer; ++j) {
+      rk[j] = 0xffffffffu;
+      if (begin + j < end) rk[j] = s_key[begin + j];
+      mine += rk[j] != 0xffffffffu;
+    }
+    uint32_t pos = block_exclusive_scan(mine, lds.wave_sum);  // synchronises before returning
+#pragma unroll
+    for (int j = 0; j < kDetLdsPer; ++j)
+      if (rk[j] != 0xffffffffu) {
+        s_key[pos] = rk[j];
+        s_val[pos] = static_cast<unsigned short>(begin + j);
+        ++pos;
+      }
+    __syncthreads();
+  }
+  block_sort_desc_lds<kDetLdsPer, unsigned short>(s_key, s_val, nvalid, &lds);
+  int ncand = nvalid;
   if (top_k > -1 && top_k < ncand) ncand = top_k;
   const DBox* cls_boxes = boxes + ((size_t)i * loc_classes + (loc_classes == 1 ? 0 : c)) * P;
   const int n_cached = min(ncand, kDetCandBoxes);
@@ -316,6 +341,9 @@ __global__ __launch_bounds__(kSortThreads) void det_class_nms_lds_kernel(
                                   &kept_count[seg]);
 }
 
+constexpr int kSelLdsPer = 16;
+constexpr int kSelLdsMax = kSelLdsPer * kSortThreads;  // 8192 entries (SSD300: 20 classes x 400)
+
 // One workgroup per image: applies keep_top_k over all classes and writes the
 // image's rows [image, label, score, xmin, ymin, xmax, ymax], labels ascending,
 // each label's boxes in NMS order.
@@ -326,6 +354,9 @@ __global__ __launch_bounds__(kSortThreads) void det_select_kernel(
     int* vals1, int* __restrict__ selected, float* __restrict__ rows_tmp,
     int* __restrict__ rows_count) {
   __shared__ BlockSortLds lds;
+  __shared__ BlockSortLds16 lds16;
+  __shared__ uint32_t s_key[kSelLdsMax];       // entry lists of up to kSelLdsMax are sorted in LDS
+  __shared__ unsigned short s_val[kSelLdsMax];
   __shared__ int s_off[1024];  // start of each class in the image's entry list
   const int i = blockIdx.x;
   const int max_entries = C * max_cand;
@@ -350,16 +381,29 @@ __global__ __launch_bounds__(kSortThreads) void det_select_kernel(
   if (keep_top_k > -1 && total > keep_top_k) {
     const int per = (total + kSortThreads - 1) / kSortThreads;
     const int begin = min(static_cast<int>(threadIdx.x) * per, total), end = min(begin + per, total);
+    const bool in_lds = total <= kSelLdsMax;
     int c = 0;
     for (int e = begin; e < end; ++e) {
       while (s_off[c + 1] <= e) ++c;
       const int idx = kept_idx[(size_t)(i * C + c) * max_cand + (e - s_off[c])];
-      k0[e] = desc_key(conf[((size_t)i * P + idx) * C + c]);
-      v0[e] = e;
+      const uint32_t key = desc_key(conf[((size_t)i * P + idx) * C + c]);
+      if (in_lds) {
+        s_key[e] = key;
+        s_val[e] = static_cast<unsigned short>(e);
+      } else {
+        k0[e] = key;
+        v0[e] = e;
+      }
     }
     __syncthreads();
-    block_sort_desc(k0, v0, k1, v1, total, &lds);
-    for (int r = threadIdx.x; r < total; r += kSortThreads) sel[v0[r]] = r < keep_top_k;
+    // both sorts are stable and see the entries in the same order: same result
+    if (in_lds) {
+      block_sort_desc_lds<kSelLdsPer, unsigned short>(s_key, s_val, total, &lds16);
+      for (int r = threadIdx.x; r < total; r += kSortThreads) sel[s_val[r]] = r < keep_top_k;
+    } else {
+      block_sort_desc(k0, v0, k1, v1, total, &lds);
+      for (int r = threadIdx.x; r < total; r += kSortThreads) sel[v0[r]] = r < keep_top_k;
+    }
     __syncthreads();
   }
   // compact the selected entries in entry order (single pass by one thread per
