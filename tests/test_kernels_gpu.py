@@ -270,6 +270,29 @@ def test_depthwise_with_epilogue(K):
     assert netrun.rel_err(got, want) < 1e-4
 
 
+@pytest.mark.parametrize("c,h,w,s,p,n", [
+    (48, 19, 19, 1, 1, 3), (7, 10, 10, 1, 0, 5), (6, 60, 60, 1, 1, 2),
+    (5, 150, 150, 1, 1, 1),    # MobileNet conv1/dw
+    (4, 75, 75, 2, 1, 2),      # stride 2, odd extents
+    (3, 8, 585, 2, 0, 2), (3, 33, 130, 1, 1, 2), (2, 6, 1024, 1, 1, 1), (2, 6, 1025, 2, 1, 1),
+])
+def test_depthwise_3x3_shapes(K, c, h, w, s, p, n):
+    """3x3 depthwise at stride 1 and 2 (four output rows per thread): small and large planes,
+    odd extents, rows wider than a workgroup, with the whole epilogue."""
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((n, c, h, w)).astype(np.float32)
+    wt = (rng.standard_normal((c, 1, 3, 3)) * 0.3).astype(np.float32)
+    sc = (rng.random(c) + 0.5).astype(np.float32)
+    sh = rng.standard_normal(c).astype(np.float32)
+    y = oracle.conv_forward(oracle.conv_geom(c, h, w, c, 3, s, p, 1, c), x, wt, None)
+    res = rng.standard_normal(y.shape).astype(np.float32)
+    want = oracle.relu(oracle.eltwise([oracle.scale(y, sc, sh), res], "SUM"), 0.1)
+    plan = K.ConvPlan(K.conv_geom(c, h, w, c, 3, s, p, 1, c))
+    got = _run_plan(K, plan, n, x, wt, want.shape, scale=sc, shift=sh, residual=res,
+                    activation=K.ACT_RELU, negative_slope=0.1)
+    assert netrun.rel_err(got, want) < 1e-4
+
+
 def test_conv_limits_are_errors(K):
     from minicaffe import MiniCaffeError
     with pytest.raises(MiniCaffeError, match="31 taps"):
