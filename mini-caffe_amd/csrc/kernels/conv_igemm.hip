@@ -1299,7 +1299,18 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
       thin_conv_kernel<<<grid, 256, 0, st>>>(batch, pointwise ? 1 : 0);
     } else {
       dim3 grid(static_cast<unsigned>(max_blocks), g.group, nsub * slices);
-      cfg.kernel[pointwise ? kModePointwise : (one_mask ? kModeOneMask : kModeMasks)]<<<grid, 256, 0, st>>>(
+      // A launch with less than one round of workgroups asks for enough LDS that
+      // at most ceil(workgroups / CUs) of them fit a CU: the dispatcher then cannot
+      // fill some CUs to eight and leave others short (1-3 % on such launches).
+      unsigned extra_lds = 0;
+      const long wgs = max_blocks * g.group * nsub * slices;
+      if (wgs < 8L * kNumCu) {
+        const int limit = std::max<long>(3, ceil_div(wgs, static_cast<long>(kNumCu)));
+        const long stat = 2L * cfg.ks * (cfg.bm + cfg.bn) * LDK * 4;
+        const long want = (160L * 1024 / limit) / 1024 * 1024;
+        if (limit < 8 && want > stat) extra_lds = static_cast<unsigned>(want - stat);
+      }
+      cfg.kernel[pointwise ? kModePointwise : (one_mask ? kModeOneMask : kModeMasks)]<<<grid, 256, extra_lds, st>>>(
           batch);
     }
     MC_LAUNCH_CHECK();
