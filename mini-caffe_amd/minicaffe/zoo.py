@@ -432,3 +432,92 @@ def mobilenet_ssd_spec(batch=1, seed=0, num_classes=21, size=300, width=1.0, dep
                    confidence_threshold=0.25)
     x = np.random.default_rng(seed + 1).uniform(-1, 1, (batch, 3, size, size)).astype(np.float32)
     return spec, {"data": x}
+
+
+def _pool(name, bottom, method, k, stride=1, pad=0, global_pooling=False):
+    p = {"pool": Enum(method)}
+    if global_pooling:
+        p["global_pooling"] = True
+    else:
+        p["kernel_size"] = k
+        p["stride"] = stride
+        if pad:
+            p["pad"] = pad
+    return {"name": name, "type": "Pooling", "bottom": [bottom], "top": [name], "pooling_param": p}
+
+
+def googlenet_spec(batch=2, size=96, seed=0, num_classes=10,
+                   modules=((64, 96, 128, 16, 32, 32), (128, 128, 192, 32, 96, 64))):
+    """The front of bvlc_googlenet (one of the three nets the reference's own test program
+    runs, tests/run_net.cpp:175-236): 7x7/2 stem, LRN, 1x1 + 3x3, LRN, then inception
+    modules (1x1 | 1x1 -> 3x3 | 1x1 -> 5x5 | 3x3/1 max pool -> 1x1, Concat), global
+    average pool, Dropout, InnerProduct, Softmax.  `modules` lists (1x1, 3x3 reduce, 3x3,
+    5x5 reduce, 5x5, pool proj) outputs; the default is inception 3a and 3b."""
+    spec = [input_layer({"data": (batch, 3, size, size)})]
+
+    def conv_relu(name, bottom, cin, cout, k, stride=1, pad=0):
+        spec.append(conv_layer(name, bottom, name, cin, cout, k, stride, pad, seed=seed, bias_value=0.2))
+        spec.append(relu_layer("relu_" + name, name))
+
+    lrn = lambda name, bottom: {"name": name, "type": "LRN", "bottom": [bottom], "top": [name],  # noqa: E731
+                                "lrn_param": {"local_size": 5, "alpha": 1e-4, "beta": 0.75}}
+    conv_relu("conv1/7x7_s2", "data", 3, 64, 7, 2, 3)
+    spec.append(_pool("pool1/3x3_s2", "conv1/7x7_s2", "MAX", 3, 2))
+    spec.append(lrn("pool1/norm1", "pool1/3x3_s2"))
+    conv_relu("conv2/3x3_reduce", "pool1/norm1", 64, 64, 1)
+    conv_relu("conv2/3x3", "conv2/3x3_reduce", 64, 192, 3, 1, 1)
+    spec.append(lrn("conv2/norm2", "conv2/3x3"))
+    spec.append(_pool("pool2/3x3_s2", "conv2/norm2", "MAX", 3, 2))
+    prev, cin = "pool2/3x3_s2", 192
+    for i, (c1, c3r, c3, c5r, c5, cp) in enumerate(modules):
+        m = "inception_%d" % i
+        conv_relu(m + "/1x1", prev, cin, c1, 1)
+        conv_relu(m + "/3x3_reduce", prev, cin, c3r, 1)
+        conv_relu(m + "/3x3", m + "/3x3_reduce", c3r, c3, 3, 1, 1)
+        conv_relu(m + "/5x5_reduce", prev, cin, c5r, 1)
+        conv_relu(m + "/5x5", m + "/5x5_reduce", c5r, c5, 5, 1, 2)
+        spec.append(_pool(m + "/pool", prev, "MAX", 3, 1, 1))
+        conv_relu(m + "/pool_proj", m + "/pool", cin, cp, 1)
+        spec.append({"name": m + "/output", "type": "Concat",
+                     "bottom": [m + "/1x1", m + "/3x3", m + "/5x5", m + "/pool_proj"], "top": [m + "/output"]})
+        prev, cin = m + "/output", c1 + c3 + c5 + cp
+    spec.append(_pool("pool5", prev, "AVE", 0, global_pooling=True))
+    spec.append({"name": "pool5/drop", "type": "Dropout", "bottom": ["pool5"], "top": ["pool5"],
+                 "dropout_param": {"dropout_ratio": 0.4}})
+    w = (_rng(seed, "loss3/classifier", "w").standard_normal((num_classes, cin)) * np.sqrt(2.0 / cin)).astype(np.float32)
+    spec.append({"name": "loss3/classifier", "type": "InnerProduct", "bottom": ["pool5"], "top": ["loss3/classifier"],
+                 "inner_product_param": {"num_output": num_classes},
+                 "blobs": [w, np.zeros(num_classes, np.float32)]})
+    spec.append({"name": "prob", "type": "Softmax", "bottom": ["loss3/classifier"], "top": ["prob"]})
+    x = np.random.default_rng(seed + 1).uniform(-1, 1, (batch, 3, size, size)).astype(np.float32)
+    return spec, {"data": x}
+
+
+def nin_spec(batch=2, size=67, seed=0, num_classes=10, width=32):
+    """Network-in-Network (another of the reference's test nets): every block is a
+    spatial convolution followed by two 1x1 "cccp" convolutions, all with ReLU; max
+    pools with Dropout between blocks; the classifier is a 1x1 convolution, a global
+    average pool and Softmax (no InnerProduct)."""
+    spec = [input_layer({"data": (batch, 3, size, size)})]
+
+    def conv_relu(name, bottom, cin, cout, k, stride=1, pad=0):
+        spec.append(conv_layer(name, bottom, name, cin, cout, k, stride, pad, seed=seed, bias_value=0.1))
+        spec.append(relu_layer("relu_" + name, name))
+
+    conv_relu("conv1", "data", 3, width * 3, 11, 4)
+    conv_relu("cccp1", "conv1", width * 3, width * 3, 1)
+    conv_relu("cccp2", "cccp1", width * 3, width * 3, 1)
+    spec.append(_pool("pool0", "cccp2", "MAX", 3, 2))
+    conv_relu("conv2", "pool0", width * 3, width * 8, 5, 1, 2)
+    conv_relu("cccp3", "conv2", width * 8, width * 8, 1)
+    conv_relu("cccp4", "cccp3", width * 8, width * 8, 1)
+    spec.append(_pool("pool2", "cccp4", "MAX", 3, 2))
+    spec.append({"name": "drop", "type": "Dropout", "bottom": ["pool2"], "top": ["pool2"],
+                 "dropout_param": {"dropout_ratio": 0.5}})
+    conv_relu("conv4-1024", "pool2", width * 8, width * 16, 3, 1, 1)
+    conv_relu("cccp7-1024", "conv4-1024", width * 16, width * 16, 1)
+    conv_relu("cccp8-1024", "cccp7-1024", width * 16, num_classes, 1)
+    spec.append(_pool("pool4", "cccp8-1024", "AVE", 0, global_pooling=True))
+    spec.append({"name": "prob", "type": "Softmax", "bottom": ["pool4"], "top": ["prob"]})
+    x = np.random.default_rng(seed + 1).uniform(-1, 1, (batch, 3, size, size)).astype(np.float32)
+    return spec, {"data": x}

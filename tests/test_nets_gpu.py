@@ -188,6 +188,39 @@ def test_flatten_and_reshape_as_views(gpu_mode):
     assert netrun.rel_err(net.get_blob("resh").data, want["resh"]) < 1e-5
 
 
+def test_googlenet_front_and_nin(gpu_mode):
+    """The other two nets the reference's test program runs (tests/run_net.cpp:175-236), at
+    reduced size: GoogLeNet's stem and first two inception modules (a blob feeding four
+    branches, 5x5 filters, LRN, 3x3/1 padded max pools, four-way Concat) and
+    Network-in-Network (11x11/4 filters, 1x1 chains, Dropout, global average pool as the
+    classifier).  Every stage against the oracle, and batch invariance as in
+    run_net.cpp:274-321."""
+    from minicaffe import zoo
+    oracle.use_openblas(False)
+    spec, inputs = zoo.googlenet_spec(batch=3, size=96, seed=4)
+    marks = ["pool1/norm1", "conv2/norm2", "pool2/3x3_s2", "inception_0/5x5", "inception_0/pool_proj",
+             "inception_0/output", "inception_1/output", "pool5", "loss3/classifier"]
+    net = run_net(gpu_mode, spec, inputs, marks)
+    want = netrun.oracle_forward(spec, inputs)
+    for name in marks + ["prob"]:
+        got = net.get_blob(name).data
+        assert got.shape == want[name].shape, name
+        assert netrun.rel_err(got, want[name]) < 1e-3, name
+    p3 = net.get_blob("prob").data.copy()
+    net.forward(data=inputs["data"][1:2])
+    assert np.abs(net.get_blob("prob").data[0] - p3[1]).max() < 1e-6
+
+    spec, inputs = zoo.nin_spec(batch=2, size=67, seed=5)
+    marks = ["conv1", "cccp2", "pool0", "conv2", "pool2", "cccp8-1024", "pool4"]
+    net = run_net(gpu_mode, spec, inputs, marks)
+    want = netrun.oracle_forward(spec, inputs)
+    for name in marks + ["prob"]:
+        got = net.get_blob(name).data
+        assert got.shape == want[name].shape, name
+        assert netrun.rel_err(got, want[name]) < 1e-3, name
+    assert np.allclose(net.get_blob("prob").data.reshape(2, -1).sum(axis=1), 1, atol=1e-5)
+
+
 def test_unfused_layers_standalone(gpu_mode):
     """BatchNorm / Scale / Bias / ReLU / TanH / Sigmoid / Eltwise that do NOT follow a
     contraction run as their own kernels; Split, Slice, Concat, Flatten, Reshape,
