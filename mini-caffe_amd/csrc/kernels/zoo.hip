@@ -113,6 +113,13 @@ __global__ __launch_bounds__(256) void prelu_kernel(const float* __restrict__ x,
 
 constexpr int kLrnChunk = 32;  // channels walked by one thread
 
+// scale^(-beta) for a scale >= k > 0 through the hardware's base-2 logarithm and
+// exponential (a few units in the last place, far inside the layer's tolerance;
+// the library powf costs several times the rest of the kernel).
+__device__ __forceinline__ float lrn_pow(float scale, float neg_beta) {
+  return __builtin_amdgcn_exp2f(neg_beta * __builtin_amdgcn_logf(scale));
+}
+
 // One thread per (image, channel chunk, pixel): the window sum of squares is
 // built directly for the chunk's first channel and then slides.
 __global__ __launch_bounds__(256) void lrn_across_kernel(const float* __restrict__ x,
@@ -138,7 +145,7 @@ __global__ __launch_bounds__(256) void lrn_across_kernel(const float* __restrict
   }
   for (int c = c0; c < c1; ++c) {
     const float v = xi[static_cast<long>(c) * spatial];
-    yi[static_cast<long>(c) * spatial] = v * powf(k + acc * alpha_over_n, neg_beta);
+    yi[static_cast<long>(c) * spatial] = v * lrn_pow(k + acc * alpha_over_n, neg_beta);
     const int head = c + 1 + post, tail = c - pre;
     if (head < C) {
       const float h = xi[static_cast<long>(head) * spatial];
@@ -148,6 +155,53 @@ __global__ __launch_bounds__(256) void lrn_across_kernel(const float* __restrict
       const float u = xi[static_cast<long>(tail) * spatial];
       acc -= u * u;
     }
+  }
+}
+
+// The same for the usual window sizes: the chunk is walked in blocks of eight
+// channels whose new values are loaded together (eight independent loads in
+// flight, every value read once per thread), and each window sum is formed
+// from the values in registers instead of sliding by add and subtract.
+template <int SIZE>
+__global__ __launch_bounds__(256) void lrn_across_fixed_kernel(const float* __restrict__ x,
+                                                               float* __restrict__ y, int num, int C,
+                                                               int spatial, float alpha_over_n,
+                                                               float neg_beta, float k, int chunks) {
+  constexpr int PRE = (SIZE - 1) / 2, B = 8;
+  const long total = static_cast<long>(num) * chunks * spatial;
+  const long gid = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x;
+  if (gid >= total) return;
+  const int p = static_cast<int>(gid % spatial);
+  const long t = gid / spatial;
+  const int chunk = static_cast<int>(t % chunks);
+  const int n = static_cast<int>(t / chunks);
+  const int c0 = chunk * kLrnChunk;
+  const int c1 = min(C, c0 + kLrnChunk);
+  const float* __restrict__ xi = x + (static_cast<long>(n) * C) * spatial + p;
+  float* __restrict__ yi = y + (static_cast<long>(n) * C) * spatial + p;
+  float win[B + SIZE - 1];  // channels cb - PRE .. cb + B - 1 + PRE of the current block
+#pragma unroll
+  for (int i = 0; i < SIZE - 1; ++i) {
+    const int c = c0 - PRE + i;
+    win[i] = (c >= 0 && c < C) ? xi[static_cast<long>(c) * spatial] : 0.f;
+  }
+  for (int cb = c0; cb < c1; cb += B) {
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      const int c = cb + PRE + j;
+      win[SIZE - 1 + j] = c < C ? xi[static_cast<long>(c) * spatial] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      if (cb + j < c1) {
+        float acc = 0.f;
+#pragma unroll
+        for (int d = 0; d < SIZE; ++d) acc += win[j + d] * win[j + d];
+        yi[static_cast<long>(cb + j) * spatial] = win[j + PRE] * lrn_pow(k + acc * alpha_over_n, neg_beta);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < SIZE - 1; ++i) win[i] = win[B + i];
   }
 }
 
@@ -177,7 +231,7 @@ __global__ __launch_bounds__(256) void lrn_within_kernel(const float* __restrict
       const float v = xp[i * W + j];
       acc += v * v;
     }
-  y[gid] = x[gid] * powf(1.f + alpha * (acc / pool), neg_beta);
+  y[gid] = x[gid] * lrn_pow(1.f + alpha * (acc / pool), neg_beta);
 }
 
 // ---- ArgMax -------------------------------------------------------------------
@@ -436,8 +490,18 @@ int mcLRNAcrossChannels(const float* bottom, float* top, int num, int channels, 
   const int chunks = ceil_div(channels, kLrnChunk);
   const long total = static_cast<long>(num) * chunks * spatial;
   MC_REQUIRE(total < (1L << 31) * 256, "mcLRNAcrossChannels: blob too large");
-  lrn_across_kernel<<<ceil_div(total, 256), 256, 0, static_cast<hipStream_t>(stream)>>>(
-      bottom, top, num, channels, spatial, local_size, alpha / local_size, -beta, k, chunks);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int blocks = ceil_div(total, 256);
+  const float an = alpha / local_size;
+  if (local_size == 3)
+    lrn_across_fixed_kernel<3><<<blocks, 256, 0, st>>>(bottom, top, num, channels, spatial, an, -beta, k, chunks);
+  else if (local_size == 5)
+    lrn_across_fixed_kernel<5><<<blocks, 256, 0, st>>>(bottom, top, num, channels, spatial, an, -beta, k, chunks);
+  else if (local_size == 7)
+    lrn_across_fixed_kernel<7><<<blocks, 256, 0, st>>>(bottom, top, num, channels, spatial, an, -beta, k, chunks);
+  else
+    lrn_across_kernel<<<blocks, 256, 0, st>>>(bottom, top, num, channels, spatial, local_size, an, -beta, k,
+                                              chunks);
   MC_LAUNCH_CHECK();
   return 0;
 }

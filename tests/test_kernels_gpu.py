@@ -677,7 +677,9 @@ def test_prelu(K, shape, shared):
 
 
 @pytest.mark.parametrize("case", [(2, 96, 27, 27, 5), (1, 7, 3, 5, 3), (2, 40, 6, 6, 9), (1, 3, 4, 4, 1),
-                                  (1, 2, 5, 5, 7)])
+                                  (1, 2, 5, 5, 7),
+                                  # chunks of 32 channels walked in blocks of 8: ragged last chunk and block
+                                  (1, 33, 5, 5, 5), (2, 64, 4, 4, 7), (1, 100, 3, 3, 3), (1, 45, 2, 3, 5)])
 def test_lrn_across_channels(K, case):
     n, c, h, w, size = case
     x = (np.random.default_rng(2).standard_normal((n, c, h, w)) * 4).astype(np.float32)
