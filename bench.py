@@ -371,6 +371,8 @@ def bandwidth_report(path):
           lambda: LIB.mcChannelTransform(P(a.data_ptr()), P(y.data_ptr()), n, c, sp, ctypes.byref(op), P(stream)))
     timed("Unary ELU, 64x256x56x56", 4 * 2 * a.numel(),
           lambda: LIB.mcUnary(5, P(a.data_ptr()), P(y.data_ptr()), a.numel(), 1.0, 0.0, 0.0, P(stream)))
+    timed("PReLU, one slope per channel, 64x256x56x56", 4 * 2 * a.numel(),
+          lambda: LIB.mcPReLU(P(a.data_ptr()), P(y.data_ptr()), n, c, sp, P(mul.data_ptr()), 0, P(stream)))
     timed("copy (Concat / Slice / Split), 64x256x56x56", 4 * 2 * a.numel(),
           lambda: LIB.mcCopy2D(P(a.data_ptr()), a.numel(), P(y.data_ptr()), a.numel(), a.numel(), 1, P(stream)))
     shape, order = ints([n, c, 56, 56]), ints([0, 2, 3, 1])

@@ -97,15 +97,29 @@ int launch_unary(const float* x, float* y, long n, float p0, float p1, float p2,
 
 // ---- PReLU --------------------------------------------------------------------
 
+// VEC = 4 requires inner % 4 == 0 (the four values share a channel) and 16-byte
+// aligned blobs.  n < 2^32 elements, so the channel comes from 32-bit divisions.
+template <int VEC>
 __global__ __launch_bounds__(256) void prelu_kernel(const float* __restrict__ x,
                                                     float* __restrict__ y, long n, int channels,
                                                     int inner, const float* __restrict__ slope,
                                                     int shared) {
+  const long nv = n / VEC;
   const long stride = static_cast<long>(gridDim.x) * blockDim.x;
-  for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < n; i += stride) {
-    const int c = shared ? 0 : static_cast<int>((i / inner) % channels);
-    const float v = x[i];
-    y[i] = fmaxf(v, 0.f) + slope[c] * fminf(v, 0.f);
+  for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < nv; i += stride) {
+    const unsigned e = static_cast<unsigned>(i) * VEC;
+    const float sl = slope[shared ? 0u : (e / static_cast<unsigned>(inner)) % static_cast<unsigned>(channels)];
+    if (VEC == 4) {
+      float4 v = reinterpret_cast<const float4*>(x)[i];
+      v.x = fmaxf(v.x, 0.f) + sl * fminf(v.x, 0.f);
+      v.y = fmaxf(v.y, 0.f) + sl * fminf(v.y, 0.f);
+      v.z = fmaxf(v.z, 0.f) + sl * fminf(v.z, 0.f);
+      v.w = fmaxf(v.w, 0.f) + sl * fminf(v.w, 0.f);
+      reinterpret_cast<float4*>(y)[i] = v;
+    } else {
+      const float v = x[i];
+      y[i] = fmaxf(v, 0.f) + sl * fminf(v, 0.f);
+    }
   }
 }
 
@@ -473,8 +487,15 @@ int mcPReLU(const float* bottom, float* top, int outer, int channels, int inner,
   const long n = static_cast<long>(outer) * channels * inner;
   if (n == 0) return 0;
   MC_REQUIRE(bottom && top && slope, "mcPReLU: null pointer");
-  prelu_kernel<<<ew_blocks(n, 256, 4), 256, 0, static_cast<hipStream_t>(stream)>>>(
-      bottom, top, n, channels, inner, slope, channel_shared);
+  MC_REQUIRE(n < (1L << 32), "mcPReLU: blob too large");
+  const bool vec = inner % 4 == 0 && (reinterpret_cast<uintptr_t>(bottom) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(top) & 15) == 0;
+  if (vec)
+    prelu_kernel<4><<<ew_blocks(n / 4, 256), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        bottom, top, n, channels, inner, slope, channel_shared);
+  else
+    prelu_kernel<1><<<ew_blocks(n, 256, 4), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        bottom, top, n, channels, inner, slope, channel_shared);
   MC_LAUNCH_CHECK();
   return 0;
 }
