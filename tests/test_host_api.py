@@ -406,3 +406,20 @@ def test_mobilenet_ssd_builder_matches_the_reference_prototxt():
     spec_dw, _ = zoo.mobilenet_ssd_spec(depthwise_type=True)
     dw = mc.Net.from_buffers(craft.to_prototxt(spec_dw))
     assert [(n, b.shape) for n, b in dw.param_list] == [(n, b.shape) for n, b in ref.param_list]
+
+
+def test_benchmark_tool_is_built_against_public_headers(tmp_path):
+    """The reference's timing tool (tools/benchmark.cpp) rebuilt from the public C++ headers:
+    same command line; without a device it builds the net and then refuses to run it."""
+    import subprocess
+    exe = os.path.join(ROOT, "mini-caffe_amd", "bin", "benchmark")
+    assert os.path.exists(exe), "run __graft_entry__.build() first"
+    from minicaffe import craft, zoo
+    spec, _ = zoo.c1_spec()
+    proto = tmp_path / "net.prototxt"
+    proto.write_text(craft.to_prototxt(spec))
+    r = subprocess.run([exe], capture_output=True, text=True, cwd=tmp_path)
+    assert r.returncode != 0 and "Usage" in (r.stdout + r.stderr)
+    r = subprocess.run([exe, str(proto), "1", "-1"], capture_output=True, text=True, cwd=tmp_path)
+    out = r.stdout + r.stderr
+    assert r.returncode == 1 and "net forward iterations: 1" in out and "HIP device path only" in out

@@ -684,3 +684,23 @@ def test_ssh_context_module_upsample_crop_and_two_top_proposal(gpu_mode):
     assert 10 < n <= 300
     assert np.array_equal(net.get_blob("m1@ssh_boxes").data[:n], rois)
     assert np.array_equal(net.get_blob("m1@ssh_cls_prob").data.reshape(-1)[:n], probs)
+
+
+def test_benchmark_tool_runs_a_prototxt(gpu_mode, tmp_path):
+    """tools/benchmark.cpp of the reference, rebuilt here: net from the prototxt alone,
+    N timed passes, layer scopes in ./profile.json."""
+    import json
+    import os
+    import subprocess
+    from minicaffe import craft, zoo
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "mini-caffe_amd", "bin", "benchmark")
+    spec, _ = zoo.resnet50_spec(batch=2, size=64, stages=(1, 1, 1, 1), width=16, num_classes=10)
+    proto = tmp_path / "net.prototxt"
+    proto.write_text(craft.to_prototxt(spec))
+    r = subprocess.run([exe, str(proto), "3", "0"], capture_output=True, text=True, cwd=tmp_path, timeout=100)
+    out = r.stdout + r.stderr
+    assert r.returncode == 0, out
+    assert out.count("Forward costs") == 3 and "run on device 0" in out
+    events = json.load(open(tmp_path / "profile.json"))["traceEvents"]
+    names = {e["name"] for e in events}
+    assert {"conv1", "pool1", "fc1000", "prob"} <= names
