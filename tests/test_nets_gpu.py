@@ -704,3 +704,33 @@ def test_benchmark_tool_runs_a_prototxt(gpu_mode, tmp_path):
     events = json.load(open(tmp_path / "profile.json"))["traceEvents"]
     names = {e["name"] for e in events}
     assert {"conv1", "pool1", "fc1000", "prob"} <= names
+
+
+def test_c_program_through_the_c_abi(gpu_mode, tmp_path):
+    """A C99 program (csrc/tools/run_net_c.c, the counterpart of the reference's
+    tests/run_net.c) creates a net from files and from buffers, fills the input, runs it
+    and lists blobs; the sum it prints for the last blob equals the oracle's."""
+    import os
+    import re
+    import subprocess
+    import wire
+    from minicaffe import craft, zoo
+    oracle.use_openblas(False)
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "mini-caffe_amd", "bin", "run_net_c")
+    spec, _ = zoo.resnet50_spec(batch=2, size=40, stages=(1, 1, 1, 1), width=8, num_classes=6, bn_seed=9)
+    (tmp_path / "n.prototxt").write_text(craft.to_prototxt(spec))
+    (tmp_path / "n.caffemodel").write_bytes(wire.net("m", [
+        wire.layer(l["name"], l["type"], l["blobs"]) for l in spec if l.get("blobs")]))
+    r = subprocess.run([exe, str(tmp_path / "n.prototxt"), str(tmp_path / "n.caffemodel")],
+                       capture_output=True, text=True, cwd=tmp_path, timeout=100)
+    out = r.stdout + r.stderr
+    assert r.returncode == 0 and "run_net_c: ok" in out, out
+    assert "data: 4 axes, [2, 3, 40, 40], 9600 values" in out
+    assert "expected error:" in out and "prob: [2, 6, 1, 1]" in out
+    # the program's deterministic input, through the oracle
+    i = np.arange(9600)
+    x = ((i * 37 % 101) / 50.0 - 1.0).astype(np.float32).reshape(2, 3, 40, 40)
+    want = netrun.oracle_forward(spec, {"data": x})["prob"]
+    m = re.search(r"sum of the last blob: ([-0-9.e]+), first value: ([-0-9.e]+)", out)
+    assert abs(float(m.group(1)) - float(want.sum())) < 1e-4
+    assert abs(float(m.group(2)) - float(want.flat[0])) < 1e-4 * float(want.max())
