@@ -423,3 +423,51 @@ def test_benchmark_tool_is_built_against_public_headers(tmp_path):
     r = subprocess.run([exe, str(proto), "1", "-1"], capture_output=True, text=True, cwd=tmp_path)
     out = r.stdout + r.stderr
     assert r.returncode == 1 and "net forward iterations: 1" in out and "HIP device path only" in out
+
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def landmark_level2_spec(batch=1):
+    """Net definition of the reference's level-2 landmark nets (example/models/deeplandmark/2_*.prototxt),
+    written from its description: 1x15x15 patch, 4x4 conv to 20, 2x2 max pool, 3x3 conv to 40,
+    2x2 max pool, 60 hidden units, 2 outputs, ReLU after every parameter layer."""
+    from minicaffe.craft import Enum, input_layer
+    conv = lambda n, b, c, k: {"name": n, "type": "Convolution", "bottom": [b], "top": [n],  # noqa: E731
+                               "convolution_param": {"num_output": c, "kernel_size": k}}
+    relu = lambda n, b: {"name": n, "type": "ReLU", "bottom": [b], "top": [b]}  # noqa: E731
+    pool = lambda n, b: {"name": n, "type": "Pooling", "bottom": [b], "top": [n],  # noqa: E731
+                         "pooling_param": {"pool": Enum("MAX"), "kernel_size": 2, "stride": 2}}
+    ip = lambda n, b, c: {"name": n, "type": "InnerProduct", "bottom": [b], "top": [n],  # noqa: E731
+                          "inner_product_param": {"num_output": c}}
+    return [input_layer({"data": (batch, 1, 15, 15)}), conv("conv1", "data", 20, 4), relu("relu1", "conv1"),
+            pool("pool1", "conv1"), conv("conv2", "pool1", 40, 3), relu("relu2", "conv2"), pool("pool2", "conv2"),
+            ip("fc1", "pool2", 60), relu("relu_fc1", "fc1"), ip("fc2", "fc1", 2), relu("relu_fc2", "fc2")]
+
+
+def test_golden_caffemodel_loads_into_the_landmark_net():
+    """tests/golden holds trained weights from the reference's example data.  The library's
+    caffemodel reader must give the values an independent wire-format walk finds."""
+    from minicaffe import craft
+    model = open(os.path.join(GOLDEN, "deeplandmark_2_LE1.caffemodel"), "rb").read()
+    want = wire.read_net_blobs(model)
+    assert sorted(want) == ["conv1", "conv2", "fc1", "fc2"]
+    net = mc.Net.from_buffers(craft.to_prototxt(landmark_level2_spec()), model)
+    params = dict(net.param_list)
+    for layer, blobs in want.items():
+        for j, arr in enumerate(blobs):
+            got = params["%s_%d" % (layer, j)].data
+            assert got.shape == arr.shape and np.array_equal(got, arr), (layer, j)
+    assert net.blobs["fc2"].shape == [1, 2]
+
+
+@needs_ref
+def test_landmark_spec_equals_the_reference_prototxt():
+    from minicaffe import craft
+    ref = mc.Net.from_buffers(open(os.path.join(REF, "example", "models", "deeplandmark", "2_LE1.prototxt")).read())
+    own = mc.Net.from_buffers(craft.to_prototxt(landmark_level2_spec()))
+    assert [(k, v.shape) for k, v in ref.blobs.items()] == [(k, v.shape) for k, v in own.blobs.items()]
+    assert [(k, v.shape) for k, v in ref.param_list] == [(k, v.shape) for k, v in own.param_list]
+    # and the fixture is the reference's file
+    a = open(os.path.join(REF, "example", "models", "deeplandmark", "2_LE1.caffemodel"), "rb").read()
+    assert a == open(os.path.join(GOLDEN, "deeplandmark_2_LE1.caffemodel"), "rb").read()

@@ -734,3 +734,34 @@ def test_c_program_through_the_c_abi(gpu_mode, tmp_path):
     m = re.search(r"sum of the last blob: ([-0-9.e]+), first value: ([-0-9.e]+)", out)
     assert abs(float(m.group(1)) - float(want.sum())) < 1e-4
     assert abs(float(m.group(2)) - float(want.flat[0])) < 1e-4 * float(want.max())
+
+
+def test_trained_landmark_net_from_the_golden_caffemodel(gpu_mode):
+    """Real trained weights (tests/golden, from the reference's deeplandmark example) through
+    CaffeNetCreateFromBuffer; forward at batch 1, as the reference's example calls it, and at
+    batch 6 after a reshape, against the oracle on the same weights."""
+    import os
+    import wire
+    from minicaffe import craft
+    from test_host_api import landmark_level2_spec
+    oracle.use_openblas(False)
+    here = os.path.dirname(os.path.abspath(__file__))
+    model = open(os.path.join(here, "golden", "deeplandmark_2_LE1.caffemodel"), "rb").read()
+    weights = wire.read_net_blobs(model)
+    rng = np.random.default_rng(31)
+    net = gpu_mode.Net.from_buffers(craft.to_prototxt(landmark_level2_spec()), model)
+    for name in ("pool1", "pool2", "fc1"):
+        net.mark_output(name)
+    for batch in (1, 6, 1):
+        spec = landmark_level2_spec(batch)
+        for layer in spec:
+            if layer["name"] in weights:
+                layer["blobs"] = weights[layer["name"]]
+        x = rng.uniform(-1, 1, (batch, 1, 15, 15)).astype(np.float32)
+        net.forward(data=x)
+        want = netrun.oracle_forward(spec, {"data": x})
+        for name in ("pool1", "pool2", "fc1", "fc2"):
+            got = net.get_blob(name).data
+            assert got.shape == want[name].shape, name
+            assert netrun.rel_err(got, want[name]) < 1e-4, (batch, name)
+        assert np.abs(want["fc2"]).max() > 1e-3   # the trained net answers with something
