@@ -19,7 +19,11 @@
 namespace mchip {
 namespace {
 
+// TRANS = false compiles only "none" and ReLU; the double-precision tanh / exp of
+// the other activations would otherwise be part of every launch's inner loop.
+template <bool TRANS>
 __device__ __forceinline__ float dw_act(float v, int act, float slope) {
+  if (!TRANS) return (act == MC_ACT_RELU && !(v > 0.f)) ? v * slope : v;
   switch (act) {
     case MC_ACT_RELU:
       return v > 0.f ? v : v * slope;
@@ -33,7 +37,7 @@ __device__ __forceinline__ float dw_act(float v, int act, float slope) {
 }
 
 // KH/KW > 0: compile-time taps (fully unrolled); 0: run-time extents.
-template <int KH, int KW>
+template <int KH, int KW, bool TRANS>
 __global__ __launch_bounds__(256) void depthwise_kernel(const DepthwiseArgs a, long count) {
   const int kh_n = KH ? KH : a.kh, kw_n = KW ? KW : a.kw;
   const int plane = a.Ho * a.Wo;
@@ -66,7 +70,7 @@ __global__ __launch_bounds__(256) void depthwise_kernel(const DepthwiseArgs a, l
     if (a.scale) acc *= a.scale[oc];
     if (a.shift) acc += a.shift[oc];
     if (a.residual) acc += a.residual[i];
-    a.y[i] = dw_act(acc, a.act, a.slope);
+    a.y[i] = dw_act<TRANS>(acc, a.act, a.slope);
   }
 }
 
@@ -75,7 +79,7 @@ __global__ __launch_bounds__(256) void depthwise_kernel(const DepthwiseArgs a, l
 // 3*SH + KH input rows, so overlapping taps are read once per thread instead of
 // once per output and the index arithmetic is shared; neighbouring threads sit on
 // neighbouring columns, so every load and store stays coalesced.
-template <int KH, int KW, int SH>
+template <int KH, int KW, int SH, bool TRANS>
 __global__ __launch_bounds__(256) void depthwise4_kernel(const DepthwiseArgs a, long groups,
                                                          int ho_groups) {
   constexpr int L = 3 * SH + KH;
@@ -128,7 +132,7 @@ __global__ __launch_bounds__(256) void depthwise4_kernel(const DepthwiseArgs a, 
       if (a.scale) val *= sc;
       if (a.shift) val += sf;
       if (a.residual) val += a.residual[out];
-      a.y[out] = dw_act(val, a.act, a.slope);
+      a.y[out] = dw_act<TRANS>(val, a.act, a.slope);
     }
   }
 }
@@ -138,24 +142,32 @@ __global__ __launch_bounds__(256) void depthwise4_kernel(const DepthwiseArgs a, 
 int depthwise_forward(const DepthwiseArgs& a, hipStream_t stream) {
   const long count = static_cast<long>(a.num) * a.C * a.mult * a.Ho * a.Wo;
   if (count == 0) return 0;
+  const bool trans = a.act == MC_ACT_TANH || a.act == MC_ACT_SIGMOID;
   if (a.kh == 3 && a.kw == 3 && a.dh == 1 && a.dw == 1 && (a.sh == 1 || a.sh == 2)) {
     const int ho_groups = ceil_div(a.Ho, 4);
     const long groups = static_cast<long>(a.num) * a.C * a.mult * ho_groups * a.Wo;
     const unsigned gb = ew_blocks(groups, 256);
-    if (a.sh == 1)
-      depthwise4_kernel<3, 3, 1><<<gb, 256, 0, stream>>>(a, groups, ho_groups);
-    else
-      depthwise4_kernel<3, 3, 2><<<gb, 256, 0, stream>>>(a, groups, ho_groups);
+    if (a.sh == 1) {
+      if (trans) depthwise4_kernel<3, 3, 1, true><<<gb, 256, 0, stream>>>(a, groups, ho_groups);
+      else depthwise4_kernel<3, 3, 1, false><<<gb, 256, 0, stream>>>(a, groups, ho_groups);
+    } else {
+      if (trans) depthwise4_kernel<3, 3, 2, true><<<gb, 256, 0, stream>>>(a, groups, ho_groups);
+      else depthwise4_kernel<3, 3, 2, false><<<gb, 256, 0, stream>>>(a, groups, ho_groups);
+    }
     MC_LAUNCH_CHECK();
     return 0;
   }
   const unsigned blocks = ew_blocks(count, 256);
-  if (a.kh == 3 && a.kw == 3)
-    depthwise_kernel<3, 3><<<blocks, 256, 0, stream>>>(a, count);
-  else if (a.kh == 5 && a.kw == 5)
-    depthwise_kernel<5, 5><<<blocks, 256, 0, stream>>>(a, count);
-  else
-    depthwise_kernel<0, 0><<<blocks, 256, 0, stream>>>(a, count);
+  if (a.kh == 3 && a.kw == 3) {
+    if (trans) depthwise_kernel<3, 3, true><<<blocks, 256, 0, stream>>>(a, count);
+    else depthwise_kernel<3, 3, false><<<blocks, 256, 0, stream>>>(a, count);
+  } else if (a.kh == 5 && a.kw == 5) {
+    if (trans) depthwise_kernel<5, 5, true><<<blocks, 256, 0, stream>>>(a, count);
+    else depthwise_kernel<5, 5, false><<<blocks, 256, 0, stream>>>(a, count);
+  } else {
+    if (trans) depthwise_kernel<0, 0, true><<<blocks, 256, 0, stream>>>(a, count);
+    else depthwise_kernel<0, 0, false><<<blocks, 256, 0, stream>>>(a, count);
+  }
   MC_LAUNCH_CHECK();
   return 0;
 }

@@ -41,30 +41,39 @@ struct ChanArgs {
   float slope;
 };
 
-__device__ __forceinline__ float chan_one(float v, int c, const ChanArgs& a) {
-  if (a.sub) v -= a.sub[c];
-  if (a.div) v /= a.div[c];
-  if (a.mul) v *= a.mul[c];
-  if (a.add) v += a.add[c];
-  return act_apply(v, a.act, a.slope);
+// The channel's four operands, fetched once per vector (absent ones are the
+// neutral element), then  ((v - sub) / div) * mul + add  and the activation.
+// TRANS = false compiles only "none" and ReLU: the double-precision tanh / exp
+// of the other two activations would otherwise sit in the loop of every launch.
+template <bool TRANS>
+__device__ __forceinline__ float chan_one(float v, float sub, float div, float mul, float add,
+                                          bool has_div, const ChanArgs& a) {
+  v -= sub;
+  if (has_div) v /= div;
+  v = v * mul + add;
+  if (TRANS) return act_apply(v, a.act, a.slope);
+  return (a.act == MC_ACT_RELU && !(v > 0.f)) ? v * a.slope : v;
 }
 
 // VEC = 4 requires inner % 4 == 0, so the four lanes of a float4 share a channel.
-template <int VEC>
+template <int VEC, bool TRANS>
 __global__ __launch_bounds__(256) void channel_transform_kernel(const ChanArgs a) {
   const long n = a.count / VEC;
+  const bool has_div = a.div != nullptr;
   for (long i = blockIdx.x * 256L + threadIdx.x; i < n; i += gridDim.x * 256L) {
     const long e = i * VEC;
     const int c = static_cast<int>((e / a.inner) % a.channels);
+    const float sub = a.sub ? a.sub[c] : 0.f, div = has_div ? a.div[c] : 1.f;
+    const float mul = a.mul ? a.mul[c] : 1.f, add = a.add ? a.add[c] : 0.f;
     if (VEC == 4) {
       float4 v = reinterpret_cast<const float4*>(a.x)[i];
-      v.x = chan_one(v.x, c, a);
-      v.y = chan_one(v.y, c, a);
-      v.z = chan_one(v.z, c, a);
-      v.w = chan_one(v.w, c, a);
+      v.x = chan_one<TRANS>(v.x, sub, div, mul, add, has_div, a);
+      v.y = chan_one<TRANS>(v.y, sub, div, mul, add, has_div, a);
+      v.z = chan_one<TRANS>(v.z, sub, div, mul, add, has_div, a);
+      v.w = chan_one<TRANS>(v.w, sub, div, mul, add, has_div, a);
       reinterpret_cast<float4*>(a.y)[i] = v;
     } else {
-      a.y[i] = chan_one(a.x[i], c, a);
+      a.y[i] = chan_one<TRANS>(a.x[i], sub, div, mul, add, has_div, a);
     }
   }
 }
@@ -290,10 +299,15 @@ int mcChannelTransform(const float* x, float* y, int outer, int channels, int in
   a.slope = op->negative_slope;
   if (a.count == 0) return 0;
   hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool trans = a.act == MC_ACT_TANH || a.act == MC_ACT_SIGMOID;
   if (inner % 4 == 0 && aligned16(x) && aligned16(y)) {
-    channel_transform_kernel<4><<<ew_blocks(a.count / 4, 256), 256, 0, st>>>(a);
+    const int blocks = ew_blocks(a.count / 4, 256);
+    if (trans) channel_transform_kernel<4, true><<<blocks, 256, 0, st>>>(a);
+    else channel_transform_kernel<4, false><<<blocks, 256, 0, st>>>(a);
   } else {
-    channel_transform_kernel<1><<<ew_blocks(a.count, 256), 256, 0, st>>>(a);
+    const int blocks = ew_blocks(a.count, 256);
+    if (trans) channel_transform_kernel<1, true><<<blocks, 256, 0, st>>>(a);
+    else channel_transform_kernel<1, false><<<blocks, 256, 0, st>>>(a);
   }
   MC_LAUNCH_CHECK();
   return 0;
