@@ -91,6 +91,9 @@ class CAFFE_API Net {
   // skipped view (Flatten, Reshape): the blob id whose memory the layer's top
   // aliases, else -1 (indexed by layer)
   vector<int> residual_alias_;
+  // for a convolution that an earlier sibling computes together with its own
+  // (same bottom, same window geometry): that sibling's layer id, else -1
+  vector<int> sibling_owner_;
   // shapes of all blobs at the last PlaceMemory
   vector<vector<int> > placed_shapes_;
   bool fusion_dirty_ = true;

@@ -99,6 +99,14 @@ class Layer {
   // activation (its own followers end without an activation).
   virtual bool AcceptsResidual() const { return false; }
   virtual void SetResidual(Blob* residual, Layer* activation) {}
+  // Sibling merge.  Two Convolution layers that read the same blob with the same
+  // window geometry, with nothing folded into either, can run as one launch over
+  // the concatenated filters (the loc and conf heads of an SSD source).  A layer
+  // that could take part describes its geometry in `key`; the first of a pair
+  // adopts the second, computes both tops in its own Forward, and the second is
+  // skipped.  AdoptSibling(nullptr, nullptr) ends the arrangement.
+  virtual bool SiblingKey(vector<int>* key) const { return false; }
+  virtual void AdoptSibling(Layer* sibling, Blob* sibling_top) {}
   // True when the top holds the bottom's values in the same order under another
   // shape (Flatten, Reshape).  When nothing reads the bottom afterwards Net lets
   // the top take over the bottom's memory and skips the layer's copy.

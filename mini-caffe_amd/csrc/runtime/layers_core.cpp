@@ -295,10 +295,103 @@ class BaseConvolutionLayer : public ContractionLayer {
 class ConvolutionLayer : public BaseConvolutionLayer {
  public:
   explicit ConvolutionLayer(const LayerParameter& param) : BaseConvolutionLayer(param) {}
+  ~ConvolutionLayer() override {
+    if (merged_plan_) mcConvPlanDestroy(merged_plan_);
+  }
   const char* type() const override { return "Convolution"; }
+
+  // ---- sibling merge: this layer and an adopted one as a single launch --------
+  bool SiblingKey(vector<int>* key) const override {
+    if (geom_.group != 1 || !followers_.empty() || residual_ != nullptr) return false;
+    *key = {geom_.channels_in, geom_.kernel_h, geom_.kernel_w, geom_.stride_h, geom_.stride_w,
+            geom_.pad_h,       geom_.pad_w,    geom_.dilation_h, geom_.dilation_w};
+    return true;
+  }
+  void AdoptSibling(Layer* sibling, Blob* sibling_top) override {
+    sibling_ = static_cast<ConvolutionLayer*>(sibling);
+    sibling_top_ = sibling_top;
+    merged_version_ = ~0ull;
+  }
+  void Reshape(const vector<Blob*>& bottom, const vector<Blob*>& top) override {
+    BaseConvolutionLayer::Reshape(bottom, top);
+    if (sibling_)
+      merged_out_.Reshape(vector<int>{top[0]->shape(0), geom_.channels_out + sibling_->geom_.channels_out,
+                                      top[0]->shape(2), top[0]->shape(3)});
+  }
+  vector<Blob*> GetTempBlobs() override {
+    vector<Blob*> t;
+    if (sibling_) t.push_back(&merged_out_);
+    return t;
+  }
 
  protected:
   bool transposed() const override { return false; }
+
+  void Forward_gpu(const vector<Blob*>& bottom, const vector<Blob*>& top) override {
+    if (!sibling_ || bottom.size() != 1) {
+      BaseConvolutionLayer::Forward_gpu(bottom, top);
+      return;
+    }
+    // One contraction over both layers' filters into a scratch blob, then each
+    // layer's channels are copied to its own top.
+    const int m1 = geom_.channels_out, m2 = sibling_->geom_.channels_out;
+    mcConvGeom g = geom_;
+    g.channels_out = m1 + m2;
+    if (!merged_plan_ || merged_h_ != g.height_in || merged_w_in_ != g.width_in || merged_m_ != m1 + m2) {
+      if (merged_plan_) mcConvPlanDestroy(merged_plan_);
+      merged_plan_ = nullptr;
+      MC_CHECK(mcConvPlanCreate(&g, &merged_plan_));
+      merged_h_ = g.height_in;
+      merged_w_in_ = g.width_in;
+      merged_m_ = m1 + m2;
+      merged_version_ = ~0ull;
+    }
+    const bool any_bias = bias_term_ || sibling_->bias_term_;
+    uint64_t v = BlobVersion(blobs_[0]) * 1000003ull + BlobVersion(sibling_->blobs_[0]);
+    if (bias_term_) v = v * 1000003ull + BlobVersion(blobs_[1]);
+    if (sibling_->bias_term_) v = v * 1000003ull + BlobVersion(sibling_->blobs_[1]);
+    if (v != merged_version_) {
+      const long w1 = blobs_[0]->count(), w2 = sibling_->blobs_[0]->count();
+      merged_filter_.Reshape(vector<int>{m1 + m2, geom_.channels_in, geom_.kernel_h, geom_.kernel_w});
+      float* w = merged_filter_.mutable_gpu_data();
+      MC_CHECK(mcCopy2D(blobs_[0]->gpu_data(), w1, w, w1, w1, 1, cur_stream()));
+      MC_CHECK(mcCopy2D(sibling_->blobs_[0]->gpu_data(), w2, w + w1, w2, w2, 1, cur_stream()));
+      if (any_bias) {
+        merged_bias_.Reshape(vector<int>{m1 + m2});
+        float* b = merged_bias_.mutable_gpu_data();
+        if (bias_term_) {
+          MC_CHECK(mcCopy2D(blobs_[1]->gpu_data(), m1, b, m1, m1, 1, cur_stream()));
+        } else {
+          MC_CHECK(mcFill(b, m1, 0.f, cur_stream()));
+        }
+        if (sibling_->bias_term_) {
+          MC_CHECK(mcCopy2D(sibling_->blobs_[1]->gpu_data(), m2, b + m1, m2, m2, 1, cur_stream()));
+        } else {
+          MC_CHECK(mcFill(b + m1, m2, 0.f, cur_stream()));
+        }
+      }
+      MC_CHECK(mcConvPlanSetWeights(merged_plan_, merged_filter_.gpu_data(), cur_stream()));
+      merged_version_ = v;
+    }
+    const int num = bottom[0]->shape(0);
+    const long plane = static_cast<long>(top[0]->shape(2)) * top[0]->shape(3);
+    merged_out_.Reshape(vector<int>{num, m1 + m2, top[0]->shape(2), top[0]->shape(3)});
+    mcEpilogue ep = {nullptr, any_bias ? merged_bias_.gpu_data() : nullptr, nullptr, MC_ACT_NONE, 0.f};
+    MC_CHECK(mcConvForward(merged_plan_, num, bottom[0]->gpu_data(), merged_out_.mutable_gpu_data(), &ep,
+                           cur_stream()));
+    const float* out = merged_out_.gpu_data();
+    MC_CHECK(mcCopy2D(out, (m1 + m2) * plane, top[0]->mutable_gpu_data(), m1 * plane, m1 * plane, num,
+                      cur_stream()));
+    MC_CHECK(mcCopy2D(out + m1 * plane, (m1 + m2) * plane, sibling_top_->mutable_gpu_data(), m2 * plane,
+                      m2 * plane, num, cur_stream()));
+  }
+
+  ConvolutionLayer* sibling_ = nullptr;
+  Blob* sibling_top_ = nullptr;
+  mcConvPlan* merged_plan_ = nullptr;
+  int merged_h_ = -1, merged_w_in_ = -1, merged_m_ = -1;
+  uint64_t merged_version_ = ~0ull;
+  Blob merged_filter_, merged_bias_, merged_out_;
 };
 REGISTER_LAYER_CLASS(Convolution);
 

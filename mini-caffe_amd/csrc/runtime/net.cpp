@@ -68,6 +68,7 @@ void Net::Init(const NetParameter& param) {
   for (size_t layer_id = 0; layer_id < layer_names_.size(); ++layer_id)
     layer_names_index_[layer_names_[layer_id]] = static_cast<int>(layer_id);
   layer_fused_.assign(layers_.size(), 0);
+  sibling_owner_.assign(layers_.size(), -1);
   residual_alias_.assign(layers_.size(), -1);
   PlaceMemory();
 }
@@ -177,10 +178,19 @@ void Net::PlaceMemory() {
         blob->ResetMemory();
         to_place.push_back(std::make_pair(static_cast<size_t>(blob->count()), blob));
       }
-      for (Blob* blob : tops) {
-        if (std::find(bottoms.begin(), bottoms.end(), blob) != bottoms.end()) continue;  // in place
-        blob->ResetMemory();
-        to_place.push_back(std::make_pair(static_cast<size_t>(blob->count()), blob));
+      if (sibling_owner_[i] < 0) {  // a merged sibling's top was placed with its owner's
+        for (Blob* blob : tops) {
+          if (std::find(bottoms.begin(), bottoms.end(), blob) != bottoms.end()) continue;  // in place
+          blob->ResetMemory();
+          to_place.push_back(std::make_pair(static_cast<size_t>(blob->count()), blob));
+        }
+      }
+      for (size_t j = i + 1; j < layers_.size() && j <= i + 8; ++j) {
+        if (sibling_owner_[j] != static_cast<int>(i)) continue;
+        for (Blob* blob : top_vecs_[j]) {  // written by this layer's launch
+          blob->ResetMemory();
+          to_place.push_back(std::make_pair(static_cast<size_t>(blob->count()), blob));
+        }
       }
     }
     std::sort(to_place.begin(), to_place.end(),
@@ -213,6 +223,8 @@ void Net::PlaceMemory() {
 void Net::PlanFusion() {
   fusion_dirty_ = false;
   layer_fused_.assign(layers_.size(), 0);
+  sibling_owner_.assign(layers_.size(), -1);
+  for (auto& l : layers_) l->AdoptSibling(nullptr, nullptr);
   for (size_t i = 0; i < layers_.size(); ++i) {
     if (layer_fused_[i] || !layers_[i]->AcceptsEpilogue()) continue;
     vector<Layer*> followers;
@@ -280,6 +292,40 @@ void Net::PlanFusion() {
     layers_[c]->SetResidual(R, layers_[e]->AbsorbedActivation());
     layer_fused_[e] = 1;
     residual_alias_[e] = t_id;
+  }
+
+  // Sibling convolutions (the loc and conf heads of an SSD source): two layers
+  // with one bottom and one top each that read the same blob with the same
+  // window geometry and have nothing folded in run as one launch of the first.
+  // The second's top must not exist before the second layer, and nothing between
+  // the two may write the shared bottom.
+  for (size_t i = 0; i < layers_.size(); ++i) {
+    vector<int> key_i, key_j;
+    if (layer_fused_[i] || bottom_vecs_[i].size() != 1 || top_vecs_[i].size() != 1) continue;
+    if (bottom_vecs_[i][0] == top_vecs_[i][0] || !layers_[i]->SiblingKey(&key_i)) continue;
+    Blob* shared = bottom_vecs_[i][0];
+    for (size_t j = i + 1; j < layers_.size() && j <= i + 8; ++j) {
+      bool writes_shared = false;
+      for (Blob* b : top_vecs_[j]) writes_shared = writes_shared || b == shared;
+      if (writes_shared) break;
+      if (layer_fused_[j] || sibling_owner_[j] >= 0) continue;
+      if (bottom_vecs_[j].size() != 1 || top_vecs_[j].size() != 1 || bottom_vecs_[j][0] != shared) continue;
+      Blob* top_j = top_vecs_[j][0];
+      if (top_j == shared || top_j == top_vecs_[i][0]) continue;
+      if (std::string(layers_[j]->type()) != layers_[i]->type()) continue;
+      if (!layers_[j]->SiblingKey(&key_j) || key_i != key_j) continue;
+      bool seen_before = false;
+      for (size_t k = 0; k < j && !seen_before; ++k) {
+        for (Blob* b : top_vecs_[k]) seen_before = seen_before || b == top_j;
+        for (Blob* b : bottom_vecs_[k]) seen_before = seen_before || b == top_j;
+      }
+      if (seen_before) continue;
+      layers_[i]->AdoptSibling(layers_[j].get(), top_j);
+      layers_[i]->Reshape(bottom_vecs_[i], top_vecs_[i]);  // sizes the scratch blob of the merged launch
+      layer_fused_[j] = 1;
+      sibling_owner_[j] = static_cast<int>(i);
+      break;  // one sibling per layer
+    }
   }
 
   // Views (Flatten, Reshape; the reference copies, src/layers/flatten_layer.cpp:34-39,

@@ -221,6 +221,63 @@ def test_googlenet_front_and_nin(gpu_mode):
     assert np.allclose(net.get_blob("prob").data.reshape(2, -1).sum(axis=1), 1, atol=1e-5)
 
 
+def test_sibling_convolutions_run_as_one_launch(gpu_mode):
+    """Convolutions that read the same blob with the same window (SSD's loc / conf heads, the
+    RPN's cls / bbox heads) are computed by one launch over the concatenated filters.  Pairs
+    with and without bias, a third sibling that stays alone, and neighbours that must not be
+    merged (other window, an in-place ReLU folded in, groups); later parameter updates of
+    either partner and a new input size are honoured."""
+    from minicaffe import zoo
+    from minicaffe.craft import input_layer
+    oracle.use_openblas(False)
+    C = 12
+    conv = lambda name, cout, k, pad, bias=True, group=1, seed=3: zoo.conv_layer(  # noqa: E731
+        name, "feat", name, C, cout, k, 1, pad, group=group, bias=bias, seed=seed, bias_value=0.3)
+    spec = [
+        input_layer({"data": (2, 3, 13, 11)}),
+        zoo.conv_layer("feat", "data", "feat", 3, C, 3, 1, 1, seed=3),
+        zoo.relu_layer("feat_relu", "feat"),
+        conv("loc", 8, 3, 1), conv("conf", 42, 3, 1),            # merged, both with bias
+        conv("third", 5, 3, 1),                                  # same window: no partner left
+        conv("a_nobias", 7, 1, 0, bias=False), conv("b_bias", 9, 1, 0),   # merged, one bias only
+        conv("c_nobias", 4, 5, 2, bias=False), conv("d_nobias", 6, 5, 2, bias=False),  # merged, no bias at all
+        conv("relu_head", 6, 3, 1), zoo.relu_layer("relu_head_relu", "relu_head"),   # has a follower: alone
+        conv("grouped", 6, 3, 1, group=3),
+    ]
+    tops = ["loc", "conf", "third", "a_nobias", "b_bias", "c_nobias", "d_nobias", "relu_head", "grouped"]
+    spec.append({"name": "cat", "type": "Concat", "bottom": tops, "top": ["cat"]})
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((2, 3, 13, 11)).astype(np.float32)
+    net = run_net(gpu_mode, spec, {"data": x}, tops)
+    want = netrun.oracle_forward(spec, {"data": x})
+    for name in tops + ["cat"]:
+        assert netrun.rel_err(net.get_blob(name).data, want[name]) < 1e-4, name
+    # which layers ran on their own: the profiler opens a scope per executed layer
+    import json
+    import tempfile
+    gpu_mode.Profiler.enable()
+    net.forward()
+    gpu_mode.Profiler.disable()
+    with tempfile.TemporaryDirectory() as d:
+        gpu_mode.Profiler.dump(d + "/p.json")
+        ran = {e["name"] for e in json.load(open(d + "/p.json"))["traceEvents"]}
+    assert {"loc", "third", "a_nobias", "c_nobias", "relu_head", "grouped"} <= ran
+    assert not ({"conf", "b_bias", "d_nobias", "relu_head_relu"} & ran)
+    # the second partner's filter and the first partner's bias change
+    params = dict(net.param_list)
+    by_name = {l["name"]: l for l in spec}
+    by_name["conf"]["blobs"][0] = by_name["conf"]["blobs"][0] * -0.5
+    params["conf_0"].data[...] = by_name["conf"]["blobs"][0]
+    by_name["loc"]["blobs"][1] = by_name["loc"]["blobs"][1] + 1.0
+    params["loc_1"].data[...] = by_name["loc"]["blobs"][1]
+    x2 = rng.standard_normal((3, 3, 9, 14)).astype(np.float32)
+    net.forward(data=x2)
+    want = netrun.oracle_forward(spec, {"data": x2})
+    for name in tops + ["cat"]:
+        got = net.get_blob(name).data
+        assert got.shape == want[name].shape and netrun.rel_err(got, want[name]) < 1e-4, name
+
+
 def test_unfused_layers_standalone(gpu_mode):
     """BatchNorm / Scale / Bias / ReLU / TanH / Sigmoid / Eltwise that do NOT follow a
     contraction run as their own kernels; Split, Slice, Concat, Flatten, Reshape,
