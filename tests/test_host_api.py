@@ -471,3 +471,13 @@ def test_landmark_spec_equals_the_reference_prototxt():
     # and the fixture is the reference's file
     a = open(os.path.join(REF, "example", "models", "deeplandmark", "2_LE1.caffemodel"), "rb").read()
     assert a == open(os.path.join(GOLDEN, "deeplandmark_2_LE1.caffemodel"), "rb").read()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asking for more ends with a message instead of a number."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=60)
+    assert r.returncode != 0 and "one GPU" in (r.stdout + r.stderr)
+    assert "{" not in r.stdout
