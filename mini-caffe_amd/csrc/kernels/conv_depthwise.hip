@@ -74,21 +74,21 @@ __global__ __launch_bounds__(256) void depthwise_kernel(const DepthwiseArgs a, l
   }
 }
 
-// Undilated kernels with stride SH down the column: a thread makes four
-// vertically neighbouring outputs (same column, rows 4*q .. 4*q+3) from
-// 3*SH + KH input rows, so overlapping taps are read once per thread instead of
+// Undilated kernels with stride SH down the column: a thread makes R
+// vertically neighbouring outputs (same column, rows R*q .. R*q+R-1) from
+// (R-1)*SH + KH input rows, so overlapping taps are read once per thread instead of
 // once per output and the index arithmetic is shared; neighbouring threads sit on
 // neighbouring columns, so every load and store stays coalesced.
-template <int KH, int KW, int SH, bool TRANS>
-__global__ __launch_bounds__(256) void depthwise4_kernel(const DepthwiseArgs a, long groups,
+template <int KH, int KW, int SH, bool TRANS, int R>
+__global__ __launch_bounds__(256) void depthwise_rows_kernel(const DepthwiseArgs a, long groups,
                                                          int ho_groups) {
-  constexpr int L = 3 * SH + KH;
+  constexpr int L = (R - 1) * SH + KH;
   for (long gi = blockIdx.x * 256L + threadIdx.x; gi < groups; gi += gridDim.x * 256L) {
     const unsigned gu = static_cast<unsigned>(gi);   // groups < 2^31
     const unsigned row = gu / static_cast<unsigned>(a.Wo);        // (n*Cout + oc)*ho_groups + q
     const int wo = static_cast<int>(gu - row * a.Wo);
     const unsigned nc = row / static_cast<unsigned>(ho_groups);
-    const int ho0 = static_cast<int>(row - nc * ho_groups) * 4;
+    const int ho0 = static_cast<int>(row - nc * ho_groups) * R;
     const unsigned cout = static_cast<unsigned>(a.C * a.mult);
     const unsigned n = nc / cout;
     const int oc = static_cast<int>(nc - n * cout);
@@ -101,7 +101,9 @@ __global__ __launch_bounds__(256) void depthwise4_kernel(const DepthwiseArgs a, 
     for (int r = 0; r < KH; ++r)
 #pragma unroll
       for (int s = 0; s < KW; ++s) wv[r][s] = wp[r * KW + s];
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    float acc[R];
+#pragma unroll
+    for (int o = 0; o < R; ++o) acc[o] = 0.f;
 #pragma unroll
     for (int t = 0; t < L; ++t) {
       const int hi = hi0 + t;
@@ -115,7 +117,7 @@ __global__ __launch_bounds__(256) void depthwise4_kernel(const DepthwiseArgs a, 
       }
       // input row t is tap row t - o*SH of output o
 #pragma unroll
-      for (int o = 0; o < 4; ++o) {
+      for (int o = 0; o < R; ++o) {
         const int r = t - o * SH;
         if (r >= 0 && r < KH) {
 #pragma unroll
@@ -125,7 +127,7 @@ __global__ __launch_bounds__(256) void depthwise4_kernel(const DepthwiseArgs a, 
     }
     const float sc = a.scale ? a.scale[oc] : 1.f, sf = a.shift ? a.shift[oc] : 0.f;
 #pragma unroll
-    for (int o = 0; o < 4; ++o) {
+    for (int o = 0; o < R; ++o) {
       if (ho0 + o >= a.Ho) break;
       const long out = (static_cast<long>(nc) * a.Ho + ho0 + o) * a.Wo + wo;
       float val = acc[o];
@@ -144,16 +146,26 @@ int depthwise_forward(const DepthwiseArgs& a, hipStream_t stream) {
   if (count == 0) return 0;
   const bool trans = a.act == MC_ACT_TANH || a.act == MC_ACT_SIGMOID;
   if (a.kh == 3 && a.kw == 3 && a.dh == 1 && a.dw == 1 && (a.sh == 1 || a.sh == 2)) {
-    const int ho_groups = ceil_div(a.Ho, 4);
+    // R output rows per thread: more rows share more of their input rows (R + 2 rows
+    // read for R outputs at stride 1), as long as the map is tall enough to keep
+    // every thread's rows inside it
+    const int rows = a.Ho >= 96 ? 16 : (a.Ho >= (a.sh == 1 ? 16 : 32) ? 8 : 4);
+    const int ho_groups = ceil_div(a.Ho, rows);
     const long groups = static_cast<long>(a.num) * a.C * a.mult * ho_groups * a.Wo;
     const unsigned gb = ew_blocks(groups, 256);
+#define MC_DW_LAUNCH(SH, R)                                                                   \
+  if (trans) depthwise_rows_kernel<3, 3, SH, true, R><<<gb, 256, 0, stream>>>(a, groups, ho_groups); \
+  else depthwise_rows_kernel<3, 3, SH, false, R><<<gb, 256, 0, stream>>>(a, groups, ho_groups)
     if (a.sh == 1) {
-      if (trans) depthwise4_kernel<3, 3, 1, true><<<gb, 256, 0, stream>>>(a, groups, ho_groups);
-      else depthwise4_kernel<3, 3, 1, false><<<gb, 256, 0, stream>>>(a, groups, ho_groups);
+      if (rows == 16) { MC_DW_LAUNCH(1, 16); }
+      else if (rows == 8) { MC_DW_LAUNCH(1, 8); }
+      else { MC_DW_LAUNCH(1, 4); }
     } else {
-      if (trans) depthwise4_kernel<3, 3, 2, true><<<gb, 256, 0, stream>>>(a, groups, ho_groups);
-      else depthwise4_kernel<3, 3, 2, false><<<gb, 256, 0, stream>>>(a, groups, ho_groups);
+      if (rows == 16) { MC_DW_LAUNCH(2, 16); }
+      else if (rows == 8) { MC_DW_LAUNCH(2, 8); }
+      else { MC_DW_LAUNCH(2, 4); }
     }
+#undef MC_DW_LAUNCH
     MC_LAUNCH_CHECK();
     return 0;
   }

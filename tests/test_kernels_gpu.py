@@ -275,10 +275,12 @@ def test_depthwise_with_epilogue(K):
     (5, 150, 150, 1, 1, 1),    # MobileNet conv1/dw
     (4, 75, 75, 2, 1, 2),      # stride 2, odd extents
     (3, 8, 585, 2, 0, 2), (3, 33, 130, 1, 1, 2), (2, 6, 1024, 1, 1, 1), (2, 6, 1025, 2, 1, 1),
+    (3, 200, 40, 2, 1, 1),     # stride 2 with 16 output rows per thread (100 rows: 6 groups + 4)
+    (2, 97, 9, 1, 0, 2),       # stride 1, 95 output rows: 8 per thread, ragged last group
 ])
 def test_depthwise_3x3_shapes(K, c, h, w, s, p, n):
-    """3x3 depthwise at stride 1 and 2 (four output rows per thread): small and large planes,
-    odd extents, rows wider than a workgroup, with the whole epilogue."""
+    """3x3 depthwise at stride 1 and 2 (4, 8 or 16 output rows per thread by map height): small
+    and large planes, odd extents, rows wider than a workgroup, with the whole epilogue."""
     rng = np.random.default_rng(21)
     x = rng.standard_normal((n, c, h, w)).astype(np.float32)
     wt = (rng.standard_normal((c, 1, 3, 3)) * 0.3).astype(np.float32)
