@@ -572,41 +572,53 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(
 // (same tap table, same packed filter, read through scalar loads) and keeps the
 // kThinM sums in registers; neighbouring threads read neighbouring addresses.
 constexpr int kThinM = 4;
+constexpr int kThinPx = 2;  // output pixels per thread: the scalar loads of a K row serve both
 __global__ __launch_bounds__(256) void thin_conv_kernel(const IgemmBatch batch, int pointwise) {
   const IgemmArgs& a = batch.sub[blockIdx.z];
-  const int p = blockIdx.x * 256 + threadIdx.x;
   const int g = blockIdx.y;
   // the gather of igemm_kernel's kModeMasks: pixel origin in the VGPR offset of a
   // buffer load, tap offset in its scalar offset, bit 31 for "outside the image"
   const __amdgpu_buffer_rsrc_t xres =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.x), 0, a.x_bytes, kBufferFlags);
-  unsigned xvoff = kNoElement;
-  unsigned row_bad = 0xFFFFFFFFu, col_bad = 0xFFFFFFFFu;
-  int n = 0, qh = 0, qw = 0;
-  if (p < a.P) {
-    n = fast_div(p, a.div_hw_mul, a.div_hw_shift);
-    const int rem = p - n * a.HqWq;
-    qh = fast_div(rem, a.div_w_mul, a.div_w_shift);
-    qw = rem - qh * a.Wq;
-    const int hi0 = qh * a.q_sh + a.in_oh;
-    const int wi0 = qw * a.q_sw + a.in_ow;
-    xvoff = static_cast<unsigned>(
-        ((n * a.x_nstride + g * a.x_gstride + hi0 * a.W + wi0) << 2) + a.pix_shift);
-    row_bad = 0x80000000u;
-    col_bad = 0u;
-    for (int b = 0; b < a.n_dh; ++b)
-      row_bad |= static_cast<unsigned>(static_cast<unsigned>(hi0 + a.tap_dh[b]) >=
-                                       static_cast<unsigned>(a.H))
-                 << b;
-    for (int b = 0; b < a.n_dw; ++b)
-      col_bad |= static_cast<unsigned>(static_cast<unsigned>(wi0 + a.tap_dw[b]) >=
-                                       static_cast<unsigned>(a.W))
-                 << b;
+  // pixel j of this thread is gridDim.x * 256 pixels after pixel j - 1, so the
+  // lanes of a wavefront stay on neighbouring pixels
+  int pix[kThinPx];
+  unsigned xvoff[kThinPx], row_bad[kThinPx], col_bad[kThinPx];
+  long ybase[kThinPx];
+#pragma unroll
+  for (int j = 0; j < kThinPx; ++j) {
+    const int p = (j * static_cast<int>(gridDim.x) + static_cast<int>(blockIdx.x)) * 256 + threadIdx.x;
+    pix[j] = p;
+    xvoff[j] = kNoElement;
+    row_bad[j] = 0xFFFFFFFFu;
+    col_bad[j] = 0xFFFFFFFFu;
+    ybase[j] = 0;
+    if (p < a.P) {
+      const int n = fast_div(p, a.div_hw_mul, a.div_hw_shift);
+      const int rem = p - n * a.HqWq;
+      const int qh = fast_div(rem, a.div_w_mul, a.div_w_shift);
+      const int qw = rem - qh * a.Wq;
+      const int hi0 = qh * a.q_sh + a.in_oh;
+      const int wi0 = qw * a.q_sw + a.in_ow;
+      xvoff[j] = static_cast<unsigned>(
+          ((n * a.x_nstride + g * a.x_gstride + hi0 * a.W + wi0) << 2) + a.pix_shift);
+      unsigned rb = 0x80000000u, cb = 0u;
+      for (int b = 0; b < a.n_dh; ++b)
+        rb |= static_cast<unsigned>(static_cast<unsigned>(hi0 + a.tap_dh[b]) >= static_cast<unsigned>(a.H)) << b;
+      for (int b = 0; b < a.n_dw; ++b)
+        cb |= static_cast<unsigned>(static_cast<unsigned>(wi0 + a.tap_dw[b]) >= static_cast<unsigned>(a.W)) << b;
+      row_bad[j] = rb;
+      col_bad[j] = cb;
+      ybase[j] = static_cast<long>(n) * a.y_nstride +
+                 static_cast<long>(qh * a.out_sh + a.out_oh) * a.Wo + qw * a.out_sw + a.out_ow;
+    }
   }
   const float* __restrict__ wg = a.wt + static_cast<size_t>(g) * a.Kpad * a.Mpad;
-  float acc[kThinM];
+  float acc[kThinPx][kThinM];
 #pragma unroll
-  for (int m = 0; m < kThinM; ++m) acc[m] = 0.f;
+  for (int j = 0; j < kThinPx; ++j)
+#pragma unroll
+    for (int m = 0; m < kThinM; ++m) acc[j][m] = 0.f;
 #define MC_LOADF(res, voff, soff) \
   __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(res, voff, soff, 0))
   // K in tiles of 16 over the padded extent (padding rows have zero filters and,
@@ -614,51 +626,54 @@ __global__ __launch_bounds__(256) void thin_conv_kernel(const IgemmBatch batch, 
   // the 16 table entries are contiguous, so they arrive in a few wide scalar loads.
   const int kmax = a.K - 1;
   const unsigned x_cbytes = static_cast<unsigned>(a.x_cstride) * 4;
-  auto gather16 = [&](int k0, float (&v)[BK]) {
+  for (int k0 = 0; k0 < a.Kpad; k0 += BK) {
+    const float* __restrict__ wk = wg + (k0 >> 4) * (a.Mpad * BK);
+    float v[kThinPx][BK];
     if (pointwise) {
 #pragma unroll
-      for (int j = 0; j < BK; ++j)
-        v[j] = MC_LOADF(xres, xvoff, static_cast<unsigned>(min(k0 + j, kmax)) * x_cbytes);
+      for (int i = 0; i < BK; ++i) {
+        const unsigned soff = static_cast<unsigned>(min(k0 + i, kmax)) * x_cbytes;
+#pragma unroll
+        for (int j = 0; j < kThinPx; ++j) v[j][i] = MC_LOADF(xres, xvoff[j], soff);
+      }
     } else {
       const int4* __restrict__ tk = a.ktab + k0;
 #pragma unroll
-      for (int j = 0; j < BK; ++j) {
-        const int4 t = tk[j];
-        const unsigned rb = __builtin_amdgcn_ubfe(row_bad, t.y, 1);
-        const unsigned cb = __builtin_amdgcn_ubfe(col_bad, t.z, 1);
-        v[j] = MC_LOADF(xres, (cb << 31) | ((rb << 31) | xvoff), t.x);
+      for (int i = 0; i < BK; ++i) {
+        const int4 t = tk[i];
+#pragma unroll
+        for (int j = 0; j < kThinPx; ++j) {
+          const unsigned rb = __builtin_amdgcn_ubfe(row_bad[j], t.y, 1);
+          const unsigned cb = __builtin_amdgcn_ubfe(col_bad[j], t.z, 1);
+          v[j][i] = MC_LOADF(xres, (cb << 31) | ((rb << 31) | xvoff[j]), t.x);
+        }
       }
     }
-  };
-  // one K tile of 16 rows per step; the loads of the next tile are issued before
-  // this one is multiplied
-  float v[BK], ahead[BK];
-  if (a.Kpad > 0) gather16(0, v);
-  for (int k0 = 0; k0 < a.Kpad; k0 += BK) {
-    const float* __restrict__ wk = wg + (k0 >> 4) * (a.Mpad * BK);
-    if (k0 + BK < a.Kpad) gather16(k0 + BK, ahead);
 #pragma unroll
-    for (int j = 0; j < BK; ++j) {
+    for (int i = 0; i < BK; ++i) {
 #pragma unroll
-      for (int m = 0; m < kThinM; ++m) acc[m] += wk[m * BK + j] * v[j];
+      for (int m = 0; m < kThinM; ++m) {
+        const float w = wk[m * BK + i];
+#pragma unroll
+        for (int j = 0; j < kThinPx; ++j) acc[j][m] += w * v[j][i];
+      }
     }
-#pragma unroll
-    for (int j = 0; j < BK; ++j) v[j] = ahead[j];
   }
 #undef MC_LOADF
-  if (p >= a.P) return;
-  const long ybase = static_cast<long>(n) * a.y_nstride +
-                     static_cast<long>(qh * a.out_sh + a.out_oh) * a.Wo + qw * a.out_sw + a.out_ow;
 #pragma unroll
-  for (int m = 0; m < kThinM; ++m) {
-    if (m >= a.M) break;
-    const int c = g * a.M + m;
-    const long idx = ybase + static_cast<long>(c) * a.y_cstride;
-    float v = acc[m];
-    if (a.scale) v *= a.scale[c];
-    if (a.shift) v += a.shift[c];
-    if (a.residual) v += a.residual[idx];
-    a.y[idx] = apply_act(v, a.act, a.slope);
+  for (int j = 0; j < kThinPx; ++j) {
+    if (pix[j] >= a.P) continue;
+#pragma unroll
+    for (int m = 0; m < kThinM; ++m) {
+      if (m >= a.M) break;
+      const int c = g * a.M + m;
+      const long idx = ybase[j] + static_cast<long>(c) * a.y_cstride;
+      float v = acc[j][m];
+      if (a.scale) v *= a.scale[c];
+      if (a.shift) v += a.shift[c];
+      if (a.residual) v += a.residual[idx];
+      a.y[idx] = apply_act(v, a.act, a.slope);
+    }
   }
 }
 
@@ -1295,7 +1310,7 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
     if (thin) {
       long most = 0;
       for (int i = 0; i < nsub; ++i) most = std::max<long>(most, batch.sub[i].P);
-      dim3 grid(static_cast<unsigned>(ceil_div(most, 256L)), g.group, nsub);
+      dim3 grid(static_cast<unsigned>(ceil_div(most, 256L * kThinPx)), g.group, nsub);
       thin_conv_kernel<<<grid, 256, 0, st>>>(batch, pointwise ? 1 : 0);
     } else {
       dim3 grid(static_cast<unsigned>(max_blocks), g.group, nsub * slices);
