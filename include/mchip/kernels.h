@@ -98,6 +98,16 @@ int mcConvPlanSetWeights(mcConvPlan* plan, const float* weights, void* stream);
 int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* top,
                   const mcEpilogue* epilogue, void* stream);
 
+/* mcConvForward for a plan whose output channels belong to two blobs: channels
+ * [0, channels_first) of every image go to top_first [num, channels_first, Ho, Wo],
+ * the others to top_second [num, Cout - channels_first, Ho, Wo].  Group 1, no
+ * residual.  No counterpart in the reference: it serves two layers
+ * that read the same blob with the same window (conv_layer.cu:7-22 twice) as one
+ * launch over the concatenated filters. */
+int mcConvForwardTwoTops(const mcConvPlan* plan, int num, const float* bottom, float* top_first,
+                         int channels_first, float* top_second, const mcEpilogue* epilogue,
+                         void* stream);
+
 /* Algorithmic FLOPs of one mcConvForward call (2*MACs, padding taps counted). */
 double mcConvPlanFlops(const mcConvPlan* plan, int num);
 

@@ -565,6 +565,33 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(
   }
 }
 
+// The same tail for a launch whose output channels belong to two blobs (two
+// sibling layers computed together): channels [0, c_first) of every image go to
+// y_first [num, c_first, plane], the others to y_second.  One thread per element;
+// such outputs are small (detection heads).
+__global__ __launch_bounds__(256) void splitk_reduce_two_kernel(
+    const float* __restrict__ part, int slices, long slice_stride, long count,
+    float* __restrict__ y_first, float* __restrict__ y_second, int c_first,
+    const float* __restrict__ scale, const float* __restrict__ shift, int plane, int C, int act,
+    float slope) {
+  const long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x;
+  if (i >= count) return;
+  float v = part[i];
+  for (int z = 1; z < slices; ++z) v += part[z * slice_stride + i];
+  const unsigned iu = static_cast<unsigned>(i);  // count < 2^29
+  const unsigned row = iu / static_cast<unsigned>(plane);  // n * C + c
+  const unsigned p = iu - row * plane;
+  const unsigned n = row / static_cast<unsigned>(C);
+  const int c = static_cast<int>(row - n * C);
+  if (scale) v *= scale[c];
+  if (shift) v += shift[c];
+  v = apply_act(v, act, slope);
+  if (c < c_first)
+    y_first[(static_cast<long>(n) * c_first + c) * plane + p] = v;
+  else
+    y_second[(static_cast<long>(n) * (C - c_first) + (c - c_first)) * plane + p] = v;
+}
+
 // Convolutions with at most kThinM output channels per group (the image-producing
 // last layer of a generator, a one-channel score map): a 32-row MFMA tile would
 // multiply mostly padding, and the layer is bound by reading its bottom blob
@@ -1154,8 +1181,14 @@ int mcConvPlanForceSplit(mcConvPlan* plan, int slices) {
   return 0;
 }
 
-int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* top,
-                  const mcEpilogue* ep, void* stream) {
+}  // extern "C"
+
+namespace {
+
+// top_second != nullptr: the plan's output channels [0, c_first) go to `top`, the
+// others to top_second.
+int conv_forward(const mcConvPlan* plan, int num, const float* bottom, float* top,
+                 const mcEpilogue* ep, void* stream, float* top_second, int c_first) {
   MC_REQUIRE(plan && bottom && top, "mcConvForward: null argument");
   MC_REQUIRE(num > 0, "mcConvForward: batch must be positive");
   const mcConvGeom& g = plan->geom;
@@ -1165,6 +1198,13 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
   MC_REQUIRE(in_count < (1L << 29) && out_count < (1L << 29),
              "mcConvForward: blob exceeds 2^29 elements");
   hipStream_t st = static_cast<hipStream_t>(stream);
+  float* const top_first = top;
+  if (top_second) {
+    MC_REQUIRE(!plan->depthwise && g.group == 1 && c_first > 0 && c_first < g.channels_out &&
+                   !(ep && ep->residual),
+               "mcConvForwardTwoTops: needs group 1, a split inside the output channels and no "
+               "residual");
+  }
   if (plan->depthwise) {
     DepthwiseArgs d = {bottom, plan->dw_weights, top, ep ? ep->scale : nullptr,
                        ep ? ep->shift : nullptr, ep ? ep->residual : nullptr, num,
@@ -1215,10 +1255,14 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
     flops += 2.0 * pixels * plan->M * g.group * s->K;
   }
   if (min_kt == (1 << 30)) min_kt = 1;
-  const bool thin = use_thin(plan, num);
+  // (the per-pixel kernel writes one top only)
+  const bool thin = !top_second && use_thin(plan, num);
   // slices are chosen for the plan as a whole: all sub-problems of a launch run
   // side by side, and one pass sums the slices of the whole top blob
-  const int slices = thin ? 1 : pick_split(plan, total_blocks, min_kt);
+  // Two tops are told apart by the pass that sums the slices, so such a launch
+  // has at least two of them (a slice past the last K tile adds zeros).
+  int slices = thin ? 1 : pick_split(plan, total_blocks, min_kt);
+  if (top_second && slices == 1) slices = 2;
   const long slice_stride = (out_count + 3) / 4 * 4;
   float* ws = nullptr;
   if (slices > 1 && get_workspace(st, sizeof(float) * slice_stride * slices, &ws)) return -1;
@@ -1330,7 +1374,13 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
     }
     MC_LAUNCH_CHECK();
   }
-  if (slices > 1) {
+  if (slices > 1 && top_second) {
+    splitk_reduce_two_kernel<<<static_cast<unsigned>(ceil_div(out_count, 256L)), 256, 0, st>>>(
+        ws, slices, slice_stride, out_count, top_first, top_second, c_first, ep ? ep->scale : nullptr,
+        ep ? ep->shift : nullptr, plan->Ho * plan->Wo, g.channels_out,
+        ep ? ep->activation : MC_ACT_NONE, ep ? ep->negative_slope : 0.f);
+    MC_LAUNCH_CHECK();
+  } else if (slices > 1) {
     splitk_reduce_kernel<<<static_cast<unsigned>(ceil_div(out_count, 1024L)), 256, 0, st>>>(
         ws, slices, slice_stride, out_count, top, ep ? ep->scale : nullptr,
         ep ? ep->shift : nullptr, ep ? ep->residual : nullptr, plan->Ho * plan->Wo,
@@ -1342,6 +1392,22 @@ int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* t
     g_timed.push_back(tl);
   }
   return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* top,
+                  const mcEpilogue* ep, void* stream) {
+  return conv_forward(plan, num, bottom, top, ep, stream, nullptr, 0);
+}
+
+int mcConvForwardTwoTops(const mcConvPlan* plan, int num, const float* bottom, float* top_first,
+                         int channels_first, float* top_second, const mcEpilogue* ep,
+                         void* stream) {
+  MC_REQUIRE(top_second, "mcConvForwardTwoTops: null argument");
+  return conv_forward(plan, num, bottom, top_first, ep, stream, top_second, channels_first);
 }
 
 int mcConvTimingEnable(int on) {

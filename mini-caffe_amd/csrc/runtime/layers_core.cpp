@@ -312,17 +312,6 @@ class ConvolutionLayer : public BaseConvolutionLayer {
     sibling_top_ = sibling_top;
     merged_version_ = ~0ull;
   }
-  void Reshape(const vector<Blob*>& bottom, const vector<Blob*>& top) override {
-    BaseConvolutionLayer::Reshape(bottom, top);
-    if (sibling_)
-      merged_out_.Reshape(vector<int>{top[0]->shape(0), geom_.channels_out + sibling_->geom_.channels_out,
-                                      top[0]->shape(2), top[0]->shape(3)});
-  }
-  vector<Blob*> GetTempBlobs() override {
-    vector<Blob*> t;
-    if (sibling_) t.push_back(&merged_out_);
-    return t;
-  }
 
  protected:
   bool transposed() const override { return false; }
@@ -332,8 +321,8 @@ class ConvolutionLayer : public BaseConvolutionLayer {
       BaseConvolutionLayer::Forward_gpu(bottom, top);
       return;
     }
-    // One contraction over both layers' filters into a scratch blob, then each
-    // layer's channels are copied to its own top.
+    // One contraction over both layers' filters; the kernel stores each layer's
+    // channels into that layer's top.
     const int m1 = geom_.channels_out, m2 = sibling_->geom_.channels_out;
     mcConvGeom g = geom_;
     g.channels_out = m1 + m2;
@@ -374,16 +363,9 @@ class ConvolutionLayer : public BaseConvolutionLayer {
       merged_version_ = v;
     }
     const int num = bottom[0]->shape(0);
-    const long plane = static_cast<long>(top[0]->shape(2)) * top[0]->shape(3);
-    merged_out_.Reshape(vector<int>{num, m1 + m2, top[0]->shape(2), top[0]->shape(3)});
     mcEpilogue ep = {nullptr, any_bias ? merged_bias_.gpu_data() : nullptr, nullptr, MC_ACT_NONE, 0.f};
-    MC_CHECK(mcConvForward(merged_plan_, num, bottom[0]->gpu_data(), merged_out_.mutable_gpu_data(), &ep,
-                           cur_stream()));
-    const float* out = merged_out_.gpu_data();
-    MC_CHECK(mcCopy2D(out, (m1 + m2) * plane, top[0]->mutable_gpu_data(), m1 * plane, m1 * plane, num,
-                      cur_stream()));
-    MC_CHECK(mcCopy2D(out + m1 * plane, (m1 + m2) * plane, sibling_top_->mutable_gpu_data(), m2 * plane,
-                      m2 * plane, num, cur_stream()));
+    MC_CHECK(mcConvForwardTwoTops(merged_plan_, num, bottom[0]->gpu_data(), top[0]->mutable_gpu_data(), m1,
+                                  sibling_top_->mutable_gpu_data(), &ep, cur_stream()));
   }
 
   ConvolutionLayer* sibling_ = nullptr;
@@ -391,7 +373,7 @@ class ConvolutionLayer : public BaseConvolutionLayer {
   mcConvPlan* merged_plan_ = nullptr;
   int merged_h_ = -1, merged_w_in_ = -1, merged_m_ = -1;
   uint64_t merged_version_ = ~0ull;
-  Blob merged_filter_, merged_bias_, merged_out_;
+  Blob merged_filter_, merged_bias_;
 };
 REGISTER_LAYER_CLASS(Convolution);
 

@@ -321,7 +321,6 @@ void Net::PlanFusion() {
       }
       if (seen_before) continue;
       layers_[i]->AdoptSibling(layers_[j].get(), top_j);
-      layers_[i]->Reshape(bottom_vecs_[i], top_vecs_[i]);  // sizes the scratch blob of the merged launch
       layer_fused_[j] = 1;
       sibling_owner_[j] = static_cast<int>(i);
       break;  // one sibling per layer

@@ -87,6 +87,8 @@ LIB.mcConvPlanOutputShape.argtypes = [c_void_p, ctypes.POINTER(c_int), ctypes.PO
 LIB.mcConvPlanSetWeights.argtypes = [c_void_p, c_void_p, c_void_p]
 LIB.mcConvForward.argtypes = [c_void_p, c_int, c_void_p, c_void_p, ctypes.POINTER(Epilogue),
                               c_void_p]
+LIB.mcConvForwardTwoTops.argtypes = [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p,
+                                     ctypes.POINTER(Epilogue), c_void_p]
 LIB.mcConvPlanFlops.argtypes = [c_void_p, c_int]
 LIB.mcConvPlanFlops.restype = ctypes.c_double
 LIB.mcConvPlanKernelName.argtypes = [c_void_p, c_int]
@@ -142,6 +144,12 @@ class ConvPlan(object):
                 activation=ACT_NONE, negative_slope=0.0, stream=0):
         ep = Epilogue(scale, shift, residual, activation, negative_slope)
         check_mc(LIB.mcConvForward(self.handle, num, x_ptr, y_ptr, ctypes.byref(ep), stream))
+
+    def forward_two_tops(self, num, x_ptr, first_ptr, channels_first, second_ptr,
+                         scale=None, shift=None, activation=ACT_NONE, negative_slope=0.0, stream=0):
+        ep = Epilogue(scale, shift, None, activation, negative_slope)
+        check_mc(LIB.mcConvForwardTwoTops(self.handle, num, x_ptr, first_ptr, channels_first,
+                                          second_ptr, ctypes.byref(ep), stream))
 
     def flops(self, num):
         return LIB.mcConvPlanFlops(self.handle, num)

@@ -34,7 +34,7 @@ def fptr(t):
     return ctypes.c_void_p(t.data_ptr())
 
 
-K_ACT_NONE, K_ACT_TANH = 0, 2
+K_ACT_NONE, K_ACT_RELU, K_ACT_TANH = 0, 1, 2
 
 CONV_CASES = [
     # cin, h, w, cout, k, s, p, d, g, transposed, batch
@@ -130,6 +130,39 @@ def test_conv_few_output_channels(K, case, act):
                  residual=rd.data_ptr(), activation=act)
     torch.cuda.synchronize()
     assert close(y2.cpu().numpy(), got)
+
+
+@pytest.mark.parametrize("c_first", [8, 64, 100, 149])
+@pytest.mark.parametrize("split", [1, 0, 3])
+def test_conv_two_tops_equals_one_top_cut_in_two(K, split, c_first):
+    """mcConvForwardTwoTops writes the same values as mcConvForward, channel ranges
+    [0, c) and [c, C) each into a blob of its own (cuts inside the first, at the edge
+    of and inside a later 32-row block, and one channel before the end): with the
+    plan's own choice of K slices, with three forced slices, and with one requested
+    (two tops always run as at least two slices, so that case is compared with the
+    two-slice single-top result)."""
+    n, cin, h, w, cout, k, c_first = 3, 48, 9, 7, 150, 3, c_first
+    rng = np.random.default_rng(31)
+    x = rng.standard_normal((n, cin, h, w)).astype(np.float32)
+    wt = (rng.standard_normal((cout, cin, k, k)) * 0.1).astype(np.float32)
+    b = rng.standard_normal(cout).astype(np.float32)
+    plan = K.ConvPlan(K.conv_geom(cin, h, w, cout, k, 1, 1))
+    xd, wd, bd = dev(x), dev(wt), dev(b)
+    plan.set_weights(wd.data_ptr())
+    whole = torch.full((n, cout, h, w), float("nan"), device="cuda")
+    plan.force_split(max(split, 2) if split else 0)
+    plan.forward(n, xd.data_ptr(), whole.data_ptr(), shift=bd.data_ptr(), activation=K_ACT_RELU)
+    plan.force_split(split)
+    first = torch.full((n, c_first, h, w), float("nan"), device="cuda")
+    second = torch.full((n, cout - c_first, h, w), float("nan"), device="cuda")
+    plan.forward_two_tops(n, xd.data_ptr(), first.data_ptr(), c_first, second.data_ptr(),
+                          shift=bd.data_ptr(), activation=K_ACT_RELU)
+    torch.cuda.synchronize()
+    assert torch.equal(first, whole[:, :c_first]) and torch.equal(second, whole[:, c_first:])
+    want = np.maximum(oracle.conv_forward(oracle.conv_geom(cin, h, w, cout, k, 1, 1), x, wt, b), 0)
+    assert netrun.rel_err(whole.cpu().numpy(), want) < 1e-4
+    with pytest.raises(Exception, match="TwoTops"):
+        plan.forward_two_tops(n, xd.data_ptr(), first.data_ptr(), cout, second.data_ptr())
 
 
 def test_conv_epilogue_matches_unfused_chain(K):
