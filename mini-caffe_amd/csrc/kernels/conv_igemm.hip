@@ -860,33 +860,6 @@ int pick_split(const mcConvPlan* plan, long blocks, int KT) {
   return std::max(s, 1);
 }
 
-// Partial sums of split-K launches: one grow-only buffer per (thread, stream);
-// launches on one stream are ordered, so consecutive layers can share it.
-struct Workspace {
-  float* ptr = nullptr;
-  size_t bytes = 0;
-};
-thread_local std::vector<std::pair<hipStream_t, Workspace>> g_workspaces;
-
-int get_workspace(hipStream_t st, size_t bytes, float** out) {
-  Workspace* ws = nullptr;
-  for (auto& e : g_workspaces)
-    if (e.first == st) ws = &e.second;
-  if (!ws) {
-    g_workspaces.emplace_back(st, Workspace());
-    ws = &g_workspaces.back().second;
-  }
-  if (ws->bytes < bytes) {
-    if (ws->ptr) MC_HIP(hipFree(ws->ptr));  // waits for the device
-    ws->ptr = nullptr;
-    ws->bytes = 0;
-    MC_HIP(hipMalloc(&ws->ptr, bytes));
-    ws->bytes = bytes;
-  }
-  *out = ws->ptr;
-  return 0;
-}
-
 int free_sub(SubProblem& s) {
   if (s.ktab_dev) (void)hipFree(s.ktab_dev);
   if (s.tap_dev) (void)hipFree(s.tap_dev);
@@ -1265,7 +1238,7 @@ int conv_forward(const mcConvPlan* plan, int num, const float* bottom, float* to
   if (top_second && slices == 1) slices = 2;
   const long slice_stride = (out_count + 3) / 4 * 4;
   float* ws = nullptr;
-  if (slices > 1 && get_workspace(st, sizeof(float) * slice_stride * slices, &ws)) return -1;
+  if (slices > 1 && stream_workspace(st, sizeof(float) * slice_stride * slices, &ws)) return -1;
 
   TimedLaunch tl;
   if (g_timing) {

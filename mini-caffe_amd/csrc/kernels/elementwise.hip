@@ -105,26 +105,33 @@ __device__ __forceinline__ float block_sum(float v, float* lds16) {
   return t;
 }
 
-// Batch statistics of one channel per workgroup (1024 threads): mean, then the
-// mean of squared deviations, as two passes over the channel's num x spatial
-// values (the second pass re-reads them from cache).  VEC = 4 walks each image's
-// plane with float4 loads; the (image, position) pair of a thread advances by a
-// fixed step, so the loops hold no division.
+// Batch statistics of one channel: mean, then the mean of squared deviations, as
+// two passes over the values (the second pass re-reads them from cache).  A
+// workgroup (up to 1024 threads) takes the images [blockIdx.y * per, + per) of
+// channel blockIdx.x.  With one part per channel it writes mean and deviation
+// itself; otherwise it leaves {mean, sum of squared deviations from that mean}
+// of its part in `partial`, and bn_batch_combine_kernel merges the parts (the
+// parallel form of the two-pass variance: M2 = sum M2_i + sum n_i (m_i - m)^2).
+// VEC = 4 walks each image's plane with float4 loads; the (image, position) pair
+// of a thread advances by a fixed step, so the loops hold no division.
 template <int VEC>
 __global__ __launch_bounds__(1024) void bn_batch_stats_kernel(const float* __restrict__ x, int num,
                                                               int C, int spatial, float eps,
                                                               float* __restrict__ mean,
-                                                              float* __restrict__ stdev) {
+                                                              float* __restrict__ stdev, int per,
+                                                              float2* __restrict__ partial) {
   __shared__ float red[16];
   const int c = blockIdx.x;
-  const int per_row = spatial / VEC;                    // vectors per image plane
+  const int first = blockIdx.y * per;
+  const int last = min(first + per, num);  // images [first, last)
+  const int per_row = spatial / VEC;       // vectors per image plane
   const int step_n = blockDim.x / per_row, step_v = blockDim.x % per_row;
-  const int n0 = threadIdx.x / per_row, v0 = threadIdx.x % per_row;
-  const float alpha = static_cast<float>(1. / (static_cast<double>(num) * spatial));
+  const int n0 = first + threadIdx.x / per_row, v0 = threadIdx.x % per_row;
+  const float alpha = static_cast<float>(1. / (static_cast<double>(last - first) * spatial));
   const long plane = spatial, image = (long)C * spatial;
   const float* __restrict__ xc = x + c * plane;
   float s = 0.f;
-  for (int n = n0, v = v0; n < num;) {
+  for (int n = n0, v = v0; n < last;) {
     const float* p = xc + n * image + v * VEC;
     if (VEC == 4) {
       const float4 t = *reinterpret_cast<const float4*>(p);
@@ -141,7 +148,7 @@ __global__ __launch_bounds__(1024) void bn_batch_stats_kernel(const float* __res
   }
   const float m = alpha * block_sum(s, red);
   float q = 0.f;
-  for (int n = n0, v = v0; n < num;) {
+  for (int n = n0, v = v0; n < last;) {
     const float* p = xc + n * image + v * VEC;
     if (VEC == 4) {
       const float4 t = *reinterpret_cast<const float4*>(p);
@@ -158,11 +165,40 @@ __global__ __launch_bounds__(1024) void bn_batch_stats_kernel(const float* __res
       ++n;
     }
   }
-  const float var = alpha * block_sum(q, red);
+  const float m2 = block_sum(q, red);
   if (threadIdx.x == 0) {
-    mean[c] = m;
-    stdev[c] = sqrtf(var + eps);
+    if (partial) {
+      partial[c * gridDim.y + blockIdx.y] = make_float2(m, m2);
+    } else {
+      mean[c] = m;
+      stdev[c] = sqrtf(alpha * m2 + eps);
+    }
   }
+}
+
+// One thread per channel merges the parts of bn_batch_stats_kernel, in part order.
+__global__ __launch_bounds__(256) void bn_batch_combine_kernel(const float2* __restrict__ partial,
+                                                               int parts, int per, int num, int C,
+                                                               int spatial, float eps,
+                                                               float* __restrict__ mean,
+                                                               float* __restrict__ stdev) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  const float total = static_cast<float>(num) * spatial;
+  float m = 0.f;
+  for (int z = 0; z < parts; ++z) {
+    const float n_z = static_cast<float>(min(per, num - z * per)) * spatial;
+    m += partial[c * parts + z].x * (n_z / total);
+  }
+  float m2 = 0.f;
+  for (int z = 0; z < parts; ++z) {
+    const float n_z = static_cast<float>(min(per, num - z * per)) * spatial;
+    const float2 t = partial[c * parts + z];
+    const float d = t.x - m;
+    m2 += t.y + n_z * d * d;
+  }
+  mean[c] = m;
+  stdev[c] = sqrtf(m2 / total + eps);
 }
 
 struct FoldArgs {
@@ -328,15 +364,34 @@ int mcBatchNormBatchStats(const float* x, int num, int channels, int spatial, fl
   MC_REQUIRE(x && mean && stdev, "mcBatchNormBatchStats: null argument");
   MC_REQUIRE(num > 0 && channels > 0 && spatial > 0, "mcBatchNormBatchStats: bad extents");
   const bool vec = spatial % 4 == 0 && aligned16(x);
-  const long per_c = (long)num * (vec ? spatial / 4 : spatial);
-  const int threads = per_c >= 1024 ? 1024 : 256;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  // Few channels would leave most of the chip idle: cut each channel's images
+  // into parts of at least 4096 values (16384 with float4 loads) until about
+  // four workgroups per compute unit exist.
+  const long part_min = vec ? 16384 : 4096;
+  int parts = 1;
+  while (channels * parts < 1024 && parts * 2 <= num && ((long)num / (parts * 2)) * spatial >= part_min) parts *= 2;
+  const int per = ceil_div(num, parts);
+  parts = ceil_div(num, per);
+  float2* partial = nullptr;
+  if (parts > 1) {
+    float* ws = nullptr;
+    if (stream_workspace(st, sizeof(float2) * channels * parts, &ws)) return -1;
+    partial = reinterpret_cast<float2*>(ws);
+  }
+  const long per_part = (long)per * (vec ? spatial / 4 : spatial);
+  const int threads = per_part >= 1024 ? 1024 : 256;
+  const dim3 grid(channels, parts);
   if (vec)
-    bn_batch_stats_kernel<4><<<channels, threads, 0, static_cast<hipStream_t>(stream)>>>(
-        x, num, channels, spatial, eps, mean, stdev);
+    bn_batch_stats_kernel<4><<<grid, threads, 0, st>>>(x, num, channels, spatial, eps, mean, stdev, per, partial);
   else
-    bn_batch_stats_kernel<1><<<channels, threads, 0, static_cast<hipStream_t>(stream)>>>(
-        x, num, channels, spatial, eps, mean, stdev);
+    bn_batch_stats_kernel<1><<<grid, threads, 0, st>>>(x, num, channels, spatial, eps, mean, stdev, per, partial);
   MC_LAUNCH_CHECK();
+  if (parts > 1) {
+    bn_batch_combine_kernel<<<ceil_div(channels, 256), 256, 0, st>>>(partial, parts, per, num, channels,
+                                                                       spatial, eps, mean, stdev);
+    MC_LAUNCH_CHECK();
+  }
   return 0;
 }
 

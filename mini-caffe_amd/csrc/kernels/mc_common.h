@@ -56,6 +56,12 @@ inline int ew_blocks(long n, int threads, int per_thread = 1) {
   return static_cast<int>(b);
 }
 
+// Device scratch for partial results that one call writes and reads back (the
+// slices of a split-K contraction, per-part statistics): one grow-only buffer per
+// (host thread, stream).  Work on one stream is ordered, so consecutive calls
+// share it.  Growing frees the old buffer, which waits for the device.
+int stream_workspace(hipStream_t st, size_t bytes, float** out);
+
 }  // namespace mchip
 
 #endif  // MCHIP_COMMON_H_

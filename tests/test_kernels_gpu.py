@@ -388,6 +388,26 @@ def test_batch_norm_batch_stats(K):
     assert np.abs(md.cpu().numpy() - x.mean(axis=(0, 2, 3))).max() < 1e-5
 
 
+@pytest.mark.parametrize("shape", [(37, 6, 32, 32), (130, 3, 24, 20), (150, 5, 9, 13), (128, 16, 64, 64),
+                                   (3, 2, 128, 128)])
+def test_batch_norm_batch_stats_of_few_channels(K, shape):
+    """With few channels each channel's images are cut into parts that run as workgroups of
+    their own and are merged afterwards (part sizes that do not divide the batch, planes that
+    are not a multiple of four, a batch too small to cut): mean and deviation against float64,
+    on data whose mean is 60 deviations away from zero."""
+    n, c, h, w = shape
+    rng = np.random.default_rng(41)
+    x = (rng.standard_normal(shape) * 0.5 + 30 + np.arange(c)[None, :, None, None]).astype(np.float32)
+    xd = dev(x)
+    md, sd = torch.empty(c, device="cuda"), torch.empty(c, device="cuda")
+    K.check_mc(K.LIB.mcBatchNormBatchStats(fptr(xd), n, c, h * w, ctypes.c_float(1e-5), fptr(md), fptr(sd), None))
+    torch.cuda.synchronize()
+    x64 = x.astype(np.float64)
+    assert np.abs(md.cpu().numpy() - x64.mean(axis=(0, 2, 3))).max() < 1e-4
+    want_sd = np.sqrt(x64.var(axis=(0, 2, 3)) + 1e-5)
+    assert np.abs(sd.cpu().numpy() / want_sd - 1).max() < 1e-4
+
+
 @pytest.mark.parametrize("method", ["MAX", "AVE"])
 @pytest.mark.parametrize("hw,k,s,p", [((112, 112), 3, 2, 0), ((75, 75), 2, 2, 0), ((19, 19), 3, 1, 1),
                                       ((7, 7), 7, 1, 0), ((6, 6), 2, 2, 1), ((9, 13), 3, 3, 1),
