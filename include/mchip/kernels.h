@@ -168,7 +168,9 @@ int mcBatchNormStored(const float* blob0, const float* blob1, const float* blob2
 
 /* BatchNorm with batch statistics (use_global_stats: false): per channel, mean
  * over num*spatial and stdev = sqrt(E[(x-mean)^2] + eps)
- * (batch_norm_layer.cpp:91-126).  One workgroup per channel, two passes. */
+ * (batch_norm_layer.cpp:91-126).  Two passes over each channel's values; with few
+ * channels a channel's images are cut into parts whose {mean, squared deviations}
+ * are merged afterwards (the parts live in a buffer the library keeps per stream). */
 int mcBatchNormBatchStats(const float* x, int num, int channels, int spatial, float eps,
                           float* mean, float* stdev, void* stream);
 
