@@ -104,27 +104,43 @@ void launch_max_pool_fixed(const PoolArgs& a, long planes, hipStream_t st) {
       <<<ceil_div(count, 256), 256, 0, st>>>(a, row_pairs, count);
 }
 
-// One wavefront per plane; 4 planes per 256-thread workgroup.
-template <int METHOD>
+// G lanes per plane (a power of two up to the wavefront), 256 / G planes per
+// workgroup: a 7x7 plane keeps 16 lanes busy for four loads each instead of 49
+// lanes of a whole wavefront for one.
+template <int METHOD, int G>
 __global__ __launch_bounds__(256) void global_pool_kernel(const float* __restrict__ x,
                                                           float* __restrict__ y, long planes,
                                                           int hw) {
-  const long plane = blockIdx.x * 4L + (threadIdx.x >> 6);
-  if (plane >= planes) return;
-  const int lane = threadIdx.x & 63;
-  const float* __restrict__ xp = x + plane * hw;
+  const long plane = blockIdx.x * static_cast<long>(256 / G) + threadIdx.x / G;
+  const int lane = threadIdx.x % G;
   float v = METHOD == MC_POOL_MAX ? -FLT_MAX : 0.f;
-  for (int i = lane; i < hw; i += 64) {
-    if (METHOD == MC_POOL_MAX) v = fmaxf(v, xp[i]);
-    else v += xp[i];
+  if (plane < planes) {
+    const float* __restrict__ xp = x + plane * hw;
+    for (int i = lane; i < hw; i += G) {
+      if (METHOD == MC_POOL_MAX) v = fmaxf(v, xp[i]);
+      else v += xp[i];
+    }
   }
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
+  for (int o = G / 2; o > 0; o >>= 1) {
     const float u = __shfl_xor(v, o, 64);
     if (METHOD == MC_POOL_MAX) v = fmaxf(v, u);
     else v += u;
   }
-  if (lane == 0) y[plane] = METHOD == MC_POOL_MAX ? v : v / static_cast<float>(hw);
+  if (lane == 0 && plane < planes) y[plane] = METHOD == MC_POOL_MAX ? v : v / static_cast<float>(hw);
+}
+
+template <int METHOD>
+void launch_global_pool(const float* x, float* y, long planes, int hw, hipStream_t st) {
+  // about four values per lane, at least 8 lanes
+  if (hw <= 32)
+    global_pool_kernel<METHOD, 8><<<ceil_div(planes, 32), 256, 0, st>>>(x, y, planes, hw);
+  else if (hw <= 64)
+    global_pool_kernel<METHOD, 16><<<ceil_div(planes, 16), 256, 0, st>>>(x, y, planes, hw);
+  else if (hw <= 128)
+    global_pool_kernel<METHOD, 32><<<ceil_div(planes, 8), 256, 0, st>>>(x, y, planes, hw);
+  else
+    global_pool_kernel<METHOD, 64><<<ceil_div(planes, 4), 256, 0, st>>>(x, y, planes, hw);
 }
 
 }  // namespace
@@ -163,11 +179,8 @@ int mcPooling(int method, const float* bottom, float* top, int planes, int H, in
   if (planes == 0) return 0;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (Ho == 1 && Wo == 1 && kh >= H && kw >= W && ph == 0 && pw == 0) {
-    const int blocks = ceil_div(planes, 4);
-    if (method == MC_POOL_MAX)
-      global_pool_kernel<MC_POOL_MAX><<<blocks, 256, 0, st>>>(bottom, top, planes, H * W);
-    else
-      global_pool_kernel<MC_POOL_AVE><<<blocks, 256, 0, st>>>(bottom, top, planes, H * W);
+    if (method == MC_POOL_MAX) launch_global_pool<MC_POOL_MAX>(bottom, top, planes, H * W, st);
+    else launch_global_pool<MC_POOL_AVE>(bottom, top, planes, H * W, st);
     MC_LAUNCH_CHECK();
     return 0;
   }

@@ -431,6 +431,24 @@ def test_pooling(K, method, hw, k, s, p):
         assert np.abs(got - want).max() < 1e-5
 
 
+@pytest.mark.parametrize("method", ["MAX", "AVE"])
+@pytest.mark.parametrize("hw", [(1, 1), (2, 3), (5, 5), (4, 8), (7, 7), (8, 8), (9, 9), (10, 13), (19, 19)])
+def test_global_pooling_plane_sizes(K, method, hw):
+    """A window that covers the whole plane: planes of 1 to 361 values (8, 16, 32 or 64 lanes
+    per plane), a plane count that fills no workgroup evenly."""
+    x = np.random.default_rng(15).standard_normal((3, 37) + hw).astype(np.float32)
+    want = x.max(axis=(2, 3)) if method == "MAX" else x.astype(np.float64).mean(axis=(2, 3))
+    xd, yd = dev(x), torch.full((3, 37, 1, 1), float("nan"), device="cuda")
+    K.check_mc(K.LIB.mcPooling(0 if method == "MAX" else 1, fptr(xd), fptr(yd), 3 * 37, hw[0], hw[1],
+                               hw[0], hw[1], 1, 1, 0, 0, None))
+    torch.cuda.synchronize()
+    got = yd.cpu().numpy().reshape(3, 37)
+    if method == "MAX":
+        assert np.array_equal(got, want)
+    else:
+        assert np.abs(got - want).max() < 1e-6
+
+
 @pytest.mark.parametrize("op,coeffs", [("SUM", None), ("SUM", [1.0, -2.0, 0.5]), ("PROD", None), ("MAX", None)])
 @pytest.mark.parametrize("count", [4096, 1001])
 def test_eltwise(K, op, coeffs, count):
