@@ -20,11 +20,18 @@
  * How each function is pinned (tests/test_oracle_det.py):
  *   anchors            the published py-faster-rcnn table for base 16
  *   proposal decode    closed form in float64 on boxes away from clip edges
- *   SortBBox           descending order on tie-free data; partial-sort contract
+ *   SortBBox           descending order on tie-free data; partial-sort contract;
+ *                      the order of EQUAL scores by seven literal vectors whose
+ *                      expected order was traced by hand from the reference text
+ *                      (a changed comparison or recursion cut fails one of them)
  *   NMS (both)         brute force: kept set is independent and maximal w.r.t.
  *                      "earlier kept box overlaps > thr"
  *   prior box          SSD300 prior count 8732 and closed-form centres / sizes
- *   detection output   brute-force greedy NMS per class in float64 on <= 64 priors
+ *   detection output   float64 walk on <= 96 priors: all three code types, variance in
+ *                      the prior or in the target, shared and per-class locations,
+ *                      any background label, adaptive eta threshold, keep_top_k.
+ *                      Not pinned: std::sort's order of equal scores at the
+ *                      keep_top_k cut (PARITY UNPINNED for that tie case)
  *   normalize          closed form
  *   roi / psroi pool   special cases that reduce to numpy routines: a roi over the
  *                      whole map with 1x1 bins is the global max / mean, with one

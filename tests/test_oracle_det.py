@@ -63,6 +63,68 @@ def test_sort_bbox_contract():
     assert np.array_equal(rois[out[:, 0].astype(int)], out)
 
 
+# Literal vectors for the order SortBBox leaves EQUAL scores in.  Each expected order was
+# traced by hand from proposal_layer.cpp:88-111 (first element is the pivot "key"; `last`
+# walks left over scores <= key, the row there moves into the hole at `first`; `first` walks
+# right over scores >= key, the row there moves into the hole at `last`; the key lands where
+# they meet; recurse left, then right only while the right part starts before num_top).
+# Rows are named a, b, c ... in input order; the trace of each case is in its comment.
+_TIE_CASES = [
+    # [a5 b5 c5], top 3.  key a: last walks 2->1->0 (5<=5 each), a stays at 0.  Right part
+    # (1,2): key b, last walks 2->1, b stays.  All-equal input keeps its order.
+    # A `<` in the last-walk would instead move c to the front: c b a.
+    ([5, 5, 5], 3, "abc"),
+    # [a3 b5 c3 d4], top 4.  key a(3): last=3 (4<=3 no) -> d into hole 0; first walks 0(d4)
+    # 1(b5) 2(c3: 3>=3) and meets last at 3; a lands at 3: d b c a.  Left part (0,2): key d(4):
+    # last 2(c3<=4)->1 (b5<=4 no) -> b into hole 0; first 0->1 meets; d lands at 1: b d c a.
+    # The equal pair ends up c before a: NOT the stable order (a before c).
+    ([3, 5, 3, 4], 4, "bdca"),
+    # [a4 b6 c4 d6 e2], top 5.  key a(4): last 4(e2<=4)->3 (d6 no) -> d into hole 0; first walks
+    # 0(d6) 1(b6) 2(c4>=4) to 3; a lands at 3: d b c a e.  Left (0,2): key d(6): last 2(c4)->1
+    # (b6<=6)->0, d stays; its right part (1,2): key b: last 2->1, b stays.  Result d b c a e:
+    # both equal pairs reversed.  A `>` in the first-walk would stop at c and give d b a c e.
+    ([4, 6, 4, 6, 2], 5, "dbcae"),
+    # [a5 b1 c2 d3 e4], top 2: the right recursion is cut by num_top.  key a(5): last walks to
+    # 0, a stays, first=0; right part (1,4) is sorted because 1 < 2: key b(1): last=4 (e4<=1 no)
+    # -> e into hole 1; first walks 1,2,3 to 4; b lands at 4: a e c d b, first=4.  Its left part
+    # (1,3): key e(4): last 3(d3)->2(c2)->1, e stays, first=1; right part (2,3) is NOT sorted
+    # because first+1 = 2 is not < num_top = 2.  c2 stays before d3.
+    ([5, 1, 2, 3, 4], 2, "aecdb"),
+    # same input, top 1: after the first partition first+1 = 1 is not < 1: nothing else moves.
+    ([5, 1, 2, 3, 4], 1, "abcde"),
+    # [a2 b7 c2 d7 e2 f7], top 3: equal scores on both sides of the cut.  key a(2): last=5
+    # (f7<=2 no) -> f into hole 0; first walks 0..4 (7,7,2,7,2 all >= 2) to 5; a lands at 5:
+    # f b c d e a.  Left (0,4): key f(7): last walks 4,3,2,1 (2,7,2,7 all <= 7) to 0, f stays,
+    # first=0.  Right (1,4) (1<3): key b(7): last walks 4,3,2 to 1, b stays, first=1.  Right
+    # (2,4) (2<3): key c(2): last 4(e2<=2)->3 (d7 no) -> d into hole 2; first 2(d7)->3 meets;
+    # c lands at 3: f b d c e a, first=3; left (2,2) and right (4<3 fails) end.  Top three are
+    # f b d (the stable order would be b d f).
+    ([2, 7, 2, 7, 2, 7], 3, "fbdcea"),
+    # [a3 b1 c3 d5 e3 f0 g5 h3], top 8: equal scores left and right of the pivot, two hole
+    # moves.  key a(3): last 7(h3<=3)->6 (g5 no) -> g into hole 0; first 0(g5)->1 (b1>=3 no) ->
+    # b into hole 6; last 6(b1)->5(f0)->4(e3<=3)->3 (d5 no) -> d into hole 1; first 1(d5)->2
+    # (c3>=3)->3 meets; a lands at 3: g d c a e f b h.  Left (0,2): key g(5): last 2(c3)->1
+    # (d5<=5)->0, g stays; right part (1,2): key d(5): last 2->1, d stays.  Right of a, (4,7)
+    # = e3 f0 b1 h3: key e(3): last 7(h3<=3)->6->5->4, e stays, first=4; right (5,7) = f0 b1 h3:
+    # key f(0): last=7 (h3<=0 no) -> h into hole 5; first 5(h3)->6(b1>=0)->7 meets; f lands at
+    # 7: h b f, first=7; left (5,6) = h3 b1: key h: last 6->5, h stays.  Result g d c a e h b f.
+    ([3, 1, 3, 5, 3, 0, 5, 3], 8, "gdcaehbf"),
+]
+
+
+@pytest.mark.parametrize("scores,top,want", _TIE_CASES)
+def test_sort_bbox_tie_order_hand_traced(scores, top, want):
+    n = len(scores)
+    rois = np.zeros((n, 5), np.float32)
+    rois[:, 0] = np.arange(n)                 # row identity travels in column 0
+    rois[:, 1] = np.arange(n) * 10 + 1        # and the other columns must travel with it
+    rois[:, 4] = scores
+    out = oracle.sort_bbox(rois, top)
+    got = "".join("abcdefgh"[int(i)] for i in out[:, 0])
+    assert got == want
+    assert np.array_equal(out, rois[out[:, 0].astype(int)])
+
+
 def brute_nms_pixel(boxes, thr, max_keep):
     b = boxes.astype(np.float64)
     area = (b[:, 2] - b[:, 0] + 1) * (b[:, 3] - b[:, 1] + 1)
@@ -139,70 +201,158 @@ def test_prior_box_ssd300():
     assert clipped[0, 0].min() == 0 and clipped[0, 0].max() == 1
 
 
+def brute_decode(code_type, var_in_target, pb, var, l):
+    """Float64 decode of P boxes for the three code types (bbox_util.cpp:242-330)."""
+    if var_in_target:
+        var = np.ones_like(var)
+    pw, ph = pb[:, 2] - pb[:, 0], pb[:, 3] - pb[:, 1]
+    if code_type == "CORNER":
+        return pb + var * l
+    if code_type == "CORNER_SIZE":
+        return pb + var * l * np.stack([pw, ph, pw, ph], 1)
+    assert code_type == "CENTER_SIZE"
+    pcx, pcy = (pb[:, 0] + pb[:, 2]) / 2, (pb[:, 1] + pb[:, 3]) / 2
+    cx, cy = var[:, 0] * l[:, 0] * pw + pcx, var[:, 1] * l[:, 1] * ph + pcy
+    w, h = np.exp(var[:, 2] * l[:, 2]) * pw, np.exp(var[:, 3] * l[:, 3]) * ph
+    return np.stack([cx - w / 2, cy - h / 2, cx + w / 2, cy + h / 2], 1)
+
+
 def brute_detection_output(param, loc, conf, prior):
-    """Independent float64 walk: decode (CENTER_SIZE), per-class greedy NMS, keep_top_k."""
+    """Independent float64 walk of detection_output_layer.cpp:74-226: decode (any code type,
+    variance in the prior or in the target, shared or per-class locations), per-class greedy
+    NMS with the adaptive threshold (bbox_util.cpp:696-715), keep_top_k."""
     num, P, C = loc.shape[0], prior.shape[2] // 4, param["num_classes"]
+    share = param.get("share_location", True)
+    bg = param.get("background_label_id", 0)
     pb = prior[0, 0].reshape(P, 4).astype(np.float64)
     var = prior[0, 1].reshape(P, 4).astype(np.float64)
     nms = param["nms_param"]
+    eta = nms.get("eta", 1.0)
     rows = []
     for i in range(num):
-        l = loc[i].reshape(P, 4).astype(np.float64)
-        pw, ph = pb[:, 2] - pb[:, 0], pb[:, 3] - pb[:, 1]
-        pcx, pcy = (pb[:, 0] + pb[:, 2]) / 2, (pb[:, 1] + pb[:, 3]) / 2
-        cx, cy = var[:, 0] * l[:, 0] * pw + pcx, var[:, 1] * l[:, 1] * ph + pcy
-        w, h = np.exp(var[:, 2] * l[:, 2]) * pw, np.exp(var[:, 3] * l[:, 3]) * ph
-        box = np.stack([cx - w / 2, cy - h / 2, cx + w / 2, cy + h / 2], 1)
-        area = np.where((box[:, 2] < box[:, 0]) | (box[:, 3] < box[:, 1]), 0, (box[:, 2] - box[:, 0]) * (box[:, 3] - box[:, 1]))
+        l_all = loc[i].reshape(P, 1 if share else C, 4).astype(np.float64)
         sc = conf[i].reshape(P, C)
-        kept = {}
-        for c in range(1, C):
+        kept, boxes = {}, {}
+        for c in range(C):
+            if c == bg:
+                continue
+            box = brute_decode(param["code_type"], param.get("variance_encoded_in_target", False),
+                               pb, var, l_all[:, 0 if share else c])
+            boxes[c] = box
+            area = np.where((box[:, 2] < box[:, 0]) | (box[:, 3] < box[:, 1]), 0,
+                            (box[:, 2] - box[:, 0]) * (box[:, 3] - box[:, 1]))
             cand = [p for p in np.argsort(-sc[:, c], kind="stable") if sc[p, c] > param["confidence_threshold"]]
-            cand = cand[:nms["top_k"]]
+            if nms.get("top_k", -1) > -1:
+                cand = cand[:nms["top_k"]]
+            thr = nms["nms_threshold"]
             ks = []
             for p in cand:
-                ok = True
-                for k in ks:
-                    iw = min(box[p, 2], box[k, 2]) - max(box[p, 0], box[k, 0])
-                    ih = min(box[p, 3], box[k, 3]) - max(box[p, 1], box[k, 1])
-                    if iw > 0 and ih > 0 and iw * ih / (area[p] + area[k] - iw * ih) > nms["nms_threshold"]:
-                        ok = False
-                        break
-                if ok:
+                iw = np.minimum(box[p, 2], box[ks, 2]) - np.maximum(box[p, 0], box[ks, 0])
+                ih = np.minimum(box[p, 3], box[ks, 3]) - np.maximum(box[p, 1], box[ks, 1])
+                inter = np.where((iw > 0) & (ih > 0), iw * ih, 0.0)
+                if not (inter / (area[p] + area[ks] - inter + 1e-300) > thr).any():
                     ks.append(p)
+                    if eta < 1 and thr > 0.5:
+                        thr *= eta
             kept[c] = ks
         allk = [(sc[p, c], c, p) for c in kept for p in kept[c]]
-        if len(allk) > param["keep_top_k"]:
+        if -1 < param["keep_top_k"] < len(allk):
             allk = sorted(allk, key=lambda t: -t[0])[:param["keep_top_k"]]
-            sel = {(c, p) for _, c, p in allk}
-            kept = {c: [p for p in kept[c] if (c, p) in sel] for c in kept}
+            kept = {c: [p for s_, c_, p in allk if c_ == c] for c in kept}
         for c in sorted(kept):
             for p in kept[c]:
-                rows.append([i, c, sc[p, c], *box[p]])
+                rows.append([i, c, sc[p, c], *boxes[c][p]])
     return np.array(rows, np.float64).reshape(-1, 7)
 
 
-def test_detection_output_brute_force():
-    r = rng(5)
-    num, P, C = 3, 64, 5
+def _detection_case(seed, num=3, P=64, C=5, per_class=False, loc_scale=0.5):
+    r = rng(seed)
     c = r.random((P, 2)) * 0.8 + 0.1
     wh = r.random((P, 2)) * 0.3 + 0.05
+    # four different variances so that a transposed or dropped variance shows
     prior = np.concatenate([np.concatenate([c - wh / 2, c + wh / 2], 1).reshape(-1),
-                            np.tile([0.1, 0.1, 0.2, 0.2], P)]).reshape(1, 2, P * 4).astype(np.float32)
-    loc = (r.standard_normal((num, P * 4)) * 0.5).astype(np.float32)
+                            np.tile([0.1, 0.15, 0.2, 0.3], P)]).reshape(1, 2, P * 4).astype(np.float32)
+    loc = (r.standard_normal((num, P * (C if per_class else 1) * 4)) * loc_scale).astype(np.float32)
     conf = oracle.softmax((r.standard_normal((num, P, C)) * 2).astype(np.float32), 2).reshape(num, P * C)
-    param = {"num_classes": C, "share_location": True, "background_label_id": 0,
-             "code_type": "CENTER_SIZE", "keep_top_k": 30, "confidence_threshold": 0.05,
-             "nms_param": {"nms_threshold": 0.45, "top_k": 20}}
-    got = oracle.detection_output(param, loc, conf, prior)
-    want = brute_detection_output(param, loc, conf, prior)
-    assert got.shape == want.shape and got.shape[0] > 10
+    return loc, conf, prior
+
+
+def _assert_rows(got, want, min_rows=10):
+    assert got.shape == want.shape and got.shape[0] > min_rows
     assert np.array_equal(got[:, :2], want[:, :2])
     assert np.abs(got - want).max() < 1e-5
+
+
+def test_detection_output_brute_force():
+    loc, conf, prior = _detection_case(5)
+    num = loc.shape[0]
+    param = {"num_classes": 5, "share_location": True, "background_label_id": 0,
+             "code_type": "CENTER_SIZE", "keep_top_k": 30, "confidence_threshold": 0.05,
+             "nms_param": {"nms_threshold": 0.45, "top_k": 20}}
+    _assert_rows(oracle.detection_output(param, loc, conf, prior),
+                 brute_detection_output(param, loc, conf, prior))
     # nothing above the threshold: one row of -1 per image with the image id
     param["confidence_threshold"] = 2.0
     none = oracle.detection_output(param, loc, conf, prior)
     assert np.array_equal(none, np.array([[i, -1, -1, -1, -1, -1, -1] for i in range(num)], np.float32))
+
+
+@pytest.mark.parametrize("code_type", ["CORNER", "CENTER_SIZE", "CORNER_SIZE"])
+@pytest.mark.parametrize("var_in_target", [False, True])
+@pytest.mark.parametrize("per_class", [False, True])
+def test_detection_output_decode_branches_brute_force(code_type, var_in_target, per_class):
+    """CORNER / CORNER_SIZE decode, variance_encoded_in_target and share_location: false
+    (bbox_util.cpp:242-330, 348-401) against the float64 walk; kept (image, label) rows
+    must be identical, scores and corners within 1e-5."""
+    loc, conf, prior = _detection_case(11 + 2 * var_in_target + per_class, per_class=per_class,
+                                       loc_scale=0.08 if code_type == "CORNER" else 0.5)
+    param = {"num_classes": 5, "share_location": not per_class, "background_label_id": 0,
+             "code_type": code_type, "variance_encoded_in_target": var_in_target,
+             "keep_top_k": 40, "confidence_threshold": 0.03,
+             "nms_param": {"nms_threshold": 0.45, "top_k": 25}}
+    got = oracle.detection_output(param, loc, conf, prior)
+    want = brute_detection_output(param, loc, conf, prior)
+    _assert_rows(got, want)
+    # the branch must matter: the other variance convention decodes different boxes
+    other = dict(param, variance_encoded_in_target=not var_in_target)
+    assert np.abs(brute_detection_output(other, loc, conf, prior)[:5, 3:] - want[:5, 3:]).max() > 1e-3
+
+
+@pytest.mark.parametrize("bg", [0, 2, -1])
+def test_detection_output_background_label_brute_force(bg):
+    """Any class can be the background (skipped); -1 keeps every class."""
+    loc, conf, prior = _detection_case(21, per_class=True)
+    param = {"num_classes": 5, "share_location": False, "background_label_id": bg,
+             "code_type": "CENTER_SIZE", "keep_top_k": -1, "confidence_threshold": 0.1,
+             "nms_param": {"nms_threshold": 0.4, "top_k": 30}}
+    got = oracle.detection_output(param, loc, conf, prior)
+    _assert_rows(got, brute_detection_output(param, loc, conf, prior))
+    assert bg not in got[:, 1]                            # the background label never appears
+    assert set(np.unique(got[:, 1]).astype(int)) == set(range(5)) - {bg}
+
+
+@pytest.mark.parametrize("eta,thr0", [(0.8, 0.9), (0.95, 0.7), (0.6, 0.55)])
+def test_detection_output_adaptive_eta_brute_force(eta, thr0):
+    """eta < 1: the overlap threshold is multiplied by eta after every kept box while it is
+    above 0.5 (bbox_util.cpp:696-715).  Overlapping priors and small offsets make the kept
+    set depend on the decaying threshold."""
+    r = rng(31)
+    num, P, C = 2, 96, 3
+    centre = r.random((P // 8, 2)) * 0.6 + 0.2                     # 12 clusters of 8 boxes
+    c = np.repeat(centre, 8, 0) + r.standard_normal((P, 2)) * 0.02
+    wh = 0.25 + r.random((P, 2)) * 0.05
+    prior = np.concatenate([np.concatenate([c - wh / 2, c + wh / 2], 1).reshape(-1),
+                            np.tile([0.1, 0.1, 0.2, 0.2], P)]).reshape(1, 2, P * 4).astype(np.float32)
+    loc = (r.standard_normal((num, P * 4)) * 0.3).astype(np.float32)
+    conf = oracle.softmax((r.standard_normal((num, P, C)) * 2).astype(np.float32), 2).reshape(num, P * C)
+    param = {"num_classes": C, "share_location": True, "background_label_id": 0,
+             "code_type": "CENTER_SIZE", "keep_top_k": -1, "confidence_threshold": 0.01,
+             "nms_param": {"nms_threshold": thr0, "top_k": -1, "eta": eta}}
+    got = oracle.detection_output(param, loc, conf, prior)
+    want = brute_detection_output(param, loc, conf, prior)
+    _assert_rows(got, want)
+    fixed = dict(param, nms_param=dict(param["nms_param"], eta=1.0))
+    assert oracle.detection_output(fixed, loc, conf, prior).shape[0] > got.shape[0]   # eta bites
 
 
 def test_normalize_closed_form():
