@@ -264,6 +264,20 @@ int mcProposal(const float* scores, const float* bbox, const float* im_info, con
                int post_nms_topn, float nms_thresh, void* workspace, size_t workspace_bytes,
                float* rois, float* roi_scores, int* num_rois, int* tie_flag, void* stream);
 
+/* mcProposal for callers that cannot allocate device memory or hand over a workspace
+ * (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc).  It
+ * has no counterpart in the reference.  Same arguments, results and kernels as
+ * mcProposal; the scratch is an 8 MiB buffer built into the library (each GPU the
+ * library runs on holds its copy until the process ends).  Problems whose scratch
+ * (mcProposalWorkspaceSize) exceeds 8 MiB are refused with an error: 1 x 18 x 38 x 63
+ * scores with pre_nms_topn 6000 need 6.7 MB.  The call itself allocates and frees
+ * nothing.  Every call on a GPU uses that GPU's one buffer: calls that overlap on one
+ * GPU (two streams, two threads) race; calls on one stream are ordered and safe. */
+int mcProposalStatic(const float* scores, const float* bbox, const float* im_info,
+                     const float* anchors, int A, int H, int W, int feat_stride, float min_size,
+                     int pre_nms_topn, int post_nms_topn, float nms_thresh, float* rois,
+                     float* roi_scores, int* num_rois, int* tie_flag, void* stream);
+
 /* Bytes of device scratch mcDetectionOutput needs, and the row capacity that can
  * never be exceeded for these parameters. */
 int mcDetectionOutputWorkspaceSize(int num, int num_priors, int num_classes, int share_location,

@@ -8,6 +8,8 @@
 //
 // This file is compiled with -ffp-contract=off: the kept-box indices must equal
 // the CPU path's bit for bit, so every a*b+c here is two roundings like there.
+#include <mutex>
+
 #include "../mc_common.h"
 #include "block_sort.h"
 #include "mchip/kernels.h"
@@ -779,18 +781,36 @@ ProposalLayout layout(int n, int pre, int post) {
 
 using namespace mchip;
 
-extern "C" {
+namespace {
 
-int mcProposalWorkspaceSize(int num_proposals, int pre_nms_topn, int post_nms_topn,
-                            size_t* bytes) {
-  MC_REQUIRE(bytes && num_proposals > 0 && pre_nms_topn > 0 && post_nms_topn > 0,
-             "mcProposalWorkspaceSize: bad argument");
-  const int pre = pre_nms_topn < num_proposals ? pre_nms_topn : num_proposals;
-  *bytes = layout(num_proposals, pre, post_nms_topn).total;
+// Scratch of mcProposalStatic: device memory that belongs to the library image, one
+// copy per GPU at its own address.  Host code must never pass the array's name to a
+// kernel or a copy (on the host it is only a handle for the symbol lookup); the
+// per-device address found by static_scratch() is what kernels receive.
+constexpr size_t kStaticScratchBytes = size_t(8) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+void* g_scratch_addr[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+// Address of the current device's copy of `scratch`, looked up once per device.
+int static_scratch(void** out) {
+  int dev = -1;
+  MC_HIP(hipGetDevice(&dev));
+  MC_REQUIRE(dev >= 0 && dev < kMaxDevices, "mcProposalStatic: device index %d not supported", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_addr[dev]) {
+    void* addr = nullptr;
+    MC_HIP(hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch)));
+    MC_REQUIRE(addr != nullptr, "mcProposalStatic: symbol lookup returned no address");
+    g_scratch_addr[dev] = addr;
+  }
+  *out = g_scratch_addr[dev];
   return 0;
 }
 
-int mcProposal(const float* scores, const float* bbox, const float* im_info, const float* anchors,
+int run_proposal(const float* scores, const float* bbox, const float* im_info, const float* anchors,
                int A, int H, int W, int feat_stride, float min_size, int pre_nms_topn,
                int post_nms_topn, float nms_thresh, void* workspace, size_t workspace_bytes,
                float* rois, float* roi_scores, int* num_rois, int* tie_flag, void* stream) {
@@ -856,6 +876,50 @@ int mcProposal(const float* scores, const float* bbox, const float* im_info, con
     MC_HIP(hipMemcpyAsync(tie_flag, flags, sizeof(int), hipMemcpyDeviceToDevice, st));
   }
   return 0;
+}
+
+
+}  // namespace
+
+extern "C" {
+
+int mcProposalWorkspaceSize(int num_proposals, int pre_nms_topn, int post_nms_topn,
+                            size_t* bytes) {
+  MC_REQUIRE(bytes && num_proposals > 0 && pre_nms_topn > 0 && post_nms_topn > 0,
+             "mcProposalWorkspaceSize: bad argument");
+  const int pre = pre_nms_topn < num_proposals ? pre_nms_topn : num_proposals;
+  *bytes = layout(num_proposals, pre, post_nms_topn).total;
+  return 0;
+}
+
+int mcProposal(const float* scores, const float* bbox, const float* im_info, const float* anchors,
+               int A, int H, int W, int feat_stride, float min_size, int pre_nms_topn,
+               int post_nms_topn, float nms_thresh, void* workspace, size_t workspace_bytes,
+               float* rois, float* roi_scores, int* num_rois, int* tie_flag, void* stream) {
+  return run_proposal(scores, bbox, im_info, anchors, A, H, W, feat_stride, min_size, pre_nms_topn,
+                      post_nms_topn, nms_thresh, workspace, workspace_bytes, rois, roi_scores,
+                      num_rois, tie_flag, stream);
+}
+
+int mcProposalStatic(const float* scores, const float* bbox, const float* im_info,
+                     const float* anchors, int A, int H, int W, int feat_stride, float min_size,
+                     int pre_nms_topn, int post_nms_topn, float nms_thresh, float* rois,
+                     float* roi_scores, int* num_rois, int* tie_flag, void* stream) {
+  MC_REQUIRE(A > 0 && H > 0 && W > 0 && pre_nms_topn > 0 && post_nms_topn > 0,
+             "mcProposalStatic: bad extents");
+  const long n_long = (long)A * H * W;
+  MC_REQUIRE(n_long < (1L << 24), "mcProposalStatic: too many proposals");
+  const int n = static_cast<int>(n_long);
+  const size_t need = layout(n, pre_nms_topn < n ? pre_nms_topn : n, post_nms_topn).total;
+  MC_REQUIRE(need <= kStaticScratchBytes,
+             "mcProposalStatic: this problem needs %zu bytes of scratch, the built-in buffer holds "
+             "%zu; use mcProposal with a caller-owned workspace",
+             need, kStaticScratchBytes);
+  void* ws = nullptr;
+  if (static_scratch(&ws) != 0) return -1;
+  return run_proposal(scores, bbox, im_info, anchors, A, H, W, feat_stride, min_size, pre_nms_topn,
+                      post_nms_topn, nms_thresh, ws, kStaticScratchBytes, rois, roi_scores, num_rois,
+                      tie_flag, stream);
 }
 
 }  // extern "C"

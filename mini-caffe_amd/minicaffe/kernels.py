@@ -80,6 +80,9 @@ LIB.mcProposalWorkspaceSize.argtypes = [c_int, c_int, c_int, ctypes.POINTER(ctyp
 LIB.mcProposal.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                            c_float, c_int, c_int, c_float, c_void_p, ctypes.c_size_t, c_void_p,
                            c_void_p, c_void_p, c_void_p, c_void_p]
+LIB.mcProposalStatic.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                 c_float, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p,
+                                 c_void_p, c_void_p]
 
 LIB.mcConvPlanCreate.argtypes = [ctypes.POINTER(ConvGeom), ctypes.POINTER(c_void_p)]
 LIB.mcConvPlanDestroy.argtypes = [c_void_p]
