@@ -43,6 +43,9 @@ class CAFFE_API Net {
   void CopyTrainedLayersFrom(const NetParameter& param);
   void CopyTrainedLayersFrom(const string& trained_filename);
 
+  /*! \brief the net's definition with every layer's current parameter blobs */
+  void ToProto(NetParameter* param) const;
+
   const string& name() const { return name_; }
   const vector<string>& blob_names() const { return blob_names_; }
   const vector<string>& param_names() const { return param_display_names_; }

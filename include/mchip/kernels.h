@@ -296,14 +296,19 @@ int mcDetectionOutputMaxRows(int num, int num_priors, int num_classes, int top_k
  * out_rows receives [image, label, score, xmin, ymin, xmax, ymax] rows, images and
  * labels ascending, each label's boxes in NMS order; *num_rows (device int) is the
  * row count, or num rows of -1 when nothing was kept (:175-185).
- * Equal scores at the keep_top_k cut are resolved by (label asc, NMS order); the
- * reference leaves that to std::sort. */
+ * When keep_top_k cuts an image's detections the reference re-sorts them with
+ * std::sort, which leaves equal scores in an order of its own.  Here equal scores
+ * at the cut are resolved by (label asc, NMS order) and a label's rows stay in NMS
+ * order.  *cut_tie_flag (optional device int) reports when that could differ, as a
+ * bit set over all images: 1 = the last score kept equals the first score dropped
+ * (which of them survive is undefined), 2 = two kept rows of one label have equal
+ * scores (their relative order is undefined); 0 = the rows are fully defined. */
 int mcDetectionOutput(const float* loc, const float* conf, const float* prior, int num,
                       int num_priors, int num_classes, int share_location, int background_label,
                       int code_type, int variance_encoded_in_target, int keep_top_k,
                       float confidence_threshold, float nms_threshold, float eta, int top_k,
                       void* workspace, size_t workspace_bytes, float* out_rows, int max_rows,
-                      int* num_rows, void* stream);
+                      int* num_rows, int* cut_tie_flag, void* stream);
 
 /* ROIPoolingLayer::Forward (roi_pooling_layer.cpp:37-110; .cu:13-81): max pooling of
  * bottom [num, channels, height, width] over num_rois regions, rois rows of

@@ -34,9 +34,11 @@ __device__ __forceinline__ float dbox_size(float xmin, float ymin, float xmax, f
 // reference's expressions promote.
 __global__ __launch_bounds__(256) void det_decode_kernel(
     const float* __restrict__ loc, const float* __restrict__ prior, int num, int P,
-    int loc_classes, int code_type, int var_in_target, DBox* __restrict__ out) {
+    int loc_classes, int code_type, int var_in_target, DBox* __restrict__ out,
+    int* __restrict__ cut_tie_flag) {
   const long total = (long)num * loc_classes * P;
   const long t = blockIdx.x * 256L + threadIdx.x;
+  if (t == 0 && cut_tie_flag) *cut_tie_flag = 0;  // raised by det_select_kernel, two launches on
   if (t >= total) return;
   const int p = static_cast<int>(t % P);
   const int c = static_cast<int>((t / P) % loc_classes);
@@ -352,7 +354,7 @@ __global__ __launch_bounds__(kSortThreads) void det_select_kernel(
     int loc_classes, int keep_top_k, int max_cand, const int* __restrict__ kept_idx,
     const int* __restrict__ kept_count, uint32_t* keys0, int* vals0, uint32_t* keys1,
     int* vals1, int* __restrict__ selected, float* __restrict__ rows_tmp,
-    int* __restrict__ rows_count) {
+    int* __restrict__ rows_count, int* __restrict__ cut_tie_flag) {
   __shared__ BlockSortLds lds;
   __shared__ BlockSortLds16 lds16;
   __shared__ uint32_t s_key[kSelLdsMax];       // entry lists of up to kSelLdsMax are sorted in LDS
@@ -403,6 +405,29 @@ __global__ __launch_bounds__(kSortThreads) void det_select_kernel(
     } else {
       block_sort_desc(k0, v0, k1, v1, total, &lds);
       for (int r = threadIdx.x; r < total; r += kSortThreads) sel[v0[r]] = r < keep_top_k;
+    }
+    // Equal scores on both sides of the cut: which of them survive is decided here
+    // by (label, NMS order) and in the reference by std::sort's internals.
+    if (threadIdx.x == 0 && cut_tie_flag && keep_top_k > 0) {
+      const uint32_t last_in = in_lds ? s_key[keep_top_k - 1] : k0[keep_top_k - 1];
+      const uint32_t first_out = in_lds ? s_key[keep_top_k] : k0[keep_top_k];
+      if (last_in == first_out) atomicOr(cut_tie_flag, 1);
+    }
+    __syncthreads();
+    // Equal scores of one label among the kept entries: the reference rebuilds each
+    // label's list in std::sort's order, here they stay in NMS order.
+    if (cut_tie_flag) {
+      int cc = 0;
+      bool tied = false;
+      for (int e = begin; e < end; ++e) {
+        while (s_off[cc + 1] <= e) ++cc;
+        if (!sel[e] || e + 1 >= s_off[cc + 1] || !sel[e + 1]) continue;
+        const int* list = kept_idx + (size_t)(i * C + cc) * max_cand;
+        const float a = conf[((size_t)i * P + list[e - s_off[cc]]) * C + cc];
+        const float b = conf[((size_t)i * P + list[e + 1 - s_off[cc]]) * C + cc];
+        tied = tied || a == b;
+      }
+      if (tied) atomicOr(cut_tie_flag, 2);
     }
     __syncthreads();
   }
@@ -534,7 +559,7 @@ int mcDetectionOutput(const float* loc, const float* conf, const float* prior, i
                       int code_type, int variance_encoded_in_target, int keep_top_k,
                       float confidence_threshold, float nms_threshold, float eta, int top_k,
                       void* workspace, size_t workspace_bytes, float* out_rows, int max_rows,
-                      int* num_rows, void* stream) {
+                      int* num_rows, int* cut_tie_flag, void* stream) {
   MC_REQUIRE(loc && conf && prior && workspace && out_rows && num_rows,
              "mcDetectionOutput: null argument");
   MC_REQUIRE(num > 0 && num <= 1024 && num_priors > 0 && num_classes > 0 && num_classes < 1024,
@@ -556,7 +581,7 @@ int mcDetectionOutput(const float* loc, const float* conf, const float* prior, i
   const long ndec = (long)num * loc_classes * num_priors;
   det_decode_kernel<<<ceil_div(ndec, 256), 256, 0, st>>>(loc, prior, num, num_priors, loc_classes,
                                                          code_type, variance_encoded_in_target,
-                                                         boxes);
+                                                         boxes, cut_tie_flag);
   MC_LAUNCH_CHECK();
   if (num_priors <= kDetLdsMax)
     det_class_nms_lds_kernel<<<dim3(num_classes, num), kSortThreads, 0, st>>>(
@@ -571,7 +596,7 @@ int mcDetectionOutput(const float* loc, const float* conf, const float* prior, i
   det_select_kernel<<<num, kSortThreads, 0, st>>>(
       conf, boxes, num_priors, num_classes, loc_classes, keep_top_k, max_cand, i32(L.kept_idx),
       i32(L.kept_count), u32(L.sk0), i32(L.sv0), u32(L.sk1), i32(L.sv1), i32(L.selected),
-      reinterpret_cast<float*>(ws + L.rows_tmp), i32(L.rows_count));
+      reinterpret_cast<float*>(ws + L.rows_tmp), i32(L.rows_count), cut_tie_flag);
   MC_LAUNCH_CHECK();
   det_emit_kernel<<<1, 256, 0, st>>>(reinterpret_cast<float*>(ws + L.rows_tmp), i32(L.rows_count),
                                      num, num_classes * max_cand, max_rows, out_rows, num_rows);

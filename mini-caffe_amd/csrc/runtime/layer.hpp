@@ -62,6 +62,13 @@ class Layer {
 
   vector<shared_ptr<Blob> >& blobs() { return blobs_; }
   const LayerParameter& layer_param() const { return layer_param_; }
+  // The layer's definition with its current parameter blobs in place of the ones
+  // it was built from (reference src/layer.hpp:282-289).
+  void ToProto(LayerParameter* param) const {
+    *param = layer_param_;
+    param->remove("blobs");
+    for (const auto& b : blobs_) b->ToProto(static_cast<BlobProto*>(param->add_sub("blobs")));
+  }
   const string name() const { return layer_param_.get_string("name"); }
 
   virtual const char* type() const { return ""; }
@@ -89,6 +96,10 @@ class Layer {
   virtual bool AcceptsEpilogue() const { return false; }
   // How many non-activation stages it can absorb (an activation may follow them).
   virtual int MaxAffineFollowers() const { return 0; }
+  // Whether `follower` (already known to be an in-place channel stage) may ride
+  // along; a layer whose own pass fixes some fields of the stage refuses
+  // followers that need those fields.
+  virtual bool AcceptsFollower(const Layer* follower) const { return true; }
   virtual void SetEpilogue(const vector<Layer*>& followers) {}
   // Residual folding.  A two-input sum with unit coefficients reports itself
   // (and the activation it absorbed, if any) so that the layer producing one of
@@ -111,6 +122,10 @@ class Layer {
   // shape (Flatten, Reshape).  When nothing reads the bottom afterwards Net lets
   // the top take over the bottom's memory and skips the layer's copy.
   virtual bool IsView() const { return false; }
+  // True when Forward gives a top a shape (and possibly new memory) that is only
+  // known after the device has run (DetectionOutput's row count).  Such a top
+  // cannot be aliased by a view that was placed before Forward.
+  virtual bool ShapesTopInForward() const { return false; }
 
  protected:
   LayerParameter layer_param_;

@@ -505,6 +505,13 @@ class BatchNormLayer : public Layer {
   // statistics -> Scale -> ReLU becomes statistics + one pass).
   bool AcceptsEpilogue() const override { return true; }
   int MaxAffineFollowers() const override { return 1; }
+  // This pass owns the stage's subtract / divide fields (mean and deviation), so
+  // only followers that fill the multiply / add fields or the activation fit:
+  // another BatchNorm or a BN would lose its own subtraction.
+  bool AcceptsFollower(const Layer* f) const override {
+    const string ty = f->type();
+    return ty == "Scale" || ty == "Bias" || ty == "ReLU" || ty == "TanH" || ty == "Sigmoid";
+  }
   void SetEpilogue(const vector<Layer*>& followers) override { followers_ = followers; }
   uint64_t ChannelStageVersion() const override {
     return (BlobVersion(blobs_[0]) * 31 + BlobVersion(blobs_[1])) * 31 + BlobVersion(blobs_[2]);

@@ -15,6 +15,7 @@ class ProposalLayer : public Layer {
  public:
   explicit ProposalLayer(const LayerParameter& param) : Layer(param) {}
   const char* type() const override { return "ProposalLayer"; }
+  bool ShapesTopInForward() const override { return true; }
   int ExactNumBottomBlobs() const override { return 3; }
   int MinTopBlobs() const override { return 1; }
   int MaxTopBlobs() const override { return 2; }
@@ -109,6 +110,7 @@ class DetectionOutputLayer : public Layer {
  public:
   explicit DetectionOutputLayer(const LayerParameter& param) : Layer(param) {}
   const char* type() const override { return "DetectionOutput"; }
+  bool ShapesTopInForward() const override { return true; }
   int ExactNumBottomBlobs() const override { return 3; }
   int ExactNumTopBlobs() const override { return 1; }
 
@@ -168,7 +170,7 @@ class DetectionOutputLayer : public Layer {
                                variance_encoded_in_target_ ? 1 : 0, keep_top_k_,
                                confidence_threshold_, nms_threshold_, eta_, top_k_,
                                workspace_.mutable_gpu_data(), bytes, top[0]->mutable_gpu_data(),
-                               max_rows, counter_.mutable_gpu_data(), cur_stream()));
+                               max_rows, counter_.mutable_gpu_data(), nullptr, cur_stream()));
     // data-dependent top shape (detection_output_layer.cpp:166-189)
     const int rows = counter_.cpu_data()[0];
     top[0]->Reshape(vector<int>{rows, 7});

@@ -179,7 +179,10 @@ class FlattenLayer : public Layer {
 
  protected:
   void Forward_gpu(const vector<Blob*>& bottom, const vector<Blob*>& top) override {
-    if (bottom[0] != top[0]) DeviceCopy(*bottom[0], top[0]);
+    if (bottom[0] == top[0]) return;
+    // the bottom's producer may have given it its final shape in its own Forward
+    if (bottom[0]->count() != top[0]->count()) Reshape(bottom, top);
+    DeviceCopy(*bottom[0], top[0]);
   }
 };
 REGISTER_LAYER_CLASS(Flatten);
@@ -246,6 +249,8 @@ class ReshapeLayer : public Layer {
 
  protected:
   void Forward_gpu(const vector<Blob*>& bottom, const vector<Blob*>& top) override {
+    // the bottom's producer may have given it its final shape in its own Forward
+    if (bottom[0]->count() != top[0]->count()) Reshape(bottom, top);
     DeviceCopy(*bottom[0], top[0]);
   }
   vector<int> dims_, copy_axes_;

@@ -238,6 +238,7 @@ void Net::PlanFusion() {
              layers_[j]->IsChannelStage(channels)) {
         const string ty = layers_[j]->type();
         const bool is_act = ty == "ReLU" || ty == "TanH" || ty == "Sigmoid";
+        if (!layers_[i]->AcceptsFollower(layers_[j].get())) break;
         if (!is_act && ++affine > layers_[i]->MaxAffineFollowers()) break;
         followers.push_back(layers_[j].get());
         ++j;
@@ -337,6 +338,14 @@ void Net::PlanFusion() {
     if (bottom_vecs_[v][0] == top_vecs_[v][0]) continue;
     const int b_id = bottom_id_vecs_[v][0];
     if (blob_life_time_[b_id] != static_cast<int>(v)) continue;
+    // a bottom that its producer re-shapes (and may re-allocate) in Forward
+    // cannot be aliased ahead of time: the view copies instead
+    bool late_shape = false;
+    for (size_t w = 0; w < v; ++w)
+      if (layers_[w]->ShapesTopInForward() &&
+          std::find(top_vecs_[w].begin(), top_vecs_[w].end(), bottom_vecs_[v][0]) != top_vecs_[w].end())
+        late_shape = true;
+    if (late_shape) continue;
     layer_fused_[v] = 1;
     residual_alias_[v] = b_id;
   }
@@ -435,6 +444,14 @@ bool Net::has_blob(const string& blob_name) const {
 const shared_ptr<Blob> Net::blob_by_name(const string& blob_name) const {
   CHECK(has_blob(blob_name)) << "Unknown blob name " << blob_name;
   return blobs_[blob_names_index_.find(blob_name)->second];
+}
+
+// reference src/net.cpp:293-301
+void Net::ToProto(NetParameter* param) const {
+  param->fields().clear();
+  param->set("name", name_, true);
+  for (const auto& layer : layers_)
+    layer->ToProto(static_cast<LayerParameter*>(param->add_sub("layer")));
 }
 
 shared_ptr<NetParameter> ReadTextNetParameterFromFile(const string& file) {

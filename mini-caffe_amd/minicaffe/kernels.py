@@ -58,7 +58,8 @@ LIB.mcDetectionOutputWorkspaceSize.argtypes = [c_int, c_int, c_int, c_int, c_int
                                                ctypes.POINTER(ctypes.c_size_t)]
 LIB.mcDetectionOutputMaxRows.argtypes = [c_int] * 5
 LIB.mcDetectionOutput.argtypes = [c_void_p, c_void_p, c_void_p] + [c_int] * 8 + \
-    [c_float, c_float, c_float, c_int, c_void_p, ctypes.c_size_t, c_void_p, c_int, c_void_p, c_void_p]
+    [c_float, c_float, c_float, c_int, c_void_p, ctypes.c_size_t, c_void_p, c_int, c_void_p, c_void_p,
+     c_void_p]
 LIB.mcROIPooling.argtypes = [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int,
                              c_float, c_void_p, c_void_p, c_void_p]
 LIB.mcPSROIPooling.argtypes = [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float,

@@ -461,6 +461,34 @@ def test_golden_caffemodel_loads_into_the_landmark_net():
     assert net.blobs["fc2"].shape == [1, 2]
 
 
+def test_net_to_proto_round_trip(tmp_path):
+    """Net::ToProto (reference src/net.cpp:293-301): the definition with the current weights
+    builds an equal net, survives the wire-format writer and reader, and the written bytes
+    hold the trained values when walked by the independent reader of tests/wire.py."""
+    import subprocess
+    from minicaffe import craft
+    exe = os.path.join(ROOT, "mini-caffe_amd", "bin", "net_roundtrip")
+    assert os.path.exists(exe), "run __graft_entry__.build() first"
+    proto = tmp_path / "net.prototxt"
+    proto.write_text(craft.to_prototxt(landmark_level2_spec(), "landmark"))
+    model = os.path.join(GOLDEN, "deeplandmark_2_LE1.caffemodel")
+    out = tmp_path / "out.caffemodel"
+    r = subprocess.run([exe, str(proto), model, str(out)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "roundtrip ok: 8 parameter blobs" in r.stdout
+    want = wire.read_net_blobs(open(model, "rb").read())
+    got = wire.read_net_blobs(out.read_bytes())
+    assert sorted(got) == sorted(want)
+    for layer in want:
+        assert len(got[layer]) == len(want[layer])
+        for a, b in zip(got[layer], want[layer]):
+            assert a.shape == b.shape and np.array_equal(a, b), layer
+    # and the library reads its own bytes back as weights through the C ABI
+    net = mc.Net.from_buffers(proto.read_text(), out.read_bytes())
+    params = dict(net.param_list)
+    assert np.array_equal(params["fc2_0"].data, want["fc2"][0])
+
+
 @needs_ref
 def test_landmark_spec_equals_the_reference_prototxt():
     from minicaffe import craft

@@ -610,22 +610,95 @@ def test_detection_output_bit_exact(K, num, P, C, share, code, keep, thr, nms, e
     if topk is not None:
         param["nms_param"]["top_k"] = topk
     want = oracle.detection_output(param, loc, conf, prior)
-    tk = -1 if topk is None else topk
+    got, flag = run_detection_output(K, param, loc, conf, prior)
+    assert got.shape == want.shape
+    assert np.array_equal(got, want)
+    want_flag = cut_tie_expected(param, loc, conf, prior)
+    assert flag == want_flag and not (want_flag & 1)      # no case here is undefined at the cut
+
+
+def run_detection_output(K, param, loc, conf, prior):
+    """mcDetectionOutput on host arrays -> (rows, cut-tie flag)."""
+    num, C = loc.shape[0], param["num_classes"]
+    P = prior.shape[2] // 4
+    nmsp = param.get("nms_param", {})
+    tk, keep = nmsp.get("top_k", -1), param.get("keep_top_k", -1)
+    share = param.get("share_location", True)
     sz = ctypes.c_size_t()
     K.check_mc(K.LIB.mcDetectionOutputWorkspaceSize(num, P, C, int(share), tk, ctypes.byref(sz)))
     max_rows = K.LIB.mcDetectionOutputMaxRows(num, P, C, tk, keep)
     ws = torch.empty(sz.value, dtype=torch.uint8, device="cuda")
     ld, cd, pd = dev(loc), dev(conf), dev(prior)
     out = torch.full((max_rows, 7), float("nan"), device="cuda")
-    cnt = torch.zeros(1, dtype=torch.int32, device="cuda")
+    cnt = torch.full((2,), -5, dtype=torch.int32, device="cuda")
+    code = {"CORNER": 1, "CENTER_SIZE": 2, "CORNER_SIZE": 3}[str(param.get("code_type", "CORNER"))]
     K.check_mc(K.LIB.mcDetectionOutput(
-        fptr(ld), fptr(cd), fptr(pd), num, P, C, int(share), 0, {"CORNER": 1, "CENTER_SIZE": 2, "CORNER_SIZE": 3}[code],
-        0, keep, ctypes.c_float(-3.4028234663852886e38 if thr is None else thr), ctypes.c_float(nms),
-        ctypes.c_float(eta), tk, fptr(ws), sz.value, fptr(out), max_rows, ctypes.c_void_p(cnt.data_ptr()), None))
+        fptr(ld), fptr(cd), fptr(pd), num, P, C, int(share), param.get("background_label_id", 0), code,
+        int(param.get("variance_encoded_in_target", False)), keep,
+        ctypes.c_float(param.get("confidence_threshold", -3.4028234663852886e38)),
+        ctypes.c_float(nmsp.get("nms_threshold", 0.3)), ctypes.c_float(nmsp.get("eta", 1.0)), tk, fptr(ws),
+        sz.value, fptr(out), max_rows, ctypes.c_void_p(cnt.data_ptr()), ctypes.c_void_p(cnt.data_ptr() + 4), None))
     torch.cuda.synchronize()
-    got = out[:int(cnt.item())].cpu().numpy()
+    return out[:int(cnt[0].item())].cpu().numpy(), int(cnt[1].item())
+
+
+def cut_tie_expected(param, loc, conf, prior):
+    """The flag's bits from the CPU side.  Over the images that keep_top_k cuts: 1 when the
+    keep_top_k-th and the next score of the per-class NMS survivors are equal, 2 when two
+    kept rows of one label have equal scores (std::sort defines neither order)."""
+    keep = param.get("keep_top_k", -1)
+    if keep < 0:
+        return 0
+    rows = oracle.detection_output(dict(param, keep_top_k=-1), loc, conf, prior)
+    flag = 0
+    for i in range(loc.shape[0]):
+        r = rows[(rows[:, 0] == i) & (rows[:, 1] >= 0)]
+        sc = np.sort(r[:, 2])[::-1]
+        if not len(sc) > keep > 0:
+            continue
+        if sc[keep - 1] == sc[keep]:
+            flag |= 1
+        for lab in np.unique(r[:, 1]):
+            s = r[(r[:, 1] == lab) & (r[:, 2] >= sc[keep - 1]), 2]
+            # of a run of equal scores at the cut only a prefix is kept: count what survives
+            room = keep - int((r[:, 2] > sc[keep - 1]).sum())
+            at_cut = r[r[:, 2] == sc[keep - 1]]
+            taken = at_cut[np.argsort(at_cut[:, 1], kind="stable")][:room]
+            s = np.concatenate([r[(r[:, 1] == lab) & (r[:, 2] > sc[keep - 1]), 2],
+                                taken[taken[:, 1] == lab, 2]])
+            if len(np.unique(s)) < len(s):
+                flag |= 2
+    return flag
+
+
+def test_detection_output_flags_equal_scores_at_the_keep_top_k_cut(K):
+    """Quantised confidences: some images have equal scores on both sides of the cut.
+    The flag says so (bit 1 = tie at the cut, bit 2 = equal scores within a kept label);
+    the rows above the tied score are the oracle's up to the order of equal scores, and
+    the kept scores are the same multiset either way."""
+    rng = np.random.default_rng(40)
+    num, P, C = 6, 300, 4
+    loc = (rng.standard_normal((num, P * 4)) * 0.5).astype(np.float32)
+    conf = (np.round(rng.random((num, P * C)) * 50) / 50).astype(np.float32)
+    c = rng.random((P, 2)) * 0.8 + 0.1
+    wh = rng.random((P, 2)) * 0.1 + 0.02
+    prior = np.concatenate([np.concatenate([c - wh / 2, c + wh / 2], 1).reshape(-1),
+                            np.tile([0.1, 0.1, 0.2, 0.2], P)]).reshape(1, 2, P * 4).astype(np.float32)
+    param = {"num_classes": C, "share_location": True, "background_label_id": 0, "code_type": "CENTER_SIZE",
+             "keep_top_k": 40, "confidence_threshold": 0.3, "nms_param": {"nms_threshold": 0.45, "top_k": 100}}
+    got, flag = run_detection_output(K, param, loc, conf, prior)
+    assert flag == 3 and cut_tie_expected(param, loc, conf, prior) == 3
+    want = oracle.detection_output(param, loc, conf, prior)
     assert got.shape == want.shape
-    assert np.array_equal(got, want)
+    for i in range(num):
+        g, w = got[got[:, 0] == i], want[want[:, 0] == i]
+        assert np.array_equal(np.sort(g[:, 2]), np.sort(w[:, 2]))
+        cut = g[:, 2].min()                       # rows strictly above the tied score are defined
+        ga, wa = g[g[:, 2] > cut], w[w[:, 2] > cut]
+        assert np.array_equal(ga[np.lexsort(ga.T[::-1])], wa[np.lexsort(wa.T[::-1])])
+    # without a cut there is nothing to flag
+    got, flag = run_detection_output(K, dict(param, keep_top_k=-1), loc, conf, prior)
+    assert flag == 0 and np.array_equal(got, oracle.detection_output(dict(param, keep_top_k=-1), loc, conf, prior))
 
 
 def _random_rois(rng, n_rois, num, img_h, img_w):

@@ -325,6 +325,77 @@ def test_unfused_layers_standalone(gpu_mode):
         assert netrun.rel_err(got, want[name]) < 1e-5, name
 
 
+def test_batch_norm_head_takes_only_scale_bias_followers(gpu_mode):
+    """A BatchNorm that runs as its own pass absorbs an in-place Scale / Bias and an
+    activation; an in-place BN or a second BatchNorm behind it carries a subtraction of
+    its own and must run as its own pass.  Both statistics modes."""
+    from minicaffe.craft import input_layer
+    rng = np.random.default_rng(14)
+    C = 5
+
+    def stats():
+        return [rng.standard_normal(C).astype(np.float32), (rng.random(C) + 0.5).astype(np.float32),
+                np.array([0.7], np.float32)]
+
+    def bn_blobs():
+        return [a.reshape(1, C) for a in (rng.standard_normal(C).astype(np.float32),
+                                          rng.standard_normal(C).astype(np.float32),
+                                          rng.standard_normal(C).astype(np.float32),
+                                          (rng.random(C) + 0.5).astype(np.float32))]
+
+    spec = [input_layer({"data": (3, C, 4, 6)}),
+            {"name": "split", "type": "Split", "bottom": ["data"], "top": ["a", "b", "c"]},
+            # batch statistics head, BN follower, ReLU
+            {"name": "bn_a", "type": "BatchNorm", "bottom": ["a"], "top": ["ya"],
+             "batch_norm_param": {"use_global_stats": False},
+             "blobs": [np.zeros(C, np.float32), np.zeros(C, np.float32), np.zeros(1, np.float32)]},
+            {"name": "fused_a", "type": "BN", "bottom": ["ya"], "top": ["ya"], "blobs": bn_blobs()},
+            {"name": "relu_a", "type": "ReLU", "bottom": ["ya"], "top": ["ya"]},
+            # stored statistics head (first layer on its blob, so it is the head), BatchNorm follower
+            {"name": "bn_b", "type": "BatchNorm", "bottom": ["b"], "top": ["yb"], "blobs": stats()},
+            {"name": "bn_b2", "type": "BatchNorm", "bottom": ["yb"], "top": ["yb"],
+             "batch_norm_param": {"eps": 1e-2}, "blobs": stats()},
+            {"name": "tanh_b", "type": "TanH", "bottom": ["yb"], "top": ["yb"]},
+            # the supported run for comparison: Scale + ReLU ride along
+            {"name": "bn_c", "type": "BatchNorm", "bottom": ["c"], "top": ["yc"], "blobs": stats()},
+            {"name": "sc_c", "type": "Scale", "bottom": ["yc"], "top": ["yc"], "scale_param": {"bias_term": True},
+             "blobs": [rng.standard_normal(C).astype(np.float32), rng.standard_normal(C).astype(np.float32)]},
+            {"name": "relu_c", "type": "ReLU", "bottom": ["yc"], "top": ["yc"]}]
+    inputs = {"data": rng.standard_normal((3, C, 4, 6)).astype(np.float32)}
+    net = run_net(gpu_mode, spec, inputs, ["ya", "yb", "yc"])
+    want = netrun.oracle_forward(spec, inputs)
+    for name in ("ya", "yb", "yc"):
+        assert netrun.rel_err(net.get_blob(name).data, want[name]) < 1e-5, name
+
+
+def test_view_behind_detection_output_sees_the_final_rows(gpu_mode):
+    """DetectionOutput sizes its top after the device has counted the rows; a Flatten
+    behind it must copy those rows (not alias the block the top had before Forward)."""
+    from minicaffe.craft import Enum, input_layer
+    rng = np.random.default_rng(15)
+    num, P, C = 2, 40, 4
+    c = rng.random((P, 2)) * 0.8 + 0.1
+    wh = rng.random((P, 2)) * 0.3 + 0.05
+    prior = np.concatenate([np.concatenate([c - wh / 2, c + wh / 2], 1).reshape(-1),
+                            np.tile([0.1, 0.1, 0.2, 0.2], P)]).reshape(1, 2, P * 4).astype(np.float32)
+    loc = (rng.standard_normal((num, P * 4)) * 0.5).astype(np.float32)
+    conf = oracle.softmax((rng.standard_normal((num, P, C)) * 2).astype(np.float32), 2).reshape(num, P * C)
+    param = {"num_classes": C, "share_location": True, "background_label_id": 0,
+             "code_type": Enum("CENTER_SIZE"), "keep_top_k": 20, "confidence_threshold": 0.05,
+             "nms_param": {"nms_threshold": 0.45, "top_k": 15}}
+    spec = [input_layer({"loc": loc.shape, "conf": conf.shape, "prior": prior.shape}),
+            {"name": "det", "type": "DetectionOutput", "bottom": ["loc", "conf", "prior"], "top": ["det"],
+             "detection_output_param": param},
+            {"name": "flat", "type": "Flatten", "bottom": ["det"], "top": ["flat"],
+             "flatten_param": {"axis": 0}}]
+    net = run_net(gpu_mode, spec, {"loc": loc, "conf": conf, "prior": prior})
+    want = oracle.detection_output(dict(param, code_type="CENTER_SIZE"), loc, conf, prior)
+    assert want.shape[0] > 5
+    assert np.array_equal(net.get_blob("flat").data.reshape(-1, 7), want)
+    net.forward(loc=loc, conf=conf, prior=prior)          # and on a repeated call
+    assert np.array_equal(net.get_blob("flat").data.reshape(-1, 7), want)
+
+
 def test_resnet50_full_graph_two_images(gpu_mode):
     """The real ResNet-50 graph at 224x224 (229 layers); the oracle uses OpenBLAS for
     its sgemm, as the reference does."""
@@ -341,18 +412,30 @@ def test_resnet50_full_graph_two_images(gpu_mode):
 
 
 def test_resnet50_b64_properties(gpu_mode):
-    """Full benchmark size: size-independent properties instead of a CPU run.
-    Rows of the batch-64 result equal the batch-1 result of the same image, rows
-    sum to one, and duplicated images give identical rows."""
+    """Full benchmark size.  Rows 0, 17 and 63 of the batch-64 result are compared with
+    the CPU oracle walking the same three images (`res5c` and `prob`); for the rest,
+    size-independent properties: rows of the batch-64 result equal the batch-1 result
+    of the same image, rows sum to one, and duplicated images give identical rows."""
     from minicaffe import zoo
     spec, inputs = zoo.resnet50_spec(batch=64, size=224, seed=0)
     x = inputs["data"]
     x[63] = x[5]
-    net = run_net(gpu_mode, spec, {"data": x})
+    net = run_net(gpu_mode, spec, {"data": x}, ["res5c"])
     p64 = net.get_blob("prob").data.copy()
+    r64 = net.get_blob("res5c").data.copy()
     assert p64.shape == (64, 1000) and np.isfinite(p64).all()
     assert np.allclose(p64.sum(axis=1), 1, atol=1e-4)
     assert np.array_equal(p64[63], p64[5])
+    rows = [0, 17, 63]
+    oracle.use_openblas(True)
+    try:
+        want = netrun.oracle_forward(spec, {"data": x[rows]}, keep={"res5c", "prob"})
+    finally:
+        oracle.use_openblas(False)
+    assert r64.shape == (64, 2048, 7, 7)
+    for k, row in enumerate(rows):
+        assert netrun.rel_err(r64[row], want["res5c"][k]) < 1e-3, row
+        assert netrun.rel_err(p64[row], want["prob"][k]) < 1e-3, row
     net.forward(data=x[17:18])
     p1 = net.get_blob("prob").data.copy()
     assert np.abs(p1[0] - p64[17]).max() < 1e-6
@@ -445,6 +528,14 @@ def _check_ssd_tail(net, spec):
     got = net.get_blob("detection_out").data.copy()
     assert got.shape == want.shape
     assert np.array_equal(got, want)
+    # the one order the reference leaves undefined (equal scores on both sides of the
+    # keep_top_k cut) does not occur in these inputs: the kernel-level call says so
+    from minicaffe import kernels
+    from test_kernels_gpu import run_detection_output
+    p = dict(spec[-1]["detection_output_param"])
+    p["code_type"] = str(p.get("code_type", "CORNER"))
+    rows, cut_tie = run_detection_output(kernels, p, loc, conf, prior)
+    assert not (cut_tie & 1) and np.array_equal(rows, want)
     return got
 
 
@@ -471,11 +562,14 @@ def test_config3_ssd_small_width_every_stage(gpu_mode):
 
 
 def test_config3_ssd_full_size_b8(gpu_mode):
-    """Benchmark size (VGG16 widths, batch 8): the dense part is checked against the
-    oracle on the first image's source layers, the tail bit for bit on all 8 images."""
+    """Benchmark size (VGG16 widths, batch 8): the dense part of image 0 (Normalize,
+    fc7, the last extra layer and the concatenated heads before and after the softmax)
+    against the oracle walking that image at full width, the tail bit for bit on all
+    8 images."""
     from minicaffe import zoo
     spec, inputs = zoo.ssd300_spec(batch=8)
-    net = run_net(gpu_mode, spec, inputs, ["mbox_loc", "mbox_conf_flatten", "mbox_priorbox", "fc7"])
+    dense = ["conv4_3_norm", "fc7", "conv9_2", "mbox_loc", "mbox_conf", "mbox_conf_flatten"]
+    net = run_net(gpu_mode, spec, inputs, dense + ["mbox_priorbox"])
     rows = _check_ssd_tail(net, spec)
     assert set(np.unique(rows[:, 0]).astype(int)) <= set(range(8))
     counts = np.bincount(rows[:, 0].astype(int), minlength=8)
@@ -486,14 +580,17 @@ def test_config3_ssd_full_size_b8(gpu_mode):
         assert (np.diff(r[:, 1]) >= 0).all()
         for lab in np.unique(r[:, 1]):
             assert (np.diff(r[r[:, 1] == lab][:, 2]) <= 0).all()
-    fc7_gpu = net.get_blob("fc7").data[:1].copy()
     oracle.use_openblas(True)
     try:
-        idx = [i for i, l in enumerate(spec) if l["name"] == "fc7_relu"][0]
-        want = netrun.oracle_forward(spec[:idx + 1], {"data": inputs["data"][:1]}, keep={"fc7"})
+        want = netrun.oracle_forward(spec[:-1], {"data": inputs["data"][:1]},
+                                     keep=set(dense + ["mbox_priorbox"]))
     finally:
         oracle.use_openblas(False)
-    assert netrun.rel_err(fc7_gpu, want["fc7"]) < 1e-3
+    assert np.array_equal(net.get_blob("mbox_priorbox").data, want["mbox_priorbox"])
+    for name in dense:
+        got = net.get_blob(name).data[:1].copy()
+        assert got.shape == want[name].shape, name
+        assert netrun.rel_err(got, want[name]) < 1e-3, name
 
 
 def test_rfcn_second_stage_on_proposal_rois(gpu_mode):
