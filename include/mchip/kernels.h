@@ -94,7 +94,8 @@ int mcConvPlanSetWeights(mcConvPlan* plan, const float* weights, void* stream);
  * Replaces ConvolutionLayer::Forward_gpu (conv_layer.cu:7-22) and
  * DeconvolutionLayer::Forward_gpu (deconv_layer.cu:7-22) including the bias
  * add; the batch is folded into the GEMM column dimension instead of the
- * reference's per-image loop. */
+ * reference's per-image loop.  Any batch an int can count is accepted: blobs of
+ * 2^29 elements or more are processed as several runs of whole images. */
 int mcConvForward(const mcConvPlan* plan, int num, const float* bottom, float* top,
                   const mcEpilogue* epilogue, void* stream);
 
@@ -124,6 +125,12 @@ int mcConvPlanForceConfig(mcConvPlan* plan, int config);
  * launches too small to fill the GPU.  No counterpart in the reference. */
 int mcConvPlanForceSplit(mcConvPlan* plan, int slices);
 
+/* Tuning/test knob: a batch whose bottom or top blob reaches 2^29 elements is cut
+ * into runs of whole images, one launch each (the reference loops over single
+ * images, base_conv_layer.cpp:254-271, so it has no such limit); this caps a run
+ * at `images` images, 0 restores the automatic choice (as many as fit).  No
+ * counterpart in the reference. */
+int mcConvPlanForceChunk(mcConvPlan* plan, int images);
 
 /* Measurement hook (no counterpart in the reference): while enabled on the
  * calling thread, every contraction kernel launch is bracketed by two HIP events

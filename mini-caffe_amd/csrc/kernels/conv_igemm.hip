@@ -797,6 +797,7 @@ struct mcConvPlan {
   int wm_stride = 0, wg_stride = 0;
   int forced_config = -1;
   int forced_split = 0;  // 0 = choose, >= 1 = this many K slices
+  int forced_chunk = 0;  // 0 = as many images per launch as fit, else at most this many
   bool force_general = false;  // use the tap-table gather even for pointwise geometry
   // group == input channels: a direct kernel reads the layer's own filter layout
   bool depthwise = false;
@@ -1149,6 +1150,12 @@ int mcConvPlanForceConfig(mcConvPlan* plan, int config) {
   return 0;
 }
 
+int mcConvPlanForceChunk(mcConvPlan* plan, int images) {
+  MC_REQUIRE(plan && images >= 0, "mcConvPlanForceChunk: bad argument");
+  plan->forced_chunk = images;
+  return 0;
+}
+
 int mcConvPlanForceSplit(mcConvPlan* plan, int slices) {
   MC_REQUIRE(plan, "mcConvPlanForceSplit: null plan");
   MC_REQUIRE(slices >= 0 && slices <= 64, "mcConvPlanForceSplit: slices out of range");
@@ -1162,16 +1169,16 @@ namespace {
 
 // top_second != nullptr: the plan's output channels [0, c_first) go to `top`, the
 // others to top_second.
-int conv_forward(const mcConvPlan* plan, int num, const float* bottom, float* top,
-                 const mcEpilogue* ep, void* stream, float* top_second, int c_first) {
-  MC_REQUIRE(plan && bottom && top, "mcConvForward: null argument");
-  MC_REQUIRE(num > 0, "mcConvForward: batch must be positive");
+// One launch (plus the pass that sums K slices) over `num` images that fit the
+// kernels' 31-bit byte offsets; conv_forward() cuts larger batches into such runs.
+int conv_forward_images(const mcConvPlan* plan, int num, const float* bottom, float* top,
+                        const mcEpilogue* ep, void* stream, float* top_second, int c_first) {
   const mcConvGeom& g = plan->geom;
   const long in_count = (long)num * g.channels_in * g.height_in * g.width_in;
   const long out_count = (long)num * g.channels_out * plan->Ho * plan->Wo;
-  // the bottom blob is addressed through a 31-bit byte offset
-  MC_REQUIRE(in_count < (1L << 29) && out_count < (1L << 29),
-             "mcConvForward: blob exceeds 2^29 elements");
+  // the blobs are addressed through 31-bit byte offsets
+  MC_REQUIRE(plan->depthwise || (in_count < (1L << 29) && out_count < (1L << 29)),
+             "mcConvForward: image run exceeds 2^29 elements");
   hipStream_t st = static_cast<hipStream_t>(stream);
   float* const top_first = top;
   if (top_second) {
@@ -1365,6 +1372,49 @@ int conv_forward(const mcConvPlan* plan, int num, const float* bottom, float* to
   if (g_timing) {
     MC_HIP(hipEventRecord(tl.stop, st));
     g_timed.push_back(tl);
+  }
+  return 0;
+}
+
+// The reference convolves image by image and so takes any blob an int can count
+// (base_conv_layer.cpp:254-271).  Here a launch covers as many images as the 31-bit
+// byte offsets of the buffer descriptors allow (fewer than 2^29 elements in the
+// bottom and in the top run, offset shifts included); a larger batch is cut into
+// equal runs of whole images, each with its own launch, epilogue and residual rows.
+int conv_forward(const mcConvPlan* plan, int num, const float* bottom, float* top,
+                 const mcEpilogue* ep, void* stream, float* top_second, int c_first) {
+  MC_REQUIRE(plan && bottom && top, "mcConvForward: null argument");
+  MC_REQUIRE(num > 0, "mcConvForward: batch must be positive");
+  const mcConvGeom& g = plan->geom;
+  if (plan->depthwise)  // indexed with 64-bit integers throughout
+    return conv_forward_images(plan, num, bottom, top, ep, stream, top_second, c_first);
+  const long in_img = (long)g.channels_in * g.height_in * g.width_in;
+  const long out_img = (long)g.channels_out * plan->Ho * plan->Wo;
+  long shift = 0;
+  for (const auto& s : plan->subs) shift = std::max(shift, (long)s.tap_shift + s.pix_shift);
+  const long lim = (1L << 29) - 1;
+  long per = std::min(lim / in_img, lim / out_img);
+  per = std::min(per, ((1L << 31) - 65 - 2 * shift) / (4 * in_img));
+  if (plan->forced_chunk > 0) per = std::min<long>(per, plan->forced_chunk);
+  MC_REQUIRE(per >= 1, "mcConvForward: a single image exceeds 2^29 elements");
+  if (num <= per)
+    return conv_forward_images(plan, num, bottom, top, ep, stream, top_second, c_first);
+  const int runs = ceil_div(num, per);
+  const int run_len = ceil_div(num, runs);
+  const long hw_out = (long)plan->Ho * plan->Wo;
+  const long first_img = top_second ? c_first * hw_out : out_img;
+  const long second_img = out_img - first_img;
+  for (int n0 = 0; n0 < num; n0 += run_len) {
+    const int n = std::min(run_len, num - n0);
+    mcEpilogue run_ep;
+    if (ep) {
+      run_ep = *ep;
+      if (ep->residual) run_ep.residual = ep->residual + n0 * out_img;
+    }
+    if (conv_forward_images(plan, n, bottom + n0 * in_img, top + n0 * first_img,
+                            ep ? &run_ep : nullptr, stream,
+                            top_second ? top_second + n0 * second_img : nullptr, c_first))
+      return -1;
   }
   return 0;
 }

@@ -99,6 +99,7 @@ LIB.mcConvPlanKernelName.argtypes = [c_void_p, c_int]
 LIB.mcConvPlanKernelName.restype = ctypes.c_char_p
 LIB.mcConvPlanForceConfig.argtypes = [c_void_p, c_int]
 LIB.mcConvPlanForceSplit.argtypes = [c_void_p, c_int]
+LIB.mcConvPlanForceChunk.argtypes = [c_void_p, c_int]
 
 
 def conv_geom(cin, h, w, cout, kernel, stride=1, pad=0, dilation=1, group=1, transposed=False):
@@ -143,6 +144,9 @@ class ConvPlan(object):
 
     def force_split(self, slices):
         check_mc(LIB.mcConvPlanForceSplit(self.handle, slices))
+
+    def force_chunk(self, images):
+        check_mc(LIB.mcConvPlanForceChunk(self.handle, images))
 
     def forward(self, num, x_ptr, y_ptr, scale=None, shift=None, residual=None,
                 activation=ACT_NONE, negative_slope=0.0, stream=0):

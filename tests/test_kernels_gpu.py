@@ -83,6 +83,95 @@ def test_conv_forward(K, case, cfg):
     assert netrun.rel_err(yd.cpu().numpy(), want) < 1e-4
 
 
+@pytest.mark.parametrize("case", [
+    # cin, h, w, cout, k, s, p, transposed, n, images per run
+    (24, 13, 11, 40, 3, 1, 1, False, 8, 3),      # runs of 3, 3, 2 images
+    (32, 9, 9, 70, 1, 1, 0, False, 7, 2),        # pointwise
+    (16, 7, 6, 20, 4, 2, 1, True, 5, 2),         # deconvolution: four parity classes per run
+    (24, 13, 11, 40, 3, 2, 1, False, 4, 1),      # one image per run
+])
+def test_conv_batch_cut_into_image_runs(K, case):
+    """A batch the buffer descriptors cannot address in one launch is cut into runs of
+    whole images (forced here with a small run length): every run must equal a call of
+    its own on those images bit for bit, epilogue and residual rows included, and the
+    whole result the oracle's."""
+    cin, h, w, cout, k, st, p, tr, n, per = case
+    rng = np.random.default_rng(51)
+    x = rng.standard_normal((n, cin, h, w)).astype(np.float32)
+    wt = (rng.standard_normal((cin, cout, k, k) if tr else (cout, cin, k, k)) * 0.1).astype(np.float32)
+    b = rng.standard_normal(cout).astype(np.float32)
+    sc = (rng.random(cout) + 0.5).astype(np.float32)
+    geom = oracle.conv_geom(cin, h, w, cout, k, st, p, 1, 1, tr)
+    raw = oracle.conv_forward(geom, x, wt, None)
+    res = rng.standard_normal(raw.shape).astype(np.float32)
+    want = np.maximum(raw * sc.reshape(1, -1, 1, 1) + b.reshape(1, -1, 1, 1) + res, 0)
+    plan = K.ConvPlan(K.conv_geom(cin, h, w, cout, k, st, p, 1, 1, tr))
+    xd, wd, bd, sd, rd = dev(x), dev(wt), dev(b), dev(sc), dev(res)
+    plan.set_weights(wd.data_ptr())
+    ep = dict(scale=sd.data_ptr(), shift=bd.data_ptr(), activation=K_ACT_RELU)
+    plan.force_chunk(per)
+    cut = torch.full(raw.shape, float("nan"), device="cuda")
+    plan.forward(n, xd.data_ptr(), cut.data_ptr(), residual=rd.data_ptr(), **ep)
+    plan.force_chunk(0)
+    runs = -(-n // per)
+    run_len = -(-n // runs)
+    parts = torch.full(raw.shape, float("nan"), device="cuda")
+    for n0 in range(0, n, run_len):
+        m = min(run_len, n - n0)
+        plan.forward(m, xd[n0:].data_ptr(), parts[n0:].data_ptr(), residual=rd[n0:].data_ptr(), **ep)
+    torch.cuda.synchronize()
+    assert torch.equal(cut, parts)
+    assert netrun.rel_err(cut.cpu().numpy(), want) < 1e-4
+    if not tr:
+        # two tops: each top advances by its own image size
+        c_first = 13
+        plan.force_chunk(per)
+        first = torch.full((n, c_first) + raw.shape[2:], float("nan"), device="cuda")
+        second = torch.full((n, cout - c_first) + raw.shape[2:], float("nan"), device="cuda")
+        plan.forward_two_tops(n, xd.data_ptr(), first.data_ptr(), c_first, second.data_ptr(), **ep)
+        torch.cuda.synchronize()
+        both = torch.cat([first, second], 1).cpu().numpy()
+        want2 = np.maximum(raw * sc.reshape(1, -1, 1, 1) + b.reshape(1, -1, 1, 1), 0)
+        assert netrun.rel_err(both, want2) < 1e-4
+
+
+def test_conv_blob_beyond_two_to_the_29_elements(K):
+    """A 1x1 convolution whose bottom and top hold more than 2^29 elements each (the
+    reference's per-image loop takes any size): the call cuts the batch itself, and
+    every image equals the result of a small call on that image."""
+    cin = cout = 64
+    h = w = 56
+    n = (1 << 29) // (cin * h * w) + 30          # 2705 images, 542.9M elements, 2.2 GB per blob
+    assert n * cin * h * w > (1 << 29)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.empty((n, cin, h, w), device="cuda").uniform_(-1, 1, generator=g)
+    wt = (torch.randn((cout, cin, 1, 1), device="cuda", generator=g) * 0.1).contiguous()
+    b = torch.randn(cout, device="cuda", generator=g)
+    plan = K.ConvPlan(K.conv_geom(cin, h, w, cout, 1, 1, 0))
+    plan.set_weights(wt.data_ptr())
+    y = torch.full((n, cout, h, w), float("nan"), device="cuda")
+    plan.forward(n, x.data_ptr(), y.data_ptr(), shift=b.data_ptr(), activation=K_ACT_RELU)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(y).all())
+    # the run length the library chose, and images on both sides of every cut
+    per = ((1 << 29) - 1) // (cin * h * w)
+    runs = -(-n // per)
+    run_len = -(-n // runs)
+    probe = sorted({0, 1, run_len - 1, run_len, run_len + 1, n - 2, n - 1})
+    small = torch.empty((1, cout, h, w), device="cuda")
+    for i in probe:
+        plan.forward(1, x[i:].data_ptr(), small.data_ptr(), shift=b.data_ptr(), activation=K_ACT_RELU)
+        torch.cuda.synchronize()
+        assert netrun.rel_err(y[i].cpu().numpy(), small[0].cpu().numpy()) < 1e-5, i
+    # and one image against the CPU oracle
+    i = run_len
+    want = np.maximum(oracle.conv_forward(oracle.conv_geom(cin, h, w, cout, 1, 1, 0), x[i:i + 1].cpu().numpy(),
+                                          wt.cpu().numpy(), b.cpu().numpy()), 0)
+    assert netrun.rel_err(y[i:i + 1].cpu().numpy(), want) < 1e-4
+    del x, y
+    torch.cuda.empty_cache()
+
+
 THIN_CASES = [
     (8, 96, 90, 3, 3, 1, 1, 1, 1, False, 8),        # 3x3 to 3 channels (one validity mask per tap pair)
     (16, 96, 90, 1, 1, 1, 0, 1, 1, False, 8),       # 1x1 score map: pointwise path
