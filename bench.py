@@ -22,10 +22,36 @@ sys.path.insert(0, os.path.join(ROOT, "mini-caffe_amd"))
 
 FP32_MFMA_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per convolution launch (mean over the 53 launches of one forward),
-# from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in
-# profiles/igemm_resnet50_b64_pmc_traffic.txt (algorithmic: 126.3e6).
-CONV_TRAFFIC_BYTES_PER_LAUNCH = 149.4e6
+CONV_SOURCE = os.path.join(ROOT, "mini-caffe_amd", "csrc", "kernels", "conv_igemm.hip")
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "igemm_resnet50_b64_pmc_traffic.txt")
+MFMA_PROFILE = os.path.join(ROOT, "profiles", "igemm_resnet50_b64_pmc_mfma_util.txt")
+
+
+def counter_figure(path, key):
+    """A figure that only a rocprofv3 --pmc run can give (HBM bytes per launch, MFMA
+    utilisation), read from the committed summary of that run.  The summary ends with
+    `key: value` lines, among them the SHA-256 of the kernel source it was taken with;
+    a summary of another kernel version is reported as stale instead of being quoted.
+    Returns (value or None, note)."""
+    import hashlib
+    fields = {}
+    try:
+        for line in open(path):
+            k, sep, v = line.partition(":")
+            if sep and " " not in k.strip():
+                fields[k.strip()] = v.strip()
+    except OSError as e:
+        return None, "no counter summary (%s)" % e
+    have = hashlib.sha256(open(CONV_SOURCE, "rb").read()).hexdigest()
+    rel = os.path.relpath(path, ROOT)
+    if key not in fields or "conv_igemm_sha256" not in fields:
+        return None, "%s holds no '%s' line" % (rel, key)
+    if fields["conv_igemm_sha256"] != have:
+        msg = ("%s was taken with another version of conv_igemm.hip (sha256 %s..., tree has %s...): "
+               "re-run the command it names" % (rel, fields["conv_igemm_sha256"][:12], have[:12]))
+        print("bench.py: STALE COUNTER SUMMARY: " + msg, file=sys.stderr)
+        return None, "stale: " + msg
+    return float(fields[key]), "%s, taken %s" % (rel, fields.get("date", "?"))
 
 
 def main():
@@ -109,9 +135,11 @@ def main():
     LIB.mcConvTimingCollect(ctypes.byref(tot_ms), ctypes.byref(launches), ctypes.byref(fl))
     LIB.mcConvTimingEnable(0)
     achieved = fl.value / (tot_ms.value * 1e-3) / 1e12 if tot_ms.value > 0 else 0.0
+    traffic, traffic_note = counter_figure(TRAFFIC_PROFILE, "traffic_bytes_per_launch")
+    mfma_util, mfma_note = counter_figure(MFMA_PROFILE, "mfma_util_pct")
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP32_MFMA_PEAK_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
-                "traffic": CONV_TRAFFIC_BYTES_PER_LAUNCH,
+                "traffic": traffic, "traffic_source": traffic_note,
                 "kernel": "igemm_f32 (Convolution + InnerProduct, fused BN/Scale/ReLU epilogue)",
                 "launches_per_step": launches.value // max(1, args.steps),
                 "kernel_ms_per_step": round(tot_ms.value / max(1, args.steps), 3),
@@ -126,6 +154,10 @@ def main():
     if args.bandwidth_report:
         bandwidth_report(args.bandwidth_report)
 
+    # the other two figures of the metric: convolution MFMA utilisation (hardware
+    # counters, quoted from the committed counter run) and the detection tails
+    del net
+    tails = detection_tails(mc, craft, zoo, LIB)
     cpu = None
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(args.cpu_batch)
@@ -139,8 +171,118 @@ def main():
                                   "(BASELINE configs[1])" % args.batch,
                       "conv_gflop_per_step": round(flops["conv"] / 1e9, 1),
                       "api": "CaffeNetForward (Net::Forward(reshape=true))"},
-           "roofline": roofline, "cpu_baseline": cpu}
+           "roofline": roofline, "cpu_baseline": cpu,
+           "conv_mfma_util_pct": mfma_util, "conv_mfma_util_source": mfma_note}
+    out.update(tails)
     print(json.dumps(out))
+
+
+def detection_tails(mc, craft, zoo, LIB):
+    """NMS / Proposal / DetectionOutput device time at the sizes of configurations 4 and 3.
+    The nets run once to produce the tails' real inputs (RPN scores and deltas; SSD
+    locations, softmaxed confidences, priors); the tails are then called alone through the
+    kernel-level C ABI, 5 warm-up + 30 calls, each call timed with HIP events on its
+    stream; medians in microseconds."""
+    import statistics
+    import numpy as np
+    import torch
+    from minicaffe import kernels as K
+    P = ctypes.c_void_p
+    stream = torch.cuda.current_stream().cuda_stream
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()  # noqa: E731
+    out = {}
+
+    # configuration 4: 1x1024x38x63 -> 21 546 anchors -> best 6000 -> NMS 0.7 -> 300 rois
+    spec, inputs = zoo.rpn_spec(seed=0)
+    net = mc.Net.from_buffers(craft.to_prototxt(spec, "rpn"))
+    craft.load_weights(net, spec)
+    for m in ("rpn_cls_prob_reshape", "rpn_bbox_pred"):
+        net.mark_output(m)
+    net.forward(**inputs)
+    prob = net.get_blob("rpn_cls_prob_reshape").data.copy()
+    bbox = net.get_blob("rpn_bbox_pred").data.copy()
+    del net
+    pp = spec[-1]["proposal_param"]
+    pre, post, thr = pp.get("pre_nms_topn", 6000), pp.get("post_nms_topn", 300), pp.get("nms_thresh", 0.7)
+    A, H, W = bbox.shape[1] // 4, bbox.shape[2], bbox.shape[3]
+    import oracle
+    sd, bd, idv, ad = dev(prob), dev(bbox), dev(inputs["im_info"]), dev(oracle.generate_anchors())
+    sz = ctypes.c_size_t()
+    K.check_mc(LIB.mcProposalWorkspaceSize(A * H * W, pre, post, ctypes.byref(sz)))
+    ws = torch.empty(sz.value, dtype=torch.uint8, device="cuda")
+    rois = torch.empty((post, 5), device="cuda")
+    cnt = torch.zeros(2, dtype=torch.int32, device="cuda")
+
+    def proposal():
+        K.check_mc(LIB.mcProposal(P(sd.data_ptr()), P(bd.data_ptr()), P(idv.data_ptr()), P(ad.data_ptr()), A, H, W, 16,
+                                  ctypes.c_float(16), pre, post, ctypes.c_float(thr), P(ws.data_ptr()), sz.value,
+                                  P(rois.data_ptr()), None, P(cnt.data_ptr()), P(cnt.data_ptr() + 4), P(stream)))
+
+    for _ in range(5):
+        proposal()
+    torch.cuda.synchronize()
+    stages = []
+    for _ in range(30):
+        LIB.mcProposalTimingEnable(1)
+        proposal()
+        LIB.mcProposalTimingEnable(0)
+        ms, calls = (ctypes.c_double * 4)(), ctypes.c_long()
+        K.check_mc(LIB.mcProposalTimingCollect(ms, ctypes.byref(calls)))
+        stages.append([1e3 * v for v in ms])
+    med = [statistics.median(s[k] for s in stages) for k in range(4)]
+    out["nms_us"] = round(med[2], 1)
+    out["proposal_us"] = round(statistics.median(sum(s) for s in stages), 1)
+    out["proposal_detail"] = {
+        "workload": "config 4: %d anchors -> best %d -> NMS %.1f -> <= %d rois (kept %d, equal scores in the "
+                    "best %d: %s)" % (A * H * W, pre, thr, post, int(cnt[0]), pre, "yes" if int(cnt[1]) else "no"),
+        "decode_sort_us": round(med[0], 1), "tie_order_replay_us": round(med[1], 1),
+        "nms_mask_scan_us": round(med[2], 1), "gather_us": round(med[3], 1),
+        "method": "mcProposal alone on the net's own scores, HIP events between stages, median of 30 calls"}
+
+    # configuration 3: SSD300 b8, 8732 priors x 21 classes, top_k 400, NMS 0.45, keep 200
+    spec, inputs = zoo.ssd300_spec(batch=8, seed=0)
+    net = mc.Net.from_buffers(craft.to_prototxt(spec, "ssd"))
+    craft.load_weights(net, spec)
+    for m in ("mbox_loc", "mbox_conf_flatten", "mbox_priorbox"):
+        net.mark_output(m)
+    net.forward(**inputs)
+    loc, conf, prior = (dev(net.get_blob(m).data.copy()) for m in ("mbox_loc", "mbox_conf_flatten", "mbox_priorbox"))
+    del net
+    dp = spec[-1]["detection_output_param"]
+    num, Pn, C = loc.shape[0], prior.shape[2] // 4, dp["num_classes"]
+    nmsp = dp["nms_param"]
+    code = {"CORNER": 1, "CENTER_SIZE": 2, "CORNER_SIZE": 3}[str(dp.get("code_type", "CORNER"))]
+    K.check_mc(LIB.mcDetectionOutputWorkspaceSize(num, Pn, C, 1, nmsp["top_k"], ctypes.byref(sz)))
+    max_rows = LIB.mcDetectionOutputMaxRows(num, Pn, C, nmsp["top_k"], dp["keep_top_k"])
+    ws = torch.empty(sz.value, dtype=torch.uint8, device="cuda")
+    rows = torch.empty((max_rows, 7), device="cuda")
+
+    def detect():
+        K.check_mc(LIB.mcDetectionOutput(
+            P(loc.data_ptr()), P(conf.data_ptr()), P(prior.data_ptr()), num, Pn, C, 1, dp.get("background_label_id", 0),
+            code, 0, dp["keep_top_k"], ctypes.c_float(dp.get("confidence_threshold", -3.4028234663852886e38)),
+            ctypes.c_float(nmsp["nms_threshold"]), ctypes.c_float(nmsp.get("eta", 1.0)), nmsp["top_k"],
+            P(ws.data_ptr()), sz.value, P(rows.data_ptr()), max_rows, P(cnt.data_ptr()), P(cnt.data_ptr() + 4),
+            P(stream)))
+
+    for _ in range(5):
+        detect()
+    torch.cuda.synchronize()
+    spans = []
+    for _ in range(30):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        detect()
+        e1.record()
+        spans.append((e0, e1))
+    torch.cuda.synchronize()
+    out["detection_output_us"] = round(1e3 * statistics.median(a.elapsed_time(b) for a, b in spans), 1)
+    out["detection_output_detail"] = {
+        "workload": "config 3: %d images x %d priors x %d classes, top_k %d, NMS %.2f, keep %d (rows %d)"
+                    % (num, Pn, C, nmsp["top_k"], nmsp["nms_threshold"], dp["keep_top_k"], int(cnt[0])),
+        "method": "mcDetectionOutput alone on the net's own tail inputs, HIP events on the launch stream, "
+                  "median of 30 calls"}
+    return out
 
 
 def configs_report(path, mc, craft, zoo, LIB):

@@ -271,6 +271,16 @@ int mcProposal(const float* scores, const float* bbox, const float* im_info, con
                int post_nms_topn, float nms_thresh, void* workspace, size_t workspace_bytes,
                float* rois, float* roi_scores, int* num_rois, int* tie_flag, void* stream);
 
+/* Measurement hook (no counterpart in the reference): while enabled on the calling
+ * thread every mcProposal / mcProposalStatic call records HIP events between its
+ * stages on the launch stream.  mcProposalTimingCollect waits for them, adds up over
+ * the calls since the last collect stage_ms[0] decode + radix sort, [1] replay of the
+ * reference's order of equal scores + gather of the best pre_nms_topn boxes,
+ * [2] NMS proper (overlap bit matrix + greedy scan), [3] roi gather and flag copy,
+ * returns the number of calls and clears the list. */
+int mcProposalTimingEnable(int on);
+int mcProposalTimingCollect(double* stage_ms, long* calls);
+
 /* mcProposal for callers that cannot allocate device memory or hand over a workspace
  * (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc).  It
  * has no counterpart in the reference.  Same arguments, results and kernels as

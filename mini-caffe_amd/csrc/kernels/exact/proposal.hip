@@ -9,6 +9,7 @@
 // This file is compiled with -ffp-contract=off: the kept-box indices must equal
 // the CPU path's bit for bit, so every a*b+c here is two roundings like there.
 #include <mutex>
+#include <vector>
 
 #include "../mc_common.h"
 #include "block_sort.h"
@@ -790,6 +791,14 @@ namespace {
 constexpr size_t kStaticScratchBytes = size_t(8) << 20;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
+// Optional stage timing (measurement hook): while enabled on the calling thread every
+// call records five HIP events on its stream.
+struct ProposalTimes {
+  hipEvent_t ev[5];
+};
+thread_local bool g_prop_timing = false;
+thread_local std::vector<ProposalTimes> g_prop_timed;
+
 constexpr int kMaxDevices = 64;
 void* g_scratch_addr[kMaxDevices];
 std::mutex g_scratch_mutex;
@@ -842,6 +851,14 @@ int run_proposal(const float* scores, const float* bbox, const float* im_info, c
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int nb = ceil_div(pre, 64);
 
+  ProposalTimes times;
+  const bool timing = g_prop_timing;
+  auto mark = [&](int k) {
+    if (!timing) return hipSuccess;
+    hipError_t e = hipEventCreate(&times.ev[k]);
+    return e != hipSuccess ? e : hipEventRecord(times.ev[k], st);
+  };
+  MC_HIP(mark(0));
   zero_ints_kernel<<<1, 64, 0, st>>>(flags, 4);
   MC_LAUNCH_CHECK();
   // foreground scores are the second half of the score blob (proposal_layer.cpp:295)
@@ -854,6 +871,7 @@ int run_proposal(const float* scores, const float* bbox, const float* im_info, c
   else
     proposal_sort_kernel<<<1, kSortThreads, 0, st>>>(k0, v0, k1, v1, n, pre, flags);
   MC_LAUNCH_CHECK();
+  MC_HIP(mark(1));
   // no-op unless equal scores reach into the first `pre` places
   quicksort_replay_kernel<<<1, kQsThreads, 0, st>>>(
       flags, korig, n, pre, k1, v1, reinterpret_cast<uint32_t*>(ws + L.kb), ints(L.vb),
@@ -864,17 +882,21 @@ int run_proposal(const float* scores, const float* bbox, const float* im_info, c
   proposal_order_gather_kernel<<<ceil_div(pre, 256), 256, 0, st>>>(v0, pre, boxes, sc, sboxes,
                                                                    sscores);
   MC_LAUNCH_CHECK();
+  MC_HIP(mark(2));
   nms_mask_kernel<<<dim3(nb, nb), 64, 0, st>>>(sboxes, pre, nms_thresh, nb, mask);
   MC_LAUNCH_CHECK();
   nms_scan_kernel<<<1, kScanThreads, sizeof(unsigned long long) * nb, st>>>(
       mask, pre, nb, post_nms_topn, kept, num_rois);
   MC_LAUNCH_CHECK();
+  MC_HIP(mark(3));
   proposal_gather_kernel<<<ceil_div(post_nms_topn, 256), 256, 0, st>>>(sboxes, sscores, kept,
                                                                        num_rois, rois, roi_scores);
   MC_LAUNCH_CHECK();
   if (tie_flag) {
     MC_HIP(hipMemcpyAsync(tie_flag, flags, sizeof(int), hipMemcpyDeviceToDevice, st));
   }
+  MC_HIP(mark(4));
+  if (timing) g_prop_timed.push_back(times);
   return 0;
 }
 
@@ -899,6 +921,29 @@ int mcProposal(const float* scores, const float* bbox, const float* im_info, con
   return run_proposal(scores, bbox, im_info, anchors, A, H, W, feat_stride, min_size, pre_nms_topn,
                       post_nms_topn, nms_thresh, workspace, workspace_bytes, rois, roi_scores,
                       num_rois, tie_flag, stream);
+}
+
+int mcProposalTimingEnable(int on) {
+  g_prop_timing = on != 0;
+  return 0;
+}
+
+int mcProposalTimingCollect(double* stage_ms, long* calls) {
+  double sum[4] = {0., 0., 0., 0.};
+  for (auto& t : g_prop_timed) {
+    MC_HIP(hipEventSynchronize(t.ev[4]));
+    for (int k = 0; k < 4; ++k) {
+      float e = 0.f;
+      MC_HIP(hipEventElapsedTime(&e, t.ev[k], t.ev[k + 1]));
+      sum[k] += e;
+    }
+    for (int k = 0; k < 5; ++k) (void)hipEventDestroy(t.ev[k]);
+  }
+  if (stage_ms)
+    for (int k = 0; k < 4; ++k) stage_ms[k] = sum[k];
+  if (calls) *calls = static_cast<long>(g_prop_timed.size());
+  g_prop_timed.clear();
+  return 0;
 }
 
 int mcProposalStatic(const float* scores, const float* bbox, const float* im_info,
