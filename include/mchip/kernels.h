@@ -261,11 +261,13 @@ int mcProposalWorkspaceSize(int num_proposals, int pre_nms_topn, int post_nms_to
  *   rois     [post_nms_topn, 5] rows (0, x1, y1, x2, y2); roi_scores optional
  *   num_rois number of valid rows (device int; the caller copies it back to
  *            shape the top blob, as Forward_cpu's final Reshape does, :313-320)
- *   tie_flag optional device int: set to 1 when two of the pre_nms_topn+1 best
- *            scores are equal.  Tie-free inputs are ordered by one radix sort; with
+ *   tie_flag optional device int: 0 when the pre_nms_topn+1 best scores are all
+ *            distinct, else 1 or 3.  Tie-free inputs are ordered by one radix sort; with
  *            ties the order is whatever the reference's quicksort SortBBox (:88-111)
- *            leaves, so that quicksort is then replayed on the device, level by
- *            level, to give the same row order. */
+ *            leaves, so that quicksort is then replayed on the device to give the
+ *            same row order: 3 = by the kernel for inputs with few equal scores (it
+ *            follows only the partitions that hold equal scores), 1 = by the general
+ *            kernel (every partition, level by level). */
 int mcProposal(const float* scores, const float* bbox, const float* im_info, const float* anchors,
                int A, int H, int W, int feat_stride, float min_size, int pre_nms_topn,
                int post_nms_topn, float nms_thresh, void* workspace, size_t workspace_bytes,
@@ -279,6 +281,10 @@ int mcProposal(const float* scores, const float* bbox, const float* im_info, con
  * [2] NMS proper (overlap bit matrix + greedy scan), [3] roi gather and flag copy,
  * returns the number of calls and clears the list. */
 int mcProposalTimingEnable(int on);
+/* Test knob (process-wide): 1 = replay the order of equal scores with the general
+ * level-by-level kernel on every input, also where the kernel for inputs with few
+ * equal scores would take over; 0 restores the automatic choice.  Results are the same. */
+int mcProposalForceGeneralReplay(int on);
 int mcProposalTimingCollect(double* stage_ms, long* calls);
 
 /* mcProposal for callers that cannot allocate device memory or hand over a workspace

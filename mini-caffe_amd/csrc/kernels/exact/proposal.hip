@@ -148,7 +148,7 @@ __global__ __launch_bounds__(kQsThreads) void quicksort_replay_kernel(
     unsigned long long* __restrict__ pref, int* __restrict__ posS, int* __restrict__ posB,
     int* __restrict__ mS, int* __restrict__ mB, int* __restrict__ hole, int* __restrict__ dest,
     int* __restrict__ nseg, unsigned char* __restrict__ cls, int* __restrict__ order_out) {
-  if (*flag == 0) return;
+  if (flag[0] == 0 || flag[1] != 0) return;  // no ties, or tie_replay_fast_kernel did the job
   __shared__ unsigned long long wave_tot[kQsThreads / 64];
   __shared__ int range_lo, range_hi, next_lo, next_hi;
   const int tid = threadIdx.x;
@@ -547,6 +547,417 @@ __global__ __launch_bounds__(kQsThreads) void quicksort_replay_kernel(
   }
 }
 
+// ---- the same replay for inputs with few equal scores ----------------------------
+//
+// When only a handful of scores are equal (real score maps: a few dozen pairs among
+// 20 000), almost every partition of the recursion holds distinct scores only, and for
+// such a partition the quicksort's result is simply the sorted order the radix sort has
+// already produced.  This kernel therefore follows the recursion only through the
+// partitions that still hold (or border on) a pair of equal scores, one partition at a
+// time instead of every place of the array on every level:
+//   * keys are replaced by their dense rank in sorted order (equal scores, equal rank),
+//     so a place is 32 bits, (rank << 16 | original index), and the whole array lives in
+//     LDS together with one 16-bit rank -> place table;
+//   * sorted places [a, b] are "clean" when no pair of equal neighbours among the sorted
+//     keys touches them (one subtraction on a prefix count); a clean child is closed at
+//     once, its places keep the radix order;
+//   * a partition longer than kFastWaveSeg is done by the whole workgroup, the others by
+//     one wavefront each, sixteen at a time.
+// A partition about pivot K = a[lo] (proposal_layer.cpp:88-111) as rank arithmetic: the
+// i-th smaller score from the left (place L_i) and the i-th larger score from the right
+// (R_i) change places through the moving hole while L_i < R_i:
+//     a[lo] <- a[R_1],  a[R_i] <- a[L_i],  a[L_i] <- a[R_(i+1)],  pivot -> last hole;
+// scores equal to the pivot's never move.  Counts come from wavefront ballots.
+// Runs when the radix sort flagged equal scores among the first num_top + 1 and the
+// input is small enough; it then sets flag[1] so that quicksort_replay_kernel, which
+// handles everything else, returns at once.
+constexpr int kFastThreads = 1024;
+constexpr int kFastWaves = kFastThreads / 64;
+constexpr int kFastMaxN = 22528;          // places held in LDS (6 bytes each)
+constexpr int kFastMaxPairs = 500;        // equal neighbour pairs among the first num_top + 1
+constexpr int kFastMaxSegs = 2 * kFastMaxPairs + 8;
+constexpr int kFastWaveSeg = 512;         // longest partition one wavefront takes
+constexpr int kFastWaveChunks = kFastWaveSeg / 64;
+constexpr int kFastChunks = kFastMaxN / 64 + 2;
+constexpr int kFastChunksPerWave = (kFastChunks + kFastWaves - 1) / kFastWaves;
+constexpr int kFastRegChunks = 8;         // chunks per wavefront whose moved places wait in registers
+
+struct FastLds {
+  uint32_t kv[kFastMaxN];                 // (dense rank << 16) | original index, by place
+  unsigned short tab[kFastMaxN + 2];      // rank -> place: smaller scores up from lo + 1,
+                                          // larger scores down from hi
+  unsigned long long ms[kFastChunks], mb[kFastChunks];  // ballots of the workgroup path
+  uint32_t cpre[kFastChunks + 1];         // exclusive chunk prefix (smaller low, larger high half)
+  uint32_t seg[2][kFastMaxSegs];          // open partitions (lo << 16 | hi), this level / next
+  unsigned short pairs[kFastMaxPairs + 2];  // sorted places j with key[j] == key[j+1], j < num_top
+  int n_pairs;
+  int n_next, moved_s, moved_b, tot, failed;
+};
+
+// Per-place step shared by both paths.  (ms, mb): ballots of the place's chunk, (ps, pb):
+// smaller / larger scores in the chunks before it.  Returns true when the place moves.
+struct FastSeg {
+  int lo, hi, nS, nB;
+};
+__device__ __forceinline__ void fast_ranks(const FastSeg& g, unsigned long long ms,
+                                           unsigned long long mb, int ps, int pb, int lane,
+                                           bool* is_s, bool* is_b, int* rank) {
+  const unsigned long long bit = 1ull << lane;
+  *is_s = (ms & bit) != 0;
+  *is_b = (mb & bit) != 0;
+  const unsigned long long lt = bit - 1ull, le = (bit << 1) - 1ull;
+  // smaller: rank from the left; larger: rank from the right (both 1-based)
+  *rank = *is_s ? ps + __popcll(ms & lt) + 1 : g.nB - (pb + __popcll(mb & le)) + 1;
+}
+
+__device__ __forceinline__ bool fast_move(const FastSeg& g, const unsigned short* tab, int q,
+                                          bool is_s, bool is_b, int rank, int* dest) {
+  if (is_s) {
+    if (rank > g.nB) return false;
+    const int r = tab[g.hi + 1 - rank];  // R_rank
+    *dest = r;
+    return q < r;
+  }
+  if (is_b) {
+    if (rank == 1) {
+      *dest = g.lo;
+      return true;
+    }
+    if (rank - 1 > g.nS) return false;
+    const int l = tab[g.lo + rank - 1];  // L_(rank-1)
+    *dest = l;
+    return q > l;
+  }
+  return false;
+}
+
+// True when a pair of equal neighbours (j, j+1) of the sorted keys, j < num_top, touches
+// the sorted places [a, b]: some j in [a - 1, b].  Binary search in the sorted pair list.
+__device__ __forceinline__ bool fast_touched(const FastLds* s, int a, int b) {
+  int lo = 0, hi = s->n_pairs;  // first pair >= a - 1
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (static_cast<int>(s->pairs[mid]) < a - 1) lo = mid + 1;
+    else hi = mid;
+  }
+  return lo < s->n_pairs && static_cast<int>(s->pairs[lo]) <= b;
+}
+
+// After the moves of a partition: place the pivot, close or queue the two children.
+// Called by one thread.
+__device__ __forceinline__ void fast_finish(FastLds* s, const FastSeg& g, uint32_t pivot, int u,
+                                            int t, int num_top, int* __restrict__ order_out,
+                                            int next) {
+  const int h = t == 0 ? g.lo : (t > u ? s->tab[g.hi + 1 - t] : s->tab[g.lo + u]);
+  if (h < g.lo || h > g.hi || t > g.nB || u > g.nS || (t != u && t != u + 1)) {
+    s->failed = 1;  // cannot happen; if it does the general kernel redoes the job
+    return;
+  }
+  s->kv[h] = pivot;
+  if (h < num_top) order_out[h] = static_cast<int>(pivot & 0xffffu);
+#pragma unroll
+  for (int side = 0; side < 2; ++side) {
+    const int a = side == 0 ? g.lo : h + 1, b = side == 0 ? h - 1 : g.hi;
+    if (a > b) continue;
+    if (side == 1 && a >= num_top) continue;  // the reference does not sort past num_top
+    if (a == b) {
+      if (a < num_top) order_out[a] = static_cast<int>(s->kv[a] & 0xffffu);
+      continue;
+    }
+    if (fast_touched(s, a, b)) {
+      const int slot = atomicAdd(&s->n_next, 1);
+      if (slot < kFastMaxSegs)
+        s->seg[next][slot] = (static_cast<uint32_t>(a) << 16) | static_cast<uint32_t>(b);
+      else
+        s->failed = 1;
+    }
+  }
+}
+
+__global__ __launch_bounds__(kFastThreads) void tie_replay_fast_kernel(
+    int* __restrict__ flag, const uint32_t* __restrict__ sorted_keys, int n, int num_top,
+    uint2* __restrict__ stage, int* __restrict__ order) {
+  if (flag[0] == 0 || n > kFastMaxN || n < 2) return;
+  __shared__ FastLds s;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  // Equal neighbour pairs of the sorted keys, 64 places per ballot: all of them give the
+  // dense ranks, those among the first num_top places are the ones the order depends on.
+  {
+    const int C = (n + 63) >> 6;
+    for (int c = wave; c < C; c += kFastWaves) {
+      const int i = (c << 6) + lane;
+      const bool eq = i + 1 < n && sorted_keys[i] == sorted_keys[i + 1];
+      const unsigned long long all = __ballot(eq), top = __ballot(eq && i < num_top);
+      if (lane == 0) {
+        s.ms[c] = all;
+        s.mb[c] = top;
+      }
+    }
+    __syncthreads();
+    if (wave == 0) {
+      uint32_t carry = 0;
+      for (int base = 0; base < C; base += 64) {
+        const int c = base + lane;
+        const uint32_t cnt = c < C ? static_cast<uint32_t>(__popcll(s.ms[c])) |
+                                         (static_cast<uint32_t>(__popcll(s.mb[c])) << 16)
+                                   : 0u;
+        uint32_t inc = cnt;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+          const uint32_t up = __shfl_up(inc, o, 64);
+          if (lane >= o) inc += up;
+        }
+        if (c < C) s.cpre[c] = carry + inc - cnt;
+        carry += __shfl(inc, 63, 64);
+      }
+      if (lane == 0) {
+        s.n_pairs = static_cast<int>(carry >> 16);
+        s.seg[0][0] = static_cast<uint32_t>(n - 1);  // lo 0, hi n - 1
+        s.n_next = 0;
+        s.failed = 0;
+      }
+    }
+    __syncthreads();
+    if (s.n_pairs > kFastMaxPairs) return;  // uniform: the general kernel runs
+    for (int c = wave; c < C; c += kFastWaves) {
+      const int i = (c << 6) + lane;
+      if (i >= n) continue;
+      const unsigned long long lt = (1ull << lane) - 1ull;
+      const int before_all = static_cast<int>(s.cpre[c] & 0xffffu) + __popcll(s.ms[c] & lt);
+      const int v = order[i];
+      s.kv[v] = (static_cast<uint32_t>(i - before_all) << 16) | static_cast<uint32_t>(v);
+      if ((s.mb[c] >> lane) & 1ull)
+        s.pairs[static_cast<int>(s.cpre[c] >> 16) + __popcll(s.mb[c] & lt)] = static_cast<unsigned short>(i);
+    }
+  }
+  __syncthreads();
+
+  // Every level shortens every open partition by at least its pivot: at most n levels.
+  int n_cur = 1, cur = 0, levels_left = n + 1;
+  while (n_cur > 0 && levels_left-- > 0) {
+    const int next = cur ^ 1;
+    // ---- long partitions: the whole workgroup, one after the other ----
+    for (int si = 0; si < n_cur; ++si) {
+      const uint32_t sg = s.seg[cur][si];
+      FastSeg g;
+      g.lo = static_cast<int>(sg >> 16);
+      g.hi = static_cast<int>(sg & 0xffffu);
+      if (g.hi - g.lo + 1 <= kFastWaveSeg) continue;  // uniform
+      const uint32_t pivot = s.kv[g.lo];
+      const uint32_t K = pivot >> 16;
+      const int places = g.hi - g.lo;  // without the pivot
+      const int C = (places + 63) >> 6;
+      if (tid == 0) {
+        s.moved_s = 0;
+        s.moved_b = 0;
+      }
+      for (int c = wave; c < C; c += kFastWaves) {
+        const int q = g.lo + 1 + (c << 6) + lane;
+        const uint32_t d = q <= g.hi ? s.kv[q] >> 16 : K;
+        const unsigned long long ms = __ballot(d > K), mb = __ballot(d < K);  // larger rank = smaller score
+        if (lane == 0) {
+          s.ms[c] = ms;
+          s.mb[c] = mb;
+        }
+      }
+      __syncthreads();
+      if (wave == 0) {
+        uint32_t carry = 0;
+        for (int base = 0; base < C; base += 64) {
+          const int c = base + lane;
+          const uint32_t cnt = c < C ? static_cast<uint32_t>(__popcll(s.ms[c])) |
+                                           (static_cast<uint32_t>(__popcll(s.mb[c])) << 16)
+                                     : 0u;
+          uint32_t inc = cnt;
+#pragma unroll
+          for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t up = __shfl_up(inc, o, 64);
+            if (lane >= o) inc += up;
+          }
+          if (c < C) s.cpre[c] = carry + inc - cnt;
+          carry += __shfl(inc, 63, 64);
+        }
+        if (lane == 0) s.tot = static_cast<int>(carry);
+      }
+      __syncthreads();
+      g.nS = s.tot & 0xffff;
+      g.nB = static_cast<int>(static_cast<uint32_t>(s.tot) >> 16);
+      if (g.nS == 0 && g.nB == 0) {
+        // every score equals the pivot's: nothing ever moves in here
+        for (int q = g.lo + tid; q <= g.hi && q < num_top; q += kFastThreads)
+          order[q] = static_cast<int>(s.kv[q] & 0xffffu);
+        __syncthreads();
+        continue;
+      }
+      for (int c = wave; c < C; c += kFastWaves) {
+        const int q = g.lo + 1 + (c << 6) + lane;
+        bool is_s, is_b;
+        int rank;
+        fast_ranks(g, s.ms[c], s.mb[c], s.cpre[c] & 0xffff, s.cpre[c] >> 16, lane, &is_s, &is_b, &rank);
+        if (is_s) s.tab[g.lo + rank] = static_cast<unsigned short>(q);
+        if (is_b) s.tab[g.hi + 1 - rank] = static_cast<unsigned short>(q);
+      }
+      __syncthreads();
+      // A moved place is read by its own lane and written to its destination after
+      // every read of the partition is done.  Up to kFastRegChunks chunks per wavefront
+      // it waits in registers, in longer partitions (the first few levels) in `stage`.
+      int u = 0, t = 0;
+      if (C <= kFastRegChunks * kFastWaves) {
+        uint32_t keep_kv[kFastRegChunks];
+        int keep_to[kFastRegChunks];
+#pragma unroll
+        for (int k = 0; k < kFastRegChunks; ++k) {
+          const int c = wave + k * kFastWaves;
+          keep_to[k] = -1;
+          if (c < C) {
+            const int q = g.lo + 1 + (c << 6) + lane;
+            bool is_s, is_b;
+            int rank, dest = 0;
+            fast_ranks(g, s.ms[c], s.mb[c], s.cpre[c] & 0xffff, s.cpre[c] >> 16, lane, &is_s, &is_b, &rank);
+            const bool mv = fast_move(g, s.tab, q, is_s, is_b, rank, &dest);
+            if (mv) {
+              keep_to[k] = dest;
+              keep_kv[k] = s.kv[q];
+            }
+            u += __popcll(__ballot(mv && is_s));
+            t += __popcll(__ballot(mv && is_b));
+          }
+        }
+        if (lane == 0) {
+          if (u) atomicAdd(&s.moved_s, u);
+          if (t) atomicAdd(&s.moved_b, t);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < kFastRegChunks; ++k)
+          if (keep_to[k] >= 0) s.kv[keep_to[k]] = keep_kv[k];
+      } else {
+        for (int c = wave; c < C; c += kFastWaves) {
+          const int q = g.lo + 1 + (c << 6) + lane;
+          bool is_s, is_b;
+          int rank, dest = 0;
+          fast_ranks(g, s.ms[c], s.mb[c], s.cpre[c] & 0xffff, s.cpre[c] >> 16, lane, &is_s, &is_b, &rank);
+          const bool mv = fast_move(g, s.tab, q, is_s, is_b, rank, &dest);
+          if (q <= g.hi) stage[q] = make_uint2(mv ? s.kv[q] : 0u, mv ? static_cast<uint32_t>(dest) : 0xffffffffu);
+          u += __popcll(__ballot(mv && is_s));
+          t += __popcll(__ballot(mv && is_b));
+        }
+        if (lane == 0) {
+          if (u) atomicAdd(&s.moved_s, u);
+          if (t) atomicAdd(&s.moved_b, t);
+        }
+        __threadfence_block();
+        __syncthreads();
+        // four loads in flight per lane
+        for (int c0 = wave; c0 < C; c0 += 4 * kFastWaves) {
+          uint2 e[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int q = g.lo + 1 + ((c0 + j * kFastWaves) << 6) + lane;
+            e[j] = q <= g.hi ? stage[q] : make_uint2(0u, 0xffffffffu);
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (e[j].y != 0xffffffffu) s.kv[e[j].y] = e[j].x;
+        }
+      }
+      __syncthreads();
+      if (tid == 0) fast_finish(&s, g, pivot, s.moved_s, s.moved_b, num_top, order, next);
+      __syncthreads();
+    }
+    // ---- short partitions: one wavefront each ----
+    for (int si = wave; si < n_cur; si += kFastWaves) {
+      const uint32_t sg = s.seg[cur][si];
+      FastSeg g;
+      g.lo = static_cast<int>(sg >> 16);
+      g.hi = static_cast<int>(sg & 0xffffu);
+      if (g.hi - g.lo + 1 > kFastWaveSeg) continue;
+      const uint32_t pivot = s.kv[g.lo];
+      const uint32_t K = pivot >> 16;
+      const int places = g.hi - g.lo;
+      const int C = (places + 63) >> 6;  // <= kFastWaveChunks
+      // this wavefront's ballots go to its own sixteen slots of the ballot arrays (the
+      // workgroup path above is finished with them)
+      unsigned long long* wms = s.ms + wave * kFastWaveChunks;
+      unsigned long long* wmb = s.mb + wave * kFastWaveChunks;
+      g.nS = 0;
+      g.nB = 0;
+      for (int c = 0; c < C; ++c) {
+        const int q = g.lo + 1 + (c << 6) + lane;
+        const uint32_t d = q <= g.hi ? s.kv[q] >> 16 : K;
+        const unsigned long long ms = __ballot(d > K), mb = __ballot(d < K);
+        if (lane == 0) {
+          wms[c] = ms;
+          wmb[c] = mb;
+        }
+        g.nS += __popcll(ms);
+        g.nB += __popcll(mb);
+      }
+      if (g.nS == 0 && g.nB == 0) {
+        for (int q = g.lo + lane; q <= g.hi && q < num_top; q += 64)
+          order[q] = static_cast<int>(s.kv[q] & 0xffffu);
+        continue;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      int ps = 0, pb = 0;
+      for (int c = 0; c < C; ++c) {
+        const int q = g.lo + 1 + (c << 6) + lane;
+        const unsigned long long ms = wms[c], mb = wmb[c];
+        bool is_s, is_b;
+        int rank;
+        fast_ranks(g, ms, mb, ps, pb, lane, &is_s, &is_b, &rank);
+        if (is_s) s.tab[g.lo + rank] = static_cast<unsigned short>(q);
+        if (is_b) s.tab[g.hi + 1 - rank] = static_cast<unsigned short>(q);
+        ps += __popcll(ms);
+        pb += __popcll(mb);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      uint32_t keep_kv[kFastWaveChunks];
+      int keep_to[kFastWaveChunks];
+      int u = 0, t = 0;
+      ps = 0;
+      pb = 0;
+#pragma unroll
+      for (int c = 0; c < kFastWaveChunks; ++c) {
+        keep_to[c] = -1;
+        if (c < C) {
+          const int q = g.lo + 1 + (c << 6) + lane;
+          const unsigned long long ms = wms[c], mb = wmb[c];
+          bool is_s, is_b;
+          int rank, dest = 0;
+          fast_ranks(g, ms, mb, ps, pb, lane, &is_s, &is_b, &rank);
+          const bool mv = fast_move(g, s.tab, q, is_s, is_b, rank, &dest);
+          if (mv) {
+            keep_to[c] = dest;
+            keep_kv[c] = s.kv[q];
+          }
+          u += __popcll(__ballot(mv && is_s));
+          t += __popcll(__ballot(mv && is_b));
+          ps += __popcll(ms);
+          pb += __popcll(mb);
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+#pragma unroll
+      for (int c = 0; c < kFastWaveChunks; ++c)
+        if (keep_to[c] >= 0) s.kv[keep_to[c]] = keep_kv[c];
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      if (lane == 0) fast_finish(&s, g, pivot, u, t, num_top, order, next);
+    }
+    __syncthreads();
+    n_cur = s.failed ? 0 : min(s.n_next, kFastMaxSegs);
+    cur = next;
+    __syncthreads();
+    if (tid == 0) s.n_next = 0;
+    __syncthreads();
+  }
+  if (tid == 0 && n_cur == 0 && !s.failed) {
+    flag[1] = 1;
+    flag[0] = 3;  // reported to the caller: equal scores, order replayed by this kernel
+  }
+}
+
 // mask[i][cb] bit j: box cb*64+j (> i) overlaps box i by more than thr, with
 // the +1 pixel extents of NonMaximumSuppressionCPU (proposal_layer.cpp:150-185).
 __global__ __launch_bounds__(64) void nms_mask_kernel(const float4* __restrict__ boxes, int n,
@@ -799,6 +1210,9 @@ struct ProposalTimes {
 thread_local bool g_prop_timing = false;
 thread_local std::vector<ProposalTimes> g_prop_timed;
 
+// Test knob: skip the few-ties replay so that the general one is exercised on every input.
+bool g_force_general_replay = false;
+
 constexpr int kMaxDevices = 64;
 void* g_scratch_addr[kMaxDevices];
 std::mutex g_scratch_mutex;
@@ -872,7 +1286,12 @@ int run_proposal(const float* scores, const float* bbox, const float* im_info, c
     proposal_sort_kernel<<<1, kSortThreads, 0, st>>>(k0, v0, k1, v1, n, pre, flags);
   MC_LAUNCH_CHECK();
   MC_HIP(mark(1));
-  // no-op unless equal scores reach into the first `pre` places
+  // both are no-ops unless equal scores reach into the first `pre` places; the first
+  // takes inputs with few equal scores, the second everything else
+  if (!g_force_general_replay) {
+    tie_replay_fast_kernel<<<1, kFastThreads, 0, st>>>(flags, k0, n, pre, reinterpret_cast<uint2*>(ws + L.pref), v0);
+    MC_LAUNCH_CHECK();
+  }
   quicksort_replay_kernel<<<1, kQsThreads, 0, st>>>(
       flags, korig, n, pre, k1, v1, reinterpret_cast<uint32_t*>(ws + L.kb), ints(L.vb),
       ints(L.seg_lo), ints(L.seg_hi), reinterpret_cast<unsigned long long*>(ws + L.pref),
@@ -921,6 +1340,11 @@ int mcProposal(const float* scores, const float* bbox, const float* im_info, con
   return run_proposal(scores, bbox, im_info, anchors, A, H, W, feat_stride, min_size, pre_nms_topn,
                       post_nms_topn, nms_thresh, workspace, workspace_bytes, rois, roi_scores,
                       num_rois, tie_flag, stream);
+}
+
+int mcProposalForceGeneralReplay(int on) {
+  g_force_general_replay = on != 0;
+  return 0;
 }
 
 int mcProposalTimingEnable(int on) {

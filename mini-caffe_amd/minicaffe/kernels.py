@@ -82,6 +82,7 @@ LIB.mcProposal.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                            c_float, c_int, c_int, c_float, c_void_p, ctypes.c_size_t, c_void_p,
                            c_void_p, c_void_p, c_void_p, c_void_p]
 LIB.mcProposalTimingEnable.argtypes = [c_int]
+LIB.mcProposalForceGeneralReplay.argtypes = [c_int]
 LIB.mcProposalTimingCollect.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(c_long)]
 LIB.mcProposalStatic.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                  c_float, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p,

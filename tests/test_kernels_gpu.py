@@ -663,7 +663,62 @@ def test_proposal_bit_exact(K, hw, pre, post, thr, quant):
     assert np.array_equal(rois, want_rois)
     assert np.array_equal(rs, want_scores)
     if quant:
-        assert ties == 1
+        assert ties & 1
+
+
+@pytest.mark.parametrize("hw,pre,post,thr,pairs,seed", [
+    ((38, 63), 6000, 300, 0.7, 1, 0),        # config 4 size, a single pair of equal scores
+    ((38, 63), 6000, 300, 0.7, 20, 1),       # about as many as the configuration's own scores hold
+    ((38, 63), 6000, 300, 0.7, 120, 2),
+    ((38, 63), 6000, 300, 0.7, 480, 3),      # close to the most the few-ties kernel takes
+    ((38, 63), 6000, 300, 0.7, 520, 4),      # just beyond: the general kernel
+    ((38, 63), 300, 100, 0.7, 200, 5),       # most pairs lie beyond the cut
+    ((20, 20), 6000, 300, 0.7, 60, 6),       # pre_nms_topn > proposals
+    ((5, 4), 100, 300, 0.3, 30, 7),          # partitions of a few places only
+    ((11, 9), 500, 60, 0.5, 8, 8),
+    ((39, 64), 6000, 300, 0.7, 25, 9),       # 22 464 proposals: the largest map the kernel holds
+    ((40, 63), 6000, 300, 0.7, 25, 10),      # 22 680: beyond it
+])
+@pytest.mark.parametrize("general", [False, True])
+def test_proposal_with_few_equal_scores(K, hw, pre, post, thr, pairs, seed, general):
+    """A few equal scores among otherwise distinct ones (what real score maps look like):
+    some pairs, some runs of three to five, some straddling the pre_nms_topn cut.  The kernel
+    that follows only the partitions holding equal scores and the general level-by-level
+    kernel must both leave the reference quicksort's order."""
+    rng = np.random.default_rng(100 + seed)
+    A, (H, W) = 9, hw
+    n = A * H * W
+    fg = (rng.permutation(n).astype(np.float32) / n * 0.9 + 0.05)
+    best = np.argsort(-fg)[:min(pre, n) // 2]
+    for g in range(pairs):
+        size = 2 if g % 5 else int(rng.integers(3, 6))
+        idx = rng.choice(best if g == 0 else n, size, replace=False)   # the first group among the best
+        fg[idx] = fg[idx[0]]
+    if pairs >= 8:                          # equal scores right at the cut
+        order = np.argsort(-fg, kind="stable")
+        cut = min(pre, n) - 1
+        fg[order[cut:cut + 3]] = fg[order[cut]]
+    scores = rng.random((1, 2 * A, H, W)).astype(np.float32)
+    scores[0, A:] = fg.reshape(H, W, A).transpose(2, 0, 1)
+    bbox = (rng.standard_normal((1, 4 * A, H, W)) * 0.3).astype(np.float32)
+    im_info = np.array([H * 16, W * 16, 1.0], np.float32)
+    param = {"pre_nms_topn": pre, "post_nms_topn": post, "nms_thresh": thr}
+    want_rois, want_scores = oracle.proposal(param, scores, bbox, im_info, 2)
+    K.check_mc(K.LIB.mcProposalForceGeneralReplay(int(general)))
+    try:
+        rois, rs, ties = run_proposal(K, scores, bbox, im_info, param)
+    finally:
+        K.check_mc(K.LIB.mcProposalForceGeneralReplay(0))
+    assert np.array_equal(rois, want_rois)
+    assert np.array_equal(rs, want_scores)
+    # which kernel did it: 3 = the few-ties one (at most 22 528 proposals and 500 equal
+    # neighbour pairs among the best pre_nms_topn + 1 sorted scores), 1 = the general one
+    props = oracle.generate_proposals(scores[0, A:], bbox[0], oracle.generate_anchors(), float(im_info[0]),
+                                      float(im_info[1]), 16.0, 16)
+    skey = np.sort(props[:, 4])[::-1]       # too small boxes score 0: more equal scores at the end
+    counted = int((skey[:-1] == skey[1:])[:min(pre, n)].sum())
+    assert counted > 0
+    assert ties == (3 if (not general and n <= 22528 and counted <= 500) else 1)
 
 
 @pytest.mark.parametrize("num,P,C,share,code,keep,thr,nms,eta,topk,sigma", [
