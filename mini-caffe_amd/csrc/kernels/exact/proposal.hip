@@ -577,10 +577,10 @@ constexpr int kFastMaxN = 22528;          // places held in LDS (6 bytes each)
 constexpr int kFastMaxPairs = 500;        // equal neighbour pairs among the first num_top + 1
 constexpr int kFastMaxSegs = 2 * kFastMaxPairs + 8;
 constexpr int kFastWaveSeg = 512;         // longest partition one wavefront takes
-constexpr int kFastWaveChunks = kFastWaveSeg / 64;
 constexpr int kFastChunks = kFastMaxN / 64 + 2;
 constexpr int kFastChunksPerWave = (kFastChunks + kFastWaves - 1) / kFastWaves;
 constexpr int kFastRegChunks = 8;         // chunks per wavefront whose moved places wait in registers
+constexpr int kFastMaxLong = kFastMaxN / kFastWaveSeg + 2;
 
 struct FastLds {
   uint32_t kv[kFastMaxN];                 // (dense rank << 16) | original index, by place
@@ -588,10 +588,13 @@ struct FastLds {
                                           // larger scores down from hi
   unsigned long long ms[kFastChunks], mb[kFastChunks];  // ballots of the workgroup path
   uint32_t cpre[kFastChunks + 1];         // exclusive chunk prefix (smaller low, larger high half)
-  uint32_t seg[2][kFastMaxSegs];          // open partitions (lo << 16 | hi), this level / next
-  unsigned short pairs[kFastMaxPairs + 2];  // sorted places j with key[j] == key[j+1], j < num_top
+  uint32_t seg[2][kFastMaxSegs];          // open short partitions (lo << 16 | hi), this level / next
+  uint32_t seg_long[2][kFastMaxLong];     // open partitions longer than kFastWaveSeg
+  uint32_t wave_cnt[kFastWaves];          // smaller / larger scores in each wavefront's chunks
+  unsigned long long pair_bits[kFastChunks];  // bit j: sorted keys j and j + 1 are equal, j < num_top
+  unsigned short pair_pre[kFastChunks];       // such pairs in the words before
   int n_pairs;
-  int n_next, moved_s, moved_b, tot, failed;
+  int n_seg[2], n_long[2], moved_s, moved_b, failed;
 };
 
 // Per-place step shared by both paths.  (ms, mb): ballots of the place's chunk, (ps, pb):
@@ -631,16 +634,14 @@ __device__ __forceinline__ bool fast_move(const FastSeg& g, const unsigned short
   return false;
 }
 
-// True when a pair of equal neighbours (j, j+1) of the sorted keys, j < num_top, touches
-// the sorted places [a, b]: some j in [a - 1, b].  Binary search in the sorted pair list.
+// Pairs of equal neighbours (j, j + 1) of the sorted keys with j < x (counted for j < num_top).
+__device__ __forceinline__ int fast_pairs_before(const FastLds* s, int x) {
+  const int w = x >> 6;
+  return s->pair_pre[w] + __popcll(s->pair_bits[w] & ((1ull << (x & 63)) - 1ull));
+}
+// True when such a pair touches the sorted places [a, b]: some j in [a - 1, b].
 __device__ __forceinline__ bool fast_touched(const FastLds* s, int a, int b) {
-  int lo = 0, hi = s->n_pairs;  // first pair >= a - 1
-  while (lo < hi) {
-    const int mid = (lo + hi) >> 1;
-    if (static_cast<int>(s->pairs[mid]) < a - 1) lo = mid + 1;
-    else hi = mid;
-  }
-  return lo < s->n_pairs && static_cast<int>(s->pairs[lo]) <= b;
+  return fast_pairs_before(s, b + 1) - fast_pairs_before(s, max(a - 1, 0)) > 0;
 }
 
 // After the moves of a partition: place the pivot, close or queue the two children.
@@ -665,13 +666,48 @@ __device__ __forceinline__ void fast_finish(FastLds* s, const FastSeg& g, uint32
       continue;
     }
     if (fast_touched(s, a, b)) {
-      const int slot = atomicAdd(&s->n_next, 1);
-      if (slot < kFastMaxSegs)
-        s->seg[next][slot] = (static_cast<uint32_t>(a) << 16) | static_cast<uint32_t>(b);
-      else
-        s->failed = 1;
+      const uint32_t entry = (static_cast<uint32_t>(a) << 16) | static_cast<uint32_t>(b);
+      if (b - a + 1 > kFastWaveSeg) {
+        const int slot = atomicAdd(&s->n_long[next], 1);
+        if (slot < kFastMaxLong) s->seg_long[next][slot] = entry;
+        else s->failed = 1;
+      } else {
+        const int slot = atomicAdd(&s->n_seg[next], 1);
+        if (slot < kFastMaxSegs) s->seg[next][slot] = entry;
+        else s->failed = 1;
+      }
     }
   }
+}
+
+// Exclusive prefix over up to kFastChunks packed chunk counts (two 16-bit halves) by one
+// wavefront: every lane adds up a run of consecutive chunks, one shuffle scan joins the
+// runs.  Returns the total in every lane.
+__device__ __forceinline__ uint32_t fast_chunk_scan(FastLds* s, int C, int lane) {
+  constexpr int kRun = (kFastChunks + 63) / 64;
+  uint32_t cnt[kRun], sum = 0;
+#pragma unroll
+  for (int j = 0; j < kRun; ++j) {
+    const int c = lane * kRun + j;
+    cnt[j] = c < C ? static_cast<uint32_t>(__popcll(s->ms[c])) |
+                         (static_cast<uint32_t>(__popcll(s->mb[c])) << 16)
+                   : 0u;
+    sum += cnt[j];
+  }
+  uint32_t inc = sum;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const uint32_t up = __shfl_up(inc, o, 64);
+    if (lane >= o) inc += up;
+  }
+  uint32_t run = inc - sum;
+#pragma unroll
+  for (int j = 0; j < kRun; ++j) {
+    const int c = lane * kRun + j;
+    if (c < C) s->cpre[c] = run;
+    run += cnt[j];
+  }
+  return __shfl(inc, 63, 64);
 }
 
 __global__ __launch_bounds__(kFastThreads) void tie_replay_fast_kernel(
@@ -696,25 +732,16 @@ __global__ __launch_bounds__(kFastThreads) void tie_replay_fast_kernel(
     }
     __syncthreads();
     if (wave == 0) {
-      uint32_t carry = 0;
-      for (int base = 0; base < C; base += 64) {
-        const int c = base + lane;
-        const uint32_t cnt = c < C ? static_cast<uint32_t>(__popcll(s.ms[c])) |
-                                         (static_cast<uint32_t>(__popcll(s.mb[c])) << 16)
-                                   : 0u;
-        uint32_t inc = cnt;
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-          const uint32_t up = __shfl_up(inc, o, 64);
-          if (lane >= o) inc += up;
-        }
-        if (c < C) s.cpre[c] = carry + inc - cnt;
-        carry += __shfl(inc, 63, 64);
-      }
+      const uint32_t carry = fast_chunk_scan(&s, C, lane);
       if (lane == 0) {
         s.n_pairs = static_cast<int>(carry >> 16);
-        s.seg[0][0] = static_cast<uint32_t>(n - 1);  // lo 0, hi n - 1
-        s.n_next = 0;
+        // the whole array, lo 0, hi n - 1, is the first partition
+        const bool is_long = n > kFastWaveSeg;
+        s.seg[0][0] = s.seg_long[0][0] = static_cast<uint32_t>(n - 1);
+        s.n_seg[0] = is_long ? 0 : 1;
+        s.n_long[0] = is_long ? 1 : 0;
+        s.n_seg[1] = 0;
+        s.n_long[1] = 0;
         s.failed = 0;
       }
     }
@@ -727,101 +754,114 @@ __global__ __launch_bounds__(kFastThreads) void tie_replay_fast_kernel(
       const int before_all = static_cast<int>(s.cpre[c] & 0xffffu) + __popcll(s.ms[c] & lt);
       const int v = order[i];
       s.kv[v] = (static_cast<uint32_t>(i - before_all) << 16) | static_cast<uint32_t>(v);
-      if ((s.mb[c] >> lane) & 1ull)
-        s.pairs[static_cast<int>(s.cpre[c] >> 16) + __popcll(s.mb[c] & lt)] = static_cast<unsigned short>(i);
+      if (lane == 0) {
+        s.pair_bits[c] = s.mb[c];
+        s.pair_pre[c] = static_cast<unsigned short>(s.cpre[c] >> 16);
+      }
+    }
+    if (tid == 0) {  // fast_pairs_before(n) reads one word past the last place when n % 64 == 0
+      s.pair_bits[C] = 0;
+      s.pair_pre[C] = static_cast<unsigned short>(s.n_pairs);
     }
   }
   __syncthreads();
 
   // Every level shortens every open partition by at least its pivot: at most n levels.
-  int n_cur = 1, cur = 0, levels_left = n + 1;
-  while (n_cur > 0 && levels_left-- > 0) {
+  int n_cur = s.n_seg[0], n_cur_long = s.n_long[0], cur = 0, levels_left = n + 1;
+  __syncthreads();
+  while (n_cur + n_cur_long > 0 && levels_left-- > 0) {
     const int next = cur ^ 1;
     // ---- long partitions: the whole workgroup, one after the other ----
-    for (int si = 0; si < n_cur; ++si) {
-      const uint32_t sg = s.seg[cur][si];
+    // Every wavefront takes a run of consecutive chunks, so that the counts before a
+    // chunk are the wavefront's running sums on top of the totals of the wavefronts
+    // before it; ballots are taken again in every pass instead of being stored.
+    for (int si = 0; si < n_cur_long; ++si) {
+      const uint32_t sg = s.seg_long[cur][si];
       FastSeg g;
       g.lo = static_cast<int>(sg >> 16);
       g.hi = static_cast<int>(sg & 0xffffu);
-      if (g.hi - g.lo + 1 <= kFastWaveSeg) continue;  // uniform
       const uint32_t pivot = s.kv[g.lo];
       const uint32_t K = pivot >> 16;
       const int places = g.hi - g.lo;  // without the pivot
       const int C = (places + 63) >> 6;
+      const int Cw = (C + kFastWaves - 1) / kFastWaves;
+      const int c_begin = min(wave * Cw, C), c_end = min(c_begin + Cw, C);
       if (tid == 0) {
         s.moved_s = 0;
         s.moved_b = 0;
       }
-      for (int c = wave; c < C; c += kFastWaves) {
-        const int q = g.lo + 1 + (c << 6) + lane;
-        const uint32_t d = q <= g.hi ? s.kv[q] >> 16 : K;
-        const unsigned long long ms = __ballot(d > K), mb = __ballot(d < K);  // larger rank = smaller score
-        if (lane == 0) {
-          s.ms[c] = ms;
-          s.mb[c] = mb;
+      {
+        int cs = 0, cb = 0;
+        for (int c = c_begin; c < c_end; ++c) {
+          const int q = g.lo + 1 + (c << 6) + lane;
+          const uint32_t d = q <= g.hi ? s.kv[q] >> 16 : K;
+          cs += __popcll(__ballot(d > K));  // larger rank = smaller score
+          cb += __popcll(__ballot(d < K));
         }
+        if (lane == 0) s.wave_cnt[wave] = static_cast<uint32_t>(cs) | (static_cast<uint32_t>(cb) << 16);
       }
       __syncthreads();
-      if (wave == 0) {
-        uint32_t carry = 0;
-        for (int base = 0; base < C; base += 64) {
-          const int c = base + lane;
-          const uint32_t cnt = c < C ? static_cast<uint32_t>(__popcll(s.ms[c])) |
-                                           (static_cast<uint32_t>(__popcll(s.mb[c])) << 16)
-                                     : 0u;
-          uint32_t inc = cnt;
+      uint32_t before = 0, total = 0;
 #pragma unroll
-          for (int o = 1; o < 64; o <<= 1) {
-            const uint32_t up = __shfl_up(inc, o, 64);
-            if (lane >= o) inc += up;
-          }
-          if (c < C) s.cpre[c] = carry + inc - cnt;
-          carry += __shfl(inc, 63, 64);
-        }
-        if (lane == 0) s.tot = static_cast<int>(carry);
+      for (int w = 0; w < kFastWaves; ++w) {
+        const uint32_t v = s.wave_cnt[w];
+        before += w < wave ? v : 0u;
+        total += v;
       }
-      __syncthreads();
-      g.nS = s.tot & 0xffff;
-      g.nB = static_cast<int>(static_cast<uint32_t>(s.tot) >> 16);
+      g.nS = static_cast<int>(total & 0xffffu);
+      g.nB = static_cast<int>(total >> 16);
       if (g.nS == 0 && g.nB == 0) {
         // every score equals the pivot's: nothing ever moves in here
         for (int q = g.lo + tid; q <= g.hi && q < num_top; q += kFastThreads)
           order[q] = static_cast<int>(s.kv[q] & 0xffffu);
-        __syncthreads();
+        __syncthreads();  // wave_cnt is reused by the next partition
         continue;
       }
-      for (int c = wave; c < C; c += kFastWaves) {
-        const int q = g.lo + 1 + (c << 6) + lane;
-        bool is_s, is_b;
-        int rank;
-        fast_ranks(g, s.ms[c], s.mb[c], s.cpre[c] & 0xffff, s.cpre[c] >> 16, lane, &is_s, &is_b, &rank);
-        if (is_s) s.tab[g.lo + rank] = static_cast<unsigned short>(q);
-        if (is_b) s.tab[g.hi + 1 - rank] = static_cast<unsigned short>(q);
+      {
+        int ps = static_cast<int>(before & 0xffffu), pb = static_cast<int>(before >> 16);
+        for (int c = c_begin; c < c_end; ++c) {
+          const int q = g.lo + 1 + (c << 6) + lane;
+          const uint32_t d = q <= g.hi ? s.kv[q] >> 16 : K;
+          const unsigned long long ms = __ballot(d > K), mb = __ballot(d < K);
+          bool is_s, is_b;
+          int rank;
+          fast_ranks(g, ms, mb, ps, pb, lane, &is_s, &is_b, &rank);
+          if (is_s) s.tab[g.lo + rank] = static_cast<unsigned short>(q);
+          if (is_b) s.tab[g.hi + 1 - rank] = static_cast<unsigned short>(q);
+          ps += __popcll(ms);
+          pb += __popcll(mb);
+        }
       }
       __syncthreads();
       // A moved place is read by its own lane and written to its destination after
       // every read of the partition is done.  Up to kFastRegChunks chunks per wavefront
       // it waits in registers, in longer partitions (the first few levels) in `stage`.
       int u = 0, t = 0;
-      if (C <= kFastRegChunks * kFastWaves) {
+      int ps = static_cast<int>(before & 0xffffu), pb = static_cast<int>(before >> 16);
+      if (Cw <= kFastRegChunks) {
         uint32_t keep_kv[kFastRegChunks];
         int keep_to[kFastRegChunks];
 #pragma unroll
         for (int k = 0; k < kFastRegChunks; ++k) {
-          const int c = wave + k * kFastWaves;
+          const int c = c_begin + k;
           keep_to[k] = -1;
-          if (c < C) {
+          if (c < c_end) {
             const int q = g.lo + 1 + (c << 6) + lane;
+            const uint32_t mine = q <= g.hi ? s.kv[q] : pivot;
+            const uint32_t d = mine >> 16;
+            const unsigned long long ms = __ballot(d > K), mb = __ballot(d < K);
             bool is_s, is_b;
             int rank, dest = 0;
-            fast_ranks(g, s.ms[c], s.mb[c], s.cpre[c] & 0xffff, s.cpre[c] >> 16, lane, &is_s, &is_b, &rank);
+            fast_ranks(g, ms, mb, ps, pb, lane, &is_s, &is_b, &rank);
             const bool mv = fast_move(g, s.tab, q, is_s, is_b, rank, &dest);
             if (mv) {
               keep_to[k] = dest;
-              keep_kv[k] = s.kv[q];
+              keep_kv[k] = mine;
             }
             u += __popcll(__ballot(mv && is_s));
             t += __popcll(__ballot(mv && is_b));
+            ps += __popcll(ms);
+            pb += __popcll(mb);
           }
         }
         if (lane == 0) {
@@ -833,29 +873,33 @@ __global__ __launch_bounds__(kFastThreads) void tie_replay_fast_kernel(
         for (int k = 0; k < kFastRegChunks; ++k)
           if (keep_to[k] >= 0) s.kv[keep_to[k]] = keep_kv[k];
       } else {
-        for (int c = wave; c < C; c += kFastWaves) {
+        for (int c = c_begin; c < c_end; ++c) {
           const int q = g.lo + 1 + (c << 6) + lane;
+          const uint32_t mine = q <= g.hi ? s.kv[q] : pivot;
+          const uint32_t d = mine >> 16;
+          const unsigned long long ms = __ballot(d > K), mb = __ballot(d < K);
           bool is_s, is_b;
           int rank, dest = 0;
-          fast_ranks(g, s.ms[c], s.mb[c], s.cpre[c] & 0xffff, s.cpre[c] >> 16, lane, &is_s, &is_b, &rank);
+          fast_ranks(g, ms, mb, ps, pb, lane, &is_s, &is_b, &rank);
           const bool mv = fast_move(g, s.tab, q, is_s, is_b, rank, &dest);
-          if (q <= g.hi) stage[q] = make_uint2(mv ? s.kv[q] : 0u, mv ? static_cast<uint32_t>(dest) : 0xffffffffu);
+          if (q <= g.hi) stage[q] = make_uint2(mv ? mine : 0u, mv ? static_cast<uint32_t>(dest) : 0xffffffffu);
           u += __popcll(__ballot(mv && is_s));
           t += __popcll(__ballot(mv && is_b));
+          ps += __popcll(ms);
+          pb += __popcll(mb);
         }
         if (lane == 0) {
           if (u) atomicAdd(&s.moved_s, u);
           if (t) atomicAdd(&s.moved_b, t);
         }
-        __threadfence_block();
         __syncthreads();
-        // four loads in flight per lane
-        for (int c0 = wave; c0 < C; c0 += 4 * kFastWaves) {
+        // every lane reads back what it staged itself, four loads in flight
+        for (int c0 = c_begin; c0 < c_end; c0 += 4) {
           uint2 e[4];
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const int q = g.lo + 1 + ((c0 + j * kFastWaves) << 6) + lane;
-            e[j] = q <= g.hi ? stage[q] : make_uint2(0u, 0xffffffffu);
+            const int q = g.lo + 1 + ((c0 + j) << 6) + lane;
+            e[j] = (c0 + j < c_end && q <= g.hi) ? stage[q] : make_uint2(0u, 0xffffffffu);
           }
 #pragma unroll
           for (int j = 0; j < 4; ++j)
@@ -863,8 +907,10 @@ __global__ __launch_bounds__(kFastThreads) void tie_replay_fast_kernel(
         }
       }
       __syncthreads();
+      // One thread places the pivot and queues the children while the others go on to
+      // the next partition: it touches the rank table and places of this partition
+      // only, and the counters it reads are reset by itself.
       if (tid == 0) fast_finish(&s, g, pivot, s.moved_s, s.moved_b, num_top, order, next);
-      __syncthreads();
     }
     // ---- short partitions: one wavefront each ----
     for (int si = wave; si < n_cur; si += kFastWaves) {
@@ -872,38 +918,31 @@ __global__ __launch_bounds__(kFastThreads) void tie_replay_fast_kernel(
       FastSeg g;
       g.lo = static_cast<int>(sg >> 16);
       g.hi = static_cast<int>(sg & 0xffffu);
-      if (g.hi - g.lo + 1 > kFastWaveSeg) continue;
       const uint32_t pivot = s.kv[g.lo];
       const uint32_t K = pivot >> 16;
       const int places = g.hi - g.lo;
-      const int C = (places + 63) >> 6;  // <= kFastWaveChunks
-      // this wavefront's ballots go to its own sixteen slots of the ballot arrays (the
-      // workgroup path above is finished with them)
-      unsigned long long* wms = s.ms + wave * kFastWaveChunks;
-      unsigned long long* wmb = s.mb + wave * kFastWaveChunks;
+      const int C = (places + 63) >> 6;
+      // The wavefront walks the chunks in order, so the counts before a chunk are running
+      // sums and nothing but the rank table is stored; the ballots are taken again in
+      // every pass (one LDS read and two compares).
       g.nS = 0;
       g.nB = 0;
       for (int c = 0; c < C; ++c) {
         const int q = g.lo + 1 + (c << 6) + lane;
         const uint32_t d = q <= g.hi ? s.kv[q] >> 16 : K;
-        const unsigned long long ms = __ballot(d > K), mb = __ballot(d < K);
-        if (lane == 0) {
-          wms[c] = ms;
-          wmb[c] = mb;
-        }
-        g.nS += __popcll(ms);
-        g.nB += __popcll(mb);
+        g.nS += __popcll(__ballot(d > K));
+        g.nB += __popcll(__ballot(d < K));
       }
       if (g.nS == 0 && g.nB == 0) {
         for (int q = g.lo + lane; q <= g.hi && q < num_top; q += 64)
           order[q] = static_cast<int>(s.kv[q] & 0xffffu);
         continue;
       }
-      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
       int ps = 0, pb = 0;
       for (int c = 0; c < C; ++c) {
         const int q = g.lo + 1 + (c << 6) + lane;
-        const unsigned long long ms = wms[c], mb = wmb[c];
+        const uint32_t d = q <= g.hi ? s.kv[q] >> 16 : K;
+        const unsigned long long ms = __ballot(d > K), mb = __ballot(d < K);
         bool is_s, is_b;
         int rank;
         fast_ranks(g, ms, mb, ps, pb, lane, &is_s, &is_b, &rank);
@@ -913,46 +952,82 @@ __global__ __launch_bounds__(kFastThreads) void tie_replay_fast_kernel(
         pb += __popcll(mb);
       }
       __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-      uint32_t keep_kv[kFastWaveChunks];
-      int keep_to[kFastWaveChunks];
       int u = 0, t = 0;
       ps = 0;
       pb = 0;
+      if (C <= kFastRegChunks) {
+        uint32_t keep_kv[kFastRegChunks];
+        int keep_to[kFastRegChunks];
 #pragma unroll
-      for (int c = 0; c < kFastWaveChunks; ++c) {
-        keep_to[c] = -1;
-        if (c < C) {
+        for (int c = 0; c < kFastRegChunks; ++c) {
+          keep_to[c] = -1;
+          if (c < C) {
+            const int q = g.lo + 1 + (c << 6) + lane;
+            const uint32_t mine = q <= g.hi ? s.kv[q] : pivot;
+            const uint32_t d = mine >> 16;
+            const unsigned long long ms = __ballot(d > K), mb = __ballot(d < K);
+            bool is_s, is_b;
+            int rank, dest = 0;
+            fast_ranks(g, ms, mb, ps, pb, lane, &is_s, &is_b, &rank);
+            const bool mv = fast_move(g, s.tab, q, is_s, is_b, rank, &dest);
+            if (mv) {
+              keep_to[c] = dest;
+              keep_kv[c] = mine;
+            }
+            u += __popcll(__ballot(mv && is_s));
+            t += __popcll(__ballot(mv && is_b));
+            ps += __popcll(ms);
+            pb += __popcll(mb);
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+#pragma unroll
+        for (int c = 0; c < kFastRegChunks; ++c)
+          if (keep_to[c] >= 0) s.kv[keep_to[c]] = keep_kv[c];
+      } else {
+        for (int c = 0; c < C; ++c) {
           const int q = g.lo + 1 + (c << 6) + lane;
-          const unsigned long long ms = wms[c], mb = wmb[c];
+          const uint32_t mine = q <= g.hi ? s.kv[q] : pivot;
+          const uint32_t d = mine >> 16;
+          const unsigned long long ms = __ballot(d > K), mb = __ballot(d < K);
           bool is_s, is_b;
           int rank, dest = 0;
           fast_ranks(g, ms, mb, ps, pb, lane, &is_s, &is_b, &rank);
           const bool mv = fast_move(g, s.tab, q, is_s, is_b, rank, &dest);
-          if (mv) {
-            keep_to[c] = dest;
-            keep_kv[c] = s.kv[q];
-          }
+          if (q <= g.hi) stage[q] = make_uint2(mv ? mine : 0u, mv ? static_cast<uint32_t>(dest) : 0xffffffffu);
           u += __popcll(__ballot(mv && is_s));
           t += __popcll(__ballot(mv && is_b));
           ps += __popcll(ms);
           pb += __popcll(mb);
         }
-      }
-      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        // every lane reads back what it staged itself, four loads in flight
+        for (int c0 = 0; c0 < C; c0 += 4) {
+          uint2 e[4];
 #pragma unroll
-      for (int c = 0; c < kFastWaveChunks; ++c)
-        if (keep_to[c] >= 0) s.kv[keep_to[c]] = keep_kv[c];
+          for (int j = 0; j < 4; ++j) {
+            const int q = g.lo + 1 + ((c0 + j) << 6) + lane;
+            e[j] = q <= g.hi ? stage[q] : make_uint2(0u, 0xffffffffu);
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (e[j].y != 0xffffffffu) s.kv[e[j].y] = e[j].x;
+        }
+      }
       __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
       if (lane == 0) fast_finish(&s, g, pivot, u, t, num_top, order, next);
     }
     __syncthreads();
-    n_cur = s.failed ? 0 : min(s.n_next, kFastMaxSegs);
+    n_cur = s.failed ? 0 : min(s.n_seg[next], kFastMaxSegs);
+    n_cur_long = s.failed ? 0 : min(s.n_long[next], kFastMaxLong);
+    if (tid == 0) {  // the lists that were just walked receive the level after next
+      s.n_seg[cur] = 0;
+      s.n_long[cur] = 0;
+    }
     cur = next;
     __syncthreads();
-    if (tid == 0) s.n_next = 0;
-    __syncthreads();
   }
-  if (tid == 0 && n_cur == 0 && !s.failed) {
+  if (tid == 0 && n_cur + n_cur_long == 0 && !s.failed) {
     flag[1] = 1;
     flag[0] = 3;  // reported to the caller: equal scores, order replayed by this kernel
   }
