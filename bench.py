@@ -458,43 +458,70 @@ def layer_roofline(path, batch):
 
 
 def bandwidth_report(path):
-    """The kernels whose bound is HBM, one launch at a time through the kernel-level C ABI
-    on torch-owned device memory: 20 warm-up launches, 100 launches timed one by one with
-    HIP events on the launch stream, median; algorithmic bytes = 4 * (elements read +
-    elements written), parameters left out."""
+    """The kernels whose bound is HBM, alone, through the kernel-level C ABI on torch-owned
+    device memory.  Two figures per kernel: `cold` rotates over enough copies of the
+    operands to exceed twice the 256 MB last-level cache and times 40 back-to-back
+    launches between two HIP events (what HBM gives; launch overhead amortised);
+    `one launch` is the median of 100 launches of one operand set, each between its own
+    two events (includes about 6 us of event and launch overhead; small operands come
+    from the cache).  Algorithmic bytes = 4 * (elements read + elements written),
+    parameters left out; Normalize counts its input twice (12 bytes per element)."""
     import statistics
     import torch
     from minicaffe import kernels as K
     from minicaffe.base import LIB
     stream = torch.cuda.current_stream().cuda_stream
     P = ctypes.c_void_p
-    ints = lambda v: (ctypes.c_int * len(v))(*v)
-    dev = lambda *shape: torch.randn(*shape, device="cuda")
+    ints = lambda v: (ctypes.c_int * len(v))(*v)  # noqa: E731
     rows = []
 
-    def timed(name, nbytes, launch):
-        for _ in range(20):
-            rc = launch()
+    def sets_for(nbytes):
+        return max(2, min(64, int(2 * 256e6 // max(nbytes, 1)) + 1))
+
+    def timed(name, nbytes, make):
+        """make() -> (launch, keepalive) for a fresh operand set."""
+        k = sets_for(nbytes)
+        launches = [make() for _ in range(k)]
+        for fn, _ in launches:
+            rc = fn()
             assert rc in (0, None), LIB.mcLastError()
+        torch.cuda.synchronize()
+        reps = 40
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(reps):
+            launches[i % k][0]()
+        e1.record()
+        torch.cuda.synchronize()
+        cold_us = e0.elapsed_time(e1) / reps * 1e3
+        fn = launches[0][0]
+        for _ in range(20):
+            fn()
         torch.cuda.synchronize()
         spans = []
         for _ in range(100):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            launch()
-            e1.record()
-            spans.append((e0, e1))
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            spans.append((a, b))
         torch.cuda.synchronize()
-        us = statistics.median(a.elapsed_time(b) for a, b in spans) * 1e3
-        gbs = nbytes / us / 1e3
-        rows.append("%-58s %9.1f MB %9.1f us %9.0f GB/s %6.1f %%" % (name, nbytes / 1e6, us, gbs, gbs / HBM_PEAK_GBS * 100))
+        one_us = statistics.median(a.elapsed_time(b) for a, b in spans) * 1e3
+        gbs = nbytes / cold_us / 1e3
+        rows.append("%-58s %9.1f MB %3d sets %9.1f us %8.0f GB/s %6.1f %% %11.1f us"
+                    % (name, nbytes / 1e6, k, cold_us, gbs, gbs / HBM_PEAK_GBS * 100, one_us))
+
+    dev = lambda *shape: torch.randn(*shape, device="cuda")  # noqa: E731
 
     def pool(name, method, planes, h, w, k, s_, pad):
         ho, wo = ctypes.c_int(), ctypes.c_int()
         LIB.mcPoolingOutputShape(h, w, k, k, s_, s_, pad, pad, ctypes.byref(ho), ctypes.byref(wo))
-        x, y = dev(planes, h, w), dev(planes, ho.value, wo.value)
-        timed(name, 4 * (x.numel() + y.numel()),
-              lambda: LIB.mcPooling(method, P(x.data_ptr()), P(y.data_ptr()), planes, h, w, k, k, s_, s_, pad, pad, P(stream)))
+
+        def make():
+            x, y = dev(planes, h, w), dev(planes, ho.value, wo.value)
+            return (lambda: LIB.mcPooling(method, P(x.data_ptr()), P(y.data_ptr()), planes, h, w, k, k, s_, s_,
+                                          pad, pad, P(stream))), (x, y)
+        timed(name, 4 * (planes * h * w + planes * ho.value * wo.value), make)
 
     pool("Pooling MAX 3x3/2, 64x64x112x112 (ResNet-50 stem)", 0, 64 * 64, 112, 112, 3, 2, 0)
     pool("Pooling MAX 2x2/2, 8x64x300x300 (SSD300 pool1)", 0, 8 * 64, 300, 300, 2, 2, 0)
@@ -502,54 +529,71 @@ def bandwidth_report(path):
     pool("Pooling AVE 7x7 global, 64x2048x7x7 (ResNet-50 pool5)", 1, 64 * 2048, 7, 7, 7, 1, 0)
 
     n, c, sp = 64, 256, 56 * 56
-    a, b, y = dev(n, c, sp), dev(n, c, sp), dev(n, c, sp)
-    bottoms = (ctypes.c_void_p * 2)(a.data_ptr(), b.data_ptr())
-    coeffs = (ctypes.c_float * 2)(1.0, 1.0)
-    timed("Eltwise SUM + ReLU, 2 x 64x256x56x56 (residual, unfused)", 4 * 3 * a.numel(),
-          lambda: LIB.mcEltwise(1, 2, bottoms, coeffs, a.numel(), P(y.data_ptr()), 1, 0.0, P(stream)))
+    numel = n * c * sp
+
+    def make_eltwise():
+        a, b, y = dev(n, c, sp), dev(n, c, sp), dev(n, c, sp)
+        bottoms = (ctypes.c_void_p * 2)(a.data_ptr(), b.data_ptr())
+        coeffs = (ctypes.c_float * 2)(1.0, 1.0)
+        return (lambda: LIB.mcEltwise(1, 2, bottoms, coeffs, numel, P(y.data_ptr()), 1, 0.0, P(stream))), (a, b, y, bottoms, coeffs)
+    timed("Eltwise SUM + ReLU, 2 x 64x256x56x56 (residual, unfused)", 4 * 3 * numel, make_eltwise)
     mul, add = dev(c), dev(c)
     op = K.ChannelOp(None, None, mul.data_ptr(), add.data_ptr(), 1, 0.0)
-    timed("channel transform x*g+b, ReLU, 64x256x56x56 (BN/Scale/ReLU)", 4 * 2 * a.numel(),
-          lambda: LIB.mcChannelTransform(P(a.data_ptr()), P(y.data_ptr()), n, c, sp, ctypes.byref(op), P(stream)))
-    timed("Unary ELU, 64x256x56x56", 4 * 2 * a.numel(),
-          lambda: LIB.mcUnary(5, P(a.data_ptr()), P(y.data_ptr()), a.numel(), 1.0, 0.0, 0.0, P(stream)))
-    timed("PReLU, one slope per channel, 64x256x56x56", 4 * 2 * a.numel(),
-          lambda: LIB.mcPReLU(P(a.data_ptr()), P(y.data_ptr()), n, c, sp, P(mul.data_ptr()), 0, P(stream)))
-    timed("copy (Concat / Slice / Split), 64x256x56x56", 4 * 2 * a.numel(),
-          lambda: LIB.mcCopy2D(P(a.data_ptr()), a.numel(), P(y.data_ptr()), a.numel(), a.numel(), 1, P(stream)))
-    shape, order = ints([n, c, 56, 56]), ints([0, 2, 3, 1])
-    timed("Permute (0,2,3,1), 64x256x56x56", 4 * 2 * a.numel(),
-          lambda: LIB.mcPermute(P(a.data_ptr()), P(y.data_ptr()), 4, shape, order, P(stream)))
-    del a, b, y
 
-    x, y = dev(8, 84, 38, 38), dev(8, 84, 38, 38)
+    def unary_like(call):
+        def make():
+            a, y = dev(n, c, sp), dev(n, c, sp)
+            return (lambda: call(a, y)), (a, y)
+        return make
+    timed("channel transform x*g+b, ReLU, 64x256x56x56 (BN/Scale/ReLU)", 4 * 2 * numel, unary_like(
+        lambda a, y: LIB.mcChannelTransform(P(a.data_ptr()), P(y.data_ptr()), n, c, sp, ctypes.byref(op), P(stream))))
+    timed("Unary ELU, 64x256x56x56", 4 * 2 * numel, unary_like(
+        lambda a, y: LIB.mcUnary(5, P(a.data_ptr()), P(y.data_ptr()), numel, 1.0, 0.0, 0.0, P(stream))))
+    timed("PReLU, one slope per channel, 64x256x56x56", 4 * 2 * numel, unary_like(
+        lambda a, y: LIB.mcPReLU(P(a.data_ptr()), P(y.data_ptr()), n, c, sp, P(mul.data_ptr()), 0, P(stream))))
+    timed("copy (Concat / Slice / Split), 64x256x56x56", 4 * 2 * numel, unary_like(
+        lambda a, y: LIB.mcCopy2D(P(a.data_ptr()), numel, P(y.data_ptr()), numel, numel, 1, P(stream))))
+    shape, order = ints([n, c, 56, 56]), ints([0, 2, 3, 1])
+    timed("Permute (0,2,3,1), 64x256x56x56", 4 * 2 * numel, unary_like(
+        lambda a, y: LIB.mcPermute(P(a.data_ptr()), P(y.data_ptr()), 4, shape, order, P(stream))))
+
+    def simple(shape_, call):
+        def make():
+            x, y = dev(*shape_), dev(*shape_)
+            return (lambda: call(x, y)), (x, y)
+        return make
     shape2 = ints([8, 84, 38, 38])
-    timed("Permute (0,2,3,1), 8x84x38x38 (SSD300 conv4_3 conf head)", 4 * 2 * x.numel(),
-          lambda: LIB.mcPermute(P(x.data_ptr()), P(y.data_ptr()), 4, shape2, order, P(stream)))
-    x, y = dev(8 * 8732, 21), dev(8 * 8732, 21)
-    timed("Softmax over 21 classes, 8x8732 rows (SSD300 mbox_conf)", 4 * 2 * x.numel(),
-          lambda: LIB.mcSoftmax(P(x.data_ptr()), P(y.data_ptr()), 8 * 8732, 21, 1, P(stream)))
-    x, y = dev(64, 1000), dev(64, 1000)
-    timed("Softmax over 1000 classes, 64 rows (ResNet-50 prob)", 4 * 2 * x.numel(),
-          lambda: LIB.mcSoftmax(P(x.data_ptr()), P(y.data_ptr()), 64, 1000, 1, P(stream)))
-    x, y, sc = dev(8, 512, 38 * 38), dev(8, 512, 38 * 38), dev(512)
-    timed("Normalize across channels, 8x512x38x38 (SSD300 conv4_3_norm)", 4 * 2 * x.numel(),
-          lambda: LIB.mcNormalize(P(x.data_ptr()), P(y.data_ptr()), 8, 512, 38 * 38, 0, 0, 1e-10, P(sc.data_ptr()), P(stream)))
-    x, y = dev(64, 96, 55, 55), dev(64, 96, 55, 55)
-    timed("LRN across 5 channels, 64x96x55x55 (AlexNet norm1)", 4 * 2 * x.numel(),
-          lambda: LIB.mcLRNAcrossChannels(P(x.data_ptr()), P(y.data_ptr()), 64, 96, 55, 55, 5, 1e-4, 0.75, 1.0, P(stream)))
+    timed("Permute (0,2,3,1), 8x84x38x38 (SSD300 conv4_3 conf head)", 4 * 2 * 8 * 84 * 38 * 38, simple(
+        (8, 84, 38, 38), lambda x, y: LIB.mcPermute(P(x.data_ptr()), P(y.data_ptr()), 4, shape2, order, P(stream))))
+    timed("Softmax over 21 classes, 8x8732 rows (SSD300 mbox_conf)", 4 * 2 * 8 * 8732 * 21, simple(
+        (8 * 8732, 21), lambda x, y: LIB.mcSoftmax(P(x.data_ptr()), P(y.data_ptr()), 8 * 8732, 21, 1, P(stream))))
+    timed("Softmax over 1000 classes, 64 rows (ResNet-50 prob)", 4 * 2 * 64 * 1000, simple(
+        (64, 1000), lambda x, y: LIB.mcSoftmax(P(x.data_ptr()), P(y.data_ptr()), 64, 1000, 1, P(stream))))
+    sc = dev(512)
+    timed("Normalize across channels, 8x512x38x38 (SSD300 conv4_3_norm)", 4 * 3 * 8 * 512 * 38 * 38, simple(
+        (8, 512, 38 * 38), lambda x, y: LIB.mcNormalize(P(x.data_ptr()), P(y.data_ptr()), 8, 512, 38 * 38, 0, 0, 1e-10,
+                                                         P(sc.data_ptr()), P(stream))))
+    timed("LRN across 5 channels, 64x96x55x55 (AlexNet norm1)", 4 * 2 * 64 * 96 * 55 * 55, simple(
+        (64, 96, 55, 55), lambda x, y: LIB.mcLRNAcrossChannels(P(x.data_ptr()), P(y.data_ptr()), 64, 96, 55, 55, 5, 1e-4,
+                                                               0.75, 1.0, P(stream))))
     for cin, h, s_ in ((512, 19, 1), (256, 38, 2), (64, 150, 1)):
         plan = K.ConvPlan(K.conv_geom(cin, h, h, cin, 3, s_, 1, group=cin))
         ho, wo = plan.output_shape()
-        x, w, y = dev(32, cin, h, h), dev(cin, 1, 3, 3), dev(32, cin, ho, wo)
+        w = dev(cin, 1, 3, 3)
         plan.set_weights(w.data_ptr())
-        timed("depthwise 3x3/%d + ReLU, 32x%dx%dx%d (MobileNet)" % (s_, cin, h, h), 4 * (x.numel() + y.numel()),
-              lambda: plan.forward(32, x.data_ptr(), y.data_ptr(), activation=K.ACT_RELU, stream=stream))
+
+        def make():
+            x, y = dev(32, cin, h, h), dev(32, cin, ho, wo)
+            return (lambda: plan.forward(32, x.data_ptr(), y.data_ptr(), activation=K.ACT_RELU, stream=stream)), (x, y)
+        timed("depthwise 3x3/%d + ReLU, 32x%dx%dx%d (MobileNet)" % (s_, cin, h, h),
+              4 * 32 * cin * (h * h + ho * wo), make)
         del plan
-    head = ["%-58s %12s %12s %14s %8s" % ("kernel, shape", "alg. bytes", "median", "achieved", "of 8 TB/s")]
-    tail = ["20 warm-up + 100 launches timed one by one with HIP events, median.  Buffers smaller than the 256 MB",
-            "last-level cache can be served from it on repeated launches (as they are inside a net, where the",
-            "producer has just written them), so small shapes may read above what HBM alone would give."]
+    head = ["%-58s %12s %8s %12s %13s %8s %14s" % ("kernel, shape", "alg. bytes", "operands", "cold", "achieved",
+                                                  "of 8 TB/s", "one launch")]
+    tail = ["cold: 40 back-to-back launches between two HIP events, rotating over `operands` sets (more than 512 MB",
+            "in total, twice the last-level cache), so every launch reads from and writes to HBM.",
+            "one launch: median of 100 launches of one operand set, each between its own two events: includes",
+            "about 6 us of event and launch overhead, and operands below 256 MB come from the last-level cache."]
     with open(path, "w") as f:
         f.write("\n".join(head + rows + tail) + "\n")
 

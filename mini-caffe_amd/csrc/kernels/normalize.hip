@@ -9,7 +9,10 @@ namespace {
 // threads each sum every eighth channel, so a half-wave reads 128 contiguous
 // bytes of a channel plane and a pixel's channels are covered by 8 threads
 // instead of one serial walk.  The 8 partial sums are added in a fixed order.
+// KEEP > 0: a thread's channels (at most KEEP of them, i.e. up to 8 * KEEP channels) stay
+// in registers between the sum and the scaling, so the blob is read once.
 constexpr int kNormPix = 32, kNormSlices = 8;
+template <int KEEP>
 __global__ __launch_bounds__(256) void normalize_pixel_kernel(
     const float* __restrict__ x, float* __restrict__ y, int C, int spatial, int tiles_per_image,
     int channel_shared, float eps, const float* __restrict__ scale) {
@@ -22,13 +25,26 @@ __global__ __launch_bounds__(256) void normalize_pixel_kernel(
   const float* __restrict__ xp = x + (long)n * C * spatial + s;
   float* __restrict__ yp = y + (long)n * C * spatial + s;
   float acc = 0.f;
+  float kept[KEEP > 0 ? KEEP : 1];
   if (live) {
-    // batches of 8 independent loads: the launch is small, so memory latency
-    // has to be covered inside a thread
+    if constexpr (KEEP > 0) {
+      // all loads are independent: the whole column of this thread is in flight at once;
+      // the squares are added in channel order, as the re-reading form below does
+#pragma unroll
+      for (int k = 0; k < KEEP; ++k) {
+        const int c = sl + k * kNormSlices;
+        kept[k] = c < C ? xp[(long)c * spatial] : 0.f;
+      }
+#pragma unroll
+      for (int k = 0; k < KEEP; ++k) acc += kept[k] * kept[k];
+    } else {
+      // batches of 8 independent loads: the launch is small, so memory latency
+      // has to be covered inside a thread
 #pragma unroll 8
-    for (int c = sl; c < C; c += kNormSlices) {
-      const float v = xp[(long)c * spatial];
-      acc += v * v;
+      for (int c = sl; c < C; c += kNormSlices) {
+        const float v = xp[(long)c * spatial];
+        acc += v * v;
+      }
     }
   }
   part[sl][px] = acc;
@@ -37,12 +53,21 @@ __global__ __launch_bounds__(256) void normalize_pixel_kernel(
 #pragma unroll
   for (int k = 0; k < kNormSlices; ++k) sum += part[k][px];
   const float norm = sqrtf(sum);
-  if (live)
+  if (live) {
+    if constexpr (KEEP > 0) {
+#pragma unroll
+      for (int k = 0; k < KEEP; ++k) {
+        const int c = sl + k * kNormSlices;
+        if (c < C) yp[(long)c * spatial] = (kept[k] / norm) * (channel_shared ? scale[0] : scale[c]);
+      }
+    } else {
 #pragma unroll 8
-    for (int c = sl; c < C; c += kNormSlices) {
-      const float v = xp[(long)c * spatial] / norm;
-      yp[(long)c * spatial] = v * (channel_shared ? scale[0] : scale[c]);
+      for (int c = sl; c < C; c += kNormSlices) {
+        const float v = xp[(long)c * spatial] / norm;
+        yp[(long)c * spatial] = v * (channel_shared ? scale[0] : scale[c]);
+      }
     }
+  }
 }
 
 // One workgroup per image.
@@ -85,8 +110,15 @@ extern "C" int mcNormalize(const float* bottom, float* top, int num, int channel
   } else {
     const int tiles = ceil_div(spatial, kNormPix);
     MC_REQUIRE((long)num * tiles < (1L << 31), "mcNormalize: too many pixels");
-    normalize_pixel_kernel<<<num * tiles, 256, 0, st>>>(bottom, top, channels, spatial, tiles,
-                                                        channel_shared, eps, scale);
+    if (channels <= 16 * kNormSlices)
+      normalize_pixel_kernel<16><<<num * tiles, 256, 0, st>>>(bottom, top, channels, spatial, tiles,
+                                                             channel_shared, eps, scale);
+    else if (channels <= 64 * kNormSlices)
+      normalize_pixel_kernel<64><<<num * tiles, 256, 0, st>>>(bottom, top, channels, spatial, tiles,
+                                                             channel_shared, eps, scale);
+    else
+      normalize_pixel_kernel<0><<<num * tiles, 256, 0, st>>>(bottom, top, channels, spatial, tiles,
+                                                            channel_shared, eps, scale);
   }
   MC_LAUNCH_CHECK();
   return 0;

@@ -5,6 +5,8 @@
 // batch of plain 2-D transposes: those go through a 64x64 LDS tile so that both
 // the reads and the writes are contiguous 256-byte rows.  Everything else falls
 // to a gather with one thread per output element.
+#include <cstdint>
+
 #include "mc_common.h"
 #include "mchip/kernels.h"
 
@@ -57,6 +59,40 @@ __global__ __launch_bounds__(256) void transpose_tile_kernel(const float* __rest
   }
 }
 
+// The same transpose with 16-byte accesses on both sides (R and C multiples of 4, both
+// blobs 16-byte aligned): a thread loads four consecutive columns of a row, and stores
+// four consecutive rows of a column.  64 x 64 tile, 256 threads, four passes each way.
+__global__ __launch_bounds__(256) void transpose_tile_vec_kernel(const float* __restrict__ x,
+                                                                 float* __restrict__ y, int R,
+                                                                 int C) {
+  __shared__ float tile[64][65];
+  const long base = (long)blockIdx.z * R * C;
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const int quad = threadIdx.x & 15, line = threadIdx.x >> 4;  // 16 quads per tile line, 16 lines per pass
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = r0 + line + 16 * i, c = c0 + 4 * quad;
+    if (r < R && c < C) {
+      const float4 v = *reinterpret_cast<const float4*>(x + base + (long)r * C + c);
+      float* t = &tile[line + 16 * i][4 * quad];
+      t[0] = v.x;
+      t[1] = v.y;
+      t[2] = v.z;
+      t[3] = v.w;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = c0 + line + 16 * i, r = r0 + 4 * quad;
+    if (r < R && c < C) {
+      const int tc = line + 16 * i, tr = 4 * quad;
+      *reinterpret_cast<float4*>(y + base + (long)c * R + r) =
+          make_float4(tile[tr][tc], tile[tr + 1][tc], tile[tr + 2][tc], tile[tr + 3][tc]);
+    }
+  }
+}
+
 }  // namespace
 }  // namespace mchip
 
@@ -96,8 +132,14 @@ extern "C" int mcPermute(const float* bottom, float* top, int n, const int* shap
     for (int i = q; i < n; ++i) C *= shape[i];
     if (R < (1L << 31) && C < (1L << 31) && batch < 65536 && ceil_div(R, 64) < 65536) {
       dim3 grid(ceil_div(C, 64), ceil_div(R, 64), static_cast<unsigned>(batch));
-      transpose_tile_kernel<<<grid, 256, 0, st>>>(bottom, top, static_cast<int>(R),
-                                                  static_cast<int>(C));
+      const bool vec = R % 4 == 0 && C % 4 == 0 &&
+                       ((reinterpret_cast<uintptr_t>(bottom) | reinterpret_cast<uintptr_t>(top)) & 15u) == 0;
+      if (vec)
+        transpose_tile_vec_kernel<<<grid, 256, 0, st>>>(bottom, top, static_cast<int>(R),
+                                                        static_cast<int>(C));
+      else
+        transpose_tile_kernel<<<grid, 256, 0, st>>>(bottom, top, static_cast<int>(R),
+                                                    static_cast<int>(C));
       MC_LAUNCH_CHECK();
       return 0;
     }

@@ -571,7 +571,12 @@ def test_softmax(K, shape, axis):
 
 @pytest.mark.parametrize("shape,order", [((8, 84, 38, 38), (0, 2, 3, 1)), ((2, 3, 4, 5), (0, 3, 1, 2)),
                                          ((2, 3, 4, 5), (3, 2, 1, 0)), ((2, 3, 4, 5), (0, 1, 2, 3)),
-                                         ((3, 70, 65), (0, 2, 1)), ((5, 6), (1, 0))])
+                                         ((3, 70, 65), (0, 2, 1)), ((5, 6), (1, 0)),
+                                         # 16-byte form of the tiled transpose: both extents multiples of 4,
+                                         # ragged tiles on both sides; then extents that rule it out
+                                         ((2, 68, 132), (0, 2, 1)), ((3, 256, 28, 28), (0, 2, 3, 1)),
+                                         ((2, 4, 4), (0, 2, 1)), ((2, 68, 130), (0, 2, 1)), ((2, 66, 132), (0, 2, 1)),
+                                         ((8, 24, 19, 19), (0, 2, 3, 1))])
 def test_permute_bit_exact(K, shape, order):
     x = np.random.default_rng(8).standard_normal(shape).astype(np.float32)
     want = np.ascontiguousarray(np.transpose(x, order))
@@ -594,14 +599,18 @@ def test_copy2d_and_fill(K):
     assert np.array_equal(got[:, 10:43], x) and np.all(got[0, :5] == 2.5) and np.all(got[1:, :10] == 0)
 
 
-def test_normalize(K):
+@pytest.mark.parametrize("shape", [(2, 12, 5, 7),       # a thread keeps its channels in registers (<= 128)
+                                   (2, 512, 9, 11),     # SSD's 512 channels, ragged pixel tile (<= 512)
+                                   (1, 130, 6, 6), (1, 515, 3, 5)])   # > 512 channels: read twice
+def test_normalize(K, shape):
     rng = np.random.default_rng(10)
-    x = rng.standard_normal((2, 12, 5, 7)).astype(np.float32)
+    x = rng.standard_normal(shape).astype(np.float32)
+    num, ch, spatial = shape[0], shape[1], shape[2] * shape[3]
     for across, shared in ((0, 0), (0, 1), (1, 0), (1, 1)):
-        s = (rng.random(1 if shared else 12) + 0.5).astype(np.float32)
+        s = (rng.random(1 if shared else ch) + 0.5).astype(np.float32)
         want = oracle.normalize(x, s, bool(across), bool(shared), 1e-10)
-        xd, sd, yd = dev(x), dev(s), torch.empty(x.shape, device="cuda")
-        K.check_mc(K.LIB.mcNormalize(fptr(xd), fptr(yd), 2, 12, 35, across, shared, ctypes.c_float(1e-10),
+        xd, sd, yd = dev(x), dev(s), torch.full(x.shape, float("nan"), device="cuda")
+        K.check_mc(K.LIB.mcNormalize(fptr(xd), fptr(yd), num, ch, spatial, across, shared, ctypes.c_float(1e-10),
                                      fptr(sd), None))
         torch.cuda.synchronize()
         assert np.abs(yd.cpu().numpy() - want).max() < 1e-6
