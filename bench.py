@@ -62,6 +62,9 @@ def main():
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-batch", type=int, default=8)
+    ap.add_argument("--no-detection-tails", action="store_true",
+                    help="skip the NMS / Proposal / DetectionOutput timings (profiling runs of the "
+                         "ResNet-50 forward alone)")
     ap.add_argument("--configs-report", metavar="PATH",
                     help="also time all five BASELINE configurations (whole forward, contraction "
                          "launches, Proposal / DetectionOutput layers) and write a text table to PATH")
@@ -157,7 +160,7 @@ def main():
     # the other two figures of the metric: convolution MFMA utilisation (hardware
     # counters, quoted from the committed counter run) and the detection tails
     del net
-    tails = detection_tails(mc, craft, zoo, LIB)
+    tails = {} if args.no_detection_tails else detection_tails(mc, craft, zoo, LIB)
     cpu = None
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(args.cpu_batch)
