@@ -9,6 +9,7 @@
 
 #include <cfloat>
 #include <cmath>
+#include <cstdint>
 
 namespace mchip {
 namespace {
@@ -102,6 +103,52 @@ void launch_max_pool_fixed(const PoolArgs& a, long planes, hipStream_t st) {
   const long count = planes * row_pairs * a.Wo;
   max_pool_fixed_kernel<KH, KW, SH, SW>
       <<<ceil_div(count, 256), 256, 0, st>>>(a, row_pairs, count);
+}
+
+// MAX 3x3 / stride 2 without padding on a width that is a multiple of 4 (the ResNet
+// stem: 112 -> 56): one thread makes a 2 x 2 block of outputs from the 5 x 5 inputs under
+// it, each input row as one aligned 16-byte load plus one more value, so neighbouring
+// threads read neighbouring 16-byte pieces and every byte fetched is used; the block's
+// two output rows leave as 8-byte stores when the output width is even.
+__global__ __launch_bounds__(256) void max_pool_3x3s2_quad_kernel(const PoolArgs a, int row_pairs,
+                                                                  int col_pairs, long count) {
+  const long i = blockIdx.x * 256L + threadIdx.x;
+  if (i >= count) return;
+  const int cp = static_cast<int>(i % col_pairs);
+  const long t = i / col_pairs;
+  const int rp = static_cast<int>(t % row_pairs);
+  const long plane = t / row_pairs;
+  const float* __restrict__ xp = a.x + plane * a.H * a.W;
+  const int h0 = 4 * rp, w0 = 4 * cp;
+  const bool last_col = w0 + 4 < a.W;  // the fifth column exists
+  float left[5], right[5];             // per input row: max of columns 0..2 and of columns 2..4
+#pragma unroll
+  for (int r = 0; r < 5; ++r) {
+    left[r] = right[r] = -FLT_MAX;
+    if (h0 + r < a.H) {
+      const float* __restrict__ row = xp + (h0 + r) * a.W + w0;
+      const float4 v = *reinterpret_cast<const float4*>(row);
+      const float e = last_col ? row[4] : -FLT_MAX;
+      left[r] = fmaxf(fmaxf(v.x, v.y), v.z);
+      right[r] = fmaxf(fmaxf(v.z, v.w), e);
+    }
+  }
+  const int oh = 2 * rp, ow = 2 * cp;
+  const float t0 = fmaxf(fmaxf(left[0], left[1]), left[2]), t1 = fmaxf(fmaxf(right[0], right[1]), right[2]);
+  const float b0 = fmaxf(fmaxf(left[2], left[3]), left[4]), b1 = fmaxf(fmaxf(right[2], right[3]), right[4]);
+  float* __restrict__ yp = a.y + (plane * a.Ho + oh) * a.Wo + ow;
+  const bool two_cols = ow + 1 < a.Wo, two_rows = oh + 1 < a.Ho;
+  if (two_cols && (a.Wo & 1) == 0) {
+    *reinterpret_cast<float2*>(yp) = make_float2(t0, t1);
+    if (two_rows) *reinterpret_cast<float2*>(yp + a.Wo) = make_float2(b0, b1);
+  } else {
+    yp[0] = t0;
+    if (two_cols) yp[1] = t1;
+    if (two_rows) {
+      yp[a.Wo] = b0;
+      if (two_cols) yp[a.Wo + 1] = b1;
+    }
+  }
 }
 
 // G lanes per plane (a power of two up to the wavefront), 256 / G planes per
@@ -202,7 +249,12 @@ int mcPooling(int method, const float* bottom, float* top, int planes, int H, in
     // every window holds at least one element (the output shape guarantees it), so
     // the padding value never reaches the output
     bool done = true;
-    if (kh == 3 && kw == 3 && sh == 2 && sw == 2) launch_max_pool_fixed<3, 3, 2, 2>(a, planes, st);
+    if (kh == 3 && kw == 3 && sh == 2 && sw == 2 && ph == 0 && pw == 0 && W % 4 == 0 &&
+        (reinterpret_cast<uintptr_t>(bottom) & 15u) == 0 && (reinterpret_cast<uintptr_t>(top) & 7u) == 0) {
+      const int row_pairs = (Ho + 1) / 2, col_pairs = (Wo + 1) / 2;
+      const long count = (long)planes * row_pairs * col_pairs;
+      max_pool_3x3s2_quad_kernel<<<ceil_div(count, 256), 256, 0, st>>>(a, row_pairs, col_pairs, count);
+    } else if (kh == 3 && kw == 3 && sh == 2 && sw == 2) launch_max_pool_fixed<3, 3, 2, 2>(a, planes, st);
     else if (kh == 2 && kw == 2 && sh == 2 && sw == 2) launch_max_pool_fixed<2, 2, 2, 2>(a, planes, st);
     else if (kh == 3 && kw == 3 && sh == 1 && sw == 1) launch_max_pool_fixed<3, 3, 1, 1>(a, planes, st);
     else done = false;

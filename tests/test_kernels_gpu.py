@@ -502,7 +502,11 @@ def test_batch_norm_batch_stats_of_few_channels(K, shape):
                                       ((7, 7), 7, 1, 0), ((6, 6), 2, 2, 1), ((9, 13), 3, 3, 1),
                                       # fixed-window max kernels: odd output heights, padding, 1-wide maps
                                       ((10, 7), 2, 2, 0), ((13, 9), 3, 2, 0), ((5, 9), 3, 2, 1), ((6, 1), 3, 1, 1),
-                                      ((3, 3), 3, 2, 0), ((300, 300), 2, 2, 0)])
+                                      ((3, 3), 3, 2, 0), ((300, 300), 2, 2, 0),
+                                      # MAX 3x3/2 on widths that are multiples of 4 (2 x 2 outputs per thread):
+                                      # odd and even output extents, the clipped last window, one block only
+                                      ((9, 12), 3, 2, 0), ((10, 16), 3, 2, 0), ((3, 4), 3, 2, 0), ((4, 8), 3, 2, 0),
+                                      ((56, 56), 3, 2, 0)])
 def test_pooling(K, method, hw, k, s, p):
     x = np.random.default_rng(5).standard_normal((2, 5) + hw).astype(np.float32)
     want = oracle.pooling(x, method, (k, k), (s, s), (p, p))
