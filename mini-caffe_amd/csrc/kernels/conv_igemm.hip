@@ -38,7 +38,7 @@ constexpr int LDK = BK + 4;  // LDS row pitch in floats
 
 typedef float acc16 __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-constexpr int kModeMasks = 0, kModeOneMask = 1, kModePointwise = 2;
+constexpr int kModeMasks = 0, kModeOneMask = 1, kModePointwise = 2, kModePointwiseQuad = 3;
 // Buffer descriptor word 3 for raw dword access on gfx9-family CDNA parts
 // (32-bit data format, no swizzle, offsets checked against num_records).
 constexpr int kBufferFlags = 0x00020000;
@@ -125,7 +125,12 @@ __device__ __forceinline__ float apply_act(float v, int act, float slope) {
 //                  (channel block of 4, tap, channel in block), so the four
 //                  rows a thread gathers per step share one tap and one
 //                  validity test;
-//   kModePointwise no table and no mask, see below.
+//   kModePointwise no table and no mask, see below;
+//   kModePointwiseQuad  the same for stride 1 on planes of a multiple of four pixels with
+//                  K a multiple of 16 (64-pixel tile only): a thread fetches four
+//                  consecutive pixels of one channel with one 16-byte load instead of
+//                  one pixel of four channels with four loads, and transposes them on
+//                  the way into LDS (four 4-byte stores).  Same products, same order.
 // Pointwise: every row k of the gather is channel k of the bottom blob
 // at the thread's own pixel (1x1 kernel, no padding), so the K loop needs no
 // tap table and no bounds handling at all.
@@ -204,11 +209,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
   const int pj = tid % BN;
   const int prow = tid / BN;  // wave-uniform because BN >= 64
   // byte offset of the pixel's origin from the descriptor base (never negative)
-  constexpr bool PW = MODE == kModePointwise;
+  constexpr bool PW4 = MODE == kModePointwiseQuad;  // pointwise, stride 1: four pixels of a channel per load
+  constexpr bool PW = MODE == kModePointwise || PW4;
+  static_assert(!PW4 || (BN == 64 && KS == 1), "the pixel-quad gather is built for the 64-pixel tile");
   unsigned xvoff = PW ? kNoElement : 0u;
   unsigned row_bad = 0xFFFFFFFFu, col_bad = 0xFFFFFFFFu;
   {
-    const int p = nt * BN + pj;
+    // PW4: thread = (K row tid % 16, pixel quad tid / 16); the plane is a multiple of four
+    // pixels, so a quad never straddles two images
+    const int p = PW4 ? nt * BN + 4 * (tid >> 4) : nt * BN + pj;
     if (p < a.P) {
       const int n = fast_div(p, a.div_hw_mul, a.div_hw_shift);
       const int rem = p - n * a.HqWq;
@@ -218,6 +227,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
       const int wi0 = qw * a.q_sw + a.in_ow;
       xvoff = static_cast<unsigned>(
           ((n * a.x_nstride + g * a.x_gstride + hi0 * a.W + wi0) << 2) + a.pix_shift);
+      if constexpr (PW4) xvoff += static_cast<unsigned>(tid & 15) * (static_cast<unsigned>(a.x_cstride) * 4u);
       if constexpr (!PW) {
         row_bad = 0x80000000u;  // bit 31: the tap of K padding rows, never valid
         col_bad = 0u;
@@ -287,7 +297,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
     _Pragma("unroll") for (int i = 0; i < B_Q; ++i) {                                        \
       const int krow =                                                                       \
           __builtin_amdgcn_readfirstlane(kt16 * BK + (i * ROWS_PER_PASS + prow) * 4);        \
-      if constexpr (PW) {                                                                    \
+      if constexpr (PW4) {                                                                   \
+        /* K is a multiple of 16 here: no padding rows */                                    \
+        const u32x4 q4 = __builtin_amdgcn_raw_buffer_load_b128(                              \
+            xres, xvoff, static_cast<unsigned>(kt16 * BK) * x_cbytes, 0);                    \
+        breg[ks][i] = __builtin_bit_cast(float4, q4);                                        \
+      } else if constexpr (PW) {                                                             \
         /* padding rows re-read the last channel; their filter rows are zero */              \
         breg[ks][i].x = MC_LOADF(xres, xvoff, static_cast<unsigned>(min(krow, kmax)) * x_cbytes);\
         breg[ks][i].y =                                                                          \
@@ -324,8 +339,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
         *reinterpret_cast<float4*>(&As[buf][ks][f / QUADS][(f % QUADS) * 4]) = areg[ks][i];  \
     }                                                                                        \
     _Pragma("unroll") for (int i = 0; i < B_Q; ++i) {                                        \
-      *reinterpret_cast<float4*>(&Bs[buf][ks][pj][(i * ROWS_PER_PASS + prow) * 4]) =         \
-          breg[ks][i];                                                                       \
+      if constexpr (PW4) {                                                                   \
+        float* col = &Bs[buf][ks][4 * (tid >> 4)][tid & 15];                                 \
+        col[0] = breg[ks][i].x;                                                              \
+        col[LDK] = breg[ks][i].y;                                                            \
+        col[2 * LDK] = breg[ks][i].z;                                                        \
+        col[3 * LDK] = breg[ks][i].w;                                                        \
+      } else {                                                                               \
+        *reinterpret_cast<float4*>(&Bs[buf][ks][pj][(i * ROWS_PER_PASS + prow) * 4]) =       \
+            breg[ks][i];                                                                     \
+      }                                                                                      \
     }                                                                                        \
   }
   // One MFMA K step multiplies k-pairs; which two physical k rows form a pair
@@ -730,7 +753,7 @@ struct TileConfig {
   int bm, bn;
   int ks;  // 16-row K tiles per stage
   const char* name;
-  void (*kernel[3])(const IgemmBatch);  // indexed by kModeMasks / kModeOneMask / kModePointwise
+  void (*kernel[4])(const IgemmBatch);  // indexed by mode; [3] (pixel-quad pointwise) may be null
 };
 
 const TileConfig kConfigs[] = {
@@ -745,7 +768,7 @@ const TileConfig kConfigs[] = {
       igemm_kernel<64, 128, 2, 2, 5, kModePointwise, 1>}},
     {64, 64, 1, "igemm_f32_64x64",
      {igemm_kernel<64, 64, 2, 2, 8, kModeMasks, 1>, igemm_kernel<64, 64, 2, 2, 8, kModeOneMask, 1>,
-      igemm_kernel<64, 64, 2, 2, 8, kModePointwise, 1>}},
+      igemm_kernel<64, 64, 2, 2, 8, kModePointwise, 1>, igemm_kernel<64, 64, 2, 2, 8, kModePointwiseQuad, 1>}},
     {32, 128, 1, "igemm_f32_32x128",
      {igemm_kernel<32, 128, 1, 4, 4, kModeMasks, 1>, igemm_kernel<32, 128, 1, 4, 4, kModeOneMask, 1>,
       igemm_kernel<32, 128, 1, 4, 4, kModePointwise, 1>}},
@@ -1227,12 +1250,15 @@ int conv_forward_images(const mcConvPlan* plan, int num, const float* bottom, fl
   long total_blocks = 0;
   int min_kt = 1 << 30;
   bool pointwise = !plan->force_general, one_mask = !plan->force_general;
+  bool quad_ok = true;  // stride-1 pointwise on planes of a multiple of four pixels, K a multiple of 16
   double flops = 0.;
   for (const SubProblem* s : live) {
     const long pixels = (long)num * s->Hq * s->Wq;
     total_blocks += (long)MT * ceil_div(pixels, cfg.bn) * g.group;
     if (s->Kpad > 0) min_kt = std::min(min_kt, s->Kpad / (BK * cfg.ks));
     pointwise = pointwise && s->pointwise;
+    quad_ok = quad_ok && s->q_sh == 1 && s->q_sw == 1 && s->Hq == g.height_in && s->Wq == g.width_in &&
+              (s->Hq * s->Wq) % 4 == 0 && s->K % 16 == 0 && s->in_oh == 0 && s->in_ow == 0;
     one_mask = one_mask && s->one_mask;
     flops += 2.0 * pixels * plan->M * g.group * s->K;
   }
@@ -1351,8 +1377,9 @@ int conv_forward_images(const mcConvPlan* plan, int num, const float* bottom, fl
         const long want = (160L * 1024 / limit) / 1024 * 1024;
         if (limit < 8 && want > stat) extra_lds = static_cast<unsigned>(want - stat);
       }
-      cfg.kernel[pointwise ? kModePointwise : (one_mask ? kModeOneMask : kModeMasks)]<<<grid, 256, extra_lds, st>>>(
-          batch);
+      int mode = pointwise ? kModePointwise : (one_mask ? kModeOneMask : kModeMasks);
+      if (pointwise && quad_ok && cfg.kernel[kModePointwiseQuad]) mode = kModePointwiseQuad;
+      cfg.kernel[mode]<<<grid, 256, extra_lds, st>>>(batch);
     }
     MC_LAUNCH_CHECK();
   }

@@ -307,11 +307,16 @@ def _run_plan(K, plan, n, x, wt, out_shape, **ep):
 @pytest.mark.parametrize("case", [
     # cin, h, w, cout, stride, batch: 1x1 kernels without padding
     (64, 14, 14, 256, 1, 3), (256, 14, 14, 128, 2, 2), (100, 1, 1, 1000, 1, 7), (40, 9, 7, 24, 1, 2),
-    (70, 5, 5, 64, 3, 2)])
+    (70, 5, 5, 64, 3, 2),
+    # stride 1, plane a multiple of four pixels, channels a multiple of 16: four pixels per load;
+    # tiles that straddle images (plane 20), a ragged last tile, then planes and channel counts
+    # that rule the form out
+    (32, 4, 5, 40, 1, 7), (48, 6, 6, 70, 1, 3), (16, 8, 8, 16, 1, 1), (32, 7, 7, 40, 1, 3), (24, 4, 4, 40, 1, 3)])
 def test_conv_pointwise_path_equals_tap_table_path(K, case):
-    """A 1x1 unpadded convolution takes a K loop without tap table; pinned to the
-    general loop (configuration + 100) it must give the same bits: both add the
-    same products in the same order."""
+    """A 1x1 unpadded convolution takes a K loop without tap table (in two forms: one
+    pixel of four channels, or four pixels of one channel per thread); pinned to the
+    general loop (configuration + 100) it must give the same bits: all add the same
+    products in the same order."""
     cin, h, w, cout, s, n = case
     rng = np.random.default_rng(3)
     x = rng.standard_normal((n, cin, h, w)).astype(np.float32)
