@@ -389,6 +389,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
   const int l32 = lane & 31;
   const int lhi = lane >> 5;
 
+  // Per-channel factors of the epilogue: thread t < BM fetches the scale of
+  // row t of this tile, thread BM + t its shift, before the K loop; after the
+  // loop they pass through the then idle A tile so that a lane reads the four
+  // consecutive rows of an accumulator group with one 16-byte LDS read instead
+  // of eight buffer loads.
+  float ep_val = tid < BM ? 1.f : 0.f;
+  {
+    const float* src = tid < BM ? a.scale : a.shift;
+    const int row = mt * BM + (tid < BM ? tid : tid - BM);
+    if (tid < 2 * BM && src != nullptr && row < a.M) ep_val = src[g * a.M + row];
+  }
+
   if (kt_end > kt_begin) {
     // Tile kt_begin + t sits in LDS buffer t % 2; the loads of the next tile
     // are in flight while the MFMA block of the current one runs.
@@ -444,15 +456,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
       __builtin_amdgcn_make_buffer_rsrc(yout, 0, a.y_bytes, kBufferFlags);
   const __amdgpu_buffer_rsrc_t rres = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<float*>(a.residual), 0, has_res ? a.y_bytes : 0, kBufferFlags);
-  const __amdgpu_buffer_rsrc_t sres = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<float*>(a.scale), 0, has_scale ? a.c_bytes : 0, kBufferFlags);
-  const __amdgpu_buffer_rsrc_t hres = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<float*>(a.shift), 0, has_shift ? a.c_bytes : 0, kBufferFlags);
   // 0: none, 1: ReLU (max with 0), 2: leaky ReLU, 3: TanH / Sigmoid
   const int act_mode = a.act == MC_ACT_NONE ? 0
                        : a.act == MC_ACT_RELU ? (a.slope == 0.f ? 1 : 2)
                                               : 3;
   const unsigned cs4 = static_cast<unsigned>(a.y_cstride) * 4;
+  float* ep = &As[0][0][0][0];
+  static_assert(2 * BM <= 256 && 2 * BM <= 2 * KS * BM * LDK, "factors must fit the A tile");
+  if (has_scale | has_shift) {
+    __syncthreads();  // every wave is done reading the last A tile
+    if (tid < 2 * BM) ep[tid] = ep_val;
+    __syncthreads();
+  }
 #define MC_ROW(r) (8 * ((r) / 4) + ((r) % 4))
 #define MC_LOADF(res, voff, soff) \
   __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(res, voff, soff, 0))
@@ -478,7 +493,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
       if (mblock + 32 <= a.M) {
         // All 32 rows are real channels.
         const unsigned c0 = g * a.M + m0;
-        const unsigned c_voff = c0 * 4;
         const unsigned y_voff =
             p < a.P ? static_cast<unsigned>(ybase + c0 * a.y_cstride) * 4 : kNoElement;
 #pragma unroll
@@ -486,11 +500,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
           if (has_scale | has_shift) {
             float sc[8], sh[8];
 #pragma unroll
-            for (int q = 0; q < 8; ++q) {
-              sc[q] = 1.f;
-              sh[q] = 0.f;
-              if (has_scale) sc[q] = MC_LOADF(sres, c_voff, MC_ROW(half * 8 + q) * 4);
-              if (has_shift) sh[q] = MC_LOADF(hres, c_voff, MC_ROW(half * 8 + q) * 4);
+            for (int qq = 0; qq < 2; ++qq) {
+              const int lrow = wm0 + i * 32 + 4 * lhi + 8 * (half * 2 + qq);
+              const float4 s4 = *reinterpret_cast<const float4*>(ep + lrow);
+              const float4 h4 = *reinterpret_cast<const float4*>(ep + BM + lrow);
+              sc[qq * 4 + 0] = s4.x; sc[qq * 4 + 1] = s4.y; sc[qq * 4 + 2] = s4.z; sc[qq * 4 + 3] = s4.w;
+              sh[qq * 4 + 0] = h4.x; sh[qq * 4 + 1] = h4.y; sh[qq * 4 + 2] = h4.z; sh[qq * 4 + 3] = h4.w;
             }
 #pragma unroll
             for (int q = 0; q < 8; ++q)
