@@ -81,6 +81,13 @@ struct IgemmArgs {
   int MT, NT;         // tile counts
   int kt_per_split;   // K tiles per blockIdx.z slice (split-K)
   int split_stride;   // elements between the partial outputs of two slices
+  // Slices summed inside the launch (counters != nullptr): every workgroup leaves
+  // its accumulators in `partial` ([slice][tile][register][thread])
+  // and counts in counters[tile]; the last one to arrive adds the slices in slice
+  // order, runs the epilogue and puts the counter back to zero.
+  float* partial;
+  int* counters;
+  int partial_tiles;  // tiles per slice in `partial`
   int act;
   float slope;
 };
@@ -251,8 +258,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
     }
   }
   const int KT = a.Kpad / (BK * KS);  // stages
-  // Split-K: slice z multiplies K stages [kt_begin, kt_end) and writes its
-  // partial sums into its own copy of the top blob.
+  // Split-K: slice z multiplies K stages [kt_begin, kt_end); its partial sums go
+  // to the workspace the last workgroup of the tile adds up (IgemmArgs::partial)
+  // or, for a launch with two tops, into its own copy of the top blob.
   const int kt_begin = kslice * a.kt_per_split;
   const int kt_end = min(KT, kt_begin + a.kt_per_split);
   float* __restrict__ yout = a.y + (size_t)kslice * a.split_stride;
@@ -442,6 +450,58 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 #undef MC_STORE_TILES
 #undef MC_COMPUTE
 
+  if (a.counters != nullptr) {
+    // K slices summed here: see IgemmArgs::partial.  The partial sums and the
+    // counter are accessed with device-scope atomic operations only (relaxed
+    // stores and loads that go past the per-XCD L2, which is not coherent with
+    // the other seven), so no cache write-back or invalidation is needed: a
+    // workgroup waits until its own stores have completed and then counts.
+    const int tile_id = (sub_index * gridDim.y + g) * gridDim.x + blockIdx.x;
+    constexpr int kRegs = TM * TN * 16;  // accumulator registers per thread
+    float* mine = a.partial +
+                  (static_cast<size_t>(kslice) * a.partial_tiles + tile_id) * (kRegs * 256) + tid;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          __hip_atomic_store(mine + ((i * TN + j) * 16 + r) * 256, acc[i][j][r], __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's partial sums have arrived
+    __syncthreads();  // ... every thread's, and every wave is done with the tiles in LDS
+    int* arrived = reinterpret_cast<int*>(&As[0][0][0][0]);
+    if (tid == 0)
+      arrived[0] = __hip_atomic_fetch_add(&a.counters[tile_id], 1, __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (arrived[0] != batch.slices - 1) return;  // uniform over the workgroup
+    // the next launch on this stream starts from zero
+    if (tid == 0)
+      __hip_atomic_store(&a.counters[tile_id], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const float* part = a.partial + static_cast<size_t>(tile_id) * (kRegs * 256) + tid;
+    const size_t slice_elems = static_cast<size_t>(a.partial_tiles) * (kRegs * 256);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          acc[i][j][r] = __hip_atomic_load(part + ((i * TN + j) * 16 + r) * 256, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+    for (int z = 1; z < batch.slices; ++z) {
+      part += slice_elems;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            acc[i][j][r] += __hip_atomic_load(part + ((i * TN + j) * 16 + r) * 256, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+
   // Epilogue.  Accumulator register r of lane l holds row 8*(r/4)+4*(l/32)+r%4,
   // column l%32 of its 32x32 block; a half-wave therefore stores 32 consecutive
   // pixels of one output channel.  Like the K loop it addresses through buffer
@@ -551,62 +611,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 #undef MC_STORE_ROWS
 }
 
-// Split-K tail: y = act((sum over slices, in slice order) * scale[c] + shift[c]
-// + residual), c = (i / cstride) % C.  One thread per four consecutive elements.
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(
-    const float* __restrict__ part, int slices, long slice_stride, long count,
-    float* __restrict__ y, const float* __restrict__ scale, const float* __restrict__ shift,
-    const float* __restrict__ residual, int cstride, int C, int act, float slope) {
-  const long i4 = (blockIdx.x * (long)blockDim.x + threadIdx.x) * 4;
-  if (i4 >= count) return;
-  float v[4];
-  if (i4 + 4 <= count) {
-    float4 s = *reinterpret_cast<const float4*>(part + i4);
-    for (int z = 1; z < slices; ++z) {
-      const float4 t = *reinterpret_cast<const float4*>(part + z * slice_stride + i4);
-      s.x += t.x;
-      s.y += t.y;
-      s.z += t.z;
-      s.w += t.w;
-    }
-    v[0] = s.x;
-    v[1] = s.y;
-    v[2] = s.z;
-    v[3] = s.w;
-  } else {
-    for (int e = 0; e < 4; ++e) {
-      v[e] = 0.f;
-      if (i4 + e < count) {
-        v[e] = part[i4 + e];
-        for (int z = 1; z < slices; ++z) v[e] += part[z * slice_stride + i4 + e];
-      }
-    }
-  }
-  const bool full = i4 + 4 <= count;
-  float4 res = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (residual && full) res = *reinterpret_cast<const float4*>(residual + i4);
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    const long i = i4 + e;
-    if (i >= count) break;
-    const int c = static_cast<int>((i / cstride) % C);
-    float r = v[e];
-    if (scale) r *= scale[c];
-    if (shift) r += shift[c];
-    if (residual) r += full ? f4at(res, e) : residual[i];
-    v[e] = apply_act(r, act, slope);
-  }
-  if (full) {
-    *reinterpret_cast<float4*>(y + i4) = make_float4(v[0], v[1], v[2], v[3]);
-  } else {
-    for (int e = 0; e < 4 && i4 + e < count; ++e) y[i4 + e] = v[e];
-  }
-}
-
-// The same tail for a launch whose output channels belong to two blobs (two
-// sibling layers computed together): channels [0, c_first) of every image go to
-// y_first [num, c_first, plane], the others to y_second.  One thread per element;
-// such outputs are small (detection heads).
+// Split-K tail for a launch whose output channels belong to two blobs (two
+// sibling layers computed together): v = act((sum over slices, in slice order) *
+// scale[c] + shift[c]); channels [0, c_first) of every image go to y_first
+// [num, c_first, plane], the others to y_second.  One thread per element; such
+// outputs are small (detection heads).
 __global__ __launch_bounds__(256) void splitk_reduce_two_kernel(
     const float* __restrict__ part, int slices, long slice_stride, long count,
     float* __restrict__ y_first, float* __restrict__ y_second, int c_first,
@@ -878,7 +887,7 @@ int pick_config(const mcConvPlan* plan, long pixels) {
 // 8 workgroup slots per CU empty, and a lone workgroup pays the full global
 // load latency on every K tile; slicing K brings the launch up to about one
 // full round of workgroups, each slice still long enough to amortise its
-// prologue and the extra pass that sums the slices.
+// prologue and the summing of the slices.
 // A handful of output channels over many pixels goes to the per-pixel kernel.
 bool use_thin(const mcConvPlan* plan, int num) {
   long total_pixels = 0;
@@ -1207,7 +1216,7 @@ namespace {
 
 // top_second != nullptr: the plan's output channels [0, c_first) go to `top`, the
 // others to top_second.
-// One launch (plus the pass that sums K slices) over `num` images that fit the
+// One launch (plus, for two tops, the pass that sums K slices) over `num` images that fit the
 // kernels' 31-bit byte offsets; conv_forward() cuts larger batches into such runs.
 int conv_forward_images(const mcConvPlan* plan, int num, const float* bottom, float* top,
                         const mcEpilogue* ep, void* stream, float* top_second, int c_first) {
@@ -1281,14 +1290,33 @@ int conv_forward_images(const mcConvPlan* plan, int num, const float* bottom, fl
   // (the per-pixel kernel writes one top only)
   const bool thin = !top_second && use_thin(plan, num);
   // slices are chosen for the plan as a whole: all sub-problems of a launch run
-  // side by side, and one pass sums the slices of the whole top blob
+  // side by side
   // Two tops are told apart by the pass that sums the slices, so such a launch
   // has at least two of them (a slice past the last K tile adds zeros).
   int slices = thin ? 1 : pick_split(plan, total_blocks, min_kt);
   if (top_second && slices == 1) slices = 2;
   const long slice_stride = (out_count + 3) / 4 * 4;
   float* ws = nullptr;
-  if (slices > 1 && stream_workspace(st, sizeof(float) * slice_stride * slices, &ws)) return -1;
+  // One top: the slices are summed inside the launch by the last workgroup of each
+  // tile.  Two tops: a pass of its own sums them and tells the tops apart.
+  const bool sum_in_launch = slices > 1 && !top_second;
+  int* counters = nullptr;
+  long partial_tiles = 0;
+  if (sum_in_launch) {
+    for (size_t first = 0; first < live.size(); first += kMaxSubs) {
+      const size_t nsub = std::min<size_t>(kMaxSubs, live.size() - first);
+      long most = 0;
+      for (size_t i = 0; i < nsub; ++i)
+        most = std::max<long>(most, (long)MT * ceil_div((long)num * live[first + i]->Hq * live[first + i]->Wq,
+                                                         cfg.bn));
+      partial_tiles = std::max<long>(partial_tiles, most * g.group * (long)nsub);
+    }
+    MC_REQUIRE(partial_tiles < (1L << 31), "mcConvForward: grid too large");
+    if (stream_workspace(st, sizeof(float) * partial_tiles * cfg.bm * cfg.bn * slices, &ws)) return -1;
+    if (stream_counters(st, static_cast<size_t>(partial_tiles), &counters)) return -1;
+  } else if (slices > 1) {
+    if (stream_workspace(st, sizeof(float) * slice_stride * slices, &ws)) return -1;
+  }
 
   TimedLaunch tl;
   if (g_timing) {
@@ -1367,7 +1395,14 @@ int conv_forward_images(const mcConvPlan* plan, int num, const float* bottom, fl
       // of a short sub-problem write zeros
       a.kt_per_split = ceil_div(std::max(s.Kpad / (BK * cfg.ks), 1), slices);
       a.split_stride = 0;
-      if (slices > 1) {
+      a.partial = nullptr;
+      a.counters = nullptr;
+      a.partial_tiles = 0;
+      if (sum_in_launch) {
+        a.partial = ws;
+        a.counters = counters;
+        a.partial_tiles = static_cast<int>(partial_tiles);
+      } else if (slices > 1) {
         a.y = ws;
         a.split_stride = static_cast<int>(slice_stride);
         a.scale = a.shift = a.residual = nullptr;
@@ -1403,12 +1438,6 @@ int conv_forward_images(const mcConvPlan* plan, int num, const float* bottom, fl
         ws, slices, slice_stride, out_count, top_first, top_second, c_first, ep ? ep->scale : nullptr,
         ep ? ep->shift : nullptr, plan->Ho * plan->Wo, g.channels_out,
         ep ? ep->activation : MC_ACT_NONE, ep ? ep->negative_slope : 0.f);
-    MC_LAUNCH_CHECK();
-  } else if (slices > 1) {
-    splitk_reduce_kernel<<<static_cast<unsigned>(ceil_div(out_count, 1024L)), 256, 0, st>>>(
-        ws, slices, slice_stride, out_count, top, ep ? ep->scale : nullptr,
-        ep ? ep->shift : nullptr, ep ? ep->residual : nullptr, plan->Ho * plan->Wo,
-        g.channels_out, ep ? ep->activation : MC_ACT_NONE, ep ? ep->negative_slope : 0.f);
     MC_LAUNCH_CHECK();
   }
   if (g_timing) {

@@ -62,6 +62,11 @@ inline int ew_blocks(long n, int threads, int per_thread = 1) {
 // share it.  Growing frees the old buffer, which waits for the device.
 int stream_workspace(hipStream_t st, size_t bytes, float** out);
 
+// Arrival counters for kernels whose workgroups hand work to the last one to
+// finish: one grow-only array of ints per (host thread, stream), zero when it is
+// handed out.  A kernel that counts in it leaves every counter at zero again.
+int stream_counters(hipStream_t st, size_t count, int** out);
+
 }  // namespace mchip
 
 #endif  // MCHIP_COMMON_H_

@@ -336,8 +336,8 @@ def test_conv_pointwise_path_equals_tap_table_path(K, case):
 @pytest.mark.parametrize("slices", [2, 3, 5, 64])
 @pytest.mark.parametrize("geom", [(96, 14, 14, 64, 3, 1, 1), (512, 7, 7, 96, 1, 1, 0), (20, 6, 5, 40, 3, 2, 1)])
 def test_conv_split_k_with_epilogue(K, geom, slices):
-    """K cut into slices whose partial sums a second kernel adds in slice order,
-    then scale, shift, residual and activation: against the oracle and against
+    """K cut into slices whose partial sums the last workgroup of each tile adds in slice
+    order, then scale, shift, residual and activation: against the oracle and against
     the unsliced launch (slices beyond the K tile count are clamped)."""
     cin, h, w, cout, k, s, p = geom
     n = 2
@@ -358,6 +358,46 @@ def test_conv_split_k_with_epilogue(K, geom, slices):
     assert netrun.rel_err(outs[0], want) < 1e-4
     assert netrun.rel_err(outs[1], want) < 1e-4
     assert netrun.rel_err(outs[1], outs[0]) < 1e-4   # summation order only
+
+
+def test_conv_slices_summed_in_launch_over_many_launches(K):
+    """The last workgroup of a tile to arrive adds the K slices of all of them, out of a
+    workspace and arrival counters that every sliced launch on the stream shares: 60
+    launches in a row, alternating between three geometries and slice counts with new
+    values each time, must each equal the launch whose slices a separate pass adds
+    (two tops: bit for bit, same partial sums in the same order) and agree with the
+    unsliced launch (summation order only).  A partial sum read before it arrived, or
+    left over from an earlier launch, would be off by whole terms."""
+    cases = [((64, 14, 14, 128, 3, 1, 1), 4, 5), ((256, 7, 7, 64, 1, 1, 0), 8, 3), ((32, 20, 12, 96, 3, 2, 1), 2, 9)]
+    plans = []
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    for geom, slices, n in cases:
+        cin, h, w, cout, k, s, p = geom
+        ho, wo = (h + 2 * p - k) // s + 1, (w + 2 * p - k) // s + 1
+        wd = torch.randn(cout, cin, k, k, device="cuda", generator=gen) * 0.1
+        pl = [K.ConvPlan(K.conv_geom(*geom)) for _ in range(3)]
+        for q in pl:
+            q.set_weights(wd.data_ptr())
+        pl[0].force_split(slices)
+        pl[1].force_split(slices)
+        pl[2].force_split(1)
+        plans.append((pl, wd, (n, cin, h, w), (n, cout, ho, wo)))
+    for it in range(60):
+        pl, wd, xs, ys = plans[it % 3]
+        n, cout = ys[0], ys[1]
+        xd = torch.randn(*xs, device="cuda", generator=gen)
+        bd = torch.randn(cout, device="cuda", generator=gen)
+        whole = torch.full(ys, float("nan"), device="cuda")
+        first = torch.full((n, 40) + ys[2:], float("nan"), device="cuda")
+        second = torch.full((n, cout - 40) + ys[2:], float("nan"), device="cuda")
+        plain = torch.full(ys, float("nan"), device="cuda")
+        pl[0].forward(n, xd.data_ptr(), whole.data_ptr(), shift=bd.data_ptr(), activation=K_ACT_RELU)
+        pl[1].forward_two_tops(n, xd.data_ptr(), first.data_ptr(), 40, second.data_ptr(),
+                               shift=bd.data_ptr(), activation=K_ACT_RELU)
+        pl[2].forward(n, xd.data_ptr(), plain.data_ptr(), shift=bd.data_ptr(), activation=K_ACT_RELU)
+        torch.cuda.synchronize()
+        assert torch.equal(first, whole[:, :40]) and torch.equal(second, whole[:, 40:]), it
+        assert netrun.rel_err(whole.cpu().numpy(), plain.cpu().numpy()) < 1e-4, it
 
 
 @pytest.mark.parametrize("act,slope", [("none", 0.0), ("relu", 0.0), ("relu", 0.2), ("tanh", 0.0),
