@@ -120,9 +120,10 @@ const char* mcConvPlanKernelName(const mcConvPlan* plan, int num);
 int mcConvPlanForceConfig(mcConvPlan* plan, int config);
 
 /* Tuning/test knob: pin the number of K slices a launch is cut into (the
- * slices' partial sums are added in slice order by a second kernel that also
- * applies the epilogue); 0 restores the automatic choice, which slices only
- * launches too small to fill the GPU.  No counterpart in the reference. */
+ * slices' partial sums are added in slice order, by the last workgroup of each
+ * tile to finish or, for two tops, by a second kernel, before the epilogue);
+ * 0 restores the automatic choice, which slices only launches too small to
+ * fill the GPU.  No counterpart in the reference. */
 int mcConvPlanForceSplit(mcConvPlan* plan, int slices);
 
 /* Tuning/test knob: a batch whose bottom or top blob reaches 2^29 elements is cut
