@@ -119,6 +119,20 @@ __device__ __forceinline__ float jaccard(const DBox& a, const DBox& b) {
   return 0.f;
 }
 
+// !(JaccardOverlap(a, b) <= thr) in straight-line code: the quotient is formed for
+// every pair and used only where the intersection has positive width and height.
+// Without the reference's early return for disjoint boxes the intersection's width
+// or height comes out negative there (fmaxf / fminf ignore a NaN operand, and the
+// comparison that found the boxes disjoint had none), which is overlap 0 as well.
+__device__ __forceinline__ bool overlap_rejects(const DBox& a, const DBox& b, float thr) {
+  const float iw = fminf(a.xmax, b.xmax) - fmaxf(a.xmin, b.xmin);
+  const float ih = fminf(a.ymax, b.ymax) - fmaxf(a.ymin, b.ymin);
+  const float isz = iw * ih;
+  const float q = isz / (a.size + b.size - isz);
+  const float overlap = (iw > 0.f && ih > 0.f) ? q : 0.f;
+  return !(overlap <= thr);
+}
+
 constexpr int kKeptLds = 512;  // kept boxes cached in LDS; further ones are read from memory
 
 // The greedy pass of ApplyNMSFast with its adaptive threshold, by one
@@ -218,48 +232,119 @@ __global__ __launch_bounds__(kSortThreads) void det_class_nms_kernel(
                        eta, &kept_count[seg]);
 }
 
-// The greedy pass for a constant threshold (eta == 1) as a bit matrix and a scan.
-// All threads of the workgroup fill row k of `mask` with one bit per later
-// candidate r > k: set when candidate r would be rejected against a kept k, the
-// same expression the greedy pass evaluates (the overlap is symmetric in its two
-// boxes bit for bit).  Then one wavefront walks the candidates in order: lane w
-// holds word w of the "rejected" set; a candidate whose bit is clear is kept and
-// its row is OR-ed into the set.  `words` = ceil(ncand / 64) <= 64.
+// The greedy pass for a constant threshold (eta == 1), 64 candidates (a block) at a
+// time, by the whole workgroup.  "Candidate r is rejected against a kept k < r" does
+// not depend on the order of decisions when the threshold is fixed, so the tests
+// can run in parallel: a wavefront holds candidate 64 w + l in lane l, tests it
+// against a candidate k (a broadcast read) and a ballot is word w of k's row.
+//   1. the block's own rows, word `blk` only (all wavefronts, eight rows each);
+//   2. one wavefront decides the block: lane l holds row 64 blk + l, a candidate
+//      whose bit in the rejected set is clear is kept and its row is OR-ed in
+//      (scalar code, no memory access); the kept ones are written by their lanes;
+//   3. only the rows of the candidates kept in this block are evaluated against the
+//      later blocks (all wavefronts) and OR-ed into the rejected set, one word per
+//      later block.  Rows of rejected candidates are never formed.
+// State: `later[w]` = word w of the rejected set, `diag[l]`, one word of kept bits.
+constexpr int kDetCandBoxes = 1024;  // candidates whose boxes are cached in LDS
+struct BlockNmsLds {
+  unsigned long long later[kDetCandBoxes / 64];
+  unsigned long long diag[64];
+  unsigned long long keep;
+  int kept_list[64];
+};
 template <typename IT>
-__device__ __forceinline__ void greedy_nms_mask(int ncand, const IT* cand_idx, const DBox* cand_box,
-                                                unsigned long long* mask, int* kept, float nms_thr,
-                                                int* kept_count_out) {
+__device__ __forceinline__ void greedy_nms_blocks(int ncand, const IT* cand_idx,
+                                                  const DBox* cand_box, BlockNmsLds* st,
+                                                  int* kept, float nms_thr, int* kept_count_out) {
   const int words = (ncand + 63) >> 6;
-  for (int item = threadIdx.x; item < ncand * words; item += kSortThreads) {
-    const int k = item / words, w = item - k * words;
-    unsigned long long bits = 0;
-    if (64 * w + 63 > k) {
-      const DBox kb = cand_box[k];
-      const int r0 = max(64 * w, k + 1), r1 = min(64 * w + 64, ncand);
-      for (int r = r0; r < r1; ++r)
-        bits |= static_cast<unsigned long long>(!(jaccard(cand_box[r], kb) <= nms_thr)) << (r & 63);
-    }
-    mask[item] = bits;
-  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  constexpr int kWaves = kSortThreads / 64;
+  if (threadIdx.x < kDetCandBoxes / 64) st->later[threadIdx.x] = 0;
+  int nkept = 0;  // used by wavefront 0
   __syncthreads();
-  if (threadIdx.x >= 64) return;
-  const int lane = threadIdx.x;
-  unsigned rej_lo = 0, rej_hi = 0;  // word `lane` of the rejected set
-  int nkept = 0;
-  for (int r = 0; r < ncand; ++r) {
-    // the row is fetched before the decision so that its latency overlaps the test
-    const unsigned long long row = lane < words ? mask[r * words + lane] : 0ull;
-    const int w = r >> 6;
-    const unsigned half = (r & 32) ? __builtin_amdgcn_readlane(rej_hi, w)
-                                   : __builtin_amdgcn_readlane(rej_lo, w);
-    if (!((half >> (r & 31)) & 1u)) {
-      if (lane == 0) kept[nkept] = static_cast<int>(cand_idx[r]);
-      ++nkept;
-      rej_lo |= static_cast<unsigned>(row);
-      rej_hi |= static_cast<unsigned>(row >> 32);
+  for (int blk = 0; blk < words; ++blk) {
+    const int bn = min(64, ncand - 64 * blk);
+    {
+      // 1. rows of the block, word blk
+      const int r = 64 * blk + lane;
+      const bool in = r < ncand;
+      const DBox rb = cand_box[min(r, ncand - 1)];
+      constexpr int kPer = 64 / kWaves;
+#pragma unroll 1
+      for (int i0 = wave * kPer; i0 < min(wave * kPer + kPer, bn); i0 += 4) {
+        DBox kb[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) kb[q] = cand_box[64 * blk + min(i0 + q, bn - 1)];
+        unsigned long long bits[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          bits[q] = __ballot(static_cast<int>(in) & static_cast<int>(lane > i0 + q) &
+                             static_cast<int>(overlap_rejects(rb, kb[q], nms_thr)));
+        if (lane < 4 && i0 + lane < bn)
+          st->diag[i0 + lane] = lane == 0 ? bits[0] : lane == 1 ? bits[1] : lane == 2 ? bits[2] : bits[3];
+      }
     }
+    __syncthreads();
+    if (wave == 0) {
+      // 2. decide the block
+      const unsigned long long diag = st->diag[min(lane, bn - 1)];
+      const unsigned long long valid = bn >= 64 ? ~0ull : ((1ull << bn) - 1ull);
+      const unsigned long long before = st->later[blk];
+      // (readfirstlane returns a signed int: through unsigned, or the low half would sign-extend)
+      const unsigned b_lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(before));
+      const unsigned b_hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(before >> 32));
+      unsigned long long rem = (static_cast<unsigned long long>(b_hi) << 32) | b_lo;
+      unsigned long long avail = ~rem & valid, keep_bits = 0;
+      while (avail != 0) {  // wave-uniform, on the scalar unit
+        const int j = __builtin_ctzll(avail);
+        keep_bits |= 1ull << j;
+        const unsigned lo = __builtin_amdgcn_readlane(static_cast<unsigned>(diag), j);
+        const unsigned hi = __builtin_amdgcn_readlane(static_cast<unsigned>(diag >> 32), j);
+        rem |= (static_cast<unsigned long long>(hi) << 32) | lo;
+        avail = ~rem & valid & ~(((1ull << j) << 1) - 1ull);  // candidates after j
+      }
+      // the block's kept candidates, in order, by their own lanes
+      if ((keep_bits >> lane) & 1ull) {
+        const int pos = __popcll(keep_bits & ((1ull << lane) - 1ull));
+        kept[nkept + pos] = static_cast<int>(cand_idx[64 * blk + lane]);
+        st->kept_list[pos] = 64 * blk + lane;
+      }
+      nkept += __popcll(keep_bits);
+      if (lane == 0) st->keep = keep_bits;
+    }
+    if (blk + 1 == words) break;  // uniform over the workgroup
+    __syncthreads();
+    {
+      // 3. kept rows against the later blocks.  nw later words for kWaves wavefronts:
+      // with fewer words than wavefronts each word's kept rows are shared by several.
+      const int nk = __popcll(st->keep);
+      const int nw = words - blk - 1;
+      const int groups = nw >= kWaves ? 1 : kWaves / nw;  // wavefronts per word
+      for (int item = wave; item < nw * groups; item += kWaves) {
+        const int w = blk + 1 + item % nw, g = item / nw;
+        const int r = 64 * w + lane;
+        const bool in = r < ncand;
+        const DBox rb = cand_box[min(r, ncand - 1)];
+        unsigned long long acc = 0;
+#pragma unroll 1
+        for (int t0 = g; t0 < nk; t0 += 4 * groups) {
+          DBox kb[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) kb[q] = cand_box[st->kept_list[min(t0 + q * groups, nk - 1)]];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            // (no short-circuit: four straight-line overlaps the scheduler can interleave)
+            const unsigned long long bits = __ballot(
+                static_cast<int>(in) & static_cast<int>(overlap_rejects(rb, kb[q], nms_thr)));
+            if (t0 + q * groups < nk) acc |= bits;
+          }
+        }
+        if (lane == 0 && acc) atomicOr(&st->later[w], acc);
+      }
+    }
+    __syncthreads();
   }
-  if (lane == 0) *kept_count_out = nkept;
+  if (threadIdx.x == 0) *kept_count_out = nkept;
 }
 
 // The same for P <= kDetLdsMax priors: scores are keyed straight into LDS and
@@ -267,7 +352,6 @@ __device__ __forceinline__ void greedy_nms_mask(int ncand, const IT* cand_idx, c
 // the candidate list.
 constexpr int kDetLdsPer = 24;
 constexpr int kDetLdsMax = kDetLdsPer * kSortThreads;  // 12288
-constexpr int kDetCandBoxes = 1024;
 __global__ __launch_bounds__(kSortThreads) void det_class_nms_lds_kernel(
     const float* __restrict__ conf, const DBox* __restrict__ boxes, int P, int C,
     int loc_classes, int background, float conf_thr, float nms_thr, float eta, int top_k,
@@ -287,12 +371,25 @@ __global__ __launch_bounds__(kSortThreads) void det_class_nms_lds_kernel(
   if (threadIdx.x == 0) s_valid = 0;
   __syncthreads();
   int valid = 0;
-  for (int p = threadIdx.x; p < P; p += kSortThreads) {
-    const float s = conf[((size_t)i * P + p) * C + c];
-    const bool ok = s > conf_thr;
-    valid += ok;
-    s_key[p] = ok ? desc_key(s) : 0xffffffffu;  // below-threshold scores sort last
-    s_val[p] = static_cast<unsigned short>(p);
+  // eight independent loads in flight per thread: the launch is one workgroup per CU
+  constexpr int kLoads = 8;
+  for (int p0 = threadIdx.x; p0 < P; p0 += kSortThreads * kLoads) {
+    float sc[kLoads];
+#pragma unroll
+    for (int q = 0; q < kLoads; ++q) {
+      const int p = p0 + q * kSortThreads;
+      sc[q] = p < P ? conf[((size_t)i * P + p) * C + c] : 0.f;
+    }
+#pragma unroll
+    for (int q = 0; q < kLoads; ++q) {
+      const int p = p0 + q * kSortThreads;
+      if (p < P) {
+        const bool ok = sc[q] > conf_thr;
+        valid += ok;
+        s_key[p] = ok ? desc_key(sc[q]) : 0xffffffffu;  // below-threshold scores sort last
+        s_val[p] = static_cast<unsigned short>(p);
+      }
+    }
   }
   if (valid) atomicAdd(&s_valid, valid);
   __syncthreads();
@@ -328,13 +425,12 @@ __global__ __launch_bounds__(kSortThreads) void det_class_nms_lds_kernel(
   const int n_cached = min(ncand, kDetCandBoxes);
   for (int r = threadIdx.x; r < n_cached; r += kSortThreads) cand_box[r] = cls_boxes[s_val[r]];
   __syncthreads();
-  // constant threshold and a bit matrix that fits the (now free) key storage:
-  // overlaps in parallel, then a scan; otherwise the greedy pass of one wavefront
-  if (eta >= 1.f && ncand <= kDetCandBoxes &&
-      ncand * ((ncand + 63) >> 6) <= static_cast<int>(sizeof(s_key) / sizeof(unsigned long long))) {
-    greedy_nms_mask<unsigned short>(ncand, s_val, cand_box,
-                                    reinterpret_cast<unsigned long long*>(s_key),
-                                    kept_idx + (size_t)seg * max_cand, nms_thr, &kept_count[seg]);
+  // constant threshold: the workgroup's block-wise pass; otherwise the greedy pass of
+  // one wavefront
+  if (eta >= 1.f && ncand <= kDetCandBoxes) {
+    greedy_nms_blocks<unsigned short>(ncand, s_val, cand_box,
+                                      reinterpret_cast<BlockNmsLds*>(s_key),
+                                      kept_idx + (size_t)seg * max_cand, nms_thr, &kept_count[seg]);
     return;
   }
   if (threadIdx.x >= 64) return;  // the greedy pass is one wavefront

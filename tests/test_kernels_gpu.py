@@ -788,11 +788,14 @@ def test_proposal_with_few_equal_scores(K, hw, pre, post, thr, pairs, seed, gene
     (1, 2000, 21, True, "CENTER_SIZE", 200, 0.01, 0.45, 1.0, 400, 0.5),
     (1, 13000, 3, True, "CENTER_SIZE", 100, 0.01, 0.45, 1.0, 1500, 2.0),   # sort through global scratch,
                                                                            # more candidates than cached
-    # candidate counts around the limits of the bit-matrix form of the greedy pass (constant threshold)
-    (2, 3000, 3, True, "CENTER_SIZE", -1, 0.001, 0.45, 1.0, 576, 1.0),     # largest matrix that fits
-    (2, 3000, 3, True, "CENTER_SIZE", -1, 0.001, 0.45, 1.0, 577, 1.0),     # one more: one-wavefront pass
-    (2, 3000, 3, True, "CENTER_SIZE", -1, 0.001, 0.3, 1.0, 64, 1.0),       # exactly one word
+    # candidate counts around the limits of the block-wise form of the greedy pass (constant threshold)
+    (2, 3000, 3, True, "CENTER_SIZE", -1, 0.001, 0.45, 1.0, 576, 1.0),     # nine blocks: more later blocks than wavefronts
+    (2, 3000, 3, True, "CENTER_SIZE", -1, 0.001, 0.45, 1.0, 577, 1.0),     # a last block of one candidate
+    (2, 3000, 3, True, "CENTER_SIZE", -1, 0.001, 0.45, 1.0, 1024, 1.0),    # as many candidates as LDS caches
+    (2, 3000, 3, True, "CENTER_SIZE", -1, 0.001, 0.45, 1.0, 1025, 1.0),    # one more: one-wavefront pass
+    (2, 3000, 3, True, "CENTER_SIZE", -1, 0.001, 0.3, 1.0, 64, 1.0),       # exactly one block
     (2, 3000, 3, True, "CENTER_SIZE", -1, 0.001, 0.3, 1.0, 65, 1.0),
+    (1, 3000, 3, True, "CENTER_SIZE", -1, 0.001, 0.95, 1.0, 300, 1.0),     # nearly everything kept
     (2, 3000, 4, False, "CORNER", -1, 0.001, 0.7, 1.0, 1, 1.0),            # a single candidate per class
     (1, 400, 2, True, "CENTER_SIZE", -1, None, 0.05, 1.0, None, 1.0),      # low threshold: long reject chains
 ])
