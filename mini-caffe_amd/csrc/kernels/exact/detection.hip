@@ -480,16 +480,40 @@ __global__ __launch_bounds__(kSortThreads) void det_select_kernel(
     const int per = (total + kSortThreads - 1) / kSortThreads;
     const int begin = min(static_cast<int>(threadIdx.x) * per, total), end = min(begin + per, total);
     const bool in_lds = total <= kSelLdsMax;
-    int c = 0;
-    for (int e = begin; e < end; ++e) {
-      while (s_off[c + 1] <= e) ++c;
-      const int idx = kept_idx[(size_t)(i * C + c) * max_cand + (e - s_off[c])];
-      const uint32_t key = desc_key(conf[((size_t)i * P + idx) * C + c]);
-      if (in_lds) {
-        s_key[e] = key;
-        s_val[e] = static_cast<unsigned short>(e);
-      } else {
-        k0[e] = key;
+    if (in_lds) {
+      // a thread's entries: first all prior indices, then all scores, so that the
+      // thread waits for two rounds of loads and not for two per entry
+      int cls[kSelLdsPer], idx[kSelLdsPer];
+      float sc[kSelLdsPer];
+      int c = 0;
+#pragma unroll
+      for (int q = 0; q < kSelLdsPer; ++q) {
+        const int e = begin + q;
+        cls[q] = 0;
+        idx[q] = 0;
+        if (e < end) {
+          while (s_off[c + 1] <= e) ++c;
+          cls[q] = c;
+          idx[q] = kept_idx[(size_t)(i * C + c) * max_cand + (e - s_off[c])];
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < kSelLdsPer; ++q)
+        sc[q] = begin + q < end ? conf[((size_t)i * P + idx[q]) * C + cls[q]] : 0.f;
+#pragma unroll
+      for (int q = 0; q < kSelLdsPer; ++q) {
+        const int e = begin + q;
+        if (e < end) {
+          s_key[e] = desc_key(sc[q]);
+          s_val[e] = static_cast<unsigned short>(e);
+        }
+      }
+    } else {
+      int c = 0;
+      for (int e = begin; e < end; ++e) {
+        while (s_off[c + 1] <= e) ++c;
+        const int idx = kept_idx[(size_t)(i * C + c) * max_cand + (e - s_off[c])];
+        k0[e] = desc_key(conf[((size_t)i * P + idx) * C + c]);
         v0[e] = e;
       }
     }
@@ -554,38 +578,50 @@ __global__ __launch_bounds__(kSortThreads) void det_select_kernel(
   if (threadIdx.x == kSortThreads - 1) rows_count[i] = static_cast<int>(pos);
 }
 
-// Concatenates the per-image rows; with no detection at all, one row of -1 per
-// image carrying the image index (detection_output_layer.cpp:175-185).
+// Concatenates the per-image rows, one workgroup per image; with no detection at
+// all, one row of -1 per image carrying the image index
+// (detection_output_layer.cpp:175-185).
 __global__ __launch_bounds__(256) void det_emit_kernel(const float* __restrict__ rows_tmp,
                                                        const int* __restrict__ rows_count,
                                                        int num, int max_entries, int max_rows,
                                                        float* __restrict__ out,
                                                        int* __restrict__ num_rows) {
-  __shared__ int s_off[1025];
-  if (threadIdx.x == 0) {
-    int off = 0;
-    for (int i = 0; i < num; ++i) {
-      s_off[i] = off;
-      off += rows_count[i];
+  __shared__ int s_before, s_total;
+  const int i = blockIdx.x;
+  if (threadIdx.x < 64) {
+    // rows of the images before this one, and of all
+    int before = 0, total = 0;
+    for (int k = threadIdx.x; k < num; k += 64) {
+      const int c = rows_count[k];
+      total += c;
+      if (k < i) before += c;
     }
-    s_off[num] = off;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      before += __shfl_xor(before, o, 64);
+      total += __shfl_xor(total, o, 64);
+    }
+    if (threadIdx.x == 0) {
+      s_before = before;
+      s_total = total;
+    }
   }
   __syncthreads();
-  const int total = s_off[num];
+  const int total = s_total;
   if (total == 0) {
-    for (int t = threadIdx.x; t < num * 7 && t < max_rows * 7; t += 256)
-      out[t] = (t % 7 == 0) ? static_cast<float>(t / 7) : -1.f;
-    if (threadIdx.x == 0) *num_rows = num;
+    if (i == 0) {
+      for (int t = threadIdx.x; t < num * 7 && t < max_rows * 7; t += 256)
+        out[t] = (t % 7 == 0) ? static_cast<float>(t / 7) : -1.f;
+      if (threadIdx.x == 0) *num_rows = num;
+    }
     return;
   }
-  for (int i = 0; i < num; ++i) {
-    const int cnt = rows_count[i];
-    const float* src = rows_tmp + (size_t)i * max_entries * 7;
-    float* dst = out + (size_t)s_off[i] * 7;
-    for (int t = threadIdx.x; t < cnt * 7; t += 256)
-      if (s_off[i] + t / 7 < max_rows) dst[t] = src[t];
-  }
-  if (threadIdx.x == 0) *num_rows = total < max_rows ? total : max_rows;
+  const int cnt = rows_count[i], off = s_before;
+  const float* src = rows_tmp + (size_t)i * max_entries * 7;
+  float* dst = out + (size_t)off * 7;
+  for (int t = threadIdx.x; t < cnt * 7; t += 256)
+    if (off + t / 7 < max_rows) dst[t] = src[t];
+  if (i == 0 && threadIdx.x == 0) *num_rows = total < max_rows ? total : max_rows;
 }
 
 struct DetLayout {
@@ -694,7 +730,7 @@ int mcDetectionOutput(const float* loc, const float* conf, const float* prior, i
       i32(L.kept_count), u32(L.sk0), i32(L.sv0), u32(L.sk1), i32(L.sv1), i32(L.selected),
       reinterpret_cast<float*>(ws + L.rows_tmp), i32(L.rows_count), cut_tie_flag);
   MC_LAUNCH_CHECK();
-  det_emit_kernel<<<1, 256, 0, st>>>(reinterpret_cast<float*>(ws + L.rows_tmp), i32(L.rows_count),
+  det_emit_kernel<<<num, 256, 0, st>>>(reinterpret_cast<float*>(ws + L.rows_tmp), i32(L.rows_count),
                                      num, num_classes * max_cand, max_rows, out_rows, num_rows);
   MC_LAUNCH_CHECK();
   return 0;
