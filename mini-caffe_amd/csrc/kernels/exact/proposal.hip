@@ -1035,32 +1035,59 @@ __global__ __launch_bounds__(kFastThreads) void tie_replay_fast_kernel(
 
 // mask[i][cb] bit j: box cb*64+j (> i) overlaps box i by more than thr, with
 // the +1 pixel extents of NonMaximumSuppressionCPU (proposal_layer.cpp:150-185).
-__global__ __launch_bounds__(64) void nms_mask_kernel(const float4* __restrict__ boxes, int n,
-                                                      float thr, int nb,
-                                                      unsigned long long* __restrict__ mask) {
-  const int rb = blockIdx.y, cb = blockIdx.x;
-  if (cb < rb) return;
-  __shared__ float4 cols[64];
-  const int cn = min(64, n - cb * 64);
-  if (static_cast<int>(threadIdx.x) < cn) cols[threadIdx.x] = boxes[cb * 64 + threadIdx.x];
-  __syncthreads();
-  const int i = rb * 64 + threadIdx.x;
-  if (i >= n) return;
-  const float4 a = boxes[i];
-  const float area_a = (a.z - a.x + 1) * (a.w - a.y + 1);
-  unsigned long long bits = 0;
-  for (int j = 0; j < cn; ++j) {
-    if (cb * 64 + j <= i) continue;
-    const float4 b = cols[j];
+// One workgroup of four wavefronts per 64 x 64 tile on or above the diagonal: lane l
+// holds column box cb*64 + l, a wavefront takes 16 of the tile's rows (a broadcast
+// read each, four independent tests in flight) and a ballot is the row's word.
+// The tiles of the upper triangle of `tiles_side` x `tiles_side` blocks are counted row
+// by row and dealt to the workgroups of the grid in turn; `nb` = words per row of `mask`.  With `done`: returns at once
+// when *done is set.
+__global__ __launch_bounds__(256) void nms_mask_kernel(const float4* __restrict__ boxes, int n,
+                                                       float thr, int nb, int tiles_side,
+                                                       unsigned long long* __restrict__ mask,
+                                                       const int* __restrict__ done) {
+  if (done != nullptr && *done != 0) return;  // uniform
+  __shared__ float4 rows[64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int total = tiles_side * (tiles_side + 1) / 2;
+  for (int t = blockIdx.x; t < total; t += gridDim.x) {
+    // tile t of the triangle -> (rb, cb), cb >= rb: row rb starts at rb*side - rb*(rb-1)/2;
+    // the largest rb with start(rb) <= t from the quadratic, corrected a step either way
+    const float sidef = static_cast<float>(tiles_side) + 0.5f;
+    int rb = static_cast<int>(sidef - sqrtf(fmaxf(sidef * sidef - 2.f * static_cast<float>(t), 0.f)));
+    rb = max(0, min(rb, tiles_side - 1));
+    auto start = [&](int r) { return r * tiles_side - r * (r - 1) / 2; };
+    while (rb > 0 && start(rb) > t) --rb;
+    while (rb + 1 < tiles_side && start(rb + 1) <= t) ++rb;
+    const int cb = rb + (t - start(rb));
+    const int rn = min(64, n - rb * 64);
+    if (static_cast<int>(threadIdx.x) < rn) rows[threadIdx.x] = boxes[rb * 64 + threadIdx.x];
+    const int c = cb * 64 + lane;
+    const bool in = c < n;
+    const float4 b = boxes[min(c, n - 1)];
     const float area_b = (b.z - b.x + 1) * (b.w - b.y + 1);
-    const float x1 = fmaxf(a.x, b.x), y1 = fmaxf(a.y, b.y);
-    const float x2 = fminf(a.z, b.z), y2 = fminf(a.w, b.w);
-    const float w = fmaxf(0.f, x2 - x1 + 1), h = fmaxf(0.f, y2 - y1 + 1);
-    const float inter = w * h;
-    const float ov = inter / (area_a + area_b - inter);
-    if (ov > thr) bits |= 1ull << j;
+    __syncthreads();
+#pragma unroll 1
+    for (int r0 = wave * 16; r0 < min(wave * 16 + 16, rn); r0 += 4) {
+      unsigned long long bits[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int r = min(r0 + q, rn - 1);
+        const float4 a = rows[r];
+        const float area_a = (a.z - a.x + 1) * (a.w - a.y + 1);
+        const float x1 = fmaxf(a.x, b.x), y1 = fmaxf(a.y, b.y);
+        const float x2 = fminf(a.z, b.z), y2 = fminf(a.w, b.w);
+        const float w = fmaxf(0.f, x2 - x1 + 1), h = fmaxf(0.f, y2 - y1 + 1);
+        const float inter = w * h;
+        const float ov = inter / (area_a + area_b - inter);
+        bits[q] = __ballot(static_cast<int>(in) & static_cast<int>(c > rb * 64 + r) &
+                           static_cast<int>(ov > thr));
+      }
+      if (lane < 4 && r0 + lane < rn)
+        mask[static_cast<size_t>(rb * 64 + r0 + lane) * nb + cb] =
+            lane == 0 ? bits[0] : lane == 1 ? bits[1] : lane == 2 ? bits[2] : bits[3];
+    }
+    __syncthreads();  // the rows are replaced by the next tile's
   }
-  mask[(size_t)i * nb + cb] = bits;
 }
 
 // Greedy scan over the boxes in score order, one workgroup.  The decisions are a
@@ -1088,10 +1115,17 @@ __device__ inline unsigned long long wave_uniform(unsigned long long v) {
   return (static_cast<unsigned long long>(hi) << 32) | lo;
 }
 
+// `n` boxes in `nb` blocks; a row of `mask` has `stride` words.  With `done`:
+// returns at once when *done is set, and sets it when this scan settles the result
+// (`final_part`: the n boxes are all there are; otherwise only if max_keep is reached).
+// `resume`: the first super-block was decided by an earlier launch (kept[0 .. *num_kept)
+// are its boxes); this one only folds their rows into the later super-blocks and goes on.
 __global__ __launch_bounds__(kScanThreads) void nms_scan_kernel(
-    const unsigned long long* __restrict__ mask, int n, int nb, int max_keep,
-    int* __restrict__ kept, int* __restrict__ num_kept) {
+    const unsigned long long* __restrict__ mask, int n, int nb, int stride, int max_keep,
+    int* __restrict__ kept, int* __restrict__ num_kept, int* __restrict__ done, int final_part,
+    int resume) {
   extern __shared__ unsigned long long removed[];  // nb words
+  if (done != nullptr && *done != 0) return;  // uniform
   __shared__ unsigned long long sub[kScanRows * kScanBlocks];
   __shared__ int sb_kept[kScanRows];
   __shared__ int s_count, s_ns;
@@ -1102,14 +1136,23 @@ __global__ __launch_bounds__(kScanThreads) void nms_scan_kernel(
     const int r = idx / kScanBlocks, c = idx % kScanBlocks;
     const long row = static_cast<long>(base_blk) * 64 + r;
     const int col = base_blk + c;
-    return (row < n && col < nb) ? mask[row * nb + col] : 0ull;
+    return (row < n && col < nb) ? mask[row * stride + col] : 0ull;
   };
   for (int w = tid; w < nb; w += kScanThreads) removed[w] = 0;
+  if (resume) {
+    const int before = *num_kept;  // at most kScanRows: all from the first super-block
+    for (int k = tid; k < before; k += kScanThreads) sb_kept[k] = kept[k];
+    if (tid == 0) {
+      s_count = before;
+      s_ns = before;
+    }
+  } else {
 #pragma unroll
-  for (int k = 0; k < kScanLoads; ++k) sub[tid + k * kScanThreads] = fetch(0, tid + k * kScanThreads);
-  if (tid == 0) {
-    s_count = 0;
-    s_ns = 0;
+    for (int k = 0; k < kScanLoads; ++k) sub[tid + k * kScanThreads] = fetch(0, tid + k * kScanThreads);
+    if (tid == 0) {
+      s_count = 0;
+      s_ns = 0;
+    }
   }
   __syncthreads();
   for (int base_blk = 0; base_blk < nb; base_blk += kScanBlocks) {
@@ -1121,7 +1164,7 @@ __global__ __launch_bounds__(kScanThreads) void nms_scan_kernel(
       for (int k = 0; k < kScanLoads; ++k)
         ahead[k] = fetch(base_blk + kScanBlocks, tid + k * kScanThreads);
     }
-    if (decider) {
+    if (decider && !(resume && base_blk == 0)) {
       int count = __builtin_amdgcn_readfirstlane(s_count);
       int ns = 0;
       const unsigned long long* sm = sub;
@@ -1133,28 +1176,40 @@ __global__ __launch_bounds__(kScanThreads) void nms_scan_kernel(
         const unsigned long long valid = bn >= 64 ? ~0ull : ((1ull << bn) - 1ull);
         unsigned long long avail = ~rem & valid;
         unsigned long long keep_bits = 0;
-        while (avail != 0 && count < max_keep) {
+        int room = max_keep - count;
+        while (avail != 0 && room > 0) {  // scalar unit only: no memory access in the chain
           const int j = __builtin_ctzll(avail);
           keep_bits |= 1ull << j;
-          if (lane == 0) {
-            kept[count] = blk * 64 + j;
-            sb_kept[ns] = blk * 64 + j;
-          }
-          ++count;
-          ++ns;
+          --room;
           const unsigned lo = __builtin_amdgcn_readlane(static_cast<unsigned>(diag), j);
           const unsigned hi = __builtin_amdgcn_readlane(static_cast<unsigned>(diag >> 32), j);
           rem |= (static_cast<unsigned long long>(hi) << 32) | lo;
           avail = ~rem & valid & ~(((1ull << j) << 1) - 1ull);  // candidates after j
         }
-        // rows kept in this block -> later words of the same super-block
+        // the block's kept boxes, in order, written by their own lanes
+        if ((keep_bits >> lane) & 1ull) {
+          const int pos = __popcll(keep_bits & ((1ull << lane) - 1ull));
+          kept[count + pos] = blk * 64 + lane;
+          sb_kept[ns + pos] = blk * 64 + lane;
+        }
+        count += __popcll(keep_bits);
+        ns += __popcll(keep_bits);
+        // rows kept in this block -> later words of the same super-block, four reads in flight
         const int wl = b + 1 + lane;
         if (wl < kScanBlocks && base_blk + wl < nb) {
           unsigned long long acc = 0, kb = keep_bits;
+          const unsigned long long* col = sm + (b * 64) * kScanBlocks + wl;
           while (kb) {
-            const int j = __builtin_ctzll(kb);
+            const int j0 = __builtin_ctzll(kb);
             kb &= kb - 1;
-            acc |= sm[(b * 64 + j) * kScanBlocks + wl];
+            const int j1 = kb ? __builtin_ctzll(kb) : j0;
+            kb &= kb - 1;
+            const int j2 = kb ? __builtin_ctzll(kb) : j0;
+            kb &= kb - 1;
+            const int j3 = kb ? __builtin_ctzll(kb) : j0;
+            kb &= kb - 1;
+            acc |= (col[j0 * kScanBlocks] | col[j1 * kScanBlocks]) |
+                   (col[j2 * kScanBlocks] | col[j3 * kScanBlocks]);
           }
           if (acc) removed[base_blk + wl] |= acc;
         }
@@ -1182,7 +1237,7 @@ __global__ __launch_bounds__(kScanThreads) void nms_scan_kernel(
         if (p < total) {
           const int k = p / far;
           w[u] = first + (p - k * far);
-          v[u] = mask[static_cast<long>(sb_kept[k]) * nb + w[u]];
+          v[u] = mask[static_cast<long>(sb_kept[k]) * stride + w[u]];
         }
       }
 #pragma unroll
@@ -1193,7 +1248,10 @@ __global__ __launch_bounds__(kScanThreads) void nms_scan_kernel(
     for (int k = 0; k < kScanLoads; ++k) sub[tid + k * kScanThreads] = ahead[k];
     __syncthreads();
   }
-  if (tid == 0) *num_kept = s_count;
+  if (tid == 0) {
+    *num_kept = s_count;
+    if (done != nullptr && (final_part || s_count >= max_keep)) *done = 1;
+  }
 }
 
 // rois[r] = (0, x1, y1, x2, y2) of the r-th kept box (proposal_layer.cpp:187-203).
@@ -1377,11 +1435,27 @@ int run_proposal(const float* scores, const float* bbox, const float* im_info, c
                                                                    sscores);
   MC_LAUNCH_CHECK();
   MC_HIP(mark(2));
-  nms_mask_kernel<<<dim3(nb, nb), 64, 0, st>>>(sboxes, pre, nms_thresh, nb, mask);
+  // The greedy pass stops at post_nms_topn kept boxes, usually long before the last
+  // candidate: first the best kScanRows candidates among themselves (a corner of the
+  // overlap matrix, one super-block of the scan).  If that settles the result the
+  // full-size launches behind it return at once; otherwise they fill the whole matrix and
+  // the scan resumes behind the first super-block.
+  int* done = flags + 2;
+  const int head = pre < kScanRows ? pre : kScanRows, head_nb = ceil_div(head, 64);
+  nms_mask_kernel<<<head_nb * (head_nb + 1) / 2, 256, 0, st>>>(sboxes, head, nms_thresh, nb, head_nb, mask,
+                                                             nullptr);
   MC_LAUNCH_CHECK();
-  nms_scan_kernel<<<1, kScanThreads, sizeof(unsigned long long) * nb, st>>>(
-      mask, pre, nb, post_nms_topn, kept, num_rois);
+  nms_scan_kernel<<<1, kScanThreads, sizeof(unsigned long long) * head_nb, st>>>(
+      mask, head, head_nb, nb, post_nms_topn, kept, num_rois, done, head == pre, 0);
   MC_LAUNCH_CHECK();
+  if (head < pre) {
+    nms_mask_kernel<<<std::min(nb * (nb + 1) / 2, 8 * kNumCu), 256, 0, st>>>(sboxes, pre, nms_thresh, nb, nb,
+                                                                           mask, done);
+    MC_LAUNCH_CHECK();
+    nms_scan_kernel<<<1, kScanThreads, sizeof(unsigned long long) * nb, st>>>(
+        mask, pre, nb, nb, post_nms_topn, kept, num_rois, done, 1, 1);
+    MC_LAUNCH_CHECK();
+  }
   MC_HIP(mark(3));
   proposal_gather_kernel<<<ceil_div(post_nms_topn, 256), 256, 0, st>>>(sboxes, sscores, kept,
                                                                        num_rois, rois, roi_scores);
