@@ -100,13 +100,32 @@ struct BlockSortLds16 {
   uint32_t wave_sum[kSortThreads / 64];
 };
 
-template <int MAXPER, typename VT>
+template <int MAXPER, typename VT, bool SKIP_CONSTANT_DIGITS = true>
 __device__ inline void block_sort_desc_lds(uint32_t* keys, VT* vals, int n, BlockSortLds16* lds) {
   const int tid = threadIdx.x;
   const int per = (n + kSortThreads - 1) / kSortThreads;
   const int begin = min(tid * per, n), end = min(begin + per, n);
   const int cnt = end - begin;
+  // Bits in which any two keys differ: a pass over a digit that is the same in every
+  // key is the identity (the sort is stable) and is skipped.  Softmax scores over many
+  // classes share their sign and most of their exponent, which saves two of the 8
+  // passes; callers whose keys spread over all exponents switch the look-ahead off.
+  uint32_t diff = 0xffffffffu;
+  if constexpr (SKIP_CONSTANT_DIGITS) {
+    diff = 0;
+    const uint32_t first = n > 0 ? keys[0] : 0u;
+    for (int j = 0; j < cnt; ++j) diff |= keys[begin + j] ^ first;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) diff |= __shfl_xor(diff, o, 64);
+    if ((tid & 63) == 0) lds->wave_sum[tid >> 6] = diff;
+    __syncthreads();
+    diff = 0;
+#pragma unroll
+    for (int w = 0; w < kSortThreads / 64; ++w) diff |= lds->wave_sum[w];
+    __syncthreads();  // wave_sum is used again by the scans below
+  }
   for (int shift = 0; shift < 32; shift += 4) {
+    if (((diff >> shift) & 15u) == 0u) continue;  // uniform over the workgroup
     uint32_t rk[MAXPER];
     VT rv[MAXPER];
 #pragma unroll

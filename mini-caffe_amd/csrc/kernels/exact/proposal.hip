@@ -102,7 +102,8 @@ __global__ __launch_bounds__(kSortThreads) void proposal_sort_lds_kernel(
     s_val[i] = static_cast<unsigned short>(i);  // v0[i] == i on entry
   }
   __syncthreads();
-  block_sort_desc_lds<kSortLdsPer, unsigned short>(s_key, s_val, n, &lds);
+  // (foreground probabilities of a two-class softmax spread over many exponents)
+  block_sort_desc_lds<kSortLdsPer, unsigned short, false>(s_key, s_val, n, &lds);
   for (int i = threadIdx.x; i < n; i += kSortThreads) {
     k0[i] = s_key[i];
     v0[i] = s_val[i];
