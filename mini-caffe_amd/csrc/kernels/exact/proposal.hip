@@ -1045,9 +1045,11 @@ __global__ __launch_bounds__(kFastThreads) void tie_replay_fast_kernel(
 __global__ __launch_bounds__(256) void nms_mask_kernel(const float4* __restrict__ boxes, int n,
                                                        float thr, int nb, int tiles_side,
                                                        unsigned long long* __restrict__ mask,
+                                                       unsigned long long* __restrict__ colmask,
                                                        const int* __restrict__ done) {
   if (done != nullptr && *done != 0) return;  // uniform
   __shared__ float4 rows[64];
+  __shared__ unsigned long long cols[64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int total = tiles_side * (tiles_side + 1) / 2;
   for (int t = blockIdx.x; t < total; t += gridDim.x) {
@@ -1066,6 +1068,8 @@ __global__ __launch_bounds__(256) void nms_mask_kernel(const float4* __restrict_
     const bool in = c < n;
     const float4 b = boxes[min(c, n - 1)];
     const float area_b = (b.z - b.x + 1) * (b.w - b.y + 1);
+    if (threadIdx.x < 64) cols[threadIdx.x] = 0;
+    unsigned long long below = 0;  // this lane's column: the earlier boxes of the tile that overlap it
     __syncthreads();
 #pragma unroll 1
     for (int r0 = wave * 16; r0 < min(wave * 16 + 16, rn); r0 += 4) {
@@ -1080,14 +1084,22 @@ __global__ __launch_bounds__(256) void nms_mask_kernel(const float4* __restrict_
         const float w = fmaxf(0.f, x2 - x1 + 1), h = fmaxf(0.f, y2 - y1 + 1);
         const float inter = w * h;
         const float ov = inter / (area_a + area_b - inter);
-        bits[q] = __ballot(static_cast<int>(in) & static_cast<int>(c > rb * 64 + r) &
-                           static_cast<int>(ov > thr));
+        const bool hit = in & (c > rb * 64 + r) & (ov > thr);
+        bits[q] = __ballot(hit);
+        if (hit && r0 + q < rn) below |= 1ull << r;
       }
       if (lane < 4 && r0 + lane < rn)
         mask[static_cast<size_t>(rb * 64 + r0 + lane) * nb + cb] =
             lane == 0 ? bits[0] : lane == 1 ? bits[1] : lane == 2 ? bits[2] : bits[3];
     }
-    __syncthreads();  // the rows are replaced by the next tile's
+    // A diagonal tile also leaves the transposed words (the overlap is symmetric bit for
+    // bit): colmask[c] = the boxes of c's own block before c that overlap it.
+    if (colmask != nullptr && rb == cb) {
+      if (below) atomicOr(&cols[lane], below);
+      __syncthreads();
+      if (threadIdx.x < 64 && in) colmask[c] = cols[lane];
+    }
+    __syncthreads();  // rows and cols are replaced by the next tile's
   }
 }
 
@@ -1124,8 +1136,9 @@ __device__ inline unsigned long long wave_uniform(unsigned long long v) {
 __global__ __launch_bounds__(kScanThreads) void nms_scan_kernel(
     const unsigned long long* __restrict__ mask, int n, int nb, int stride, int max_keep,
     int* __restrict__ kept, int* __restrict__ num_kept, int* __restrict__ done, int final_part,
-    int resume) {
+    int resume, const unsigned long long* __restrict__ colmask) {
   extern __shared__ unsigned long long removed[];  // nb words
+  __shared__ unsigned long long subcol[kScanRows];  // colmask of the super-block's boxes
   if (done != nullptr && *done != 0) return;  // uniform
   __shared__ unsigned long long sub[kScanRows * kScanBlocks];
   __shared__ int sb_kept[kScanRows];
@@ -1150,6 +1163,8 @@ __global__ __launch_bounds__(kScanThreads) void nms_scan_kernel(
   } else {
 #pragma unroll
     for (int k = 0; k < kScanLoads; ++k) sub[tid + k * kScanThreads] = fetch(0, tid + k * kScanThreads);
+    static_assert(kScanRows == kScanThreads, "one column word per thread");
+    subcol[tid] = tid < n ? colmask[tid] : 0ull;
     if (tid == 0) {
       s_count = 0;
       s_ns = 0;
@@ -1165,28 +1180,37 @@ __global__ __launch_bounds__(kScanThreads) void nms_scan_kernel(
       for (int k = 0; k < kScanLoads; ++k)
         ahead[k] = fetch(base_blk + kScanBlocks, tid + k * kScanThreads);
     }
+    const long next_row = static_cast<long>(base_blk + kScanBlocks) * 64 + tid;
+    const unsigned long long ahead_col = (more && next_row < n) ? colmask[next_row] : 0ull;
     if (decider && !(resume && base_blk == 0)) {
       int count = __builtin_amdgcn_readfirstlane(s_count);
       int ns = 0;
       const unsigned long long* sm = sub;
       for (int b = 0; b < kScanBlocks && base_blk + b < nb && count < max_keep; ++b) {
         const int blk = base_blk + b;
-        const unsigned long long diag = sm[(b * 64 + lane) * kScanBlocks + b];
         unsigned long long rem = wave_uniform(removed[blk]);
         const int bn = min(64, n - blk * 64);
         const unsigned long long valid = bn >= 64 ? ~0ull : ((1ull << bn) - 1ull);
-        unsigned long long avail = ~rem & valid;
-        unsigned long long keep_bits = 0;
-        int room = max_keep - count;
-        while (avail != 0 && room > 0) {  // scalar unit only: no memory access in the chain
-          const int j = __builtin_ctzll(avail);
-          keep_bits |= 1ull << j;
-          --room;
-          const unsigned lo = __builtin_amdgcn_readlane(static_cast<unsigned>(diag), j);
-          const unsigned hi = __builtin_amdgcn_readlane(static_cast<unsigned>(diag >> 32), j);
-          rem |= (static_cast<unsigned long long>(hi) << 32) | lo;
-          avail = ~rem & valid & ~(((1ull << j) << 1) - 1ull);  // candidates after j
+        // The block's decisions in rounds instead of one box at a time: lane j holds the
+        // boxes of the block before j that overlap it (colmask).  A box none of whose
+        // overlapping predecessors is still open is settled: removed if one of them is
+        // kept, else kept.  The first open box always settles, so at most 64 rounds; boxes
+        // suppress few of their neighbours, so a handful.  Same result as the serial pass:
+        // a box is settled only when every box that could suppress it has been.
+        const unsigned long long before = subcol[b * 64 + lane];
+        unsigned long long open = ~rem & valid, keep_bits = 0;
+        while (open != 0) {  // wave-uniform
+          const bool mine = (open >> lane) & 1ull;
+          const bool suppressed = (before & keep_bits) != 0;
+          const bool waits = (before & open) != 0;
+          const unsigned long long now_removed = __ballot(mine && suppressed);
+          const unsigned long long now_kept = __ballot(mine && !suppressed && !waits);
+          keep_bits |= now_kept;
+          open &= ~(now_kept | now_removed);
         }
+        // the serial pass stops at max_keep kept boxes: drop the ones it would not have reached
+        for (int extra = __popcll(keep_bits) - (max_keep - count); extra > 0; --extra)
+          keep_bits &= ~(1ull << (63 - __builtin_clzll(keep_bits)));
         // the block's kept boxes, in order, written by their own lanes
         if ((keep_bits >> lane) & 1ull) {
           const int pos = __popcll(keep_bits & ((1ull << lane) - 1ull));
@@ -1195,24 +1219,46 @@ __global__ __launch_bounds__(kScanThreads) void nms_scan_kernel(
         }
         count += __popcll(keep_bits);
         ns += __popcll(keep_bits);
-        // rows kept in this block -> later words of the same super-block, four reads in flight
-        const int wl = b + 1 + lane;
-        if (wl < kScanBlocks && base_blk + wl < nb) {
-          unsigned long long acc = 0, kb = keep_bits;
-          const unsigned long long* col = sm + (b * 64) * kScanBlocks + wl;
-          while (kb) {
-            const int j0 = __builtin_ctzll(kb);
-            kb &= kb - 1;
-            const int j1 = kb ? __builtin_ctzll(kb) : j0;
-            kb &= kb - 1;
-            const int j2 = kb ? __builtin_ctzll(kb) : j0;
-            kb &= kb - 1;
-            const int j3 = kb ? __builtin_ctzll(kb) : j0;
-            kb &= kb - 1;
-            acc |= (col[j0 * kScanBlocks] | col[j1 * kScanBlocks]) |
-                   (col[j2 * kScanBlocks] | col[j3 * kScanBlocks]);
+        // rows kept in this block -> later words of the same super-block
+        if (__popcll(keep_bits) > 12) {
+          // many: lane (g, w) = (lane / 8, lane % 8) reads word w of rows g, g + 8, ... of the
+          // block (the 64 lanes read 512 contiguous bytes at a time), keeps those of kept
+          // rows, and the eight row groups are OR-ed across lanes
+          const int w8 = lane & 7, g = lane >> 3;
+          const unsigned long long* rowp = sm + (b * 64 + g) * kScanBlocks + w8;
+          unsigned long long v[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) v[i] = rowp[i * 8 * kScanBlocks];
+          unsigned long long acc = 0;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) acc |= ((keep_bits >> (g + 8 * i)) & 1ull) ? v[i] : 0ull;
+#pragma unroll
+          for (int o = 8; o < 64; o <<= 1) {
+            const unsigned lo = __shfl_xor(static_cast<unsigned>(acc), o, 64);
+            const unsigned hi = __shfl_xor(static_cast<unsigned>(acc >> 32), o, 64);
+            acc |= (static_cast<unsigned long long>(hi) << 32) | lo;
           }
-          if (acc) removed[base_blk + wl] |= acc;
+          if (lane < 8 && w8 > b && base_blk + w8 < nb && acc) removed[base_blk + w8] |= acc;
+        } else {
+          // few: lane w walks the kept rows, four reads in flight
+          const int wl = b + 1 + lane;
+          if (wl < kScanBlocks && base_blk + wl < nb) {
+            unsigned long long acc = 0, kb = keep_bits;
+            const unsigned long long* col = sm + (b * 64) * kScanBlocks + wl;
+            while (kb) {
+              const int j0 = __builtin_ctzll(kb);
+              kb &= kb - 1;
+              const int j1 = kb ? __builtin_ctzll(kb) : j0;
+              kb &= kb - 1;
+              const int j2 = kb ? __builtin_ctzll(kb) : j0;
+              kb &= kb - 1;
+              const int j3 = kb ? __builtin_ctzll(kb) : j0;
+              kb &= kb - 1;
+              acc |= (col[j0 * kScanBlocks] | col[j1 * kScanBlocks]) |
+                     (col[j2 * kScanBlocks] | col[j3 * kScanBlocks]);
+            }
+            if (acc) removed[base_blk + wl] |= acc;
+          }
         }
         __builtin_amdgcn_wave_barrier();
       }
@@ -1247,6 +1293,7 @@ __global__ __launch_bounds__(kScanThreads) void nms_scan_kernel(
     }
 #pragma unroll
     for (int k = 0; k < kScanLoads; ++k) sub[tid + k * kScanThreads] = ahead[k];
+    subcol[tid] = ahead_col;
     __syncthreads();
   }
   if (tid == 0) {
@@ -1443,18 +1490,20 @@ int run_proposal(const float* scores, const float* bbox, const float* im_info, c
   // the scan resumes behind the first super-block.
   int* done = flags + 2;
   const int head = pre < kScanRows ? pre : kScanRows, head_nb = ceil_div(head, 64);
+  // (the equal-score replay is over: its prefix-count array holds the column words now)
+  unsigned long long* colmask = reinterpret_cast<unsigned long long*>(ws + L.pref);
   nms_mask_kernel<<<head_nb * (head_nb + 1) / 2, 256, 0, st>>>(sboxes, head, nms_thresh, nb, head_nb, mask,
-                                                             nullptr);
+                                                             colmask, nullptr);
   MC_LAUNCH_CHECK();
   nms_scan_kernel<<<1, kScanThreads, sizeof(unsigned long long) * head_nb, st>>>(
-      mask, head, head_nb, nb, post_nms_topn, kept, num_rois, done, head == pre, 0);
+      mask, head, head_nb, nb, post_nms_topn, kept, num_rois, done, head == pre, 0, colmask);
   MC_LAUNCH_CHECK();
   if (head < pre) {
     nms_mask_kernel<<<std::min(nb * (nb + 1) / 2, 8 * kNumCu), 256, 0, st>>>(sboxes, pre, nms_thresh, nb, nb,
-                                                                           mask, done);
+                                                                           mask, colmask, done);
     MC_LAUNCH_CHECK();
     nms_scan_kernel<<<1, kScanThreads, sizeof(unsigned long long) * nb, st>>>(
-        mask, pre, nb, nb, post_nms_topn, kept, num_rois, done, 1, 1);
+        mask, pre, nb, nb, post_nms_topn, kept, num_rois, done, 1, 1, colmask);
     MC_LAUNCH_CHECK();
   }
   MC_HIP(mark(3));
