@@ -237,18 +237,22 @@ __global__ __launch_bounds__(kSortThreads) void det_class_nms_kernel(
 // not depend on the order of decisions when the threshold is fixed, so the tests
 // can run in parallel: a wavefront holds candidate 64 w + l in lane l, tests it
 // against a candidate k (a broadcast read) and a ballot is word w of k's row.
-//   1. the block's own rows, word `blk` only (all wavefronts, eight rows each);
-//   2. one wavefront decides the block: lane l holds row 64 blk + l, a candidate
-//      whose bit in the rejected set is clear is kept and its row is OR-ed in
-//      (scalar code, no memory access); the kept ones are written by their lanes;
+//   1. the block's own pairs (all wavefronts, eight of the block's candidates each as
+//      the earlier box): lane l collects in `before[l]` the earlier candidates of the block
+//      that candidate l is rejected against;
+//   2. one wavefront decides the block in rounds: a candidate none of whose rejecting
+//      predecessors is still open is settled, rejected if one of them is kept, else kept
+//      (two ballots per round; the first open candidate always settles, and candidates
+//      reject few of their neighbours, so a few rounds instead of one step per kept
+//      candidate); the kept ones are written by their lanes;
 //   3. only the rows of the candidates kept in this block are evaluated against the
 //      later blocks (all wavefronts) and OR-ed into the rejected set, one word per
 //      later block.  Rows of rejected candidates are never formed.
-// State: `later[w]` = word w of the rejected set, `diag[l]`, one word of kept bits.
+// State: `later[w]` = word w of the rejected set, `before[l]`, one word of kept bits.
 constexpr int kDetCandBoxes = 1024;  // candidates whose boxes are cached in LDS
 struct BlockNmsLds {
   unsigned long long later[kDetCandBoxes / 64];
-  unsigned long long diag[64];
+  unsigned long long before[64];  // per candidate of the block: the earlier ones of the block it is rejected against
   unsigned long long keep;
   int kept_list[64];
 };
@@ -260,48 +264,54 @@ __device__ __forceinline__ void greedy_nms_blocks(int ncand, const IT* cand_idx,
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   constexpr int kWaves = kSortThreads / 64;
   if (threadIdx.x < kDetCandBoxes / 64) st->later[threadIdx.x] = 0;
+  if (threadIdx.x < 64) st->before[threadIdx.x] = 0;
   int nkept = 0;  // used by wavefront 0
   __syncthreads();
   for (int blk = 0; blk < words; ++blk) {
     const int bn = min(64, ncand - 64 * blk);
     {
-      // 1. rows of the block, word blk
+      // 1. the block's own pairs: lane l collects the earlier candidates of the block that
+      // candidate 64 blk + l is rejected against (the test is symmetric in its two boxes)
       const int r = 64 * blk + lane;
       const bool in = r < ncand;
       const DBox rb = cand_box[min(r, ncand - 1)];
       constexpr int kPer = 64 / kWaves;
+      unsigned long long mine = 0;
 #pragma unroll 1
       for (int i0 = wave * kPer; i0 < min(wave * kPer + kPer, bn); i0 += 4) {
         DBox kb[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) kb[q] = cand_box[64 * blk + min(i0 + q, bn - 1)];
-        unsigned long long bits[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-          bits[q] = __ballot(static_cast<int>(in) & static_cast<int>(lane > i0 + q) &
-                             static_cast<int>(overlap_rejects(rb, kb[q], nms_thr)));
-        if (lane < 4 && i0 + lane < bn)
-          st->diag[i0 + lane] = lane == 0 ? bits[0] : lane == 1 ? bits[1] : lane == 2 ? bits[2] : bits[3];
+        for (int q = 0; q < 4; ++q) {
+          const bool hit = in & (lane > i0 + q) & (i0 + q < bn) & overlap_rejects(rb, kb[q], nms_thr);
+          mine |= hit ? 1ull << (i0 + q) : 0ull;
+        }
       }
+      if (mine) atomicOr(&st->before[lane], mine);
     }
     __syncthreads();
     if (wave == 0) {
-      // 2. decide the block
-      const unsigned long long diag = st->diag[min(lane, bn - 1)];
+      // 2. decide the block in rounds: a candidate none of whose rejecting predecessors is
+      // still open is settled, rejected if one of them is kept, else kept.  The first open
+      // candidate always settles; candidates reject few of their neighbours, so a few rounds.
+      const unsigned long long before = st->before[lane];
+      st->before[lane] = 0;  // for the next block (two barriers away)
       const unsigned long long valid = bn >= 64 ? ~0ull : ((1ull << bn) - 1ull);
-      const unsigned long long before = st->later[blk];
+      const unsigned long long prior = st->later[blk];
       // (readfirstlane returns a signed int: through unsigned, or the low half would sign-extend)
-      const unsigned b_lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(before));
-      const unsigned b_hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(before >> 32));
-      unsigned long long rem = (static_cast<unsigned long long>(b_hi) << 32) | b_lo;
-      unsigned long long avail = ~rem & valid, keep_bits = 0;
-      while (avail != 0) {  // wave-uniform, on the scalar unit
-        const int j = __builtin_ctzll(avail);
-        keep_bits |= 1ull << j;
-        const unsigned lo = __builtin_amdgcn_readlane(static_cast<unsigned>(diag), j);
-        const unsigned hi = __builtin_amdgcn_readlane(static_cast<unsigned>(diag >> 32), j);
-        rem |= (static_cast<unsigned long long>(hi) << 32) | lo;
-        avail = ~rem & valid & ~(((1ull << j) << 1) - 1ull);  // candidates after j
+      const unsigned b_lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(prior));
+      const unsigned b_hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(prior >> 32));
+      const unsigned long long rem = (static_cast<unsigned long long>(b_hi) << 32) | b_lo;
+      unsigned long long open = ~rem & valid, keep_bits = 0;
+      while (open != 0) {  // wave-uniform
+        const bool is_open = (open >> lane) & 1ull;
+        const bool rejected = (before & keep_bits) != 0;
+        const bool waits = (before & open) != 0;
+        const unsigned long long now_rejected = __ballot(is_open && rejected);
+        const unsigned long long now_kept = __ballot(is_open && !rejected && !waits);
+        keep_bits |= now_kept;
+        open &= ~(now_kept | now_rejected);
       }
       // the block's kept candidates, in order, by their own lanes
       if ((keep_bits >> lane) & 1ull) {
