@@ -449,8 +449,159 @@ __global__ __launch_bounds__(kSortThreads) void det_class_nms_lds_kernel(
                                   &kept_count[seg]);
 }
 
+// Sum of one int per thread over the workgroup, returned to every thread.  `slots` has
+// one entry per wavefront and may be reused right after the call returns.
+__device__ __forceinline__ int block_sum(int v, uint32_t* slots) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  if ((threadIdx.x & 63) == 0) slots[threadIdx.x >> 6] = static_cast<uint32_t>(v);
+  __syncthreads();
+  int total = 0;
+#pragma unroll
+  for (int w = 0; w < kSortThreads / 64; ++w) total += static_cast<int>(slots[w]);
+  __syncthreads();
+  return total;
+}
+
 constexpr int kSelLdsPer = 16;
-constexpr int kSelLdsMax = kSelLdsPer * kSortThreads;  // 8192 entries (SSD300: 20 classes x 400)
+constexpr int kSelLdsMax = kSelLdsPer * kSortThreads;  // 8192 entries held in registers (SSD300: 20 classes x 400)
+
+// keep_top_k and the rows of one image whose entry list has at most kSelLdsMax entries:
+// every thread keeps its run of up to kSelLdsPer entries (class, prior, score) in
+// registers from the first gather to the rows, so the list is read once.
+struct SelectShortLds {
+  uint32_t slots[2][kSortThreads / 64];
+  uint32_t scan[kSortThreads / 64];
+  // first entry of every thread's run, for the neighbour test across two runs
+  int first_cls[kSortThreads];
+  float first_score[kSortThreads];
+  unsigned char first_in[kSortThreads];
+};
+__device__ __forceinline__ void select_short(
+    const float* __restrict__ conf, const DBox* __restrict__ boxes, int P, int C, int loc_classes,
+    int keep_top_k, int max_cand, const int* __restrict__ kept_idx, const int* s_off, int total,
+    int i, float* __restrict__ rows_image, int* __restrict__ rows_count,
+    int* __restrict__ cut_tie_flag, SelectShortLds* st) {
+  const int tid = threadIdx.x;
+  const int per = (total + kSortThreads - 1) / kSortThreads;
+  const int begin = min(tid * per, total), end = min(begin + per, total);
+  const int cnt = end - begin;
+  // first all prior indices, then all scores: two rounds of loads per thread
+  int cls[kSelLdsPer], idx[kSelLdsPer];
+  float sc[kSelLdsPer];
+  {
+    int c = 0;
+#pragma unroll
+    for (int q = 0; q < kSelLdsPer; ++q) {
+      cls[q] = 0;
+      idx[q] = 0;
+      if (q < cnt) {
+        const int e = begin + q;
+        while (s_off[c + 1] <= e) ++c;
+        cls[q] = c;
+        idx[q] = kept_idx[(size_t)(i * C + c) * max_cand + (e - s_off[c])];
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < kSelLdsPer; ++q)
+      sc[q] = q < cnt ? conf[((size_t)i * P + idx[q]) * C + cls[q]] : 0.f;
+  }
+  uint32_t in_mask = cnt >= 32 ? 0xffffffffu : ((1u << cnt) - 1u);  // bit q: entry begin + q is kept
+  if (keep_top_k > -1 && total > keep_top_k) {
+    // Which entries are among the keep_top_k best needs no sort: T = the keep_top_k-th
+    // smallest key, found bit by bit from the top with one count over the workgroup per
+    // bit; entries with a smaller key are in, those equal to T fill the remaining places
+    // in entry order -- what a stable sort cut at keep_top_k selects.  The counts: ballots
+    // within a wavefront (scalar population counts), the eight wavefront counts through
+    // LDS with one barrier (two alternating sets of slots: a set is rewritten two rounds
+    // later, when every reader has passed the barrier in between).  Unused register slots
+    // hold the largest key; `padding` takes them out of a count that reaches it.
+    uint32_t rk[kSelLdsPer];
+#pragma unroll
+    for (int q = 0; q < kSelLdsPer; ++q) rk[q] = q < cnt ? desc_key(sc[q]) : 0xffffffffu;
+    const int padding = kSortThreads * kSelLdsPer - total;
+    uint32_t T = 0;
+    int parity = 0;
+    for (int bit = 31; bit >= 0 && keep_top_k > 0; --bit) {
+      const uint32_t mid = T | ((1u << bit) - 1u);
+      int below = 0;  // of this wavefront
+#pragma unroll
+      for (int q = 0; q < kSelLdsPer; ++q) below += __popcll(__ballot(rk[q] <= mid));
+      if ((tid & 63) == 0) st->slots[parity][tid >> 6] = static_cast<uint32_t>(below);
+      __syncthreads();
+      const uint4 a = *reinterpret_cast<const uint4*>(&st->slots[parity][0]);
+      const uint4 b = *reinterpret_cast<const uint4*>(&st->slots[parity][4]);
+      static_assert(kSortThreads / 64 == 8, "eight wavefront counts");
+      int total_below = static_cast<int>(a.x + a.y + a.z + a.w + b.x + b.y + b.z + b.w);
+      if (mid == 0xffffffffu) total_below -= padding;
+      if (total_below < keep_top_k) T |= 1u << bit;
+      parity ^= 1;
+    }
+    int less = 0, equal = 0;
+#pragma unroll
+    for (int q = 0; q < kSelLdsPer; ++q) {
+      less += (q < cnt) && rk[q] < T;
+      equal += (q < cnt) && rk[q] == T;
+    }
+    const int need_equal = keep_top_k - block_sum(less, st->scan);
+    const int equal_total = block_sum(equal, st->scan);
+    int rank = static_cast<int>(block_exclusive_scan(static_cast<uint32_t>(equal), st->scan));
+    in_mask = 0;
+#pragma unroll
+    for (int q = 0; q < kSelLdsPer; ++q)
+      if (q < cnt) {
+        bool in = rk[q] < T;
+        if (rk[q] == T) in = rank++ < need_equal;
+        in_mask |= static_cast<uint32_t>(in) << q;
+      }
+    // Equal scores on both sides of the cut: which of them survive is decided here
+    // by (label, NMS order) and in the reference by std::sort's internals.
+    if (tid == 0 && cut_tie_flag && keep_top_k > 0 && equal_total > need_equal)
+      atomicOr(cut_tie_flag, 1);
+    // Equal scores of one label among the kept entries: the reference rebuilds each
+    // label's list in std::sort's order, here they stay in NMS order.
+    if (cut_tie_flag) {
+      st->first_cls[tid] = cnt > 0 ? cls[0] : -1;
+      st->first_score[tid] = sc[0];
+      st->first_in[tid] = static_cast<unsigned char>(in_mask & 1u);
+      __syncthreads();
+      bool tied = false;
+#pragma unroll
+      for (int q = 0; q < kSelLdsPer; ++q) {
+        if (q >= cnt || !((in_mask >> q) & 1u)) continue;
+        if (q + 1 < cnt) {
+          tied = tied || (((in_mask >> (q + 1)) & 1u) && cls[q + 1] == cls[q] && sc[q + 1] == sc[q]);
+        } else if (tid + 1 < kSortThreads && begin + q + 1 < total) {
+          // the next entry opens the next thread's run (runs are contiguous and in order)
+          tied = tied || (st->first_in[tid + 1] && st->first_cls[tid + 1] == cls[q] &&
+                          st->first_score[tid + 1] == sc[q]);
+        }
+      }
+      if (tied) atomicOr(cut_tie_flag, 2);
+    }
+  }
+  // the kept entries in entry order
+  uint32_t pos = block_exclusive_scan(static_cast<uint32_t>(__popc(in_mask)), st->scan);
+  DBox bx[kSelLdsPer];
+#pragma unroll
+  for (int q = 0; q < kSelLdsPer; ++q)
+    if ((in_mask >> q) & 1u)
+      bx[q] = boxes[((size_t)i * loc_classes + (loc_classes == 1 ? 0 : cls[q])) * P + idx[q]];
+#pragma unroll
+  for (int q = 0; q < kSelLdsPer; ++q)
+    if ((in_mask >> q) & 1u) {
+      float* row = rows_image + static_cast<size_t>(pos) * 7;
+      row[0] = static_cast<float>(i);
+      row[1] = static_cast<float>(cls[q]);
+      row[2] = sc[q];
+      row[3] = bx[q].xmin;
+      row[4] = bx[q].ymin;
+      row[5] = bx[q].xmax;
+      row[6] = bx[q].ymax;
+      ++pos;
+    }
+  if (tid == kSortThreads - 1) rows_count[i] = static_cast<int>(pos);
+}
 
 // One workgroup per image: applies keep_top_k over all classes and writes the
 // image's rows [image, label, score, xmin, ymin, xmax, ymax], labels ascending,
@@ -462,9 +613,7 @@ __global__ __launch_bounds__(kSortThreads) void det_select_kernel(
     int* vals1, int* __restrict__ selected, float* __restrict__ rows_tmp,
     int* __restrict__ rows_count, int* __restrict__ cut_tie_flag) {
   __shared__ BlockSortLds lds;
-  __shared__ BlockSortLds16 lds16;
-  __shared__ uint32_t s_key[kSelLdsMax];       // entry lists of up to kSelLdsMax are sorted in LDS
-  __shared__ unsigned short s_val[kSelLdsMax];
+  __shared__ SelectShortLds short_lds;
   __shared__ int s_off[1024];  // start of each class in the image's entry list
   const int i = blockIdx.x;
   const int max_entries = C * max_cand;
@@ -473,52 +622,34 @@ __global__ __launch_bounds__(kSortThreads) void det_select_kernel(
   uint32_t* k1 = keys1 + (size_t)i * max_entries;
   int* v1 = vals1 + (size_t)i * max_entries;
   int* sel = selected + (size_t)i * max_entries;
+  // (the counts are fetched by one thread each: a single thread adding them up straight
+  // from memory would pay one load latency per class)
+  for (int c = threadIdx.x; c < C; c += kSortThreads) s_off[c + 1] = kept_count[i * C + c];
+  __syncthreads();
   if (threadIdx.x == 0) {
     int off = 0;
     for (int c = 0; c < C; ++c) {
+      const int cnt = s_off[c + 1];
       s_off[c] = off;
-      off += kept_count[i * C + c];
+      off += cnt;
     }
     s_off[C] = off;
   }
   __syncthreads();
   const int total = s_off[C];
   // entry e = (label, position in that label's NMS order), labels ascending
+  if (total <= kSelLdsMax) {  // uniform
+    select_short(conf, boxes, P, C, loc_classes, keep_top_k, max_cand, kept_idx, s_off, total, i,
+                 rows_tmp + (size_t)i * max_entries * 7, rows_count, cut_tie_flag, &short_lds);
+    return;
+  }
+  // Longer lists go through global scratch: flags, a stable sort cut at keep_top_k.
   for (int e = threadIdx.x; e < total; e += kSortThreads) sel[e] = 1;
   __syncthreads();
+  const int per = (total + kSortThreads - 1) / kSortThreads;
+  const int begin = min(static_cast<int>(threadIdx.x) * per, total), end = min(begin + per, total);
   if (keep_top_k > -1 && total > keep_top_k) {
-    const int per = (total + kSortThreads - 1) / kSortThreads;
-    const int begin = min(static_cast<int>(threadIdx.x) * per, total), end = min(begin + per, total);
-    const bool in_lds = total <= kSelLdsMax;
-    if (in_lds) {
-      // a thread's entries: first all prior indices, then all scores, so that the
-      // thread waits for two rounds of loads and not for two per entry
-      int cls[kSelLdsPer], idx[kSelLdsPer];
-      float sc[kSelLdsPer];
-      int c = 0;
-#pragma unroll
-      for (int q = 0; q < kSelLdsPer; ++q) {
-        const int e = begin + q;
-        cls[q] = 0;
-        idx[q] = 0;
-        if (e < end) {
-          while (s_off[c + 1] <= e) ++c;
-          cls[q] = c;
-          idx[q] = kept_idx[(size_t)(i * C + c) * max_cand + (e - s_off[c])];
-        }
-      }
-#pragma unroll
-      for (int q = 0; q < kSelLdsPer; ++q)
-        sc[q] = begin + q < end ? conf[((size_t)i * P + idx[q]) * C + cls[q]] : 0.f;
-#pragma unroll
-      for (int q = 0; q < kSelLdsPer; ++q) {
-        const int e = begin + q;
-        if (e < end) {
-          s_key[e] = desc_key(sc[q]);
-          s_val[e] = static_cast<unsigned short>(e);
-        }
-      }
-    } else {
+    {
       int c = 0;
       for (int e = begin; e < end; ++e) {
         while (s_off[c + 1] <= e) ++c;
@@ -528,21 +659,12 @@ __global__ __launch_bounds__(kSortThreads) void det_select_kernel(
       }
     }
     __syncthreads();
-    // both sorts are stable and see the entries in the same order: same result
-    if (in_lds) {
-      block_sort_desc_lds<kSelLdsPer, unsigned short>(s_key, s_val, total, &lds16);
-      for (int r = threadIdx.x; r < total; r += kSortThreads) sel[s_val[r]] = r < keep_top_k;
-    } else {
-      block_sort_desc(k0, v0, k1, v1, total, &lds);
-      for (int r = threadIdx.x; r < total; r += kSortThreads) sel[v0[r]] = r < keep_top_k;
-    }
+    block_sort_desc(k0, v0, k1, v1, total, &lds);
+    for (int r = threadIdx.x; r < total; r += kSortThreads) sel[v0[r]] = r < keep_top_k;
     // Equal scores on both sides of the cut: which of them survive is decided here
     // by (label, NMS order) and in the reference by std::sort's internals.
-    if (threadIdx.x == 0 && cut_tie_flag && keep_top_k > 0) {
-      const uint32_t last_in = in_lds ? s_key[keep_top_k - 1] : k0[keep_top_k - 1];
-      const uint32_t first_out = in_lds ? s_key[keep_top_k] : k0[keep_top_k];
-      if (last_in == first_out) atomicOr(cut_tie_flag, 1);
-    }
+    if (threadIdx.x == 0 && cut_tie_flag && keep_top_k > 0 && k0[keep_top_k - 1] == k0[keep_top_k])
+      atomicOr(cut_tie_flag, 1);
     __syncthreads();
     // Equal scores of one label among the kept entries: the reference rebuilds each
     // label's list in std::sort's order, here they stay in NMS order.
@@ -561,10 +683,7 @@ __global__ __launch_bounds__(kSortThreads) void det_select_kernel(
     }
     __syncthreads();
   }
-  // compact the selected entries in entry order (single pass by one thread per
-  // class would serialise; a block scan over `sel` keeps it parallel)
-  const int per = (total + kSortThreads - 1) / kSortThreads;
-  const int begin = min(static_cast<int>(threadIdx.x) * per, total), end = min(begin + per, total);
+  // compact the selected entries in entry order (a block scan over `sel`)
   uint32_t mine = 0;
   for (int e = begin; e < end; ++e) mine += sel[e];
   uint32_t pos = block_exclusive_scan(mine, lds.wave_sum);

@@ -796,6 +796,10 @@ def test_proposal_with_few_equal_scores(K, hw, pre, post, thr, pairs, seed, gene
     (2, 3000, 3, True, "CENTER_SIZE", -1, 0.001, 0.3, 1.0, 64, 1.0),       # exactly one block
     (2, 3000, 3, True, "CENTER_SIZE", -1, 0.001, 0.3, 1.0, 65, 1.0),
     (1, 3000, 3, True, "CENTER_SIZE", -1, 0.001, 0.95, 1.0, 300, 1.0),     # nearly everything kept
+    # keep_top_k over more kept boxes than the selection holds in registers (8192): through global scratch
+    (1, 6000, 12, True, "CENTER_SIZE", 300, 0.001, 0.95, 1.0, 900, 1.0),
+    (1, 6000, 12, True, "CENTER_SIZE", -1, 0.001, 0.95, 1.0, 900, 1.0),    # ... and without a cut
+    (2, 700, 13, True, "CENTER_SIZE", 0, 0.001, 0.6, 1.0, 100, 1.0),       # keep_top_k 0: nothing kept
     (2, 3000, 4, False, "CORNER", -1, 0.001, 0.7, 1.0, 1, 1.0),            # a single candidate per class
     (1, 400, 2, True, "CENTER_SIZE", -1, None, 0.05, 1.0, None, 1.0),      # low threshold: long reject chains
 ])
