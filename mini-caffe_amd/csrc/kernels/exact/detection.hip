@@ -826,6 +826,10 @@ int mcDetectionOutput(const float* loc, const float* conf, const float* prior, i
   MC_REQUIRE(num > 0 && num <= 1024 && num_priors > 0 && num_classes > 0 && num_classes < 1024,
              "mcDetectionOutput: bad extents");
   MC_REQUIRE(code_type >= 1 && code_type <= 3, "Unknown LocLossType.");
+  // shared locations carry the label -1, which DecodeBBoxesAll then skips as background
+  // (bbox_util.cpp:366-371; the layer aborts at detection_output_layer.cpp:122-126)
+  MC_REQUIRE(!(share_location && background_label == -1),
+             "Could not find location predictions for label -1");
   MC_REQUIRE(nms_threshold >= 0.f, "nms_threshold must be non negative.");
   MC_REQUIRE(eta > 0.f && eta <= 1.f, "eta must be in (0, 1]");
   MC_REQUIRE(max_rows >= num, "mcDetectionOutput: output needs at least one row per image");

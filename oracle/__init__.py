@@ -478,6 +478,8 @@ def detection_output(param, loc, conf, prior):
         float(param.get("confidence_threshold", -3.4028234663852886e38)),
         float(nms.get("nms_threshold", 0.3)), float(nms.get("eta", 1.0)), int(nms.get("top_k", -1)),
         _fp(out), max_rows)
+    if n == -2:
+        raise ValueError("Could not find location predictions for label -1")  # the reference's LOG(FATAL)
     assert n >= 0, "detection_output: row buffer too small"
     return out[:n].copy()
 

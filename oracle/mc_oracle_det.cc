@@ -425,12 +425,16 @@ static void nms_fast(const std::vector<Box>& boxes, const float* scores, int str
 /* DetectionOutputLayer::Forward_cpu.  loc: num x (P*loc_classes*4); conf: num x
  * (P*num_classes), prior-major; prior: 2 x (P*4).  out receives rows of 7 floats
  * (capacity max_rows); returns the number of rows (num rows of -1 when nothing
- * is kept, as :175-185). */
+ * is kept, as :175-185), -1 when out is too small, -2 where the reference aborts. */
 int orc_detection_output(const float* loc, const float* conf, const float* prior, int num,
                          int num_priors, int num_classes, int share_location, int background_label,
                          int code_type, int var_in_target, int keep_top_k, float conf_thr,
                          float nms_thr, float eta, int top_k, float* out, int max_rows) {
   const int loc_classes = share_location ? 1 : num_classes;
+  /* Shared locations carry the label -1; with background_label_id == -1 DecodeBBoxesAll
+   * (bbox_util.cpp:366-371) skips them as "background" and the layer then dies with
+   * "Could not find location predictions for label -1" (detection_output_layer.cpp:122-126). */
+  if (share_location && background_label == -1) return -2;
   std::vector<std::map<int, std::vector<int> > > all_indices(num);
   std::vector<std::vector<std::vector<Box> > > decoded(num);
   int num_kept = 0;

@@ -779,6 +779,20 @@ def test_proposal_with_few_equal_scores(K, hw, pre, post, thr, pairs, seed, gene
     assert ties == (3 if (not general and n <= 22528 and counted <= 500) else 1)
 
 
+def test_detection_output_shared_locations_without_background_fail(K):
+    """share_location with background_label_id -1 aborts in the reference ("Could not find
+    location predictions for label -1", detection_output_layer.cpp:122-126): an error here."""
+    rng = np.random.default_rng(3)
+    P, C = 6, 3
+    loc = rng.standard_normal((1, P * 4)).astype(np.float32)
+    conf = oracle.softmax(rng.standard_normal((1, P, C)).astype(np.float32), 2).reshape(1, P * C)
+    prior = np.tile(np.float32([0.1, 0.1, 0.4, 0.4]), 2 * P).reshape(1, 2, P * 4)
+    param = {"num_classes": C, "share_location": True, "background_label_id": -1,
+             "nms_param": {"nms_threshold": 0.5}}
+    with pytest.raises(Exception, match="label -1"):
+        run_detection_output(K, param, loc, conf, prior)
+
+
 @pytest.mark.parametrize("num,P,C,share,code,keep,thr,nms,eta,topk,sigma", [
     (2, 64, 4, True, "CENTER_SIZE", 10, 0.01, 0.45, 1.0, 20, 2.0),
     (8, 8732, 21, True, "CENTER_SIZE", 200, 0.01, 0.45, 1.0, 400, 2.0),   # config 3 tail, logits N(0, sigma=2)

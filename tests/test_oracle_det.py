@@ -318,6 +318,21 @@ def test_detection_output_decode_branches_brute_force(code_type, var_in_target, 
     assert np.abs(brute_detection_output(other, loc, conf, prior)[:5, 3:] - want[:5, 3:]).max() > 1e-3
 
 
+def test_detection_output_shared_locations_without_background_fail():
+    """share_location with background_label_id -1: the reference skips the shared boxes
+    (label -1) as background and aborts (bbox_util.cpp:366-371,
+    detection_output_layer.cpp:122-126); the restatement reports it."""
+    rng = np.random.default_rng(3)
+    P, C = 6, 3
+    loc = rng.standard_normal((1, P * 4)).astype(np.float32)
+    conf = oracle.softmax(rng.standard_normal((1, P, C)).astype(np.float32), 2).reshape(1, P * C)
+    prior = np.tile(np.float32([0.1, 0.1, 0.4, 0.4]), 2 * P).reshape(1, 2, P * 4)
+    param = {"num_classes": C, "share_location": True, "background_label_id": -1,
+             "nms_param": {"nms_threshold": 0.5}}
+    with pytest.raises(ValueError, match="label -1"):
+        oracle.detection_output(param, loc, conf, prior)
+
+
 @pytest.mark.parametrize("bg", [0, 2, -1])
 def test_detection_output_background_label_brute_force(bg):
     """Any class can be the background (skipped); -1 keeps every class."""
