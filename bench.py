@@ -22,7 +22,8 @@ sys.path.insert(0, os.path.join(ROOT, "mini-caffe_amd"))
 
 FP32_MFMA_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBS = 8000.0
-CONV_SOURCE = os.path.join(ROOT, "mini-caffe_amd", "csrc", "kernels", "conv_igemm.hip")
+CONV_SOURCES = [os.path.join(ROOT, "mini-caffe_amd", "csrc", "kernels", f)
+                for f in ("conv_igemm.hip", "conv_winograd.hip")]
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "igemm_resnet50_b64_pmc_traffic.txt")
 MFMA_PROFILE = os.path.join(ROOT, "profiles", "igemm_resnet50_b64_pmc_mfma_util.txt")
 
@@ -30,8 +31,8 @@ MFMA_PROFILE = os.path.join(ROOT, "profiles", "igemm_resnet50_b64_pmc_mfma_util.
 def counter_figure(path, key):
     """A figure that only a rocprofv3 --pmc run can give (HBM bytes per launch, MFMA
     utilisation), read from the committed summary of that run.  The summary ends with
-    `key: value` lines, among them the SHA-256 of the kernel source it was taken with;
-    a summary of another kernel version is reported as stale instead of being quoted.
+    `key: value` lines, among them the SHA-256 of the convolution kernel sources it was
+    taken with; a summary of another kernel version is reported as stale instead of being quoted.
     Returns (value or None, note)."""
     import hashlib
     fields = {}
@@ -42,13 +43,13 @@ def counter_figure(path, key):
                 fields[k.strip()] = v.strip()
     except OSError as e:
         return None, "no counter summary (%s)" % e
-    have = hashlib.sha256(open(CONV_SOURCE, "rb").read()).hexdigest()
+    have = hashlib.sha256(b"".join(open(f, "rb").read() for f in CONV_SOURCES)).hexdigest()
     rel = os.path.relpath(path, ROOT)
-    if key not in fields or "conv_igemm_sha256" not in fields:
+    if key not in fields or "conv_sources_sha256" not in fields:
         return None, "%s holds no '%s' line" % (rel, key)
-    if fields["conv_igemm_sha256"] != have:
-        msg = ("%s was taken with another version of conv_igemm.hip (sha256 %s..., tree has %s...): "
-               "re-run the command it names" % (rel, fields["conv_igemm_sha256"][:12], have[:12]))
+    if fields["conv_sources_sha256"] != have:
+        msg = ("%s was taken with another version of conv_igemm.hip + conv_winograd.hip (sha256 %s..., tree "
+               "has %s...): re-run the command it names" % (rel, fields["conv_sources_sha256"][:12], have[:12]))
         print("bench.py: STALE COUNTER SUMMARY: " + msg, file=sys.stderr)
         return None, "stale: " + msg
     return float(fields[key]), "%s, taken %s" % (rel, fields.get("date", "?"))
@@ -135,19 +136,33 @@ def main():
     for _ in range(args.steps):
         net.forward()
     tot_ms, launches, fl = ctypes.c_double(), ctypes.c_long(), ctypes.c_double()
-    LIB.mcConvTimingCollect(ctypes.byref(tot_ms), ctypes.byref(launches), ctypes.byref(fl))
+    issued, wino = ctypes.c_double(), ctypes.c_long()
+    LIB.mcConvTimingCollectDetail(ctypes.byref(tot_ms), ctypes.byref(launches), ctypes.byref(fl),
+                                  ctypes.byref(issued), ctypes.byref(wino))
     LIB.mcConvTimingEnable(0)
-    achieved = fl.value / (tot_ms.value * 1e-3) / 1e12 if tot_ms.value > 0 else 0.0
+    # achieved: the layers' algorithmic FLOPs (2 x MACs of the direct sum) over the device time
+    # of their launches.  A 3x3 layer on the Winograd path counts with its direct-sum FLOPs and
+    # with all three of its launches (transforms included); mfma_issued_* is what the matrix
+    # pipe was actually handed in the same time.
+    secs = tot_ms.value * 1e-3
+    achieved = fl.value / secs / 1e12 if secs > 0 else 0.0
+    issued_tflops = issued.value / secs / 1e12 if secs > 0 else 0.0
     traffic, traffic_note = counter_figure(TRAFFIC_PROFILE, "traffic_bytes_per_launch")
     mfma_util, mfma_note = counter_figure(MFMA_PROFILE, "mfma_util_pct")
+    steps = max(1, args.steps)
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP32_MFMA_PEAK_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
                 "traffic": traffic, "traffic_source": traffic_note,
-                "kernel": "igemm_f32 (Convolution + InnerProduct, fused BN/Scale/ReLU epilogue)",
-                "launches_per_step": launches.value // max(1, args.steps),
-                "kernel_ms_per_step": round(tot_ms.value / max(1, args.steps), 3),
-                "gflop_per_step": round(fl.value / max(1, args.steps) / 1e9, 1)}
-
+                "kernel": "igemm_f32 (Convolution + InnerProduct, fused BN/Scale/ReLU epilogue; %d of the %d "
+                          "contractions per step run it as the sixteen products of F(2x2,3x3) Winograd, "
+                          "timed with their two transform kernels)" % (wino.value // steps, launches.value // steps),
+                "launches_per_step": launches.value // steps,
+                "winograd_per_step": wino.value // steps,
+                "kernel_ms_per_step": round(tot_ms.value / steps, 3),
+                "gflop_per_step": round(fl.value / steps / 1e9, 1),
+                "mfma_issued_gflop_per_step": round(issued.value / steps / 1e9, 1),
+                "mfma_issued_tflops": round(issued_tflops, 2),
+                "mfma_issued_frac": round(issued_tflops / FP32_MFMA_PEAK_TFLOPS, 4)}
     if args.configs_report:
         configs_report(args.configs_report, mc, craft, zoo, LIB)
     if args.layer_scaling:
@@ -432,30 +447,38 @@ def layer_roofline(path, batch):
         w = torch.randn(cout, cin, k, k, device="cuda") * 0.05
         y = torch.empty(batch, cout, ho, wo, device="cuda")
         plan.set_weights(w.data_ptr())
-        for _ in range(5):
-            plan.forward(batch, x.data_ptr(), y.data_ptr(), activation=K.ACT_RELU, stream=stream)
-        torch.cuda.synchronize()
-        reps = 20
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(reps):
-            plan.forward(batch, x.data_ptr(), y.data_ptr(), activation=K.ACT_RELU, stream=stream)
-        e1.record()
-        torch.cuda.synchronize()
-        us = e0.elapsed_time(e1) / reps * 1e3
         fl = plan.flops(batch)
         nbytes = 4.0 * (x.numel() + y.numel() + w.numel())
         t_mfma, t_hbm = fl / (FP32_MFMA_PEAK_TFLOPS * 1e6), nbytes / (HBM_PEAK_GBS * 1e3)
         roof = max(t_mfma, t_hbm)
-        sum_roof += roof * cnt
-        sum_meas += us * cnt
-        lines.append("%-24s %3d %8.2f %9.1f %8.1f %6s %9.1f %9.1f %9.1f %6.1f%%" % (
-            "%d->%d %dx%d/%d @%d" % (cin, cout, k, k, s_, h), cnt, fl / 1e9, nbytes / 1e6, fl / nbytes,
-            "mfma" if t_mfma >= t_hbm else "hbm", roof, us, fl / us / 1e6, 100 * roof / us))
+        winograd = plan.kernel_name(batch) == "winograd_f32"
+        # a layer the library runs on the Winograd path is also timed on the direct one
+        for mode in ((-1, 0) if winograd else (-1,)):
+            plan.force_winograd(mode)
+            for _ in range(5):
+                plan.forward(batch, x.data_ptr(), y.data_ptr(), activation=K.ACT_RELU, stream=stream)
+            torch.cuda.synchronize()
+            reps = 20
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                plan.forward(batch, x.data_ptr(), y.data_ptr(), activation=K.ACT_RELU, stream=stream)
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) / reps * 1e3
+            if mode == -1:
+                sum_roof += roof * cnt
+                sum_meas += us * cnt
+            lines.append("%-24s %3d %8.2f %9.1f %8.1f %6s %9.1f %9.1f %9.1f %6.1f%%  %s" % (
+                "%d->%d %dx%d/%d @%d" % (cin, cout, k, k, s_, h), cnt, fl / 1e9, nbytes / 1e6, fl / nbytes,
+                "mfma" if t_mfma >= t_hbm else "hbm", roof, us, fl / us / 1e6, 100 * roof / us,
+                "" if not winograd else ("Winograd F(2x2,3x3): transforms + 16 products" if mode == -1
+                                         else "(same layer pinned to the direct path; not in the total)")))
         del x, y, w, plan
     lines.append("all 53 convolutions: roofline %.0f us, measured %.0f us = %.1f%% of the per-layer roofline"
                  % (sum_roof, sum_meas, 100 * sum_roof / sum_meas))
-    lines.append("roof us = max(FLOP / 157.3 TFLOP/s, bytes / 8 TB/s); 20 back-to-back launches between two events.")
+    lines.append("roof us = max(FLOP / 157.3 TFLOP/s, bytes / 8 TB/s) with the FLOPs and bytes of the direct sum; 20 "
+                 "back-to-back calls between two events.")
     with open(path, "w") as f:
         f.write("\n".join(lines) + "\n")
 

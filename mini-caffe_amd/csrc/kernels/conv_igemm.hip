@@ -849,6 +849,9 @@ struct mcConvPlan {
   // group == input channels: a direct kernel reads the layer's own filter layout
   bool depthwise = false;
   float* dw_weights = nullptr;  // copy of the [Cout, 1, kh, kw] filter blob
+  // 3x3 stride 1: the Winograd path, and who decides (-1 = by size, 0 = never, 1 = always)
+  WinogradState* winograd = nullptr;
+  int winograd_mode = -1;
   std::vector<SubProblem> subs;
 };
 
@@ -858,10 +861,13 @@ namespace {
 // bracketed by HIP events on the stream it runs on.
 struct TimedLaunch {
   hipEvent_t start, stop;
-  double flops;
+  double flops;   // algorithmic: what the layer's direct sum takes
+  double issued;  // what the matrix pipe is given (less on the Winograd path)
   const char* name;
 };
 thread_local bool g_timing = false;
+thread_local bool g_timing_outer = false;  // a Winograd layer is timed as a whole
+int g_winograd_default = -1;  // mode new plans start with
 thread_local std::vector<TimedLaunch> g_timed;
 
 // Tile choice.  With 256 CUs the tile count per CU is small for most layers, so
@@ -1125,6 +1131,8 @@ int mcConvPlanCreate(const mcConvGeom* gp, mcConvPlan** out) {
                   : fail("mcConvPlanCreate: device set-up failed: %s", hipGetErrorString(e));
     }
   }
+  plan->winograd = winograd_create(g, plan->Ho, plan->Wo);
+  plan->winograd_mode = g_winograd_default;
   *out = plan;
   return 0;
 }
@@ -1153,6 +1161,7 @@ int mcInnerProductPlanCreate(int K, int N, int transpose, mcConvPlan** out) {
 int mcConvPlanDestroy(mcConvPlan* plan) {
   if (!plan) return 0;
   if (plan->dw_weights) (void)hipFree(plan->dw_weights);
+  winograd_destroy(plan->winograd);
   for (auto& s : plan->subs) free_sub(s);
   delete plan;
   return 0;
@@ -1183,6 +1192,23 @@ int mcConvPlanSetWeights(mcConvPlan* plan, const float* weights, void* stream) {
         plan->wm_stride, plan->wg_stride);
     MC_LAUNCH_CHECK();
   }
+  if (plan->winograd && winograd_set_weights(plan->winograd, weights, st)) return -1;
+  return 0;
+}
+
+int mcConvPlanForceWinograd(mcConvPlan* plan, int mode) {
+  MC_REQUIRE(plan && mode >= -1 && mode <= 1, "mcConvPlanForceWinograd: bad argument");
+  MC_REQUIRE(mode != 1 || plan->winograd,
+             "mcConvPlanForceWinograd: not a 3x3 stride-1 convolution of one group");
+  plan->winograd_mode = mode;
+  return 0;
+}
+
+int mcConvWinogradRunBytes(long bytes) { return winograd_set_run_bytes(bytes); }
+
+int mcConvWinogradDefault(int mode) {
+  MC_REQUIRE(mode >= -1 && mode <= 1, "mcConvWinogradDefault: bad argument");
+  g_winograd_default = mode;
   return 0;
 }
 
@@ -1245,7 +1271,7 @@ int conv_forward_images(const mcConvPlan* plan, int num, const float* bottom, fl
     if (g_timing) {
       MC_HIP(hipEventCreate(&tl.start));
       MC_HIP(hipEventCreate(&tl.stop));
-      tl.flops = mcConvPlanFlops(plan, num);
+      tl.flops = tl.issued = mcConvPlanFlops(plan, num);
       tl.name = "depthwise_f32";
       MC_HIP(hipEventRecord(tl.start, st));
     }
@@ -1319,10 +1345,11 @@ int conv_forward_images(const mcConvPlan* plan, int num, const float* bottom, fl
   }
 
   TimedLaunch tl;
-  if (g_timing) {
+  const bool timed = g_timing && !g_timing_outer;
+  if (timed) {
     MC_HIP(hipEventCreate(&tl.start));
     MC_HIP(hipEventCreate(&tl.stop));
-    tl.flops = flops;
+    tl.flops = tl.issued = flops;
     tl.name = thin ? "thin_f32" : cfg.name;
     MC_HIP(hipEventRecord(tl.start, st));
   }
@@ -1440,7 +1467,7 @@ int conv_forward_images(const mcConvPlan* plan, int num, const float* bottom, fl
         ep ? ep->activation : MC_ACT_NONE, ep ? ep->negative_slope : 0.f);
     MC_LAUNCH_CHECK();
   }
-  if (g_timing) {
+  if (timed) {
     MC_HIP(hipEventRecord(tl.stop, st));
     g_timed.push_back(tl);
   }
@@ -1459,6 +1486,30 @@ int conv_forward(const mcConvPlan* plan, int num, const float* bottom, float* to
   const mcConvGeom& g = plan->geom;
   if (plan->depthwise)  // indexed with 64-bit integers throughout
     return conv_forward_images(plan, num, bottom, top, ep, stream, top_second, c_first);
+  if (plan->winograd && !top_second && plan->winograd_mode != 0 && plan->forced_config < 0 &&
+      plan->forced_split == 0 && plan->forced_chunk == 0 && winograd_fits(plan->winograd, num) &&
+      (plan->winograd_mode == 1 || winograd_pays(plan->winograd, num))) {
+    // timed as one contraction: both transforms belong to the layer's cost
+    TimedLaunch tl;
+    const bool timed = g_timing && !g_timing_outer;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (timed) {
+      MC_HIP(hipEventCreate(&tl.start));
+      MC_HIP(hipEventCreate(&tl.stop));
+      tl.flops = mcConvPlanFlops(plan, num);
+      tl.issued = winograd_issued_flops(plan->winograd, num);
+      tl.name = "winograd_f32";
+      MC_HIP(hipEventRecord(tl.start, st));
+      g_timing_outer = true;
+    }
+    const int rc = winograd_forward(plan->winograd, num, bottom, top, ep, stream);
+    if (timed) {
+      g_timing_outer = false;
+      MC_HIP(hipEventRecord(tl.stop, st));
+      g_timed.push_back(tl);
+    }
+    return rc;
+  }
   const long in_img = (long)g.channels_in * g.height_in * g.width_in;
   const long out_img = (long)g.channels_out * plan->Ho * plan->Wo;
   long shift = 0;
@@ -1511,22 +1562,32 @@ int mcConvTimingEnable(int on) {
   return 0;
 }
 
-int mcConvTimingCollect(double* total_ms, long* launches, double* flops) {
-  double ms = 0., fl = 0.;
+int mcConvTimingCollectDetail(double* total_ms, long* launches, double* flops, double* issued_flops,
+                              long* winograd) {
+  double ms = 0., fl = 0., is = 0.;
+  long wino = 0;
   for (auto& t : g_timed) {
     MC_HIP(hipEventSynchronize(t.stop));
     float e = 0.f;
     MC_HIP(hipEventElapsedTime(&e, t.start, t.stop));
     ms += e;
     fl += t.flops;
+    is += t.issued;
+    wino += t.issued != t.flops;
     (void)hipEventDestroy(t.start);
     (void)hipEventDestroy(t.stop);
   }
   if (total_ms) *total_ms = ms;
   if (launches) *launches = static_cast<long>(g_timed.size());
   if (flops) *flops = fl;
+  if (issued_flops) *issued_flops = is;
+  if (winograd) *winograd = wino;
   g_timed.clear();
   return 0;
+}
+
+int mcConvTimingCollect(double* total_ms, long* launches, double* flops) {
+  return mcConvTimingCollectDetail(total_ms, launches, flops, nullptr, nullptr);
 }
 
 double mcConvPlanFlops(const mcConvPlan* plan, int num) {
@@ -1541,6 +1602,10 @@ double mcConvPlanFlops(const mcConvPlan* plan, int num) {
 const char* mcConvPlanKernelName(const mcConvPlan* plan, int num) {
   if (plan && plan->depthwise) return "depthwise_f32";
   if (!plan || plan->subs.empty()) return "";
+  if (plan->winograd && plan->winograd_mode != 0 && plan->forced_config < 0 &&
+      plan->forced_split == 0 && plan->forced_chunk == 0 && winograd_fits(plan->winograd, num) &&
+      (plan->winograd_mode == 1 || winograd_pays(plan->winograd, num)))
+    return "winograd_f32";
   if (use_thin(plan, num)) return "thin_f32";
   const auto& s = plan->subs[0];
   return kConfigs[pick_config(plan, (long)num * s.Hq * s.Wq)].name;

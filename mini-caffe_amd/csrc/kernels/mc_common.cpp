@@ -15,7 +15,7 @@ struct Workspace {
   float* ptr = nullptr;
   size_t bytes = 0;
 };
-thread_local std::vector<std::pair<hipStream_t, Workspace>> g_workspaces;
+thread_local std::vector<std::pair<hipStream_t, Workspace>> g_workspaces[2];
 struct Counters {
   int* ptr = nullptr;
   size_t count = 0;
@@ -45,13 +45,14 @@ int stream_counters(hipStream_t st, size_t count, int** out) {
   return 0;
 }
 
-int stream_workspace(hipStream_t st, size_t bytes, float** out) {
+int stream_workspace(hipStream_t st, size_t bytes, float** out, int slot) {
   Workspace* ws = nullptr;
-  for (auto& e : g_workspaces)
+  auto& all = g_workspaces[slot != 0];
+  for (auto& e : all)
     if (e.first == st) ws = &e.second;
   if (!ws) {
-    g_workspaces.emplace_back(st, Workspace());
-    ws = &g_workspaces.back().second;
+    all.emplace_back(st, Workspace());
+    ws = &all.back().second;
   }
   if (ws->bytes < bytes) {
     if (ws->ptr) MC_HIP(hipFree(ws->ptr));  // waits for the device

@@ -59,8 +59,9 @@ inline int ew_blocks(long n, int threads, int per_thread = 1) {
 // Device scratch for partial results that one call writes and reads back (the
 // slices of a split-K contraction, per-part statistics): one grow-only buffer per
 // (host thread, stream).  Work on one stream is ordered, so consecutive calls
-// share it.  Growing frees the old buffer, which waits for the device.
-int stream_workspace(hipStream_t st, size_t bytes, float** out);
+// share it.  Growing frees the old buffer, which waits for the device.  A caller
+// that keeps its buffer across a call that takes one itself uses another slot.
+int stream_workspace(hipStream_t st, size_t bytes, float** out, int slot = 0);
 
 // Arrival counters for kernels whose workgroups hand work to the last one to
 // finish: one grow-only array of ints per (host thread, stream), zero when it is

@@ -53,6 +53,9 @@ LIB.mcNormalize.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_in
                             c_void_p]
 LIB.mcConvTimingCollect.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(c_long),
                                     ctypes.POINTER(ctypes.c_double)]
+LIB.mcConvTimingCollectDetail.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(c_long),
+                                          ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
+                                          ctypes.POINTER(c_long)]
 
 LIB.mcDetectionOutputWorkspaceSize.argtypes = [c_int, c_int, c_int, c_int, c_int,
                                                ctypes.POINTER(ctypes.c_size_t)]
@@ -102,6 +105,9 @@ LIB.mcConvPlanKernelName.argtypes = [c_void_p, c_int]
 LIB.mcConvPlanKernelName.restype = ctypes.c_char_p
 LIB.mcConvPlanForceConfig.argtypes = [c_void_p, c_int]
 LIB.mcConvPlanForceSplit.argtypes = [c_void_p, c_int]
+LIB.mcConvPlanForceWinograd.argtypes = [c_void_p, c_int]
+LIB.mcConvWinogradDefault.argtypes = [c_int]
+LIB.mcConvWinogradRunBytes.argtypes = [ctypes.c_long]
 LIB.mcConvPlanForceChunk.argtypes = [c_void_p, c_int]
 
 
@@ -147,6 +153,10 @@ class ConvPlan(object):
 
     def force_split(self, slices):
         check_mc(LIB.mcConvPlanForceSplit(self.handle, slices))
+
+    def force_winograd(self, mode):
+        """-1: the library decides by size, 0: direct path, 1: Winograd whenever the geometry allows."""
+        check_mc(LIB.mcConvPlanForceWinograd(self.handle, mode))
 
     def force_chunk(self, images):
         check_mc(LIB.mcConvPlanForceChunk(self.handle, images))

@@ -360,6 +360,74 @@ def test_conv_split_k_with_epilogue(K, geom, slices):
     assert netrun.rel_err(outs[1], outs[0]) < 1e-4   # summation order only
 
 
+WINOGRAD_CASES = [
+    # cin, h, w, cout, pad, batch: odd and even maps, every padding, one-pixel maps,
+    # channel counts off every tile size, more blocks than one plane row of the inner blob
+    (8, 6, 6, 8, 1, 1), (20, 7, 7, 33, 1, 3), (16, 14, 15, 16, 0, 2), (5, 9, 4, 7, 2, 2),
+    (64, 13, 13, 70, 1, 5), (3, 1, 1, 4, 1, 2), (7, 3, 3, 5, 0, 1), (130, 28, 28, 128, 1, 2),
+    (4, 200, 190, 6, 1, 2)]
+
+
+@pytest.mark.parametrize("case", WINOGRAD_CASES)
+def test_conv_winograd_path(K, case):
+    """3x3 stride-1 convolutions pinned to the Winograd path, with the whole epilogue,
+    against the oracle's direct sum; the same plan pinned to the direct path as well."""
+    cin, h, w, cout, pad, n = case
+    rng = np.random.default_rng(17)
+    x = rng.standard_normal((n, cin, h, w)).astype(np.float32)
+    wt = (rng.standard_normal((cout, cin, 3, 3)) * 0.2).astype(np.float32)
+    b = rng.standard_normal(cout).astype(np.float32)
+    sc = (rng.random(cout) + 0.5).astype(np.float32)
+    y = oracle.conv_forward(oracle.conv_geom(cin, h, w, cout, 3, 1, pad), x, wt, None)
+    res = rng.standard_normal(y.shape).astype(np.float32)
+    want = oracle.relu(oracle.eltwise([oracle.scale(y, sc, b), res], "SUM"), 0.1)
+    plan = K.ConvPlan(K.conv_geom(cin, h, w, cout, 3, 1, pad))
+    ep = dict(scale=sc, shift=b, residual=res, activation=K.ACT_RELU, negative_slope=0.1)
+    tol = 4e-6 * max(1.0, float(np.abs(y).max()))
+    for mode in (1, 0):
+        plan.force_winograd(mode)
+        got = _run_plan(K, plan, n, x, wt, want.shape, **ep)
+        assert np.abs(got - want).max() < tol, (case, mode)
+    # no epilogue at all
+    plan.force_winograd(1)
+    got = _run_plan(K, plan, n, x, wt, y.shape)
+    assert np.abs(got - y).max() < tol
+
+
+def test_conv_winograd_runs_batches_and_new_weights(K):
+    """One plan on the Winograd path over changing batch sizes (its inner plans are kept
+    by size, two at a time), with the batch cut into runs of images, and after the weights
+    change."""
+    cin, h, w, cout = 12, 10, 11, 9
+    rng = np.random.default_rng(18)
+    plan = K.ConvPlan(K.conv_geom(cin, h, w, cout, 3, 1, 1))
+    plan.force_winograd(1)
+    per_image = 64 * (cin + cout) * 5 * 6
+    try:
+        for round_, n in enumerate((5, 2, 7, 5, 1)):
+            K.LIB.mcConvWinogradRunBytes(max(1 << 20, 2 * per_image) if round_ % 2 else 1 << 30)
+            x = rng.standard_normal((n, cin, h, w)).astype(np.float32)
+            wt = (rng.standard_normal((cout, cin, 3, 3)) * 0.2).astype(np.float32)
+            b = rng.standard_normal(cout).astype(np.float32)
+            res = rng.standard_normal((n, cout, h, w)).astype(np.float32)
+            want = oracle.conv_forward(oracle.conv_geom(cin, h, w, cout, 3, 1, 1), x, wt, b) + res
+            got = _run_plan(K, plan, n, x, wt, want.shape, shift=b, residual=res)
+            assert np.abs(got - want).max() < 1e-5, (round_, n)
+    finally:
+        K.LIB.mcConvWinogradRunBytes(1 << 30)
+
+
+def test_conv_winograd_refused_where_it_does_not_apply(K):
+    for geom in (K.conv_geom(8, 9, 9, 8, 3, 2, 1), K.conv_geom(8, 9, 9, 8, 5, 1, 2),
+                 K.conv_geom(8, 9, 9, 8, 3, 1, 1, group=2), K.conv_geom(8, 9, 9, 8, 3, 1, 1, dilation=2),
+                 K.conv_geom(8, 9, 9, 8, 3, 1, 1, transposed=True)):
+        plan = K.ConvPlan(geom)
+        with pytest.raises(Exception, match="not a 3x3 stride-1 convolution"):
+            plan.force_winograd(1)
+        plan.force_winograd(0)
+        plan.force_winograd(-1)
+
+
 def test_conv_slices_summed_in_launch_over_many_launches(K):
     """The last workgroup of a tile to arrive adds the K slices of all of them, out of a
     workspace and arrival counters that every sliced launch on the stream shares: 60
