@@ -63,6 +63,11 @@ def main():
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-batch", type=int, default=8)
+    ap.add_argument("--no-winograd", action="store_true",
+                    help="keep every convolution on the direct implicit-GEMM path (3x3 stride-1 layers with "
+                         "128 or more channels otherwise run as F(2x2,3x3) Winograd)")
+    ap.add_argument("--no-direct-comparison", action="store_true",
+                    help="skip the second, shorter measurement with every convolution on the direct path")
     ap.add_argument("--no-detection-tails", action="store_true",
                     help="skip the NMS / Proposal / DetectionOutput timings (profiling runs of the "
                          "ResNet-50 forward alone)")
@@ -113,6 +118,8 @@ def main():
 
     spec, inputs = zoo.resnet50_spec(batch=args.batch, size=224, seed=0)
     flops = zoo.conv_flops(spec, inputs)
+    if args.no_winograd:
+        LIB.mcConvWinogradDefault(0)
     net = mc.Net.from_buffers(craft.to_prototxt(spec, "ResNet-50"))
     craft.load_weights(net, spec)
     net.forward(**inputs)          # uploads input + weights, packs filters
@@ -163,6 +170,37 @@ def main():
                 "mfma_issued_gflop_per_step": round(issued.value / steps / 1e9, 1),
                 "mfma_issued_tflops": round(issued_tflops, 2),
                 "mfma_issued_frac": round(issued_tflops / FP32_MFMA_PEAK_TFLOPS, 4)}
+    # The same net with every convolution on the direct path (no Winograd), shorter: what
+    # the implicit-GEMM kernel alone gives, for comparison with the figures above.
+    direct = None
+    if not args.no_winograd and not args.no_direct_comparison:
+        LIB.mcConvWinogradDefault(0)
+        net0 = mc.Net.from_buffers(craft.to_prototxt(spec, "ResNet-50"))
+        craft.load_weights(net0, spec)
+        net0.forward(**inputs)
+        n0 = max(10, args.steps // 2)
+        for _ in range(max(5, args.warmup // 2)):
+            net0.forward()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n0):
+            net0.forward()
+        torch.cuda.synchronize()
+        el0 = time.perf_counter() - t0
+        LIB.mcConvTimingEnable(1)
+        for _ in range(n0):
+            net0.forward()
+        LIB.mcConvTimingCollectDetail(ctypes.byref(tot_ms), ctypes.byref(launches), ctypes.byref(fl),
+                                      ctypes.byref(issued), ctypes.byref(wino))
+        LIB.mcConvTimingEnable(0)
+        LIB.mcConvWinogradDefault(-1)
+        rate0 = fl.value / (tot_ms.value * 1e-3) / 1e12
+        direct = {"value": round(args.batch * n0 / el0, 1), "unit": "images/s", "steps": n0,
+                  "ms_per_step": round(1e3 * el0 / n0, 3), "kernel_ms_per_step": round(tot_ms.value / n0, 3),
+                  "achieved": round(rate0, 2), "frac": round(rate0 / FP32_MFMA_PEAK_TFLOPS, 4),
+                  "note": "same net, mcConvWinogradDefault(0): all 53 convolutions on the direct implicit-GEMM path"}
+        del net0
+
     if args.configs_report:
         configs_report(args.configs_report, mc, craft, zoo, LIB)
     if args.layer_scaling:
@@ -190,7 +228,8 @@ def main():
                       "conv_gflop_per_step": round(flops["conv"] / 1e9, 1),
                       "api": "CaffeNetForward (Net::Forward(reshape=true))"},
            "roofline": roofline, "cpu_baseline": cpu,
-           "conv_mfma_util_pct": mfma_util, "conv_mfma_util_source": mfma_note}
+           "conv_mfma_util_pct": mfma_util, "conv_mfma_util_source": mfma_note,
+           "direct_path_only": direct}
     out.update(tails)
     print(json.dumps(out))
 
@@ -381,8 +420,10 @@ def configs_report(path, mc, craft, zoo, LIB):
 
 
 def layer_scaling(path):
-    """One convolution launch (ReLU epilogue) at growing batch sizes: time per launch and
-    TFLOP/s, through the kernel-level C ABI on torch-owned device memory."""
+    """One convolution launch of the implicit-GEMM kernel (ReLU epilogue, pinned to the direct
+    path) at growing batch sizes: time per launch and TFLOP/s, through the kernel-level C ABI
+    on torch-owned device memory; the 3x3 layers that the library would run as Winograd are
+    listed a second time on that path (algorithmic TFLOP/s: the direct sum's FLOPs)."""
     import torch
     from minicaffe import kernels as K
     # cin, height = width, cout, kernel, stride, pad: shapes of ResNet-50 stages 2-5
@@ -392,13 +433,15 @@ def layer_scaling(path):
     batches = (16, 32, 64, 128, 256, 512)
     lines = ["%-22s" % "convolution" + "".join("%16s" % ("batch %d" % n) for n in batches)]
     stream = torch.cuda.current_stream().cuda_stream
-    for cin, h, cout, k, s, p in shapes:
+    wino = [sh + (1,) for sh in shapes if sh[3] == 3 and sh[0] >= 128]
+    for cin, h, cout, k, s, p, mode in [sh + (0,) for sh in shapes] + wino:
         cells = []
         for n in batches:
-            if n * max(cin, cout) * h * h > 2 ** 28:
+            if n * max(cin, cout) * h * h > 2 ** 28 or (mode == 1 and 4 * n * max(cin, cout) * h * h >= 2 ** 29):
                 cells.append("%16s" % "-")
                 continue
             plan = K.ConvPlan(K.conv_geom(cin, h, h, cout, k, s, p))
+            plan.force_winograd(mode)
             ho, wo = plan.output_shape()
             x = torch.randn(n, cin, h, h, device="cuda")
             w = torch.randn(cout, cin, k, k, device="cuda") * 0.05
@@ -417,8 +460,9 @@ def layer_scaling(path):
             ms = e0.elapsed_time(e1) / reps
             cells.append("%8.0f us %4.0f" % (ms * 1e3, plan.flops(n) / ms / 1e9))
             del x, y, w, plan
-        lines.append("%-22s" % ("%d->%d %dx%d @%d" % (cin, cout, k, k, h)) + "".join(cells))
-    lines.append("cells: time per launch (10 back-to-back launches between two events) and TFLOP/s")
+        lines.append("%-22s" % ("%d->%d %dx%d @%d%s" % (cin, cout, k, k, h, " W" if mode else "")) + "".join(cells))
+    lines.append("cells: time per launch (10 back-to-back launches between two events) and TFLOP/s; W = the layer as "
+                 "F(2x2,3x3) Winograd (three launches, TFLOP/s in the direct sum's FLOPs)")
     with open(path, "w") as f:
         f.write("\n".join(lines) + "\n")
 
