@@ -31,7 +31,15 @@ namespace mchip {
 
 namespace {
 
-constexpr int kChannelsPerThread = 4;
+// Channels a thread of a transform kernel walks with one decomposition of its
+// block index: four where the launch still has a few workgroups per CU, fewer on
+// small maps (7x7 maps of 64 images are 1024 blocks: four workgroups per channel
+// group), so that the launch keeps enough loads in flight.
+inline int channels_per_thread(long tblocks, int channels, int least) {
+  for (int cpt = 4; cpt > least; cpt /= 2)
+    if (tblocks * ((channels + cpt - 1) / cpt) >= 8L * kNumCu) return cpt;
+  return least;
+}
 
 __device__ __forceinline__ float act_value(float v, int act, float slope) {
   switch (act) {
@@ -85,9 +93,11 @@ struct WinogradShape {
 // the padding (zeros outside the map).  Lanes run along t, so the sixteen stores
 // of a channel are contiguous rows; a thread walks kChannelsPerThread channels
 // with one decomposition of t.
+template <int CPT>
 __global__ __launch_bounds__(256) void winograd_input_kernel(const float* __restrict__ x,
                                                              float* __restrict__ v,
                                                              const WinogradShape s) {
+  constexpr int kChannelsPerThread = CPT;
   const int t = blockIdx.x * 256 + threadIdx.x;
   if (t >= s.Tpad) return;
   const int c0 = blockIdx.y * kChannelsPerThread;
@@ -148,11 +158,12 @@ struct WinogradEpilogue {
 // Y = A^T m A, A^T = [1 1 1 0; 0 1 -1 -1], m[f] = M[f][co][t]; then the layer's
 // epilogue  act(Y * scale[co] + shift[co] + residual)  on the up to four outputs
 // of block t that lie inside the map.
-template <bool PAIRS>
+template <bool PAIRS, int CPT>
 __global__ __launch_bounds__(256) void winograd_output_kernel(const float* __restrict__ m,
                                                               float* __restrict__ y,
                                                               const WinogradShape s,
                                                               const WinogradEpilogue e) {
+  constexpr int kChannelsPerThread = CPT;
   const int t = blockIdx.x * 256 + threadIdx.x;
   if (t >= s.T) return;
   const int c0 = blockIdx.y * kChannelsPerThread;
@@ -413,19 +424,36 @@ int winograd_forward(WinogradState* w, int num, const float* bottom, float* top,
     float* v = ws;
     float* m = ws + v_floats;
     const unsigned tblocks = static_cast<unsigned>(ceil_div(s.Tpad, 256));
-    winograd_input_kernel<<<dim3(tblocks, ceil_div(s.C, kChannelsPerThread)), 256, 0, st>>>(
-        bottom + n0 * in_img, v, s);
+    const float* run_bottom = bottom + n0 * in_img;
+    float* run_top = top + n0 * out_img;
+    switch (channels_per_thread(tblocks, s.C, 1)) {
+      case 4:
+        winograd_input_kernel<4><<<dim3(tblocks, ceil_div(s.C, 4)), 256, 0, st>>>(run_bottom, v, s);
+        break;
+      case 2:
+        winograd_input_kernel<2><<<dim3(tblocks, ceil_div(s.C, 2)), 256, 0, st>>>(run_bottom, v, s);
+        break;
+      default:
+        winograd_input_kernel<1><<<dim3(tblocks, s.C), 256, 0, st>>>(run_bottom, v, s);
+    }
     MC_LAUNCH_CHECK();
     if (mcConvForward(inner, 1, v, m, nullptr, stream)) return -1;
     e.residual = (ep && ep->residual) ? ep->residual + n0 * out_img : nullptr;
-    const dim3 ogrid(static_cast<unsigned>(ceil_div(s.T, 256)), ceil_div(s.Cout, kChannelsPerThread));
+    const unsigned oblocks = static_cast<unsigned>(ceil_div(s.T, 256));
     // (top and residual rows are 8-byte aligned when the width is even and the blob is)
     const bool pairs = s.Wo % 2 == 0 && reinterpret_cast<uintptr_t>(top) % 8 == 0 &&
                        (!ep || !ep->residual || reinterpret_cast<uintptr_t>(ep->residual) % 8 == 0);
-    if (pairs)
-      winograd_output_kernel<true><<<ogrid, 256, 0, st>>>(m, top + n0 * out_img, s, e);
-    else
-      winograd_output_kernel<false><<<ogrid, 256, 0, st>>>(m, top + n0 * out_img, s, e);
+    const int cpt = channels_per_thread(oblocks, s.Cout, 2);  // (one channel per thread measured slower here)
+    const dim3 ogrid(oblocks, ceil_div(s.Cout, cpt));
+#define MC_WINOGRAD_OUT(P, C) winograd_output_kernel<P, C><<<ogrid, 256, 0, st>>>(m, run_top, s, e)
+    if (pairs) {
+      if (cpt == 4) MC_WINOGRAD_OUT(true, 4);
+      else MC_WINOGRAD_OUT(true, 2);
+    } else {
+      if (cpt == 4) MC_WINOGRAD_OUT(false, 4);
+      else MC_WINOGRAD_OUT(false, 2);
+    }
+#undef MC_WINOGRAD_OUT
     MC_LAUNCH_CHECK();
   }
   return 0;
