@@ -59,6 +59,49 @@ def test_small_resnet_every_marked_blob(gpu_mode):
     assert np.allclose(net.get_blob("prob").data.sum(axis=1), 1, atol=1e-5)
 
 
+def test_nets_with_every_3x3_layer_on_the_winograd_path(gpu_mode):
+    """The library takes the Winograd path by size, which small test nets never reach:
+    with mcConvWinogradDefault(1) every 3x3 stride-1 convolution of a small ResNet (folded
+    BatchNorm / Scale / ReLU and residual sums in the output transform), of it again at another
+    batch size and after a weight update, and of a quarter-width SSD300 runs through it."""
+    from minicaffe import zoo
+    from minicaffe.base import LIB
+    oracle.use_openblas(False)
+    LIB.mcConvWinogradDefault(1)
+    try:
+        spec, inputs = zoo.resnet50_spec(batch=3, size=65, stages=(2, 2, 1, 1), width=16,
+                                         num_classes=10, bn_seed=3)
+        marks = ["conv1", "res2a", "res2b", "res3a", "res5a", "fc1000"]
+        net = run_net(gpu_mode, spec, inputs, marks)
+        want = netrun.oracle_forward(spec, inputs)
+        for name in marks + ["prob"]:
+            assert netrun.rel_err(net.get_blob(name).data, want[name]) < 1e-3, name
+        # a filter of a Winograd layer changes: its transformed copy must follow
+        params = dict(net.param_list)
+        idx = next(i for i, layer in enumerate(spec) if layer["name"] == "res2a_branch2b")
+        spec[idx]["blobs"][0] = spec[idx]["blobs"][0] * -0.7
+        params["res2a_branch2b_0"].data[...] = spec[idx]["blobs"][0]
+        net.forward()
+        want = netrun.oracle_forward(spec, inputs)
+        assert netrun.rel_err(net.get_blob("fc1000").data, want["fc1000"]) < 1e-3
+        # another batch size through the same plans
+        spec2, inputs2 = zoo.resnet50_spec(batch=5, size=65, stages=(2, 2, 1, 1), width=16,
+                                           num_classes=10, bn_seed=3)
+        spec2[idx]["blobs"][0] = spec[idx]["blobs"][0]
+        net.forward(**inputs2)
+        want2 = netrun.oracle_forward(spec2, inputs2)
+        assert netrun.rel_err(net.get_blob("fc1000").data, want2["fc1000"]) < 1e-3
+        del net
+
+        spec, inputs = zoo.ssd300_spec(batch=2, seed=4, width=16)
+        net = run_net(gpu_mode, spec, inputs, ["conv4_3_norm", "fc7", "mbox_loc", "mbox_conf"])
+        want = netrun.oracle_forward(spec, inputs)
+        for name in ("conv4_3_norm", "fc7", "mbox_loc", "mbox_conf"):
+            assert netrun.rel_err(net.get_blob(name).data, want[name]) < 1e-3, name
+    finally:
+        LIB.mcConvWinogradDefault(-1)
+
+
 def test_forward_twice_and_weight_update(gpu_mode):
     """A second forward reuses packed filters and folded epilogues; changing a
     parameter blob through the C ABI must invalidate both."""
