@@ -1486,7 +1486,7 @@ int conv_forward(const mcConvPlan* plan, int num, const float* bottom, float* to
   const mcConvGeom& g = plan->geom;
   if (plan->depthwise)  // indexed with 64-bit integers throughout
     return conv_forward_images(plan, num, bottom, top, ep, stream, top_second, c_first);
-  if (plan->winograd && !top_second && plan->winograd_mode != 0 && plan->forced_config < 0 &&
+  if (plan->winograd && plan->winograd_mode != 0 && plan->forced_config < 0 &&
       plan->forced_split == 0 && plan->forced_chunk == 0 && winograd_fits(plan->winograd, num) &&
       (plan->winograd_mode == 1 || winograd_pays(plan->winograd, num))) {
     // timed as one contraction: both transforms belong to the layer's cost
@@ -1502,7 +1502,7 @@ int conv_forward(const mcConvPlan* plan, int num, const float* bottom, float* to
       MC_HIP(hipEventRecord(tl.start, st));
       g_timing_outer = true;
     }
-    const int rc = winograd_forward(plan->winograd, num, bottom, top, ep, stream);
+    const int rc = winograd_forward(plan->winograd, num, bottom, top, ep, stream, top_second, c_first);
     if (timed) {
       g_timing_outer = false;
       MC_HIP(hipEventRecord(tl.stop, st));

@@ -36,8 +36,9 @@ bool winograd_fits(const WinogradState* w, int num);  // intermediates addressab
 bool winograd_pays(const WinogradState* w, int num);  // the automatic choice
 double winograd_issued_flops(const WinogradState* w, int num);  // of the sixteen products
 int winograd_set_run_bytes(long bytes);  // budget for V + M of one run of images
+// top_second / c_first as in mcConvForwardTwoTops (null / ignored for one top)
 int winograd_forward(WinogradState* w, int num, const float* bottom, float* top,
-                     const mcEpilogue* ep, void* stream);
+                     const mcEpilogue* ep, void* stream, float* top_second, int c_first);
 
 }  // namespace mchip
 

@@ -153,6 +153,10 @@ struct WinogradEpilogue {
   const float* residual;
   int act;
   float slope;
+  // two sibling layers computed together: channels [0, c_first) of every image go
+  // to the first top [N, c_first, Ho, Wo], the others to y_second; one top: c_first = Cout
+  float* y_second;
+  int c_first;
 };
 
 // Y = A^T m A, A^T = [1 1 1 0; 0 1 -1 -1], m[f] = M[f][co][t]; then the layer's
@@ -196,7 +200,10 @@ __global__ __launch_bounds__(256) void winograd_output_kernel(const float* __res
     }
     const float sc = e.scale ? e.scale[c] : 1.f;
     const float sh = e.shift ? e.shift[c] : 0.f;
-    const long base = (((long)n * s.Cout + c) * s.Ho + ho) * s.Wo + wo;
+    const bool first = c < e.c_first;
+    float* __restrict__ yc = first ? y : e.y_second;
+    const long base = first ? (((long)n * e.c_first + c) * s.Ho + ho) * s.Wo + wo
+                            : (((long)n * (s.Cout - e.c_first) + (c - e.c_first)) * s.Ho + ho) * s.Wo + wo;
     if (e.scale) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) out[i][0] *= sc, out[i][1] *= sc;
@@ -219,7 +226,7 @@ __global__ __launch_bounds__(256) void winograd_output_kernel(const float* __res
         }
         val.x = act_value(val.x, e.act, e.slope);
         val.y = act_value(val.y, e.act, e.slope);
-        *reinterpret_cast<float2*>(y + o) = val;
+        *reinterpret_cast<float2*>(yc + o) = val;
       }
     } else {
 #pragma unroll
@@ -231,7 +238,7 @@ __global__ __launch_bounds__(256) void winograd_output_kernel(const float* __res
           const long o = base + i * s.Wo + j;
           float val = out[i][j];
           if (e.residual) val += e.residual[o];
-          y[o] = act_value(val, e.act, e.slope);
+          yc[o] = act_value(val, e.act, e.slope);
         }
       }
     }
@@ -329,15 +336,21 @@ bool winograd_fits(const WinogradState* w, int num) {
 // against 209 on 56x56 maps); 128 -> 128 gains while V and M fit the 256 MB
 // last-level cache (152 -> 108 us on 28x28 maps) and loses beyond it (428 -> 478
 // on 150x150); 128 -> 256 gains 1.17x; 256 and 512 channels gain 1.4x to 1.8x on
-// every map; launches of a few hundred blocks are latency bound either way.
+// every map.  One narrow side is fine when the other is wide (SSD's merged heads,
+// 512 -> 100 on 38x38 b8: 147 -> 92 us; 1024 -> 150 on 19x19: 113 -> 81; 96 -> 512:
+// 91 -> 76) down to about 96 channels (256 -> 64 and 64 -> 512 break even, 1024 ->
+// 64 loses); 200 blocks still gain or break even (512 -> 150 on 10x10 b8: 42 -> 30 us).
 bool winograd_pays(const WinogradState* w, int num) {
   const mcConvGeom& g = w->geom;
   const long blocks = (long)num * ((w->Ho + 1) / 2) * ((w->Wo + 1) / 2);
   const int least = std::min(g.channels_in, g.channels_out);
   const int most = std::max(g.channels_in, g.channels_out);
-  if (blocks < 512 || least < 128) return false;
+  if (blocks < 192 || least < 96) return false;
+  // odd and tiny maps compute blocks that hang over the edge: a 3x3 map is four
+  // blocks for nine outputs (16 x 4 products against 36 x 9 / 4 useful ones)
+  if (10L * w->Ho * w->Wo < 26L * ((w->Ho + 1) / 2) * ((w->Wo + 1) / 2)) return false;
   if (most >= 256) return true;
-  return 64L * (g.channels_in + g.channels_out) * blocks <= (256L << 20);
+  return least >= 128 && 64L * (g.channels_in + g.channels_out) * blocks <= (256L << 20);
 }
 
 int winograd_set_weights(WinogradState* w, const float* weights, hipStream_t st) {
@@ -396,8 +409,12 @@ int winograd_set_run_bytes(long bytes) {
 }
 
 int winograd_forward(WinogradState* w, int num, const float* bottom, float* top,
-                     const mcEpilogue* ep, void* stream) {
+                     const mcEpilogue* ep, void* stream, float* top_second, int c_first) {
   MC_REQUIRE(w->have_weights, "mcConvForward: the plan has no weights yet");
+  MC_REQUIRE(!top_second || (c_first > 0 && c_first < w->geom.channels_out && !(ep && ep->residual)),
+             "mcConvForwardTwoTops: needs group 1, a split inside the output channels and no "
+             "residual");
+  if (!top_second) c_first = w->geom.channels_out;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const mcConvGeom& g = w->geom;
   // equal runs of whole images whose V and M fit the budget
@@ -407,8 +424,10 @@ int winograd_forward(WinogradState* w, int num, const float* bottom, float* top,
   const int runs = ceil_div(num, fit);
   const int run_len = ceil_div(num, runs);
   const long in_img = (long)g.channels_in * g.height_in * g.width_in;
-  const long out_img = (long)g.channels_out * w->Ho * w->Wo;
+  const long hw_out = (long)w->Ho * w->Wo;
+  const long out_img = c_first * hw_out, second_img = (g.channels_out - c_first) * hw_out;
   WinogradEpilogue e;
+  e.c_first = c_first;
   e.scale = ep ? ep->scale : nullptr;
   e.shift = ep ? ep->shift : nullptr;
   e.act = ep ? ep->activation : MC_ACT_NONE;
@@ -441,7 +460,9 @@ int winograd_forward(WinogradState* w, int num, const float* bottom, float* top,
     e.residual = (ep && ep->residual) ? ep->residual + n0 * out_img : nullptr;
     const unsigned oblocks = static_cast<unsigned>(ceil_div(s.T, 256));
     // (top and residual rows are 8-byte aligned when the width is even and the blob is)
+    e.y_second = top_second ? top_second + n0 * second_img : nullptr;
     const bool pairs = s.Wo % 2 == 0 && reinterpret_cast<uintptr_t>(top) % 8 == 0 &&
+                       reinterpret_cast<uintptr_t>(top_second) % 8 == 0 &&
                        (!ep || !ep->residual || reinterpret_cast<uintptr_t>(ep->residual) % 8 == 0);
     const int cpt = channels_per_thread(oblocks, s.Cout, 2);  // (one channel per thread measured slower here)
     const dim3 ogrid(oblocks, ceil_div(s.Cout, cpt));

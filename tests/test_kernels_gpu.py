@@ -394,6 +394,41 @@ def test_conv_winograd_path(K, case):
     assert np.abs(got - y).max() < tol
 
 
+@pytest.mark.parametrize("c_first", [1, 16, 50, 99])
+def test_conv_winograd_two_tops(K, c_first):
+    """The Winograd path with the output channels split over two blobs (merged sibling
+    layers): the same values as with one top, odd and even maps, batch cut into runs."""
+    rng = np.random.default_rng(19)
+    for h, w, n in ((9, 7, 3), (10, 12, 5)):
+        cin, cout = 24, 100
+        x = rng.standard_normal((n, cin, h, w)).astype(np.float32)
+        wt = (rng.standard_normal((cout, cin, 3, 3)) * 0.2).astype(np.float32)
+        b = rng.standard_normal(cout).astype(np.float32)
+        sc = (rng.random(cout) + 0.5).astype(np.float32)
+        plan = K.ConvPlan(K.conv_geom(cin, h, w, cout, 3, 1, 1))
+        plan.force_winograd(1)
+        xd, wd, bd, sd = dev(x), dev(wt), dev(b), dev(sc)
+        plan.set_weights(wd.data_ptr())
+        ep = dict(scale=sd.data_ptr(), shift=bd.data_ptr(), activation=K_ACT_RELU)
+        whole = torch.full((n, cout, h, w), float("nan"), device="cuda")
+        plan.forward(n, xd.data_ptr(), whole.data_ptr(), **ep)
+        try:
+            for run_bytes in (1 << 30, 1 << 20):
+                K.LIB.mcConvWinogradRunBytes(run_bytes)
+                first = torch.full((n, c_first, h, w), float("nan"), device="cuda")
+                second = torch.full((n, cout - c_first, h, w), float("nan"), device="cuda")
+                plan.forward_two_tops(n, xd.data_ptr(), first.data_ptr(), c_first, second.data_ptr(), **ep)
+                torch.cuda.synchronize()
+                assert torch.equal(first, whole[:, :c_first]) and torch.equal(second, whole[:, c_first:])
+        finally:
+            K.LIB.mcConvWinogradRunBytes(1 << 30)
+        want = np.maximum(oracle.scale(oracle.conv_forward(oracle.conv_geom(cin, h, w, cout, 3, 1, 1), x, wt, None),
+                                       sc, b), 0)
+        assert netrun.rel_err(whole.cpu().numpy(), want) < 1e-4
+        with pytest.raises(Exception, match="TwoTops"):
+            plan.forward_two_tops(n, xd.data_ptr(), first.data_ptr(), cout, second.data_ptr())
+
+
 def test_conv_winograd_runs_batches_and_new_weights(K):
     """One plan on the Winograd path over changing batch sizes (its inner plans are kept
     by size, two at a time), with the batch cut into runs of images, and after the weights
