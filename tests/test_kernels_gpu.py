@@ -394,6 +394,34 @@ def test_conv_winograd_path(K, case):
     assert np.abs(got - y).max() < tol
 
 
+@pytest.mark.parametrize("case", [(512, 19, 512, 2), (128, 28, 128, 3), (1024, 13, 256, 1)])
+def test_conv_winograd_error_at_layer_sizes(K, case):
+    """Sums over thousands of products, post-ReLU bottoms and He-scaled filters: the direct
+    path, the Winograd path and the reference's own algorithm (im2col + OpenBLAS sgemm, the
+    oracle) are all held against a float64 convolution with the parity metric (floor 1e-2 of
+    the largest output, bar 1e-4); the Winograd path may not be further from float64 than
+    three times the reference's algorithm is."""
+    cin, hw, cout, n = case
+    rng = np.random.default_rng(23)
+    x = np.maximum(rng.standard_normal((n, cin, hw, hw)), 0).astype(np.float32)
+    wt = (rng.standard_normal((cout, cin, 3, 3)) * np.sqrt(2.0 / (9 * cin))).astype(np.float32)
+    oracle.use_openblas(True)
+    try:
+        want = oracle.conv_forward(oracle.conv_geom(cin, hw, hw, cout, 3, 1, 1), x, wt, None)
+    finally:
+        oracle.use_openblas(False)
+    exact = torch.nn.functional.conv2d(torch.from_numpy(x).double(), torch.from_numpy(wt).double(),
+                                       padding=1).numpy()
+    plan = K.ConvPlan(K.conv_geom(cin, hw, hw, cout, 3, 1, 1))
+    err = {}
+    for mode in (0, 1):
+        plan.force_winograd(mode)
+        got = _run_plan(K, plan, n, x, wt, want.shape)
+        err[mode] = netrun.rel_err(got, exact)
+        assert err[mode] < 1e-4 and netrun.rel_err(got, want) < 1e-4, (case, mode, err)
+    assert err[1] < 3 * max(netrun.rel_err(want, exact), 1e-5), (case, err)
+
+
 @pytest.mark.parametrize("c_first", [1, 16, 50, 99])
 def test_conv_winograd_two_tops(K, c_first):
     """The Winograd path with the output channels split over two blobs (merged sibling
