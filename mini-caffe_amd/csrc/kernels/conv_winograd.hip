@@ -325,7 +325,9 @@ bool winograd_fits(const WinogradState* w, int num) {
   const long blocks = (long)num * ((w->Ho + 1) / 2) * ((w->Wo + 1) / 2);
   const long T = padded_blocks(blocks);
   const long most = 16L * std::max(w->geom.channels_in, w->geom.channels_out) * T;
-  return plane_rows(blocks) < 16384 && most < (1L << 29);
+  // (the transform kernels put channels on the grid's y axis)
+  return plane_rows(blocks) < 16384 && most < (1L << 29) &&
+         std::max(w->geom.channels_in, w->geom.channels_out) <= 65535;
 }
 
 // The automatic choice.  Per output block the direct path multiplies 36 Cin Cout

@@ -19,7 +19,8 @@ dev, fptr = T.dev, T.fptr
 
 def test_random_convolutions(K):
     """Convolution / Deconvolution with random extents, kernel, stride, pad, dilation and
-    groups (depthwise included), random tile configuration and K slices, and a random
+    groups (depthwise included), random tile configuration and K slices (3x3 stride-1 cases
+    left to the automatic choice run on the Winograd path half of the time), and a random
     epilogue (scale, shift, residual, ReLU / leaky ReLU / TanH)."""
     rng = np.random.default_rng(2024)
     done = 0
@@ -32,7 +33,9 @@ def test_random_convolutions(K):
         kh, kw = int(rng.integers(1, 6)), int(rng.integers(1, 6))
         if rng.integers(0, 3) == 0:
             kw = kh
-        sh, sw = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        if rng.integers(0, 5) == 0:
+            kh = kw = 3
+        sh, sw = (1, 1) if rng.integers(0, 3) == 0 else (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
         dh, dw = (int(rng.integers(1, 3)), int(rng.integers(1, 3))) if rng.integers(0, 4) == 0 else (1, 1)
         ph, pw = int(rng.integers(0, 3)), int(rng.integers(0, 3))
         h, w = int(rng.integers(1, 30)), int(rng.integers(1, 30))
@@ -66,6 +69,8 @@ def test_random_convolutions(K):
         slices, config = int(rng.choice([0, 0, 1, 2, 3, 7])), int(rng.choice([-1, -1, 0, 1, 2, 3, 4, 5, 6, 7]))
         plan.force_split(slices)
         plan.force_config(config)
+        if (kh, kw, sh, sw, dh, dw, g, tr) == (3, 3, 1, 1, 1, 1, 1, False) and slices == 0 and config == -1:
+            plan.force_winograd(int(rng.integers(0, 2)))
         ep = dict(scale=sc, shift=b, activation=act, negative_slope=slope)
         if use_res:
             ep["residual"] = res
@@ -73,7 +78,7 @@ def test_random_convolutions(K):
         # absolute against the largest pre-activation value: TanH squeezes a sum of
         # hundreds of products into [-1, 1] without shrinking its rounding noise
         scale_of_sums = max(1.0, float(np.abs(y).max()))
-        assert np.abs(got - want).max() < 2e-6 * scale_of_sums + 1e-6, (geom, n, slices, config, act, use_res)
+        assert np.abs(got - want).max() < 3e-6 * scale_of_sums + 1e-6, (geom, n, slices, config, act, use_res)
         done += 1
     assert done > 200
 
