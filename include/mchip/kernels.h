@@ -162,6 +162,11 @@ int mcConvTimingEnable(int on);
 int mcConvTimingCollect(double* total_ms, long* launches, double* flops);
 int mcConvTimingCollectDetail(double* total_ms, long* launches, double* flops, double* issued_flops,
                               long* winograd);
+/* Of the last collection: device time and FLOPs of the contraction kernel's own
+ * launches alone, the transform kernels left out.  The launches inside Winograd
+ * layers are timed by themselves only under mcConvTimingEnable(2) (two more events
+ * inside the layer's own pair, which lengthen the layer's time a little). */
+int mcConvTimingKernelTotals(double* kernel_ms, double* kernel_flops);
 
 /* HIP stream of the calling thread's Mini-Caffe context (created on first use);
  * lets a harness record events around Net::Forward.  NULL if no device. */

@@ -866,7 +866,10 @@ struct TimedLaunch {
   const char* name;
 };
 thread_local bool g_timing = false;
-thread_local bool g_timing_outer = false;  // a Winograd layer is timed as a whole
+thread_local bool g_timing_nested = false;  // also time the launch inside a Winograd layer
+thread_local bool g_timing_outer = false;  // a Winograd layer is timed as a whole ...
+thread_local std::vector<TimedLaunch> g_timed_inner;  // ... and its contraction launch by itself
+thread_local double g_kernel_ms = 0., g_kernel_flops = 0.;  // of the last collection
 int g_winograd_default = -1;  // mode new plans start with
 thread_local std::vector<TimedLaunch> g_timed;
 
@@ -1345,7 +1348,7 @@ int conv_forward_images(const mcConvPlan* plan, int num, const float* bottom, fl
   }
 
   TimedLaunch tl;
-  const bool timed = g_timing && !g_timing_outer;
+  const bool timed = g_timing && (!g_timing_outer || g_timing_nested);
   if (timed) {
     MC_HIP(hipEventCreate(&tl.start));
     MC_HIP(hipEventCreate(&tl.stop));
@@ -1469,7 +1472,7 @@ int conv_forward_images(const mcConvPlan* plan, int num, const float* bottom, fl
   }
   if (timed) {
     MC_HIP(hipEventRecord(tl.stop, st));
-    g_timed.push_back(tl);
+    (g_timing_outer ? g_timed_inner : g_timed).push_back(tl);
   }
   return 0;
 }
@@ -1559,6 +1562,7 @@ int mcConvForwardTwoTops(const mcConvPlan* plan, int num, const float* bottom, f
 
 int mcConvTimingEnable(int on) {
   g_timing = on != 0;
+  g_timing_nested = on == 2;
   return 0;
 }
 
@@ -1566,6 +1570,7 @@ int mcConvTimingCollectDetail(double* total_ms, long* launches, double* flops, d
                               long* winograd) {
   double ms = 0., fl = 0., is = 0.;
   long wino = 0;
+  g_kernel_ms = g_kernel_flops = 0.;
   for (auto& t : g_timed) {
     MC_HIP(hipEventSynchronize(t.stop));
     float e = 0.f;
@@ -1574,15 +1579,35 @@ int mcConvTimingCollectDetail(double* total_ms, long* launches, double* flops, d
     fl += t.flops;
     is += t.issued;
     wino += t.issued != t.flops;
+    if (t.issued == t.flops) {
+      g_kernel_ms += e;
+      g_kernel_flops += t.issued;
+    }
     (void)hipEventDestroy(t.start);
     (void)hipEventDestroy(t.stop);
   }
+  for (auto& t : g_timed_inner) {  // the contraction launches inside Winograd layers
+    MC_HIP(hipEventSynchronize(t.stop));
+    float e = 0.f;
+    MC_HIP(hipEventElapsedTime(&e, t.start, t.stop));
+    g_kernel_ms += e;
+    g_kernel_flops += t.issued;
+    (void)hipEventDestroy(t.start);
+    (void)hipEventDestroy(t.stop);
+  }
+  g_timed_inner.clear();
   if (total_ms) *total_ms = ms;
   if (launches) *launches = static_cast<long>(g_timed.size());
   if (flops) *flops = fl;
   if (issued_flops) *issued_flops = is;
   if (winograd) *winograd = wino;
   g_timed.clear();
+  return 0;
+}
+
+int mcConvTimingKernelTotals(double* kernel_ms, double* kernel_flops) {
+  if (kernel_ms) *kernel_ms = g_kernel_ms;
+  if (kernel_flops) *kernel_flops = g_kernel_flops;
   return 0;
 }
 

@@ -57,6 +57,7 @@ LIB.mcConvTimingCollectDetail.argtypes = [ctypes.POINTER(ctypes.c_double), ctype
                                           ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
                                           ctypes.POINTER(c_long)]
 
+LIB.mcConvTimingKernelTotals.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
 LIB.mcDetectionOutputWorkspaceSize.argtypes = [c_int, c_int, c_int, c_int, c_int,
                                                ctypes.POINTER(ctypes.c_size_t)]
 LIB.mcDetectionOutputMaxRows.argtypes = [c_int] * 5
