@@ -384,7 +384,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
     }                                                                                        \
   }
 
-  // Order of a stage's instructions inside a wavefront: the LDS reads, three quarters
+  // Order of a stage's instructions inside a wavefront: the global loads of the next
+  // stage (as a group the scheduler keeps first, not behind a hard scheduling barrier:
+  // their scalar address arithmetic may mix with what follows), the LDS reads, three quarters
   // of the stage's MFMAs, the LDS stores of the next stage (which wait for its global
   // loads), the last quarter.  The last MFMAs work on registers only, so the compiler
   // lets them sink below the barrier that follows, next to the loads and LDS reads of
@@ -393,6 +395,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
   // path) 5.01 ms per forward, stores after half of the block 4.86, after a quarter
   // 4.91, after three quarters 4.87 (4.64 -> 4.54 with the Winograd layers).
 #define MC_INTERLEAVE()                                                   \
+  __builtin_amdgcn_sched_group_barrier(0x020, 32, 0);                     \
   __builtin_amdgcn_sched_group_barrier(0x100, 2 * KS * (TM + TN), 0);     \
   __builtin_amdgcn_sched_group_barrier(0x008, 6 * KS * TM * TN, 0);       \
   __builtin_amdgcn_sched_group_barrier(0x200, 16, 0);                     \
@@ -433,13 +436,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
     int t = 0;
     for (; t + 2 < nk; t += 2) {
       MC_LOAD_TILES(kt_begin + t + 1);
-      __builtin_amdgcn_sched_barrier(0);  // keep the global loads ahead of the MFMA block
       MC_COMPUTE(0);
       MC_STORE_TILES(1);
       MC_INTERLEAVE();
       __syncthreads();
       MC_LOAD_TILES(kt_begin + t + 2);
-      __builtin_amdgcn_sched_barrier(0);
       MC_COMPUTE(1);
       MC_STORE_TILES(0);
       MC_INTERLEAVE();
@@ -448,10 +449,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
     // one or two tiles left; tile t is in buffer 0
     if (t + 1 < nk) {
       MC_LOAD_TILES(kt_begin + t + 1);
-      __builtin_amdgcn_sched_barrier(0);
       MC_COMPUTE(0);
-      __builtin_amdgcn_sched_barrier(0);
       MC_STORE_TILES(1);
+      MC_INTERLEAVE();
       __syncthreads();
       MC_COMPUTE(1);
     } else {
