@@ -134,39 +134,29 @@ int mcConvPlanForceSplit(mcConvPlan* plan, int slices);
 int mcConvPlanForceChunk(mcConvPlan* plan, int images);
 
 /* A 3x3 convolution with stride 1, no dilation and one group can run as
- * F(2x2, 3x3) Winograd: the bottom is transformed into sixteen [Cin, blocks]
- * matrices, the sixteen products with the transformed filters run as one grouped
- * 1x1 contraction on the same kernel, and the output transform applies the
- * epilogue (2.25 times fewer multiplications, four times the intermediate
- * traffic; the sums associate differently from the direct path, both within fp32
- * rounding of conv_layer.cpp:27-42).  mode -1 lets the library decide by size,
- * 0 keeps the direct path, 1 takes this one whenever the geometry allows.
+ * F(2x2, 3x3) Winograd in one launch: the loader transforms the 4x4 input patches
+ * on their way into LDS, sixteen products with the transformed filters run on the
+ * matrix cores, and the output transform applies the epilogue before the store
+ * (2.25 times fewer multiplications and no intermediate in memory; the sums
+ * associate differently from the direct path, both within fp32 rounding of
+ * conv_layer.cpp:27-42).  mode -1 lets the library decide by size, 0 keeps the
+ * direct path, 1 takes this one whenever the geometry allows.
  * mcConvWinogradDefault sets the mode that plans created afterwards start with.
  * No counterpart in the reference. */
 int mcConvPlanForceWinograd(mcConvPlan* plan, int mode);
 int mcConvWinogradDefault(int mode);
-/* Tuning knob: the transformed bottom and the products of one run of images may
- * take this many bytes of workspace together; a larger batch is cut into equal
- * runs of whole images that fit (default 1 GiB).  No counterpart in the reference. */
-int mcConvWinogradRunBytes(long bytes);
 
 /* Measurement hook (no counterpart in the reference): while enabled on the
- * calling thread, every contraction (one kernel launch; on the Winograd path the
- * input transform, the contraction launch and the output transform together) is
- * bracketed by two HIP events recorded on the launch stream.  mcConvTimingCollect
- * waits for them, returns the summed device time, the number of contractions and
- * their algorithmic FLOPs (those of the direct sum), and clears the list;
+ * calling thread, every contraction (one kernel launch) is bracketed by two HIP
+ * events recorded on the launch stream.  mcConvTimingCollect waits for them,
+ * returns the summed device time, the number of contractions and their
+ * algorithmic FLOPs (those of the direct sum), and clears the list;
  * mcConvTimingCollectDetail also returns the FLOPs handed to the matrix pipe
  * (fewer on the Winograd path) and the number of Winograd contractions. */
 int mcConvTimingEnable(int on);
 int mcConvTimingCollect(double* total_ms, long* launches, double* flops);
 int mcConvTimingCollectDetail(double* total_ms, long* launches, double* flops, double* issued_flops,
                               long* winograd);
-/* Of the last collection: device time and FLOPs of the contraction kernel's own
- * launches alone, the transform kernels left out.  The launches inside Winograd
- * layers are timed by themselves only under mcConvTimingEnable(2) (two more events
- * inside the layer's own pair, which lengthen the layer's time a little). */
-int mcConvTimingKernelTotals(double* kernel_ms, double* kernel_flops);
 
 /* HIP stream of the calling thread's Mini-Caffe context (created on first use);
  * lets a harness record events around Net::Forward.  NULL if no device. */

@@ -104,11 +104,6 @@ __device__ __forceinline__ float f4at(const float4& v, int e) {
   return e == 0 ? v.x : (e == 1 ? v.y : (e == 2 ? v.z : v.w));
 }
 
-// n / d for the d the host prepared (mul, shift) for; shift == 32 means d == 1.
-__device__ __forceinline__ int fast_div(int n, unsigned mul, unsigned shift) {
-  return shift == 32 ? n : static_cast<int>(__umulhi(static_cast<unsigned>(n), mul) >> shift);
-}
-
 __device__ __forceinline__ float apply_act(float v, int act, float slope) {
   switch (act) {
     case MC_ACT_RELU:
@@ -881,10 +876,6 @@ struct TimedLaunch {
   const char* name;
 };
 thread_local bool g_timing = false;
-thread_local bool g_timing_nested = false;  // also time the launch inside a Winograd layer
-thread_local bool g_timing_outer = false;  // a Winograd layer is timed as a whole ...
-thread_local std::vector<TimedLaunch> g_timed_inner;  // ... and its contraction launch by itself
-thread_local double g_kernel_ms = 0., g_kernel_flops = 0.;  // of the last collection
 int g_winograd_default = -1;  // mode new plans start with
 thread_local std::vector<TimedLaunch> g_timed;
 
@@ -944,26 +935,6 @@ int free_sub(SubProblem& s) {
   s.wk_off_dev = nullptr;
   s.wt_dev = nullptr;
   return 0;
-}
-
-// Multiplier and shift with  n / d == mulhi(n, mul) >> shift  for 0 <= n < n_max.
-// shift 32 stands for d == 1 (no 32-bit multiplier exists for it).
-void make_fast_div(unsigned d, unsigned long long n_max, unsigned* mul, unsigned* shift) {
-  *mul = 0;
-  *shift = 32;
-  if (d <= 1) return;
-  for (int s = 31; s >= 0; --s) {
-    const unsigned __int128 pow = (unsigned __int128)1 << (32 + s);
-    const unsigned __int128 m = (pow + d - 1) / d;
-    if (m >> 32) continue;
-    const unsigned __int128 err = m * d - pow;  // 0 <= err < d
-    if (err * n_max < pow) {
-      *mul = static_cast<unsigned>(m);
-      *shift = static_cast<unsigned>(s);
-      return;
-    }
-  }
-  // unreachable for n_max < 2^32: s = 0 gives err * n_max < d * 2^32 / d
 }
 
 // floor division for possibly negative numerators
@@ -1222,8 +1193,6 @@ int mcConvPlanForceWinograd(mcConvPlan* plan, int mode) {
   return 0;
 }
 
-int mcConvWinogradRunBytes(long bytes) { return winograd_set_run_bytes(bytes); }
-
 int mcConvWinogradDefault(int mode) {
   MC_REQUIRE(mode >= -1 && mode <= 1, "mcConvWinogradDefault: bad argument");
   g_winograd_default = mode;
@@ -1363,7 +1332,7 @@ int conv_forward_images(const mcConvPlan* plan, int num, const float* bottom, fl
   }
 
   TimedLaunch tl;
-  const bool timed = g_timing && (!g_timing_outer || g_timing_nested);
+  const bool timed = g_timing;
   if (timed) {
     MC_HIP(hipEventCreate(&tl.start));
     MC_HIP(hipEventCreate(&tl.stop));
@@ -1487,9 +1456,16 @@ int conv_forward_images(const mcConvPlan* plan, int num, const float* bottom, fl
   }
   if (timed) {
     MC_HIP(hipEventRecord(tl.stop, st));
-    (g_timing_outer ? g_timed_inner : g_timed).push_back(tl);
+    g_timed.push_back(tl);
   }
   return 0;
+}
+
+// Whether a call with `num` images runs on the Winograd path.
+bool takes_winograd(const mcConvPlan* plan, int num) {
+  return plan->winograd && plan->winograd_mode != 0 && plan->forced_config < 0 &&
+         winograd_fits(plan->winograd, num) &&
+         (plan->winograd_mode == 1 || winograd_pays(plan->winograd, num));
 }
 
 // The reference convolves image by image and so takes any blob an int can count
@@ -1504,12 +1480,9 @@ int conv_forward(const mcConvPlan* plan, int num, const float* bottom, float* to
   const mcConvGeom& g = plan->geom;
   if (plan->depthwise)  // indexed with 64-bit integers throughout
     return conv_forward_images(plan, num, bottom, top, ep, stream, top_second, c_first);
-  if (plan->winograd && plan->winograd_mode != 0 && plan->forced_config < 0 &&
-      plan->forced_split == 0 && plan->forced_chunk == 0 && winograd_fits(plan->winograd, num) &&
-      (plan->winograd_mode == 1 || winograd_pays(plan->winograd, num))) {
-    // timed as one contraction: both transforms belong to the layer's cost
+  if (takes_winograd(plan, num)) {
     TimedLaunch tl;
-    const bool timed = g_timing && !g_timing_outer;
+    const bool timed = g_timing;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (timed) {
       MC_HIP(hipEventCreate(&tl.start));
@@ -1518,11 +1491,10 @@ int conv_forward(const mcConvPlan* plan, int num, const float* bottom, float* to
       tl.issued = winograd_issued_flops(plan->winograd, num);
       tl.name = "winograd_f32";
       MC_HIP(hipEventRecord(tl.start, st));
-      g_timing_outer = true;
     }
-    const int rc = winograd_forward(plan->winograd, num, bottom, top, ep, stream, top_second, c_first);
+    const int rc = winograd_forward(plan->winograd, num, bottom, top, ep, stream, top_second, c_first,
+                                    plan->forced_chunk, plan->forced_split);
     if (timed) {
-      g_timing_outer = false;
       MC_HIP(hipEventRecord(tl.stop, st));
       g_timed.push_back(tl);
     }
@@ -1577,7 +1549,6 @@ int mcConvForwardTwoTops(const mcConvPlan* plan, int num, const float* bottom, f
 
 int mcConvTimingEnable(int on) {
   g_timing = on != 0;
-  g_timing_nested = on == 2;
   return 0;
 }
 
@@ -1585,7 +1556,6 @@ int mcConvTimingCollectDetail(double* total_ms, long* launches, double* flops, d
                               long* winograd) {
   double ms = 0., fl = 0., is = 0.;
   long wino = 0;
-  g_kernel_ms = g_kernel_flops = 0.;
   for (auto& t : g_timed) {
     MC_HIP(hipEventSynchronize(t.stop));
     float e = 0.f;
@@ -1594,35 +1564,15 @@ int mcConvTimingCollectDetail(double* total_ms, long* launches, double* flops, d
     fl += t.flops;
     is += t.issued;
     wino += t.issued != t.flops;
-    if (t.issued == t.flops) {
-      g_kernel_ms += e;
-      g_kernel_flops += t.issued;
-    }
     (void)hipEventDestroy(t.start);
     (void)hipEventDestroy(t.stop);
   }
-  for (auto& t : g_timed_inner) {  // the contraction launches inside Winograd layers
-    MC_HIP(hipEventSynchronize(t.stop));
-    float e = 0.f;
-    MC_HIP(hipEventElapsedTime(&e, t.start, t.stop));
-    g_kernel_ms += e;
-    g_kernel_flops += t.issued;
-    (void)hipEventDestroy(t.start);
-    (void)hipEventDestroy(t.stop);
-  }
-  g_timed_inner.clear();
   if (total_ms) *total_ms = ms;
   if (launches) *launches = static_cast<long>(g_timed.size());
   if (flops) *flops = fl;
   if (issued_flops) *issued_flops = is;
   if (winograd) *winograd = wino;
   g_timed.clear();
-  return 0;
-}
-
-int mcConvTimingKernelTotals(double* kernel_ms, double* kernel_flops) {
-  if (kernel_ms) *kernel_ms = g_kernel_ms;
-  if (kernel_flops) *kernel_flops = g_kernel_flops;
   return 0;
 }
 
@@ -1642,10 +1592,7 @@ double mcConvPlanFlops(const mcConvPlan* plan, int num) {
 const char* mcConvPlanKernelName(const mcConvPlan* plan, int num) {
   if (plan && plan->depthwise) return "depthwise_f32";
   if (!plan || plan->subs.empty()) return "";
-  if (plan->winograd && plan->winograd_mode != 0 && plan->forced_config < 0 &&
-      plan->forced_split == 0 && plan->forced_chunk == 0 && winograd_fits(plan->winograd, num) &&
-      (plan->winograd_mode == 1 || winograd_pays(plan->winograd, num)))
-    return "winograd_f32";
+  if (takes_winograd(plan, num)) return "winograd_f32";
   if (use_thin(plan, num)) return "thin_f32";
   const auto& s = plan->subs[0];
   return kConfigs[pick_config(plan, (long)num * s.Hq * s.Wq)].name;

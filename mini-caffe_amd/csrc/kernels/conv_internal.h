@@ -25,20 +25,48 @@ struct DepthwiseArgs {
 // y[n][c*mult+j][ho][wo] = act((sum over taps w * x) * scale + shift + residual).
 int depthwise_forward(const DepthwiseArgs& a, hipStream_t stream);
 
-// 3x3 stride-1 convolution as F(2x2, 3x3) Winograd: input transform, sixteen
-// grouped 1x1 contractions on the implicit-GEMM kernel, output transform with
-// the layer's epilogue.  winograd_create returns null for any other geometry.
+// Multiplier and shift with  n / d == mulhi(n, mul) >> shift  for 0 <= n < n_max.
+// shift 32 stands for d == 1 (no 32-bit multiplier exists for it).
+inline void make_fast_div(unsigned d, unsigned long long n_max, unsigned* mul, unsigned* shift) {
+  *mul = 0;
+  *shift = 32;
+  if (d <= 1) return;
+  for (int s = 31; s >= 0; --s) {
+    const unsigned __int128 pow = (unsigned __int128)1 << (32 + s);
+    const unsigned __int128 m = (pow + d - 1) / d;
+    if (m >> 32) continue;
+    const unsigned __int128 err = m * d - pow;  // 0 <= err < d
+    if (err * n_max < pow) {
+      *mul = static_cast<unsigned>(m);
+      *shift = static_cast<unsigned>(s);
+      return;
+    }
+  }
+  // unreachable for n_max < 2^32: s = 0 gives err * n_max < d * 2^32 / d
+}
+
+// n / d for the d the host prepared (mul, shift) for; shift == 32 means d == 1.
+__device__ __forceinline__ int fast_div(int n, unsigned mul, unsigned shift) {
+  return shift == 32 ? n : static_cast<int>(__umulhi(static_cast<unsigned>(n), mul) >> shift);
+}
+
+// 3x3 stride-1 convolution as F(2x2, 3x3) Winograd in one launch: the input
+// transform in the loader, the sixteen products on the matrix cores, the output
+// transform and the layer's epilogue before the store.  winograd_create returns
+// null for any other geometry.
 struct WinogradState;
 WinogradState* winograd_create(const mcConvGeom& geom, int Ho, int Wo);
 void winograd_destroy(WinogradState* w);
 int winograd_set_weights(WinogradState* w, const float* weights, hipStream_t stream);
-bool winograd_fits(const WinogradState* w, int num);  // intermediates addressable
+bool winograd_fits(const WinogradState* w, int num);  // one image addressable by the kernel
 bool winograd_pays(const WinogradState* w, int num);  // the automatic choice
 double winograd_issued_flops(const WinogradState* w, int num);  // of the sixteen products
-int winograd_set_run_bytes(long bytes);  // budget for V + M of one run of images
-// top_second / c_first as in mcConvForwardTwoTops (null / ignored for one top)
+// top_second / c_first as in mcConvForwardTwoTops (null / ignored for one top);
+// images_per_run > 0 caps the images one launch takes, forced_slices > 0 fixes the
+// number of slices the input channels are cut into
 int winograd_forward(WinogradState* w, int num, const float* bottom, float* top,
-                     const mcEpilogue* ep, void* stream, float* top_second, int c_first);
+                     const mcEpilogue* ep, void* stream, float* top_second, int c_first,
+                     int images_per_run, int forced_slices);
 
 }  // namespace mchip
 

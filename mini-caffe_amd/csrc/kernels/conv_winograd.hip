@@ -7,20 +7,26 @@
 // d the 4x4 input patch under the block, g the 3x3 filter.  Summed over the
 // input channels the element-wise products are sixteen independent matrix
 // products  M_f[Cout][T] = U_f[Cout][Cin] * V_f[Cin][T]  (f = position in the
-// 4x4 transform, T = 2x2 output blocks of the whole batch), which is exactly a
-// 1x1 convolution with sixteen groups: it runs on the implicit-GEMM kernel of
-// conv_igemm.hip through the plan interface.  Three launches per layer:
+// 4x4 transform, T = 2x2 output blocks of the whole batch).  One kernel does all
+// of it for a tile of 64 output channels x 32 blocks:
 //
-//   winograd_input_kernel    bottom [N, C, H, W]        -> V [16, C, Tpad]
-//   igemm (pointwise, g=16)  V, U                       -> M [16, Cout, Tpad]
-//   winograd_output_kernel   M (+ scale/shift/residual) -> top [N, Cout, Ho, Wo]
+//   loader    every thread fetches three rows of a block's 4x4 patch of one
+//             channel straight from the bottom blob, forms eight of the sixteen
+//             V values in registers and stores them as the B operands in LDS;
+//             the transformed filters U (packed once per weight change in the
+//             order the tile consumes them) are copied to LDS as they are;
+//   products  wavefront w multiplies the four transform positions of row w,
+//             f = 4 w .. 4 w + 3: 8 accumulator blocks of 32 x 32 per wavefront,
+//             v_mfma_f32_32x32x2_f32;
+//   finish    A^T m A: the sums over a transform row in registers, the sums
+//             over the four rows (= wavefronts) through LDS, then the layer's
+//             epilogue (scale, shift, residual, activation) and the store.
 //
-// V and M are four times the size of bottom and top, so the detour pays where
-// the contraction dominates the traffic: many channels on both sides.  Replaces
-// the same reference code as the direct path (conv_layer.cu:7-22 with
-// base_conv_layer.cpp:254-278); sums are associated differently from a direct
-// convolution (transformed operands, K order over input channels only), within
-// the usual fp32 rounding of either.
+// Neither V nor M ever exists in memory: the launch reads the bottom blob and
+// the filters and writes the top blob.  Replaces the same reference code as the
+// direct path (conv_layer.cu:7-22 with base_conv_layer.cpp:254-278); sums are
+// associated differently from a direct convolution (transformed operands, K
+// order over input channels only), within the usual fp32 rounding of either.
 #include "conv_internal.h"
 #include "mc_common.h"
 #include "mchip/kernels.h"
@@ -31,15 +37,17 @@ namespace mchip {
 
 namespace {
 
-// Channels a thread of a transform kernel walks with one decomposition of its
-// block index: four where the launch still has a few workgroups per CU, fewer on
-// small maps (7x7 maps of 64 images are 1024 blocks: four workgroups per channel
-// group), so that the launch keeps enough loads in flight.
-inline int channels_per_thread(long tblocks, int channels, int least) {
-  for (int cpt = 4; cpt > least; cpt /= 2)
-    if (tblocks * ((channels + cpt - 1) / cpt) >= 8L * kNumCu) return cpt;
-  return least;
-}
+constexpr int kTileM = 64;   // output channels of a tile
+constexpr int kTileT = 32;   // 2x2 output blocks of a tile
+constexpr int kStageC = 4;   // input channels per K stage
+constexpr int kAStage = 16 * kTileM * kStageC;  // floats of U per stage and tile
+constexpr int kBStage = 16 * kTileT * kStageC;  // floats of V per stage and tile
+constexpr int kBufferFlags = 0x00020000;        // raw dword buffer, offsets range-checked
+constexpr unsigned kNoElement = 0x80000000u;    // beyond every buffer this file builds
+
+typedef float acc16 __attribute__((ext_vector_type(16)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float act_value(float v, int act, float slope) {
   switch (act) {
@@ -54,17 +62,24 @@ __device__ __forceinline__ float act_value(float v, int act, float slope) {
   }
 }
 
-// U[f][co][ci] = (G g G^T)[f / 4][f % 4], G = [1 0 0; 1/2 1/2 1/2; 1/2 -1/2 1/2; 0 0 1].
-// One thread per filter.
-__global__ __launch_bounds__(256) void winograd_filter_kernel(const float* __restrict__ w,
-                                                              float* __restrict__ u, long filters) {
+// Transformed filters in the order a tile's stages read them:
+//   u[mt][kt][f][kp][m][e] = (G g G^T)[f / 4][f % 4]  of filter (co, ci),
+//   co = 64 mt + m, ci = 4 kt + 2 kp + e,  G = [1 0 0; 1/2 1/2 1/2; 1/2 -1/2 1/2; 0 0 1],
+// zero where co or ci lie past the layer's channels (KT is even: the loader works in
+// rounds of eight channels).  One thread per (co, ci) of the padded extents.
+__global__ __launch_bounds__(256) void winograd_pack_filter_kernel(const float* __restrict__ w,
+                                                                   float* __restrict__ u, int Cout,
+                                                                   int C, int MT, int KT) {
   const long i = blockIdx.x * 256L + threadIdx.x;
-  if (i >= filters) return;
+  const int cpad = KT * kStageC;
+  if (i >= (long)MT * kTileM * cpad) return;
+  const int co = static_cast<int>(i / cpad), ci = static_cast<int>(i % cpad);
   float g[3][3];
 #pragma unroll
   for (int r = 0; r < 3; ++r)
 #pragma unroll
-    for (int c = 0; c < 3; ++c) g[r][c] = w[i * 9 + r * 3 + c];
+    for (int c = 0; c < 3; ++c)
+      g[r][c] = (co < Cout && ci < C) ? w[((long)co * C + ci) * 9 + r * 3 + c] : 0.f;
   float t[4][3];
 #pragma unroll
   for (int c = 0; c < 3; ++c) {
@@ -73,159 +88,403 @@ __global__ __launch_bounds__(256) void winograd_filter_kernel(const float* __res
     t[2][c] = 0.5f * (g[0][c] - g[1][c] + g[2][c]);
     t[3][c] = g[2][c];
   }
+  const int mt = co / kTileM, m = co % kTileM;
+  const int kt = ci / kStageC, kp = (ci % kStageC) / 2, e = ci % 2;
+  float* out = u + ((long)mt * KT + kt) * kAStage + kp * (kTileM * 2) + m * 2 + e;
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    u[(r * 4 + 0) * filters + i] = t[r][0];
-    u[(r * 4 + 1) * filters + i] = 0.5f * (t[r][0] + t[r][1] + t[r][2]);
-    u[(r * 4 + 2) * filters + i] = 0.5f * (t[r][0] - t[r][1] + t[r][2]);
-    u[(r * 4 + 3) * filters + i] = t[r][2];
+    out[(r * 4 + 0) * (kTileM * kStageC)] = t[r][0];
+    out[(r * 4 + 1) * (kTileM * kStageC)] = 0.5f * (t[r][0] + t[r][1] + t[r][2]);
+    out[(r * 4 + 2) * (kTileM * kStageC)] = 0.5f * (t[r][0] - t[r][1] + t[r][2]);
+    out[(r * 4 + 3) * (kTileM * kStageC)] = t[r][2];
   }
 }
 
-struct WinogradShape {
-  int C, H, W, Cout, Ho, Wo, pad_h, pad_w;
-  int Th, Tw;       // 2x2 output blocks per image, down and across
-  int T, Tpad;      // blocks of the batch; columns of V and M
-};
-
-// V[f][c][t] = (B^T d B)[f / 4][f % 4], B^T = [1 0 -1 0; 0 1 1 0; 0 -1 1 0; 0 1 0 -1];
-// d = the 4x4 patch of channel c whose corner is output block t's corner minus
-// the padding (zeros outside the map).  Lanes run along t, so the sixteen stores
-// of a channel are contiguous rows; a thread walks kChannelsPerThread channels
-// with one decomposition of t.
-template <int CPT>
-__global__ __launch_bounds__(256) void winograd_input_kernel(const float* __restrict__ x,
-                                                             float* __restrict__ v,
-                                                             const WinogradShape s) {
-  constexpr int kChannelsPerThread = CPT;
-  const int t = blockIdx.x * 256 + threadIdx.x;
-  if (t >= s.Tpad) return;
-  const int c0 = blockIdx.y * kChannelsPerThread;
-  const long fstride = (long)s.C * s.Tpad;
-  if (t >= s.T) {
-    for (int c = c0; c < min(c0 + kChannelsPerThread, s.C); ++c)
-#pragma unroll
-      for (int f = 0; f < 16; ++f) v[f * fstride + (long)c * s.Tpad + t] = 0.f;
-    return;
-  }
-  const int per_image = s.Th * s.Tw;
-  const int n = t / per_image;
-  const int rem = t - n * per_image;
-  const int ty = rem / s.Tw;
-  const int tx = rem - ty * s.Tw;
-  const int h0 = 2 * ty - s.pad_h, w0 = 2 * tx - s.pad_w;
-  bool row_ok[4], col_ok[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    row_ok[i] = static_cast<unsigned>(h0 + i) < static_cast<unsigned>(s.H);
-    col_ok[i] = static_cast<unsigned>(w0 + i) < static_cast<unsigned>(s.W);
-  }
-  for (int c = c0; c < min(c0 + kChannelsPerThread, s.C); ++c) {
-    const float* plane = x + ((long)n * s.C + c) * s.H * s.W;
-    float d[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        d[i][j] = (row_ok[i] && col_ok[j]) ? plane[(h0 + i) * s.W + w0 + j] : 0.f;
-    float r[4][4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      r[0][j] = d[0][j] - d[2][j];
-      r[1][j] = d[1][j] + d[2][j];
-      r[2][j] = d[2][j] - d[1][j];
-      r[3][j] = d[1][j] - d[3][j];
-    }
-    float* out = v + (long)c * s.Tpad + t;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      out[(i * 4 + 0) * fstride] = r[i][0] - r[i][2];
-      out[(i * 4 + 1) * fstride] = r[i][1] + r[i][2];
-      out[(i * 4 + 2) * fstride] = r[i][2] - r[i][1];
-      out[(i * 4 + 3) * fstride] = r[i][1] - r[i][3];
-    }
-  }
-}
-
-struct WinogradEpilogue {
-  const float* scale;
-  const float* shift;
-  const float* residual;
+struct WinogradArgs {
+  const float* __restrict__ x;   // bottom [num, C, H, W]
+  const float* __restrict__ u;   // packed filters, see winograd_pack_filter_kernel
+  float* __restrict__ y;         // top [num, c_first, Ho, Wo]
+  float* __restrict__ y_second;  // [num, Cout - c_first, Ho, Wo] or null
+  const float* __restrict__ scale;
+  const float* __restrict__ shift;
+  const float* __restrict__ residual;
+  unsigned x_bytes, u_bytes;
+  int C, H, W, HW;
+  int x_nstride;  // C * H * W
+  int Cout, Ho, Wo, HoWo;
+  int pad_h, pad_w;
+  int Tw, ThTw, T;  // blocks across, per image, in the run
+  unsigned div_img_mul, div_img_shift;  // t / ThTw
+  unsigned div_tw_mul, div_tw_shift;    // rem / Tw
+  unsigned div_mt_mul, div_mt_shift;    // logical tile / MT
+  int MT, NT, KT;
+  int c_first;
   int act;
   float slope;
-  // two sibling layers computed together: channels [0, c_first) of every image go
-  // to the first top [N, c_first, Ho, Wo], the others to y_second; one top: c_first = Cout
-  float* y_second;
-  int c_first;
+  int pairs;  // a block's two outputs of a row may go out as one 8-byte store
+  // The channel rounds cut into slices (blockIdx.y), summed inside the launch: every
+  // workgroup leaves its 64 row sums per thread in `partial`
+  // ([slice][tile][value][thread]) and counts in counters[tile]; the last one to arrive
+  // adds the slices in slice order, finishes the tile and puts the counter back to zero.
+  int rounds_per_slice;
+  float* partial;
+  int* counters;
 };
 
-// Y = A^T m A, A^T = [1 1 1 0; 0 1 -1 -1], m[f] = M[f][co][t]; then the layer's
-// epilogue  act(Y * scale[co] + shift[co] + residual)  on the up to four outputs
-// of block t that lie inside the map.
-template <bool PAIRS, int CPT>
-__global__ __launch_bounds__(256) void winograd_output_kernel(const float* __restrict__ m,
-                                                              float* __restrict__ y,
-                                                              const WinogradShape s,
-                                                              const WinogradEpilogue e) {
-  constexpr int kChannelsPerThread = CPT;
-  const int t = blockIdx.x * 256 + threadIdx.x;
-  if (t >= s.T) return;
-  const int c0 = blockIdx.y * kChannelsPerThread;
-  const long fstride = (long)s.Cout * s.Tpad;
-  const int per_image = s.Th * s.Tw;
-  const int n = t / per_image;
-  const int rem = t - n * per_image;
-  const int ty = rem / s.Tw;
-  const int tx = rem - ty * s.Tw;
-  const int ho = 2 * ty, wo = 2 * tx;
-  const bool row1 = ho + 1 < s.Ho, col1 = wo + 1 < s.Wo;
-  for (int c = c0; c < min(c0 + kChannelsPerThread, s.Cout); ++c) {
-    const float* in = m + (long)c * s.Tpad + t;
-    float q[4][4];
+// Lane l of v_mfma_f32_32x32x2_f32 supplies A[l % 32][l / 32] and B[l / 32][l % 32];
+// which two physical K rows form a step is free as long as both operands agree,
+// so half-wave h reads the stage's channels 2 h and 2 h + 1 with one 8-byte LDS read
+// and step e multiplies channels {e, 2 + e}.
+template <int DIAG>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void winograd_fused_kernel(
+    const WinogradArgs a) {
+  // K loop: As[2][f 16][kp 2][m 64][e 2], Bs[2][2][f 16][kp 2][t 32][e 2]  (64 KB);
+  // finish: Es[dj 2][i 4][co 64][t 32]                                     (64 KB)
+  __shared__ __attribute__((aligned(16))) float lds[2 * 4 * kTileM * kTileT];
+  float* const As = lds;
+  float* const Bs = lds + 2 * kAStage;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31;
+  const int lhi = lane >> 5;
+
+  // Workgroup ids are dealt round-robin to the 8 XCDs: give each XCD a contiguous
+  // run of logical tiles (channel tiles fastest), so the tiles that share a patch
+  // tile and neighbouring patch tiles meet in one L2.
+  int mt, nt;
+  {
+    const int total = a.MT * a.NT;
+    const int bid = blockIdx.x;
+    const int q = total / kNumXcd, r = total % kNumXcd;
+    const int xcd = bid % kNumXcd, local = bid / kNumXcd;
+    const int logical = xcd * q + (xcd < r ? xcd : r) + local;
+    nt = fast_div(logical, a.div_mt_mul, a.div_mt_shift);
+    mt = logical - nt * a.MT;
+  }
+
+  const __amdgpu_buffer_rsrc_t xres =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.x), 0, a.x_bytes, kBufferFlags);
+  const __amdgpu_buffer_rsrc_t ures =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.u), 0, a.u_bytes, kBufferFlags);
+
+  // Loader of the bottom blob: a round covers eight channels (two K stages).
+  // Wavefront w takes channels 2 w and 2 w + 1 of the round (lane / 32), lane % 32 is
+  // the block; a thread fetches the block's whole 4x4 patch of its channel with
+  // sixteen dword loads whose byte offsets are fixed over the K loop (the round's
+  // first channel rides in the scalar offset), forms the sixteen V values in
+  // registers and stores them where the products read them.  An element outside the
+  // map or past the last block has bit 31 set, which is beyond the buffer: it reads
+  // as zero.  The loads of round s + 1 are issued before the products of round s and
+  // first touched after them: two K stages to cover the latency of memory.
+  unsigned boff[4][4];
+  {
+    const int t = nt * kTileT + l32;
+    const bool tv = t < a.T;
+    const int n = fast_div(t, a.div_img_mul, a.div_img_shift);
+    const int rem = t - n * a.ThTw;
+    const int ty = fast_div(rem, a.div_tw_mul, a.div_tw_shift);
+    const int tx = rem - ty * a.Tw;
+    const int h0 = 2 * ty - a.pad_h, w0 = 2 * tx - a.pad_w;
+    const unsigned origin =
+        (static_cast<unsigned>(n) * a.x_nstride + static_cast<unsigned>(2 * wave + lhi) * a.HW) * 4u;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 4; ++i) {
+      const int hh = h0 + i;
+      const bool row_ok = tv && static_cast<unsigned>(hh) < static_cast<unsigned>(a.H);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) q[i][j] = in[(i * 4 + j) * fstride];
-    float a[2][4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      a[0][j] = q[0][j] + q[1][j] + q[2][j];
-      a[1][j] = q[1][j] - q[2][j] - q[3][j];
+      for (int j = 0; j < 4; ++j) {
+        const int ww = w0 + j;
+        const bool ok = row_ok && static_cast<unsigned>(ww) < static_cast<unsigned>(a.W);
+        boff[i][j] = ok ? origin + static_cast<unsigned>(hh * a.W + ww) * 4u : kNoElement;
+      }
     }
+  }
+  const int rounds = a.KT / 2;
+  const int s_begin = blockIdx.y * a.rounds_per_slice;  // this slice's rounds (never empty)
+  const int s_end = min(rounds, s_begin + a.rounds_per_slice);
+  // the last round of a channel count that is no multiple of eight: a lane whose
+  // channel does not exist gets the "no element" offsets before that round is fetched
+  const bool ragged = (a.C & 7) != 0;
+  const bool no_channel = 8 * (rounds - 1) + 2 * wave + lhi >= a.C;
+#define MC_DROP_MISSING_CHANNELS()                                           \
+  _Pragma("unroll") for (int i = 0; i < 4; ++i) {                            \
+    _Pragma("unroll") for (int j = 0; j < 4; ++j)                            \
+      boff[i][j] = no_channel ? kNoElement : boff[i][j];                     \
+  }
+  // LDS places (in floats) of what this thread stores and reads
+  const int a_st = tid * 4;
+  // (the two B buffers alternate by round: both places flip by the size of one)
+  int b_st = (wave >> 1) * kBStage + (wave & 1) * (kTileT * 2) + l32 * 2 + lhi;
+  const int a_rd = wave * 4 * (kTileM * kStageC) + lhi * (kTileM * 2) + l32 * 2;
+  int b_rd = wave * 4 * (kTileT * kStageC) + lhi * (kTileT * 2) + l32 * 2;
+  const unsigned a_voff = static_cast<unsigned>(tid) * 16u;
+  const unsigned round_bytes = static_cast<unsigned>(a.HW) * 32u;  // eight channels
+
+  float4 areg[4];
+  float ereg[4][4];
+
+#define MC_LOADF(res, voff, soff) \
+  __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(res, voff, soff, 0))
+#define MC_LOAD_A(kt)                                                                           \
+  if (!(DIAG & 2)) {                                                                            \
+    const unsigned a_soff = static_cast<unsigned>((mt * a.KT + (kt)) * kAStage) * 4u;           \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                             \
+      const u32x4 w4 = __builtin_amdgcn_raw_buffer_load_b128(ures, a_voff, a_soff + i * 4096u, 0); \
+      areg[i] = __builtin_bit_cast(float4, w4);                                                 \
+    }                                                                                           \
+  }
+#define MC_LOAD_B(s)                                                                            \
+  if (!(DIAG & 1)) {                                                                            \
+    const unsigned b_soff = static_cast<unsigned>(s) * round_bytes;                             \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                             \
+      _Pragma("unroll") for (int j = 0; j < 4; ++j) ereg[i][j] = MC_LOADF(xres, boff[i][j], b_soff); \
+    }                                                                                           \
+  }
+#define MC_STORE_A(buf)                                                                         \
+  if (!(DIAG & 4)) {                                                                            \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                               \
+      *reinterpret_cast<float4*>(As + (buf)*kAStage + a_st + i * 1024) = areg[i];               \
+  }
+  // V = B^T d B, B^T = [1 0 -1 0; 0 1 1 0; 0 -1 1 0; 0 1 0 -1]
+#define MC_STORE_B()                                                                       \
+  if (!(DIAG & 4)) {                                                                            \
+    float* bw = Bs + (b_st ^ (2 * kBStage));                                                    \
+    _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                             \
+      const float r0 = ereg[0][j] - ereg[2][j], r1 = ereg[1][j] + ereg[2][j];                   \
+      const float r2 = ereg[2][j] - ereg[1][j], r3 = ereg[1][j] - ereg[3][j];                   \
+      ereg[0][j] = r0;                                                                          \
+      ereg[1][j] = r1;                                                                          \
+      ereg[2][j] = r2;                                                                          \
+      ereg[3][j] = r3;                                                                          \
+    }                                                                                           \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                             \
+      bw[(i * 4 + 0) * (kTileT * kStageC)] = ereg[i][0] - ereg[i][2];                           \
+      bw[(i * 4 + 1) * (kTileT * kStageC)] = ereg[i][1] + ereg[i][2];                           \
+      bw[(i * 4 + 2) * (kTileT * kStageC)] = ereg[i][2] - ereg[i][1];                           \
+      bw[(i * 4 + 3) * (kTileT * kStageC)] = ereg[i][1] - ereg[i][3];                           \
+    }                                                                                           \
+  }
+#define MC_COMPUTE(abuf, sub)                                                             \
+  {                                                                                             \
+    f32x2 av[4][2], bv[4];                                                                      \
+    _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                             \
+      _Pragma("unroll") for (int mb = 0; mb < 2; ++mb) av[j][mb] = *reinterpret_cast<const f32x2*>( \
+          As + (abuf)*kAStage + a_rd + j * (kTileM * kStageC) + mb * 64);                       \
+      bv[j] = *reinterpret_cast<const f32x2*>(Bs + b_rd + (sub)*kBStage + j * (kTileT * kStageC)); \
+    }                                                                                           \
+    _Pragma("unroll") for (int e = 0; e < 2; ++e) {                                             \
+      _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                           \
+        _Pragma("unroll") for (int mb = 0; mb < 2; ++mb)                                        \
+          acc[j][mb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j][mb][e], bv[j][e], acc[j][mb], 0, 0, 0); \
+      }                                                                                         \
+    }                                                                                           \
+  }
+  // Order of a stage's instructions inside a wavefront.  A wavefront issues in order, and
+  // a global load can wait for room in the memory pipeline: twenty loads at the head of
+  // a stage keep the wavefront from feeding the matrix pipe for as long.  So every
+  // product is followed by one or two loads (first stage of a round: the filters of
+  // the second stage, then the patches of the next round) or by a share of the
+  // transform and of the LDS stores (second stage), whose issue then hides under the
+  // product's 64 cycles.
+#define MC_SG(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+#define MC_ORDER_FIRST()                                                                     \
+  MC_SG(0x100, 6);                                                                           \
+  MC_SG(0x008, 1); MC_SG(0x020, 2); MC_SG(0x008, 1); MC_SG(0x020, 2);                        \
+  MC_SG(0x008, 1); MC_SG(0x020, 2); MC_SG(0x008, 1); MC_SG(0x020, 2);                        \
+  MC_SG(0x008, 1); MC_SG(0x020, 2); MC_SG(0x008, 1); MC_SG(0x020, 2);                        \
+  MC_SG(0x008, 1); MC_SG(0x020, 2); MC_SG(0x008, 1); MC_SG(0x020, 2);                        \
+  MC_SG(0x008, 1); MC_SG(0x020, 1); MC_SG(0x008, 1); MC_SG(0x020, 1);                        \
+  MC_SG(0x008, 1); MC_SG(0x020, 1); MC_SG(0x008, 1); MC_SG(0x020, 1);                        \
+  MC_SG(0x008, 1); MC_SG(0x200, 1); MC_SG(0x008, 1); MC_SG(0x200, 1);                        \
+  MC_SG(0x008, 1); MC_SG(0x200, 1); MC_SG(0x008, 1); MC_SG(0x200, 1)
+#define MC_ORDER_SECOND()                                                                    \
+  MC_SG(0x100, 6);                                                                           \
+  MC_SG(0x008, 1); MC_SG(0x020, 1); MC_SG(0x008, 1); MC_SG(0x020, 1);                        \
+  MC_SG(0x008, 1); MC_SG(0x020, 1); MC_SG(0x008, 1); MC_SG(0x020, 1);                        \
+  MC_SG(0x008, 1); MC_SG(0x002, 4); MC_SG(0x008, 1); MC_SG(0x002, 4);                        \
+  MC_SG(0x008, 1); MC_SG(0x002, 4); MC_SG(0x008, 1); MC_SG(0x002, 4);                        \
+  MC_SG(0x008, 1); MC_SG(0x002, 4); MC_SG(0x008, 1); MC_SG(0x002, 4);                        \
+  MC_SG(0x008, 1); MC_SG(0x002, 4); MC_SG(0x008, 1); MC_SG(0x002, 4);                        \
+  MC_SG(0x008, 1); MC_SG(0x200, 4); MC_SG(0x008, 1); MC_SG(0x200, 4);                        \
+  MC_SG(0x008, 1); MC_SG(0x200, 2); MC_SG(0x008, 1); MC_SG(0x200, 2)
+  // Round s: its V sits in the B buffer b_rd points into (both halves), the filters of
+  // its first stage in A buffer 0.  Every round fetches what the next one needs; the
+  // last round fetches its own operands once more (nobody reads them), so all rounds
+  // are the same code.
+#define MC_ROUND(s)                                                      \
+  {                                                                      \
+    const int s_next = min((s) + 1, rounds - 1);                         \
+    MC_LOAD_A(2 * (s) + 1);                                              \
+    MC_LOAD_B(s_next);                                                   \
+    MC_COMPUTE(0, 0);                                                    \
+    MC_STORE_A(1);                                                       \
+    MC_ORDER_FIRST();                                                    \
+    __syncthreads();                                                     \
+    __builtin_amdgcn_sched_barrier(0);                                   \
+    MC_LOAD_A(2 * s_next);                                               \
+    MC_COMPUTE(1, 1);                                                    \
+    MC_STORE_B();                                                        \
+    MC_STORE_A(0);                                                       \
+    b_st ^= 2 * kBStage;                                                 \
+    b_rd ^= 2 * kBStage;                                                 \
+    MC_ORDER_SECOND();                                                   \
+    __syncthreads();                                                     \
+    __builtin_amdgcn_sched_barrier(0);                                   \
+  }
+
+  acc16 acc[4][2];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[j][mb][r] = 0.f;
+
+  {
+    if (ragged && s_begin + 1 == rounds) MC_DROP_MISSING_CHANNELS();
+    MC_LOAD_B(s_begin);
+    MC_LOAD_A(2 * s_begin);
+    MC_STORE_A(0);
+    b_st ^= 2 * kBStage;  // (MC_STORE_B fills the buffer the products do not read)
+    MC_STORE_B();
+    b_st ^= 2 * kBStage;
+    __syncthreads();
+    for (int s = s_begin; s < s_end; ++s) {
+      if (ragged && s + 2 == rounds) MC_DROP_MISSING_CHANNELS();
+      MC_ROUND(s);
+    }
+  }
+#undef MC_LOADF
+#undef MC_LOAD_A
+#undef MC_LOAD_B
+#undef MC_DROP_MISSING_CHANNELS
+#undef MC_STORE_A
+#undef MC_STORE_B
+#undef MC_COMPUTE
+#undef MC_ORDER_FIRST
+#undef MC_ORDER_SECOND
+#undef MC_SG
+#undef MC_ROUND
+
+  // Finish.  Y = A^T m A, A^T = [1 1 1 0; 0 1 -1 -1].  This wavefront holds row i =
+  // wave of m (columns j = 0 .. 3): the sums over j stay in registers,
+  //   s[0] = m0 + m1 + m2,  s[1] = m1 - m2 - m3,
+  // and go to Es[dj][i][co][t]; accumulator register r of lane l is channel
+  // 32 mb + 8 (r / 4) + 4 (l / 32) + r % 4, block l % 32.
+  float sv[2][2][16];
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float m0 = acc[0][mb][r], m1 = acc[1][mb][r], m2 = acc[2][mb][r], m3 = acc[3][mb][r];
+      sv[0][mb][r] = m0 + m1 + m2;
+      sv[1][mb][r] = m1 - m2 - m3;
+    }
+  __syncthreads();  // every wavefront is done with the stage buffers
+  if (a.counters != nullptr) {
+    // The partial sums and the counter are accessed with device-scope atomic operations
+    // only (relaxed stores and loads that go past the per-XCD L2, which is not coherent
+    // with the other seven), so no cache write-back or invalidation is needed: a
+    // workgroup waits until its own stores have completed and then counts.
+    const int tile_id = blockIdx.x;
+    const size_t slice_elems = static_cast<size_t>(gridDim.x) * (64 * 256);
+    float* mine = a.partial + blockIdx.y * slice_elems + static_cast<size_t>(tile_id) * (64 * 256) + tid;
+#pragma unroll
+    for (int v = 0; v < 64; ++v)
+      __hip_atomic_store(mine + v * 256, sv[v >> 5][(v >> 4) & 1][v & 15], __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's partial sums have arrived
+    __syncthreads();                                   // ... and every thread's
+    int* arrived = reinterpret_cast<int*>(lds);
+    if (tid == 0)
+      arrived[0] = __hip_atomic_fetch_add(&a.counters[tile_id], 1, __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const int before = arrived[0];
+    __syncthreads();  // (lds is about to be reused)
+    if (before != static_cast<int>(gridDim.y) - 1) return;  // uniform over the workgroup
+    // the next launch on this stream starts from zero
+    if (tid == 0)
+      __hip_atomic_store(&a.counters[tile_id], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const float* part = a.partial + static_cast<size_t>(tile_id) * (64 * 256) + tid;
+#pragma unroll
+    for (int v = 0; v < 64; ++v)
+      sv[v >> 5][(v >> 4) & 1][v & 15] =
+          __hip_atomic_load(part + v * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (unsigned z = 1; z < gridDim.y; ++z) {
+      part += slice_elems;
+#pragma unroll
+      for (int v = 0; v < 64; ++v)
+        sv[v >> 5][(v >> 4) & 1][v & 15] +=
+            __hip_atomic_load(part + v * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  float* const Es = lds;
+#pragma unroll
+  for (int dj = 0; dj < 2; ++dj)
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int co = 32 * mb + 8 * (r / 4) + 4 * lhi + (r % 4);
+        Es[((dj * 4 + wave) * kTileM + co) * kTileT + l32] = sv[dj][mb][r];
+      }
+  __syncthreads();
+
+  // Thread = (block tid % 32, channels tid / 32 + 8 q): the sums over the four rows,
+  //   out[0][dj] = s0 + s1 + s2,  out[1][dj] = s1 - s2 - s3,
+  // then the layer's epilogue on the up to four outputs of the block inside the map.
+  const int tq = tid & 31, cq = tid >> 5;
+  const int t = nt * kTileT + tq;
+  if (t >= a.T) return;
+  const int n = fast_div(t, a.div_img_mul, a.div_img_shift);
+  const int rem = t - n * a.ThTw;
+  const int ty = fast_div(rem, a.div_tw_mul, a.div_tw_shift);
+  const int tx = rem - ty * a.Tw;
+  const int ho = 2 * ty, wo = 2 * tx;
+  const bool row1 = ho + 1 < a.Ho, col1 = wo + 1 < a.Wo;
+  const int c_second = a.Cout - a.c_first;
+#pragma unroll 2
+  for (int q = 0; q < 8; ++q) {
+    const int cl = cq + 8 * q;
+    const int c = mt * kTileM + cl;
+    if (c >= a.Cout) break;
     float out[2][2];
 #pragma unroll
+    for (int dj = 0; dj < 2; ++dj) {
+      const float s0 = Es[((dj * 4 + 0) * kTileM + cl) * kTileT + tq];
+      const float s1 = Es[((dj * 4 + 1) * kTileM + cl) * kTileT + tq];
+      const float s2 = Es[((dj * 4 + 2) * kTileM + cl) * kTileT + tq];
+      const float s3 = Es[((dj * 4 + 3) * kTileM + cl) * kTileT + tq];
+      out[0][dj] = s0 + s1 + s2;
+      out[1][dj] = s1 - s2 - s3;
+    }
+    const float sc = a.scale ? a.scale[c] : 1.f;
+    const float sh = a.shift ? a.shift[c] : 0.f;
+    const bool first = c < a.c_first;
+    float* __restrict__ yc = first ? a.y : a.y_second;
+    const long base = first ? (((long)n * a.c_first + c) * a.Ho + ho) * a.Wo + wo
+                            : (((long)n * c_second + (c - a.c_first)) * a.Ho + ho) * a.Wo + wo;
+#pragma unroll
     for (int i = 0; i < 2; ++i) {
-      out[i][0] = a[i][0] + a[i][1] + a[i][2];
-      out[i][1] = a[i][1] - a[i][2] - a[i][3];
+      out[i][0] = out[i][0] * sc + sh;
+      out[i][1] = out[i][1] * sc + sh;
     }
-    const float sc = e.scale ? e.scale[c] : 1.f;
-    const float sh = e.shift ? e.shift[c] : 0.f;
-    const bool first = c < e.c_first;
-    float* __restrict__ yc = first ? y : e.y_second;
-    const long base = first ? (((long)n * e.c_first + c) * s.Ho + ho) * s.Wo + wo
-                            : (((long)n * (s.Cout - e.c_first) + (c - e.c_first)) * s.Ho + ho) * s.Wo + wo;
-    if (e.scale) {
-#pragma unroll
-      for (int i = 0; i < 2; ++i) out[i][0] *= sc, out[i][1] *= sc;
-    }
-    if (e.shift) {
-#pragma unroll
-      for (int i = 0; i < 2; ++i) out[i][0] += sh, out[i][1] += sh;
-    }
-    if (PAIRS) {
-      // even width: a block's two outputs of a row are one aligned 8-byte access
+    if (a.pairs) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         if (i == 1 && !row1) break;
-        const long o = base + i * s.Wo;
+        const long o = base + i * a.Wo;
         float2 val = make_float2(out[i][0], out[i][1]);
-        if (e.residual) {
-          const float2 r = *reinterpret_cast<const float2*>(e.residual + o);
+        if (a.residual) {
+          const float2 r = *reinterpret_cast<const float2*>(a.residual + o);
           val.x += r.x;
           val.y += r.y;
         }
-        val.x = act_value(val.x, e.act, e.slope);
-        val.y = act_value(val.y, e.act, e.slope);
+        val.x = act_value(val.x, a.act, a.slope);
+        val.y = act_value(val.y, a.act, a.slope);
         *reinterpret_cast<float2*>(yc + o) = val;
       }
     } else {
@@ -235,10 +494,10 @@ __global__ __launch_bounds__(256) void winograd_output_kernel(const float* __res
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
           if (j == 1 && !col1) break;
-          const long o = base + i * s.Wo + j;
+          const long o = base + i * a.Wo + j;
           float val = out[i][j];
-          if (e.residual) val += e.residual[o];
-          yc[o] = act_value(val, e.act, e.slope);
+          if (a.residual) val += a.residual[o];
+          yc[o] = act_value(val, a.act, a.slope);
         }
       }
     }
@@ -250,23 +509,10 @@ __global__ __launch_bounds__(256) void winograd_output_kernel(const float* __res
 struct WinogradState {
   mcConvGeom geom;
   int Ho = 0, Wo = 0;
-  float* u = nullptr;          // transformed filters [16 * Cout, Cin]
+  int MT = 0, KT = 0;
+  float* u = nullptr;  // packed transformed filters, allocated when weights first arrive
   bool have_weights = false;
-  // 1x1 plans with sixteen groups on a one-image blob of Tpad pixels, by Tpad: a
-  // batch runs in at most two different run lengths
-  struct Inner {
-    int tpad = 0;
-    mcConvPlan* plan = nullptr;
-  };
-  Inner inner[2];
-  int next_inner = 0;
 };
-
-// Bytes of V and M one run of images may take; a larger batch is cut into equal
-// runs of whole images.  It bounds the workspace, nothing else: shorter runs that
-// keep V and M in the last-level cache were measured and are slower (every run
-// pays the ramp and tail of three launches).
-long g_winograd_run_bytes = 1L << 30;
 
 bool winograd_eligible(const mcConvGeom& g) {
   return !g.transposed && g.group == 1 && g.kernel_h == 3 && g.kernel_w == 3 && g.stride_h == 1 &&
@@ -279,69 +525,29 @@ WinogradState* winograd_create(const mcConvGeom& g, int Ho, int Wo) {
   w->geom = g;
   w->Ho = Ho;
   w->Wo = Wo;
+  w->MT = ceil_div(g.channels_out, kTileM);
+  w->KT = 2 * ceil_div(g.channels_in, 2 * kStageC);
   return w;
 }
 
 void winograd_destroy(WinogradState* w) {
   if (!w) return;
-  for (auto& in : w->inner)
-    if (in.plan) (void)mcConvPlanDestroy(in.plan);
   if (w->u) (void)hipFree(w->u);
   delete w;
 }
 
-namespace {
-// The contraction sees V as a one-image blob of `rows` x (Tpad / rows) pixels; both
-// extents stay below its limit of 16384, and a row is a multiple of four pixels
-// (16-byte gathers).
-inline long plane_rows(long T) { return (T + 8191) / 8192; }
-inline long padded_blocks(long T) {
-  const long unit = 4 * plane_rows(T);
-  return (T + unit - 1) / unit * unit;
-}
-
-WinogradShape shape_of(const WinogradState* w, int num) {
-  WinogradShape s;
-  s.C = w->geom.channels_in;
-  s.H = w->geom.height_in;
-  s.W = w->geom.width_in;
-  s.Cout = w->geom.channels_out;
-  s.Ho = w->Ho;
-  s.Wo = w->Wo;
-  s.pad_h = w->geom.pad_h;
-  s.pad_w = w->geom.pad_w;
-  s.Th = (w->Ho + 1) / 2;
-  s.Tw = (w->Wo + 1) / 2;
-  const long T = (long)num * s.Th * s.Tw;
-  s.T = static_cast<int>(T);
-  s.Tpad = static_cast<int>(padded_blocks(T));
-  return s;
-}
-}  // namespace
-
-// Whether a batch of `num` images can take this path at all: V and M must stay
-// below the 2^29 elements one contraction launch addresses.
-bool winograd_fits(const WinogradState* w, int num) {
-  const long blocks = (long)num * ((w->Ho + 1) / 2) * ((w->Wo + 1) / 2);
-  const long T = padded_blocks(blocks);
-  const long most = 16L * std::max(w->geom.channels_in, w->geom.channels_out) * T;
-  // (the transform kernels put channels on the grid's y axis)
-  return plane_rows(blocks) < 16384 && most < (1L << 29) &&
-         std::max(w->geom.channels_in, w->geom.channels_out) <= 65535;
+// Whether one image can take this path at all: bottom, top and the packed filters
+// are addressed with 31-bit byte offsets.
+bool winograd_fits(const WinogradState* w, int /*num*/) {
+  const mcConvGeom& g = w->geom;
+  const long in_img = (long)g.channels_in * g.height_in * g.width_in;
+  const long out_img = (long)g.channels_out * w->Ho * w->Wo;
+  const long u_floats = (long)w->MT * w->KT * kAStage;
+  return in_img < (1L << 29) && out_img < (1L << 29) && u_floats < (1L << 29);
 }
 
 // The automatic choice.  Per output block the direct path multiplies 36 Cin Cout
-// times and moves 4 (Cin + Cout) floats; this path multiplies 16 Cin Cout times
-// and moves 16 (Cin + Cout) floats twice (V and M, written and read) besides.
-// Measured on the 3x3 layers of ResNet-50 (batch 64), VGG-16 / SSD300 (batch 8)
-// and an RPN head, direct against this path: 64 channels lose everywhere (151 us
-// against 209 on 56x56 maps); 128 -> 128 gains while V and M fit the 256 MB
-// last-level cache (152 -> 108 us on 28x28 maps) and loses beyond it (428 -> 478
-// on 150x150); 128 -> 256 gains 1.17x; 256 and 512 channels gain 1.4x to 1.8x on
-// every map.  One narrow side is fine when the other is wide (SSD's merged heads,
-// 512 -> 100 on 38x38 b8: 147 -> 92 us; 1024 -> 150 on 19x19: 113 -> 81; 96 -> 512:
-// 91 -> 76) down to about 96 channels (256 -> 64 and 64 -> 512 break even, 1024 ->
-// 64 loses); 200 blocks still gain or break even (512 -> 150 on 10x10 b8: 42 -> 30 us).
+// times, this path 16 Cin Cout times; both read the bottom and write the top once.
 bool winograd_pays(const WinogradState* w, int num) {
   const mcConvGeom& g = w->geom;
   const long blocks = (long)num * ((w->Ho + 1) / 2) * ((w->Wo + 1) / 2);
@@ -351,67 +557,28 @@ bool winograd_pays(const WinogradState* w, int num) {
   // odd and tiny maps compute blocks that hang over the edge: a 3x3 map is four
   // blocks for nine outputs (16 x 4 products against 36 x 9 / 4 useful ones)
   if (10L * w->Ho * w->Wo < 26L * ((w->Ho + 1) / 2) * ((w->Wo + 1) / 2)) return false;
-  if (most >= 256) return true;
-  return least >= 128 && 64L * (g.channels_in + g.channels_out) * blocks <= (256L << 20);
+  return most >= 128;
 }
 
 int winograd_set_weights(WinogradState* w, const float* weights, hipStream_t st) {
-  const long filters = (long)w->geom.channels_out * w->geom.channels_in;
-  if (!w->u) MC_HIP(hipMalloc(&w->u, sizeof(float) * 16 * filters));
-  winograd_filter_kernel<<<ew_blocks(filters, 256), 256, 0, st>>>(weights, w->u, filters);
+  const long floats = (long)w->MT * w->KT * kAStage;
+  if (!w->u) MC_HIP(hipMalloc(&w->u, sizeof(float) * floats));
+  const long threads = (long)w->MT * kTileM * w->KT * kStageC;
+  winograd_pack_filter_kernel<<<static_cast<unsigned>(ceil_div(threads, 256)), 256, 0, st>>>(
+      weights, w->u, w->geom.channels_out, w->geom.channels_in, w->MT, w->KT);
   MC_LAUNCH_CHECK();
   w->have_weights = true;
-  for (auto& in : w->inner)
-    if (in.plan && mcConvPlanSetWeights(in.plan, w->u, st)) return -1;
   return 0;
 }
-
-namespace {
-int inner_plan(WinogradState* w, const WinogradShape& s, hipStream_t st, mcConvPlan** out) {
-  for (auto& in : w->inner)
-    if (in.plan && in.tpad == s.Tpad) {
-      *out = in.plan;
-      return 0;
-    }
-  WinogradState::Inner& slot = w->inner[w->next_inner];
-  w->next_inner ^= 1;
-  if (slot.plan) {
-    // kernels of an earlier call may still read the old plan's filter copy
-    MC_HIP(hipStreamSynchronize(st));
-    (void)mcConvPlanDestroy(slot.plan);
-    slot.plan = nullptr;
-  }
-  mcConvGeom g;
-  g.channels_in = 16 * s.C;
-  g.height_in = static_cast<int>(plane_rows(s.T));
-  g.width_in = s.Tpad / g.height_in;
-  g.channels_out = 16 * s.Cout;
-  g.kernel_h = g.kernel_w = 1;
-  g.stride_h = g.stride_w = 1;
-  g.pad_h = g.pad_w = 0;
-  g.dilation_h = g.dilation_w = 1;
-  g.group = 16;
-  g.transposed = 0;
-  if (mcConvPlanCreate(&g, &slot.plan)) return -1;
-  slot.tpad = s.Tpad;
-  if (mcConvPlanSetWeights(slot.plan, w->u, st)) return -1;
-  *out = slot.plan;
-  return 0;
-}
-}  // namespace
 
 double winograd_issued_flops(const WinogradState* w, int num) {
   const double blocks = (double)num * ((w->Ho + 1) / 2) * ((w->Wo + 1) / 2);
   return 2. * 16. * w->geom.channels_in * w->geom.channels_out * blocks;
 }
 
-int winograd_set_run_bytes(long bytes) {
-  g_winograd_run_bytes = std::max(bytes, 1L << 20);
-  return 0;
-}
-
 int winograd_forward(WinogradState* w, int num, const float* bottom, float* top,
-                     const mcEpilogue* ep, void* stream, float* top_second, int c_first) {
+                     const mcEpilogue* ep, void* stream, float* top_second, int c_first,
+                     int images_per_run, int forced_slices) {
   MC_REQUIRE(w->have_weights, "mcConvForward: the plan has no weights yet");
   MC_REQUIRE(!top_second || (c_first > 0 && c_first < w->geom.channels_out && !(ep && ep->residual)),
              "mcConvForwardTwoTops: needs group 1, a split inside the output channels and no "
@@ -419,64 +586,84 @@ int winograd_forward(WinogradState* w, int num, const float* bottom, float* top,
   if (!top_second) c_first = w->geom.channels_out;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const mcConvGeom& g = w->geom;
-  // equal runs of whole images whose V and M fit the budget
-  const long per_image =
-      64L * (g.channels_in + g.channels_out) * ((w->Ho + 1) / 2) * ((w->Wo + 1) / 2);
-  const long fit = std::max(1L, g_winograd_run_bytes / per_image);
-  const int runs = ceil_div(num, fit);
-  const int run_len = ceil_div(num, runs);
   const long in_img = (long)g.channels_in * g.height_in * g.width_in;
   const long hw_out = (long)w->Ho * w->Wo;
+  const long top_img = (long)g.channels_out * hw_out;
   const long out_img = c_first * hw_out, second_img = (g.channels_out - c_first) * hw_out;
-  WinogradEpilogue e;
-  e.c_first = c_first;
-  e.scale = ep ? ep->scale : nullptr;
-  e.shift = ep ? ep->shift : nullptr;
-  e.act = ep ? ep->activation : MC_ACT_NONE;
-  e.slope = ep ? ep->negative_slope : 0.f;
+  const int Th = (w->Ho + 1) / 2, Tw = (w->Wo + 1) / 2;
+  // equal runs of whole images that the 31-bit byte offsets reach
+  const long lim = (1L << 29) - 1;
+  long per = std::min(lim / in_img, lim / top_img);
+  per = std::min(per, lim / ((long)Th * Tw));
+  if (images_per_run > 0) per = std::min<long>(per, images_per_run);
+  MC_REQUIRE(per >= 1, "mcConvForward: a single image exceeds 2^29 elements");
+  const int runs = ceil_div(num, per);
+  const int run_len = ceil_div(num, runs);
+
+  WinogradArgs a;
+  a.u = w->u;
+  a.u_bytes = static_cast<unsigned>(sizeof(float) * (long)w->MT * w->KT * kAStage);
+  a.scale = ep ? ep->scale : nullptr;
+  a.shift = ep ? ep->shift : nullptr;
+  a.C = g.channels_in;
+  a.H = g.height_in;
+  a.W = g.width_in;
+  a.HW = g.height_in * g.width_in;
+  a.x_nstride = static_cast<int>(in_img);
+  a.Cout = g.channels_out;
+  a.Ho = w->Ho;
+  a.Wo = w->Wo;
+  a.HoWo = static_cast<int>(hw_out);
+  a.pad_h = g.pad_h;
+  a.pad_w = g.pad_w;
+  a.Tw = Tw;
+  a.ThTw = Th * Tw;
+  a.MT = w->MT;
+  a.KT = w->KT;
+  a.c_first = c_first;
+  a.act = ep ? ep->activation : MC_ACT_NONE;
+  a.slope = ep ? ep->negative_slope : 0.f;
+  // (top and residual rows are 8-byte aligned when the width is even and the blob is)
+  a.pairs = w->Wo % 2 == 0 && reinterpret_cast<uintptr_t>(top) % 8 == 0 &&
+            reinterpret_cast<uintptr_t>(top_second) % 8 == 0 &&
+            (!ep || !ep->residual || reinterpret_cast<uintptr_t>(ep->residual) % 8 == 0);
   for (int n0 = 0; n0 < num; n0 += run_len) {
     const int n = std::min(run_len, num - n0);
-    const WinogradShape s = shape_of(w, n);
-    mcConvPlan* inner = nullptr;
-    if (inner_plan(w, s, st, &inner)) return -1;
-    float* ws = nullptr;
-    const size_t v_floats = 16ul * s.C * s.Tpad, m_floats = 16ul * s.Cout * s.Tpad;
-    if (stream_workspace(st, sizeof(float) * (v_floats + m_floats), &ws, 1)) return -1;
-    float* v = ws;
-    float* m = ws + v_floats;
-    const unsigned tblocks = static_cast<unsigned>(ceil_div(s.Tpad, 256));
-    const float* run_bottom = bottom + n0 * in_img;
-    float* run_top = top + n0 * out_img;
-    switch (channels_per_thread(tblocks, s.C, 1)) {
-      case 4:
-        winograd_input_kernel<4><<<dim3(tblocks, ceil_div(s.C, 4)), 256, 0, st>>>(run_bottom, v, s);
-        break;
-      case 2:
-        winograd_input_kernel<2><<<dim3(tblocks, ceil_div(s.C, 2)), 256, 0, st>>>(run_bottom, v, s);
-        break;
-      default:
-        winograd_input_kernel<1><<<dim3(tblocks, s.C), 256, 0, st>>>(run_bottom, v, s);
+    a.x = bottom + n0 * in_img;
+    a.x_bytes = static_cast<unsigned>(n * in_img * 4);
+    a.y = top + n0 * out_img;
+    a.y_second = top_second ? top_second + n0 * second_img : nullptr;
+    a.residual = (ep && ep->residual) ? ep->residual + n0 * out_img : nullptr;
+    a.T = n * a.ThTw;
+    a.NT = ceil_div(a.T, kTileT);
+    make_fast_div(a.ThTw, (unsigned long long)a.NT * kTileT + 1, &a.div_img_mul, &a.div_img_shift);
+    make_fast_div(a.Tw, (unsigned long long)a.ThTw + 1, &a.div_tw_mul, &a.div_tw_shift);
+    make_fast_div(a.MT, (unsigned long long)a.MT * a.NT + 1, &a.div_mt_mul, &a.div_mt_shift);
+    const long tiles = (long)a.MT * a.NT;
+    MC_REQUIRE(tiles < (1L << 31), "mcConvForward: grid too large");
+    // A launch that leaves workgroup slots empty (two per CU) cuts the channel rounds
+    // into slices, each at least four rounds long.
+    const int rounds = w->KT / 2;
+    int slices = forced_slices > 0 ? forced_slices : static_cast<int>(2L * kNumCu / tiles);
+    slices = std::max(1, std::min(std::min(slices, 16), forced_slices > 0 ? rounds : rounds / 4));
+    a.rounds_per_slice = ceil_div(rounds, slices);
+    slices = ceil_div(rounds, a.rounds_per_slice);  // no empty slice
+    a.partial = nullptr;
+    a.counters = nullptr;
+    if (slices > 1) {
+      if (stream_workspace(st, sizeof(float) * tiles * slices * 64 * 256, &a.partial)) return -1;
+      if (stream_counters(st, static_cast<size_t>(tiles), &a.counters)) return -1;
     }
-    MC_LAUNCH_CHECK();
-    if (mcConvForward(inner, 1, v, m, nullptr, stream)) return -1;
-    e.residual = (ep && ep->residual) ? ep->residual + n0 * out_img : nullptr;
-    const unsigned oblocks = static_cast<unsigned>(ceil_div(s.T, 256));
-    // (top and residual rows are 8-byte aligned when the width is even and the blob is)
-    e.y_second = top_second ? top_second + n0 * second_img : nullptr;
-    const bool pairs = s.Wo % 2 == 0 && reinterpret_cast<uintptr_t>(top) % 8 == 0 &&
-                       reinterpret_cast<uintptr_t>(top_second) % 8 == 0 &&
-                       (!ep || !ep->residual || reinterpret_cast<uintptr_t>(ep->residual) % 8 == 0);
-    const int cpt = channels_per_thread(oblocks, s.Cout, 2);  // (one channel per thread measured slower here)
-    const dim3 ogrid(oblocks, ceil_div(s.Cout, cpt));
-#define MC_WINOGRAD_OUT(P, C) winograd_output_kernel<P, C><<<ogrid, 256, 0, st>>>(m, run_top, s, e)
-    if (pairs) {
-      if (cpt == 4) MC_WINOGRAD_OUT(true, 4);
-      else MC_WINOGRAD_OUT(true, 2);
-    } else {
-      if (cpt == 4) MC_WINOGRAD_OUT(false, 4);
-      else MC_WINOGRAD_OUT(false, 2);
+    static const int diag = getenv("MC_WINO_DIAG") ? atoi(getenv("MC_WINO_DIAG")) : 0;
+    const dim3 grid(static_cast<unsigned>(tiles), slices);
+    switch (diag) {
+      case 1: winograd_fused_kernel<1><<<grid, 256, 0, st>>>(a); break;
+      case 2: winograd_fused_kernel<2><<<grid, 256, 0, st>>>(a); break;
+      case 3: winograd_fused_kernel<3><<<grid, 256, 0, st>>>(a); break;
+      case 4: winograd_fused_kernel<4><<<grid, 256, 0, st>>>(a); break;
+      case 7: winograd_fused_kernel<7><<<grid, 256, 0, st>>>(a); break;
+      default: winograd_fused_kernel<0><<<grid, 256, 0, st>>>(a);
     }
-#undef MC_WINOGRAD_OUT
     MC_LAUNCH_CHECK();
   }
   return 0;

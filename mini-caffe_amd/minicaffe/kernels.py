@@ -57,7 +57,6 @@ LIB.mcConvTimingCollectDetail.argtypes = [ctypes.POINTER(ctypes.c_double), ctype
                                           ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
                                           ctypes.POINTER(c_long)]
 
-LIB.mcConvTimingKernelTotals.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
 LIB.mcDetectionOutputWorkspaceSize.argtypes = [c_int, c_int, c_int, c_int, c_int,
                                                ctypes.POINTER(ctypes.c_size_t)]
 LIB.mcDetectionOutputMaxRows.argtypes = [c_int] * 5
@@ -108,7 +107,6 @@ LIB.mcConvPlanForceConfig.argtypes = [c_void_p, c_int]
 LIB.mcConvPlanForceSplit.argtypes = [c_void_p, c_int]
 LIB.mcConvPlanForceWinograd.argtypes = [c_void_p, c_int]
 LIB.mcConvWinogradDefault.argtypes = [c_int]
-LIB.mcConvWinogradRunBytes.argtypes = [ctypes.c_long]
 LIB.mcConvPlanForceChunk.argtypes = [c_void_p, c_int]
 
 

@@ -440,16 +440,14 @@ def test_conv_winograd_two_tops(K, c_first):
         ep = dict(scale=sd.data_ptr(), shift=bd.data_ptr(), activation=K_ACT_RELU)
         whole = torch.full((n, cout, h, w), float("nan"), device="cuda")
         plan.forward(n, xd.data_ptr(), whole.data_ptr(), **ep)
-        try:
-            for run_bytes in (1 << 30, 1 << 20):
-                K.LIB.mcConvWinogradRunBytes(run_bytes)
-                first = torch.full((n, c_first, h, w), float("nan"), device="cuda")
-                second = torch.full((n, cout - c_first, h, w), float("nan"), device="cuda")
-                plan.forward_two_tops(n, xd.data_ptr(), first.data_ptr(), c_first, second.data_ptr(), **ep)
-                torch.cuda.synchronize()
-                assert torch.equal(first, whole[:, :c_first]) and torch.equal(second, whole[:, c_first:])
-        finally:
-            K.LIB.mcConvWinogradRunBytes(1 << 30)
+        for per_run in (0, 2):
+            plan.force_chunk(per_run)
+            first = torch.full((n, c_first, h, w), float("nan"), device="cuda")
+            second = torch.full((n, cout - c_first, h, w), float("nan"), device="cuda")
+            plan.forward_two_tops(n, xd.data_ptr(), first.data_ptr(), c_first, second.data_ptr(), **ep)
+            torch.cuda.synchronize()
+            assert torch.equal(first, whole[:, :c_first]) and torch.equal(second, whole[:, c_first:])
+        plan.force_chunk(0)
         want = np.maximum(oracle.scale(oracle.conv_forward(oracle.conv_geom(cin, h, w, cout, 3, 1, 1), x, wt, None),
                                        sc, b), 0)
         assert netrun.rel_err(whole.cpu().numpy(), want) < 1e-4
@@ -458,26 +456,21 @@ def test_conv_winograd_two_tops(K, c_first):
 
 
 def test_conv_winograd_runs_batches_and_new_weights(K):
-    """One plan on the Winograd path over changing batch sizes (its inner plans are kept
-    by size, two at a time), with the batch cut into runs of images, and after the weights
-    change."""
+    """One plan on the Winograd path over changing batch sizes, with the batch cut into
+    runs of images, and after the weights change."""
     cin, h, w, cout = 12, 10, 11, 9
     rng = np.random.default_rng(18)
     plan = K.ConvPlan(K.conv_geom(cin, h, w, cout, 3, 1, 1))
     plan.force_winograd(1)
-    per_image = 64 * (cin + cout) * 5 * 6
-    try:
-        for round_, n in enumerate((5, 2, 7, 5, 1)):
-            K.LIB.mcConvWinogradRunBytes(max(1 << 20, 2 * per_image) if round_ % 2 else 1 << 30)
-            x = rng.standard_normal((n, cin, h, w)).astype(np.float32)
-            wt = (rng.standard_normal((cout, cin, 3, 3)) * 0.2).astype(np.float32)
-            b = rng.standard_normal(cout).astype(np.float32)
-            res = rng.standard_normal((n, cout, h, w)).astype(np.float32)
-            want = oracle.conv_forward(oracle.conv_geom(cin, h, w, cout, 3, 1, 1), x, wt, b) + res
-            got = _run_plan(K, plan, n, x, wt, want.shape, shift=b, residual=res)
-            assert np.abs(got - want).max() < 1e-5, (round_, n)
-    finally:
-        K.LIB.mcConvWinogradRunBytes(1 << 30)
+    for round_, n in enumerate((5, 2, 7, 5, 1)):
+        plan.force_chunk(2 if round_ % 2 else 0)
+        x = rng.standard_normal((n, cin, h, w)).astype(np.float32)
+        wt = (rng.standard_normal((cout, cin, 3, 3)) * 0.2).astype(np.float32)
+        b = rng.standard_normal(cout).astype(np.float32)
+        res = rng.standard_normal((n, cout, h, w)).astype(np.float32)
+        want = oracle.conv_forward(oracle.conv_geom(cin, h, w, cout, 3, 1, 1), x, wt, b) + res
+        got = _run_plan(K, plan, n, x, wt, want.shape, shift=b, residual=res)
+        assert np.abs(got - want).max() < 1e-5, (round_, n)
 
 
 def test_conv_winograd_refused_where_it_does_not_apply(K):
