@@ -68,9 +68,6 @@ def main():
                          "128 or more channels otherwise run as F(2x2,3x3) Winograd)")
     ap.add_argument("--no-direct-comparison", action="store_true",
                     help="skip the second, shorter measurement with every convolution on the direct path")
-    ap.add_argument("--no-kernel-pass", action="store_true",
-                    help="skip the extra pass that times the contraction launch inside every Winograd layer "
-                         "by itself (igemm_launch_* in the roofline block)")
     ap.add_argument("--no-detection-tails", action="store_true",
                     help="skip the NMS / Proposal / DetectionOutput timings (profiling runs of the "
                          "ResNet-50 forward alone)")
@@ -150,21 +147,10 @@ def main():
     LIB.mcConvTimingCollectDetail(ctypes.byref(tot_ms), ctypes.byref(launches), ctypes.byref(fl),
                                   ctypes.byref(issued), ctypes.byref(wino))
     LIB.mcConvTimingEnable(0)
-    # a shorter pass with the contraction launch inside every Winograd layer timed by itself
-    # as well: what the kernel alone reaches (these extra events would lengthen the layers above)
-    k_steps = 0 if args.no_kernel_pass else max(5, args.steps // 4)
-    k_ms, k_fl = ctypes.c_double(), ctypes.c_double()
-    if k_steps:
-        LIB.mcConvTimingEnable(2)
-        for _ in range(k_steps):
-            net.forward()
-        LIB.mcConvTimingCollectDetail(None, None, None, None, None)
-        LIB.mcConvTimingKernelTotals(ctypes.byref(k_ms), ctypes.byref(k_fl))
-        LIB.mcConvTimingEnable(0)
     # achieved: the layers' algorithmic FLOPs (2 x MACs of the direct sum) over the device time
-    # of their launches.  A 3x3 layer on the Winograd path counts with its direct-sum FLOPs and
-    # with all three of its launches (transforms included); mfma_issued_* is what the matrix
-    # pipe was actually handed in the same time.
+    # of their launches (one launch per contraction).  A 3x3 layer on the Winograd path counts
+    # with its direct-sum FLOPs; mfma_issued_* is what the matrix pipe was actually handed in
+    # the same time (2.25 times fewer products for those layers).
     secs = tot_ms.value * 1e-3
     achieved = fl.value / secs / 1e12 if secs > 0 else 0.0
     issued_tflops = issued.value / secs / 1e12 if secs > 0 else 0.0
@@ -174,22 +160,16 @@ def main():
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP32_MFMA_PEAK_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
                 "traffic": traffic, "traffic_source": traffic_note,
-                "kernel": "igemm_f32 (Convolution + InnerProduct, fused BN/Scale/ReLU epilogue; %d of the %d "
-                          "contractions per step run it as the sixteen products of F(2x2,3x3) Winograd, "
-                          "timed with their two transform kernels)" % (wino.value // steps, launches.value // steps),
+                "kernel": "igemm_f32 / winograd_fused (Convolution + InnerProduct, fused BN/Scale/ReLU epilogue; "
+                          "%d of the %d contractions per step are 3x3 stride-1 layers run as F(2x2,3x3) Winograd "
+                          "in one launch each)" % (wino.value // steps, launches.value // steps),
                 "launches_per_step": launches.value // steps,
                 "winograd_per_step": wino.value // steps,
                 "kernel_ms_per_step": round(tot_ms.value / steps, 3),
                 "gflop_per_step": round(fl.value / steps / 1e9, 1),
                 "mfma_issued_gflop_per_step": round(issued.value / steps / 1e9, 1),
                 "mfma_issued_tflops": round(issued_tflops, 2),
-                "mfma_issued_frac": round(issued_tflops / FP32_MFMA_PEAK_TFLOPS, 4),
-                # the contraction kernel's launches by themselves (Winograd transforms left out):
-                # the FLOPs it is handed over its own device time
-                "igemm_launch_ms_per_step": round(k_ms.value / k_steps, 3) if k_steps else None,
-                "igemm_launch_tflops": round(k_fl.value / (k_ms.value * 1e-3) / 1e12, 2) if k_ms.value > 0 else None,
-                "igemm_launch_frac": round(k_fl.value / (k_ms.value * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS, 4)
-                if k_ms.value > 0 else None}
+                "mfma_issued_frac": round(issued_tflops / FP32_MFMA_PEAK_TFLOPS, 4)}
     # The same net with every convolution on the direct path (no Winograd), shorter: what
     # the implicit-GEMM kernel alone gives, for comparison with the figures above.
     direct = None

@@ -224,6 +224,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
   float4 areg[4];
   float ereg[4][4];
+  const float sgv = a.slope + lane;  // (diagnosis builds only)
 
 #define MC_LOADF(res, voff, soff) \
   __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(res, voff, soff, 0))
@@ -269,6 +270,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #define MC_COMPUTE(abuf, sub)                                                             \
   {                                                                                             \
     f32x2 av[4][2], bv[4];                                                                      \
+    if (DIAG & 8) { _Pragma("unroll") for (int j = 0; j < 4; ++j) { av[j][0] = av[j][1] = bv[j] = f32x2{sgv, sgv}; } } else \
     _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                             \
       _Pragma("unroll") for (int mb = 0; mb < 2; ++mb) av[j][mb] = *reinterpret_cast<const f32x2*>( \
           As + (abuf)*kAStage + a_rd + j * (kTileM * kStageC) + mb * 64);                       \
@@ -321,7 +323,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     MC_COMPUTE(0, 0);                                                    \
     MC_STORE_A(1);                                                       \
     MC_ORDER_FIRST();                                                    \
-    __syncthreads();                                                     \
+    if (!(DIAG & 16)) __syncthreads();                                   \
     __builtin_amdgcn_sched_barrier(0);                                   \
     MC_LOAD_A(2 * s_next);                                               \
     MC_COMPUTE(1, 1);                                                    \
@@ -330,7 +332,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     b_st ^= 2 * kBStage;                                                 \
     b_rd ^= 2 * kBStage;                                                 \
     MC_ORDER_SECOND();                                                   \
-    __syncthreads();                                                     \
+    if (!(DIAG & 16)) __syncthreads();                                   \
     __builtin_amdgcn_sched_barrier(0);                                   \
   }
 
@@ -548,16 +550,27 @@ bool winograd_fits(const WinogradState* w, int /*num*/) {
 
 // The automatic choice.  Per output block the direct path multiplies 36 Cin Cout
 // times, this path 16 Cin Cout times; both read the bottom and write the top once.
+// Measured, this path against the direct one: launches of some size win whenever both
+// channel counts reach 64 (64 -> 64 on 56x56, batch 64: 97 us against 128; 128 -> 128
+// on 28x28: 95 / 141; 256 -> 256 on 14x14: 91 / 148; 512 -> 512 on 7x7, which pads to
+// 8x8: 101 / 156; VGG's 64 -> 64 on 300x300, batch 8: 295 / 423, 512 -> 512 on 38x38:
+// 245 / 430; the RPN head 1024 -> 512 on 38x63: 110 / 197; SSD's merged heads 512 -> 100
+// on 38x38: 86 / 124, 1024 -> 150 on 19x19: 66 / 97, 512 -> 150 on 10x10: 35 / 39).
+// What loses: 32 input channels (the loop is four rounds long: 56 / 47 us), an
+// output tile that is half padding (64 -> 32: 86 / 82), and launches of a few tiles,
+// whose time is this kernel's longer prologue and finish (256 -> 150 on 5x5 maps, 9
+// tiles: 25 / 19 us; one image of 256 channels on 14x14: 22 / 19; config 1's single
+// 64 -> 64 layer on one 56x56 image, 25 tiles of 8 rounds: 17 / 12).
 bool winograd_pays(const WinogradState* w, int num) {
   const mcConvGeom& g = w->geom;
   const long blocks = (long)num * ((w->Ho + 1) / 2) * ((w->Wo + 1) / 2);
-  const int least = std::min(g.channels_in, g.channels_out);
-  const int most = std::max(g.channels_in, g.channels_out);
-  if (blocks < 192 || least < 96) return false;
+  if (g.channels_in < 64) return false;
+  if (4 * g.channels_out < 3 * w->MT * kTileM) return false;
   // odd and tiny maps compute blocks that hang over the edge: a 3x3 map is four
   // blocks for nine outputs (16 x 4 products against 36 x 9 / 4 useful ones)
   if (10L * w->Ho * w->Wo < 26L * ((w->Ho + 1) / 2) * ((w->Wo + 1) / 2)) return false;
-  return most >= 128;
+  const long tiles = (long)w->MT * ceil_div(blocks, kTileT);
+  return tiles * (w->KT / 2) >= 1200;
 }
 
 int winograd_set_weights(WinogradState* w, const float* weights, hipStream_t st) {
@@ -662,6 +675,9 @@ int winograd_forward(WinogradState* w, int num, const float* bottom, float* top,
       case 3: winograd_fused_kernel<3><<<grid, 256, 0, st>>>(a); break;
       case 4: winograd_fused_kernel<4><<<grid, 256, 0, st>>>(a); break;
       case 7: winograd_fused_kernel<7><<<grid, 256, 0, st>>>(a); break;
+      case 15: winograd_fused_kernel<15><<<grid, 256, 0, st>>>(a); break;
+      case 20: winograd_fused_kernel<20><<<grid, 256, 0, st>>>(a); break;
+      case 31: winograd_fused_kernel<31><<<grid, 256, 0, st>>>(a); break;
       default: winograd_fused_kernel<0><<<grid, 256, 0, st>>>(a);
     }
     MC_LAUNCH_CHECK();
