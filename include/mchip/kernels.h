@@ -279,25 +279,49 @@ int mcProposalWorkspaceSize(int num_proposals, int pre_nms_topn, int post_nms_to
  *   rois     [post_nms_topn, 5] rows (0, x1, y1, x2, y2); roi_scores optional
  *   num_rois number of valid rows (device int; the caller copies it back to
  *            shape the top blob, as Forward_cpu's final Reshape does, :313-320)
- *   tie_flag optional device int: 0 when the pre_nms_topn+1 best scores are all
- *            distinct, else 1 or 3.  Tie-free inputs are ordered by one radix sort; with
- *            ties the order is whatever the reference's quicksort SortBBox (:88-111)
- *            leaves, so that quicksort is then replayed on the device to give the
- *            same row order: 3 = by the kernel for inputs with few equal scores (it
- *            follows only the partitions that hold equal scores), 1 = by the general
- *            kernel (every partition, level by level). */
+ *   tie_flag optional device int: 0 when no order of equal scores had to be looked up,
+ *            else 1 or 3 (see below).
+ * Two steps, both queued by this call.  (1) The head of the table: the best 512
+ * proposals are selected, ordered by (score descending, index ascending) and scanned;
+ * the greedy pass usually reaches post_nms_topn kept boxes inside them.  Equal scores
+ * among them matter only when two proposals of one score are both still alive when
+ * the scan reaches them (the reference's quicksort SortBBox, :88-111, leaves equal
+ * scores in an order of its own); a kernel checks that for every such group.  (2)
+ * The full-size path, which skips itself on the device when step 1 settled the
+ * result: all proposals are ordered by one radix sort; if equal scores reach into
+ * the first pre_nms_topn + 1 places, SortBBox is replayed on the device to give the
+ * same row order (tie_flag 3 = by the kernel for inputs with few equal scores, which
+ * follows only the partitions that hold equal scores, 1 = by the general kernel,
+ * every partition, level by level); then the overlap bit matrix and the scan. */
 int mcProposal(const float* scores, const float* bbox, const float* im_info, const float* anchors,
                int A, int H, int W, int feat_stride, float min_size, int pre_nms_topn,
                int post_nms_topn, float nms_thresh, void* workspace, size_t workspace_bytes,
                float* rois, float* roi_scores, int* num_rois, int* tie_flag, void* stream);
 
+/* The two steps of mcProposal as calls of their own, for a caller that reads num_rois
+ * back anyway (the top's shape depends on it) and can read two more ints with it:
+ * state[0] = tie_flag as above, state[1] = 1 when rois / num_rois are final.
+ * mcProposalHead queues step 1 only (state[1] = 0: call mcProposalRest with the same
+ * arguments, which starts over with the full-size path and always ends with
+ * state[1] = 1).  Saves the launches of step 2 that would return at once.  No
+ * counterpart in the reference. */
+int mcProposalHead(const float* scores, const float* bbox, const float* im_info, const float* anchors,
+                   int A, int H, int W, int feat_stride, float min_size, int pre_nms_topn,
+                   int post_nms_topn, float nms_thresh, void* workspace, size_t workspace_bytes,
+                   float* rois, float* roi_scores, int* num_rois, int* state, void* stream);
+int mcProposalRest(const float* scores, const float* bbox, const float* im_info, const float* anchors,
+                   int A, int H, int W, int feat_stride, float min_size, int pre_nms_topn,
+                   int post_nms_topn, float nms_thresh, void* workspace, size_t workspace_bytes,
+                   float* rois, float* roi_scores, int* num_rois, int* state, void* stream);
+
 /* Measurement hook (no counterpart in the reference): while enabled on the calling
- * thread every mcProposal / mcProposalStatic call records HIP events between its
- * stages on the launch stream.  mcProposalTimingCollect waits for them, adds up over
- * the calls since the last collect stage_ms[0] decode + radix sort, [1] replay of the
- * reference's order of equal scores + gather of the best pre_nms_topn boxes,
- * [2] NMS proper (overlap bit matrix + greedy scan), [3] roi gather and flag copy,
- * returns the number of calls and clears the list. */
+ * thread every mcProposal* call records HIP events between its stages on the launch
+ * stream.  mcProposalTimingCollect waits for them, adds up over the calls since the
+ * last collect stage_ms[0] decode + ordering of the head, [1] overlap matrix, scan and
+ * check of the head + roi gather, [2] full-size path: radix sort, replay of the
+ * reference's order of equal scores, gather of the best pre_nms_topn boxes, [3]
+ * full-size path: NMS proper (overlap bit matrix + greedy scan) + roi gather; returns
+ * the number of calls and clears the list. */
 int mcProposalTimingEnable(int on);
 /* Test knob (process-wide): 1 = replay the order of equal scores with the general
  * level-by-level kernel on every input, also where the kernel for inputs with few

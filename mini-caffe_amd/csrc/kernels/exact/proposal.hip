@@ -50,9 +50,10 @@ __global__ __launch_bounds__(256) void proposal_decode_kernel(
     const float* __restrict__ fg, const float* __restrict__ bbox, const float* __restrict__ anchors,
     const float* __restrict__ im_info, int A, int H, int W, int feat_stride, float min_size_param,
     float4* __restrict__ boxes, uint32_t* __restrict__ keys, uint32_t* __restrict__ keys_orig,
-    int* __restrict__ vals, float* __restrict__ scores) {
+    int* __restrict__ vals, float* __restrict__ scores, int* __restrict__ flags) {
   const int n = A * H * W;
   const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < 8) flags[i] = 0;  // the call's flag words (nothing reads them before this kernel ends)
   if (i >= n) return;
   const int k = i % A;
   const int pix = i / A;
@@ -78,7 +79,9 @@ __global__ __launch_bounds__(256) void proposal_decode_kernel(
 // Orders all proposals by (score desc, index asc) and flags score ties that
 // reach into the first `pre` places.
 __global__ __launch_bounds__(kSortThreads) void proposal_sort_kernel(
-    uint32_t* k0, int* v0, uint32_t* k1, int* v1, int n, int pre, int* __restrict__ tie_flag) {
+    uint32_t* k0, int* v0, uint32_t* k1, int* v1, int n, int pre, int* __restrict__ tie_flag,
+    const int* __restrict__ skip) {
+  if (*skip != 0) return;  // uniform: the head of the table settled the result
   __shared__ BlockSortLds lds;
   block_sort_desc(k0, v0, k1, v1, n, &lds);
   int ties = 0;
@@ -93,7 +96,9 @@ __global__ __launch_bounds__(kSortThreads) void proposal_sort_kernel(
 constexpr int kSortLdsPer = 44;
 constexpr int kSortLdsMax = kSortLdsPer * kSortThreads;  // 22528
 __global__ __launch_bounds__(kSortThreads) void proposal_sort_lds_kernel(
-    uint32_t* k0, int* v0, int n, int pre, int* __restrict__ tie_flag) {
+    uint32_t* k0, int* v0, int n, int pre, int* __restrict__ tie_flag,
+    const int* __restrict__ skip) {
+  if (*skip != 0) return;  // uniform: the head of the table settled the result
   __shared__ BlockSortLds16 lds;
   __shared__ uint32_t s_key[kSortLdsMax];
   __shared__ unsigned short s_val[kSortLdsMax];
@@ -118,12 +123,297 @@ __global__ __launch_bounds__(kSortThreads) void proposal_sort_lds_kernel(
 __global__ __launch_bounds__(256) void proposal_order_gather_kernel(
     const int* __restrict__ order, int pre, const float4* __restrict__ boxes,
     const float* __restrict__ scores, float4* __restrict__ sorted_boxes,
-    float* __restrict__ sorted_scores) {
+    float* __restrict__ sorted_scores, const int* __restrict__ skip) {
+  if (skip != nullptr && *skip != 0) return;
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i >= pre) return;
   const int src = order[i];
   sorted_boxes[i] = boxes[src];
   sorted_scores[i] = scores[src];
+}
+
+// ---- the head of the table first ---------------------------------------------------
+//
+// The greedy pass stops at post_nms_topn kept boxes, usually a few hundred candidates
+// into the table (config 4: the 300th kept box is candidate 461 of 6000), so ordering
+// all proposals, and replaying the reference's order of equal scores over all of
+// them, is mostly work whose result nobody reads.  The first step therefore orders
+// only the best `want` proposals (one super-block of the scan): the want-th best score
+// is found by bisection on the key bits, the proposals at or above it are compacted in
+// index order and sorted by (score descending, index ascending).  The scan over them
+// either reaches post_nms_topn kept boxes, or the full-size path behind it starts over.
+//
+// Equal scores: SortBBox (proposal_layer.cpp:88-111) leaves them in an order of its own,
+// which only the replay kernels below know.  It cannot matter when, of the proposals
+// that share a score, at most one is still alive when the scan reaches them (alive:
+// overlaps no box kept before the group): the others are dropped wherever they stand,
+// the live one is kept wherever it stands, and the kept sequence is the same for every
+// order of the group.  proposal_head_check_kernel verifies exactly that for every group
+// of equal scores the scan reached (a group that hangs over the end of the head, where
+// the order would also decide who is in, counts as not settled), and only then reports
+// the result as complete.
+constexpr int kHeadWant = 512;                        // = kScanRows, one super-block of the scan
+constexpr int kHeadThreads = 512;
+constexpr int kHeadPer = 44;                          // keys per thread
+constexpr int kHeadMaxN = kHeadPer * kHeadThreads;    // 22528 proposals
+constexpr int kHeadCandPer = 8;                       // candidates per thread after the first cut
+constexpr int kHeadCand = kHeadCandPer * kHeadThreads;
+
+// Compare-exchange network over one (key, index) pair per thread of the workgroup
+// (kHeadThreads entries, the unused ones hold the largest pair): ascending by key, then
+// index.  Partners closer than a wavefront are reached by lane shuffles, the others
+// through LDS.  Fully unrolled: every shuffle has a constant distance.
+template <int K, int J>
+__device__ __forceinline__ void bitonic_step(uint32_t& key, uint32_t& idx, uint32_t* xk, uint32_t* xi) {
+  const int tid = threadIdx.x;
+  uint32_t ok, oi;
+  if constexpr (J >= 64) {
+    __syncthreads();
+    xk[tid] = key;
+    xi[tid] = idx;
+    __syncthreads();
+    ok = xk[tid ^ J];
+    oi = xi[tid ^ J];
+  } else {
+    ok = __shfl_xor(key, J, 64);
+    oi = __shfl_xor(idx, J, 64);
+  }
+  const bool up = (tid & K) == 0;          // this run sorts ascending
+  const bool lower = (tid & J) == 0;       // this thread keeps the smaller of the two
+  const bool other_less = ok < key || (ok == key && oi < idx);
+  const bool take = (lower == up) ? other_less : !other_less;
+  key = take ? ok : key;
+  idx = take ? oi : idx;
+  if constexpr (J > 1) bitonic_step<K, J / 2>(key, idx, xk, xi);
+}
+template <int K>
+__device__ __forceinline__ void bitonic_merge_up_to(uint32_t& key, uint32_t& idx, uint32_t* xk, uint32_t* xi) {
+  if constexpr (K > 2) bitonic_merge_up_to<K / 2>(key, idx, xk, xi);
+  bitonic_step<K, K / 2>(key, idx, xk, xi);
+}
+
+// info[0] = number of ordered entries m >= want (the keys at or below the want-th smallest),
+// 0 when the head could not be ordered here (more candidates than the kernel holds: equal
+// scores in crowds; the full-size path takes over).  out_keys / out_order[0 .. m): (key
+// ascending = score descending, index ascending); the boxes and scores of the first
+// `want` of them go to sorted_boxes / sorted_scores.
+__global__ __launch_bounds__(kHeadThreads) void proposal_head_kernel(
+    const uint32_t* __restrict__ keys, int n, int want, uint32_t* __restrict__ out_keys,
+    int* __restrict__ out_order, int* __restrict__ info, const float4* __restrict__ boxes,
+    const float* __restrict__ scores, float4* __restrict__ sorted_boxes,
+    float* __restrict__ sorted_scores) {
+  __shared__ uint32_t s_ckey[kHeadCand];
+  __shared__ unsigned short s_cidx[kHeadCand];
+  __shared__ uint32_t s_x[2 * kHeadThreads];
+  __shared__ int s_cnt[2][3][kHeadThreads / 64];
+  __shared__ uint32_t s_red[kHeadThreads / 64];
+  __shared__ uint32_t s_wave_sum[kHeadThreads / 64];
+  __shared__ int s_tot;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // any thread may hold any key: coalesced loads, key i in thread i % threads (no branches
+  // around the loads: all of them are in flight together)
+  uint32_t rk[kHeadPer];
+#pragma unroll
+  for (int j = 0; j < kHeadPer; ++j) {
+    const int i = tid + j * kHeadThreads;
+    const uint32_t k = keys[min(i, n - 1)];
+    rk[j] = i < n ? k : 0xffffffffu;
+  }
+  // First cut.  Every thread has a smallest key; the largest of those has at least one key
+  // per thread at or below it, kHeadThreads >= want in all, and (the threads hold strided
+  // samples of the table) usually a few thousand: the candidates.
+  uint32_t lowest = 0xffffffffu;
+#pragma unroll
+  for (int j = 0; j < kHeadPer; ++j) lowest = min(lowest, rk[j]);
+  uint32_t cut = lowest;  // a thread without keys (n < threads) holds all ones: every key passes
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) cut = max(cut, __shfl_xor(cut, o, 64));
+  if (lane == 0) s_red[wave] = cut;
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < kHeadThreads / 64; ++w) cut = max(cut, s_red[w]);
+  int mine = 0;
+#pragma unroll
+  for (int j = 0; j < kHeadPer; ++j) mine += (tid + j * kHeadThreads < n && rk[j] <= cut) ? 1 : 0;
+  uint32_t base = block_exclusive_scan(static_cast<uint32_t>(mine), s_wave_sum);
+  if (tid == kHeadThreads - 1) s_tot = static_cast<int>(base) + mine;
+  __syncthreads();
+  const int ncand = s_tot;
+  if (ncand > kHeadCand) {  // uniform
+    if (tid == 0) info[0] = 0;
+    return;
+  }
+  {
+    int at = static_cast<int>(base);
+#pragma unroll
+    for (int j = 0; j < kHeadPer; ++j)
+      if (tid + j * kHeadThreads < n && rk[j] <= cut) {
+        s_ckey[at] = rk[j];
+        s_cidx[at] = static_cast<unsigned short>(tid + j * kHeadThreads);
+        ++at;
+      }
+  }
+  __syncthreads();
+  uint32_t ck[kHeadCandPer];
+  uint32_t diff = 0;
+  const uint32_t first = s_ckey[0];
+#pragma unroll
+  for (int j = 0; j < kHeadCandPer; ++j) {
+    const int i = tid + j * kHeadThreads;
+    ck[j] = i < ncand ? s_ckey[i] : 0xffffffffu;
+    diff |= (i < ncand ? ck[j] : first) ^ first;
+  }
+  // bits that are the same in every candidate are tau's as well: their rounds are skipped
+  // (the best scores share sign, exponent and often the first bits of the mantissa)
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) diff |= __shfl_xor(diff, o, 64);
+  if (lane == 0) s_red[wave] = diff;  // (all reads of the cut are behind two barriers)
+  __syncthreads();
+  diff = 0;
+#pragma unroll
+  for (int w = 0; w < kHeadThreads / 64; ++w) diff |= s_red[w];
+  diff = __builtin_amdgcn_readfirstlane(diff);
+  // tau = the smallest value with at least `want` candidates <= tau, two bits per round from
+  // the top: of the four values of the pair the smallest whose trial (prefix | pair | all
+  // lower bits set) has enough candidates at or below.  (A padding entry, all ones, is
+  // never at or below a trial value that has a zero bit; the all-ones trial is not counted.)
+  uint32_t tau = first & ~diff;
+  for (int bit = 31; bit >= 1; bit -= 2) {
+    if (!((diff >> (bit - 1)) & 3u)) continue;  // uniform
+    const uint32_t pair = 3u << (bit - 1), low = (1u << (bit - 1)) - 1u;
+    const uint32_t prefix = tau & ~pair;
+    const uint32_t t0 = prefix | low, t1 = prefix | (1u << (bit - 1)) | low, t2 = prefix | (1u << bit) | low;
+    int c0 = 0, c1 = 0, c2 = 0;
+#pragma unroll
+    for (int j = 0; j < kHeadCandPer; ++j) {
+      c0 += __popcll(__ballot(ck[j] <= t0));  // scalar: the wavefront's count
+      c1 += __popcll(__ballot(ck[j] <= t1));
+      c2 += __popcll(__ballot(ck[j] <= t2));
+    }
+    const int slot = (bit >> 1) & 1;
+    if (lane == 0) {
+      s_cnt[slot][0][wave] = c0;
+      s_cnt[slot][1][wave] = c1;
+      s_cnt[slot][2][wave] = c2;
+    }
+    __syncthreads();
+    int n0 = 0, n1 = 0, n2 = 0;
+#pragma unroll
+    for (int w = 0; w < kHeadThreads / 64; ++w) {
+      n0 += s_cnt[slot][0][w];
+      n1 += s_cnt[slot][1][w];
+      n2 += s_cnt[slot][2][w];
+    }
+    tau = prefix | (n0 >= want ? 0u : n1 >= want ? (1u << (bit - 1)) : n2 >= want ? (1u << bit) : pair);
+  }
+  // the candidates at or below tau, at most one per thread from here on
+  mine = 0;
+#pragma unroll
+  for (int j = 0; j < kHeadCandPer; ++j) mine += ck[j] <= tau ? 1 : 0;  // (padding: tau < all ones, or no padding passes below)
+  base = block_exclusive_scan(static_cast<uint32_t>(mine), s_wave_sum);
+  if (tid == kHeadThreads - 1) s_tot = static_cast<int>(base) + mine;
+  __syncthreads();
+  const int m = s_tot;
+  if (m > kHeadThreads) {  // uniform: equal scores hang over the end of the head
+    if (tid == 0) info[0] = 0;
+    return;
+  }
+  {
+    int at = static_cast<int>(base);
+#pragma unroll
+    for (int j = 0; j < kHeadCandPer; ++j)
+      if (ck[j] <= tau) {
+        s_x[at] = ck[j];
+        s_x[kHeadThreads + at] = s_cidx[tid + j * kHeadThreads];
+        ++at;
+      }
+  }
+  __syncthreads();
+  uint32_t key = tid < m ? s_x[tid] : 0xffffffffu;
+  uint32_t idx = tid < m ? s_x[kHeadThreads + tid] : 0xffffffffu;
+  // ((key, index) pairs are all different, so the network's order is the stable one)
+  bitonic_merge_up_to<kHeadThreads>(key, idx, s_x, s_x + kHeadThreads);
+  if (tid < m) {
+    out_keys[tid] = key;
+    out_order[tid] = static_cast<int>(idx);
+  }
+  if (tid < want) {
+    sorted_boxes[tid] = boxes[idx];
+    sorted_scores[tid] = scores[idx];
+  }
+  if (tid == 0) info[0] = m;
+}
+
+// After the scan over the head: is its result the whole layer's?  flags[2] (done): the
+// scan settled (post_nms_topn kept boxes, or the head was the whole table); flags[3]
+// (complete) is set when, besides, no group of equal scores that the scan reached has two
+// live members or hangs over the end of the head.  Otherwise done is cleared again and
+// the full-size path behind this kernel runs.  mask: rows of the head corner, `stride`
+// words each.
+__global__ __launch_bounds__(512) void proposal_head_check_kernel(
+    const uint32_t* __restrict__ head_keys, const int* __restrict__ info, int want,
+    const int* __restrict__ kept, const int* __restrict__ num_kept, int max_keep,
+    const unsigned long long* __restrict__ mask, int stride, int* __restrict__ flags,
+    const float4* __restrict__ sorted_boxes, const float* __restrict__ sorted_scores,
+    float* __restrict__ rois, float* __restrict__ roi_scores, int* __restrict__ state) {
+  __shared__ unsigned char alive[kHeadWant];
+  __shared__ int s_need;
+  const int z = threadIdx.x;
+  const int m = info[0];
+  const int count = *num_kept;
+  if (z == 0) s_need = (m == 0 || flags[2] == 0) ? 1 : 0;
+  // the last candidate the scan examined
+  const int last = count >= max_keep ? kept[max_keep - 1] : want - 1;
+  bool member = false;
+  int first = z;
+  if (z < kHeadWant) alive[z] = 0;
+  if (m > 0 && z < want) {
+    const uint32_t k = head_keys[z];
+    member = (z > 0 && head_keys[z - 1] == k) || (z + 1 < m && head_keys[z + 1] == k);
+    if (member) {
+      while (first > 0 && head_keys[first - 1] == k) --first;
+      bool live = true;
+      if (first <= last) {
+        for (int r = 0; r < count && live; ++r) {
+          const int kb = kept[r];
+          if (kb >= first) break;  // kept[] ascends
+          live = !((mask[static_cast<size_t>(kb) * stride + (z >> 6)] >> (z & 63)) & 1ull);
+        }
+      }
+      alive[z] = live ? 1 : 0;
+    }
+  }
+  __syncthreads();
+  if (member && first == z && z <= last) {
+    // this thread owns the group that starts here
+    const uint32_t k = head_keys[z];
+    int live = 0, end = z;
+    while (end < want && end < m && head_keys[end] == k) live += alive[end++];
+    // more of the group beyond the head (which is also the table's cut when the head is all of it)
+    const bool hangs_over = end == want && end < m && head_keys[end] == k;
+    if (live >= 2 || hangs_over) s_need = 1;
+  }
+  __syncthreads();
+  const int complete = s_need ? 0 : 1;
+  if (z == 0) {
+    flags[3] = complete;
+    if (!complete) flags[2] = 0;
+    if (state != nullptr) {  // (the step was called by itself)
+      state[0] = 0;
+      state[1] = complete;
+    }
+  }
+  // rois[r] = (0, x1, y1, x2, y2) of the r-th kept box (proposal_layer.cpp:187-203); the
+  // head holds at most 512 kept boxes
+  if (complete && z < count) {
+    const float4 b = sorted_boxes[kept[z]];
+    rois[z * 5 + 0] = 0.f;
+    rois[z * 5 + 1] = b.x;
+    rois[z * 5 + 2] = b.y;
+    rois[z * 5 + 3] = b.z;
+    rois[z * 5 + 4] = b.w;
+    if (roi_scores) roi_scores[z] = sorted_scores[kept[z]];
+  }
 }
 
 // Exact replay of the reference's SortBBox (proposal_layer.cpp:88-111) for inputs
@@ -1121,6 +1411,7 @@ constexpr int kScanThreads = 512;
 constexpr int kScanBlocks = 8;                    // blocks of 64 boxes per super-block
 constexpr int kScanRows = kScanBlocks * 64;       // boxes per super-block
 constexpr int kScanLoads = kScanRows * kScanBlocks / kScanThreads;  // staged words per thread
+static_assert(kHeadWant == kScanRows, "the head is one super-block of the scan");
 
 __device__ inline unsigned long long wave_uniform(unsigned long long v) {
   const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v));
@@ -1307,7 +1598,14 @@ __global__ void proposal_gather_kernel(const float4* __restrict__ sorted_boxes,
                                        const float* __restrict__ sorted_scores,
                                        const int* __restrict__ kept,
                                        const int* __restrict__ num_kept, float* __restrict__ rois,
-                                       float* __restrict__ roi_scores) {
+                                       float* __restrict__ roi_scores, const int* __restrict__ flags,
+                                       int* __restrict__ state, int state_ints) {
+  // what the caller learns: state[0] = which equal-score replay ran, state[1] = the result is final
+  if (state != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
+    state[0] = flags[0];
+    if (state_ints > 1) state[1] = 1;
+  }
+  if (flags[3] != 0) return;  // the head step wrote the rows
   const int r = blockIdx.x * blockDim.x + threadIdx.x;
   if (r >= *num_kept) return;
   const float4 b = sorted_boxes[kept[r]];
@@ -1364,7 +1662,7 @@ ProposalLayout layout(int n, int pre, int post) {
   L.sorted_scores = take(sizeof(float) * pre);
   L.mask = take(sizeof(unsigned long long) * (size_t)pre * nb);
   L.kept = take(sizeof(int) * post);
-  L.flags = take(sizeof(int) * 4);
+  L.flags = take(sizeof(int) * 8);
   L.total = off;
   return L;
 }
@@ -1414,10 +1712,17 @@ int static_scratch(void** out) {
   return 0;
 }
 
-int run_proposal(const float* scores, const float* bbox, const float* im_info, const float* anchors,
-               int A, int H, int W, int feat_stride, float min_size, int pre_nms_topn,
-               int post_nms_topn, float nms_thresh, void* workspace, size_t workspace_bytes,
-               float* rois, float* roi_scores, int* num_rois, int* tie_flag, void* stream) {
+// Steps of run_proposal: the head of the table alone, the full-size path alone, or both
+// (the second then skips itself on the device when the first one settled the result).
+constexpr int kStepHead = 1, kStepRest = 2;
+
+// state (device, optional): [0] which equal-score replay ran (0 none, 1 general, 3 few
+// ties), [1] 1 when rois / num_rois are final.
+int run_proposal(int steps, const float* scores, const float* bbox, const float* im_info,
+                 const float* anchors, int A, int H, int W, int feat_stride, float min_size,
+                 int pre_nms_topn, int post_nms_topn, float nms_thresh, void* workspace,
+                 size_t workspace_bytes, float* rois, float* roi_scores, int* num_rois, int* state,
+                 int state_ints, void* stream) {
   MC_REQUIRE(scores && bbox && im_info && anchors && workspace && rois && num_rois,
              "mcProposal: null argument");
   MC_REQUIRE(A > 0 && H > 0 && W > 0 && pre_nms_topn > 0 && post_nms_topn > 0,
@@ -1442,9 +1747,18 @@ int run_proposal(const float* scores, const float* bbox, const float* im_info, c
   float* sscores = reinterpret_cast<float*>(ws + L.sorted_scores);
   unsigned long long* mask = reinterpret_cast<unsigned long long*>(ws + L.mask);
   int* kept = reinterpret_cast<int*>(ws + L.kept);
+  // flags: [0] equal scores among the first pre + 1 sorted places (| 2: the few-ties replay
+  // took them), [1] few-ties replay done, [2] the scan settled the result, [3] the head of
+  // the table settled it (the full-size path skips itself), [4] entries the head ordered
   int* flags = reinterpret_cast<int*>(ws + L.flags);
+  int* done = flags + 2;
+  int* complete = flags + 3;
+  int* head_info = flags + 4;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int nb = ceil_div(pre, 64);
+  // (the equal-score replay's prefix-count array holds the column words of the overlap matrix
+  // whenever the replay is not running)
+  unsigned long long* colmask = reinterpret_cast<unsigned long long*>(ws + L.pref);
 
   ProposalTimes times;
   const bool timing = g_prop_timing;
@@ -1454,64 +1768,86 @@ int run_proposal(const float* scores, const float* bbox, const float* im_info, c
     return e != hipSuccess ? e : hipEventRecord(times.ev[k], st);
   };
   MC_HIP(mark(0));
-  zero_ints_kernel<<<1, 64, 0, st>>>(flags, 4);
-  MC_LAUNCH_CHECK();
   // foreground scores are the second half of the score blob (proposal_layer.cpp:295)
   proposal_decode_kernel<<<ceil_div(n, 256), 256, 0, st>>>(scores + n, bbox, anchors, im_info, A, H,
                                                           W, feat_stride, min_size, boxes, k0,
-                                                          korig, v0, sc);
+                                                          korig, v0, sc, flags);
   MC_LAUNCH_CHECK();
-  if (n <= kSortLdsMax)
-    proposal_sort_lds_kernel<<<1, kSortThreads, 0, st>>>(k0, v0, n, pre, flags);
-  else
-    proposal_sort_kernel<<<1, kSortThreads, 0, st>>>(k0, v0, k1, v1, n, pre, flags);
-  MC_LAUNCH_CHECK();
-  MC_HIP(mark(1));
-  // both are no-ops unless equal scores reach into the first `pre` places; the first
-  // takes inputs with few equal scores, the second everything else
-  if (!g_force_general_replay) {
-    tie_replay_fast_kernel<<<1, kFastThreads, 0, st>>>(flags, k0, n, pre, reinterpret_cast<uint2*>(ws + L.pref), v0);
+  // The head can settle the result only if post_nms_topn kept boxes fit it (or it is the
+  // whole table).
+  const bool head_possible = n <= kHeadMaxN && (post_nms_topn < kHeadWant || pre <= kHeadWant);
+  if ((steps & kStepHead) && head_possible) {
+    const int want = pre < kHeadWant ? pre : kHeadWant, head_nb = ceil_div(want, 64);
+    proposal_head_kernel<<<1, kHeadThreads, 0, st>>>(korig, n, want, k1, v1, head_info, boxes, sc,
+                                                     sboxes, sscores);
     MC_LAUNCH_CHECK();
+    MC_HIP(mark(1));
+    nms_mask_kernel<<<head_nb * (head_nb + 1) / 2, 256, 0, st>>>(sboxes, want, nms_thresh, nb, head_nb,
+                                                               mask, colmask, nullptr);
+    MC_LAUNCH_CHECK();
+    nms_scan_kernel<<<1, kScanThreads, sizeof(unsigned long long) * head_nb, st>>>(
+        mask, want, head_nb, nb, post_nms_topn, kept, num_rois, done, want == pre, 0, colmask);
+    MC_LAUNCH_CHECK();
+    proposal_head_check_kernel<<<1, 512, 0, st>>>(k1, head_info, want, kept, num_rois, post_nms_topn,
+                                                  mask, nb, flags, sboxes, sscores, rois, roi_scores,
+                                                  (steps & kStepRest) ? nullptr : state);
+    MC_LAUNCH_CHECK();
+  } else {
+    MC_HIP(mark(1));
   }
-  quicksort_replay_kernel<<<1, kQsThreads, 0, st>>>(
-      flags, korig, n, pre, k1, v1, reinterpret_cast<uint32_t*>(ws + L.kb), ints(L.vb),
-      ints(L.seg_lo), ints(L.seg_hi), reinterpret_cast<unsigned long long*>(ws + L.pref),
-      ints(L.posS), ints(L.posB), ints(L.mS), ints(L.mB), ints(L.hole), ints(L.dest), ints(L.nseg),
-      reinterpret_cast<unsigned char*>(ws + L.cls), v0);
-  MC_LAUNCH_CHECK();
-  proposal_order_gather_kernel<<<ceil_div(pre, 256), 256, 0, st>>>(v0, pre, boxes, sc, sboxes,
-                                                                   sscores);
-  MC_LAUNCH_CHECK();
   MC_HIP(mark(2));
-  // The greedy pass stops at post_nms_topn kept boxes, usually long before the last
-  // candidate: first the best kScanRows candidates among themselves (a corner of the
-  // overlap matrix, one super-block of the scan).  If that settles the result the
-  // full-size launches behind it return at once; otherwise they fill the whole matrix and
-  // the scan resumes behind the first super-block.
-  int* done = flags + 2;
-  const int head = pre < kScanRows ? pre : kScanRows, head_nb = ceil_div(head, 64);
-  // (the equal-score replay is over: its prefix-count array holds the column words now)
-  unsigned long long* colmask = reinterpret_cast<unsigned long long*>(ws + L.pref);
-  nms_mask_kernel<<<head_nb * (head_nb + 1) / 2, 256, 0, st>>>(sboxes, head, nms_thresh, nb, head_nb, mask,
-                                                             colmask, nullptr);
-  MC_LAUNCH_CHECK();
-  nms_scan_kernel<<<1, kScanThreads, sizeof(unsigned long long) * head_nb, st>>>(
-      mask, head, head_nb, nb, post_nms_topn, kept, num_rois, done, head == pre, 0, colmask);
-  MC_LAUNCH_CHECK();
-  if (head < pre) {
-    nms_mask_kernel<<<std::min(nb * (nb + 1) / 2, 8 * kNumCu), 256, 0, st>>>(sboxes, pre, nms_thresh, nb, nb,
-                                                                           mask, colmask, done);
+  if (steps & kStepRest) {
+    if (n <= kSortLdsMax)
+      proposal_sort_lds_kernel<<<1, kSortThreads, 0, st>>>(k0, v0, n, pre, flags, complete);
+    else
+      proposal_sort_kernel<<<1, kSortThreads, 0, st>>>(k0, v0, k1, v1, n, pre, flags, complete);
     MC_LAUNCH_CHECK();
-    nms_scan_kernel<<<1, kScanThreads, sizeof(unsigned long long) * nb, st>>>(
-        mask, pre, nb, nb, post_nms_topn, kept, num_rois, done, 1, 1, colmask);
+    // both are no-ops unless equal scores reach into the first `pre` places; the first
+    // takes inputs with few equal scores, the second everything else
+    if (!g_force_general_replay) {
+      tie_replay_fast_kernel<<<1, kFastThreads, 0, st>>>(flags, k0, n, pre, reinterpret_cast<uint2*>(ws + L.pref), v0);
+      MC_LAUNCH_CHECK();
+    }
+    quicksort_replay_kernel<<<1, kQsThreads, 0, st>>>(
+        flags, korig, n, pre, k1, v1, reinterpret_cast<uint32_t*>(ws + L.kb), ints(L.vb),
+        ints(L.seg_lo), ints(L.seg_hi), reinterpret_cast<unsigned long long*>(ws + L.pref),
+        ints(L.posS), ints(L.posB), ints(L.mS), ints(L.mB), ints(L.hole), ints(L.dest), ints(L.nseg),
+        reinterpret_cast<unsigned char*>(ws + L.cls), v0);
     MC_LAUNCH_CHECK();
-  }
-  MC_HIP(mark(3));
-  proposal_gather_kernel<<<ceil_div(post_nms_topn, 256), 256, 0, st>>>(sboxes, sscores, kept,
-                                                                       num_rois, rois, roi_scores);
-  MC_LAUNCH_CHECK();
-  if (tie_flag) {
-    MC_HIP(hipMemcpyAsync(tie_flag, flags, sizeof(int), hipMemcpyDeviceToDevice, st));
+    proposal_order_gather_kernel<<<ceil_div(pre, 256), 256, 0, st>>>(v0, pre, boxes, sc, sboxes, sscores,
+                                                                     complete);
+    MC_LAUNCH_CHECK();
+    MC_HIP(mark(3));
+    // The greedy pass stops at post_nms_topn kept boxes, usually long before the last
+    // candidate: first the best kScanRows candidates among themselves (a corner of the
+    // overlap matrix, one super-block of the scan).  If that settles the result the
+    // full-size launches behind it return at once; otherwise they fill the whole matrix and
+    // the scan resumes behind the first super-block.  (`done` is also set when the head
+    // step was complete: all four launches return at once then.)
+    const int head = pre < kScanRows ? pre : kScanRows, head_nb = ceil_div(head, 64);
+    nms_mask_kernel<<<head_nb * (head_nb + 1) / 2, 256, 0, st>>>(sboxes, head, nms_thresh, nb, head_nb, mask,
+                                                               colmask, done);
+    MC_LAUNCH_CHECK();
+    nms_scan_kernel<<<1, kScanThreads, sizeof(unsigned long long) * head_nb, st>>>(
+        mask, head, head_nb, nb, post_nms_topn, kept, num_rois, done, head == pre, 0, colmask);
+    MC_LAUNCH_CHECK();
+    if (head < pre) {
+      nms_mask_kernel<<<std::min(nb * (nb + 1) / 2, 8 * kNumCu), 256, 0, st>>>(sboxes, pre, nms_thresh, nb, nb,
+                                                                             mask, colmask, done);
+      MC_LAUNCH_CHECK();
+      nms_scan_kernel<<<1, kScanThreads, sizeof(unsigned long long) * nb, st>>>(
+          mask, pre, nb, nb, post_nms_topn, kept, num_rois, done, 1, 1, colmask);
+      MC_LAUNCH_CHECK();
+    }
+    proposal_gather_kernel<<<ceil_div(post_nms_topn, 256), 256, 0, st>>>(
+        sboxes, sscores, kept, num_rois, rois, roi_scores, flags, state, state_ints);
+    MC_LAUNCH_CHECK();
+  } else {
+    MC_HIP(mark(3));
+    if (state && !head_possible) {  // the head step was asked for and cannot run: not final
+      zero_ints_kernel<<<1, 64, 0, st>>>(state, state_ints);
+      MC_LAUNCH_CHECK();
+    }
   }
   MC_HIP(mark(4));
   if (timing) g_prop_timed.push_back(times);
@@ -1536,9 +1872,28 @@ int mcProposal(const float* scores, const float* bbox, const float* im_info, con
                int A, int H, int W, int feat_stride, float min_size, int pre_nms_topn,
                int post_nms_topn, float nms_thresh, void* workspace, size_t workspace_bytes,
                float* rois, float* roi_scores, int* num_rois, int* tie_flag, void* stream) {
-  return run_proposal(scores, bbox, im_info, anchors, A, H, W, feat_stride, min_size, pre_nms_topn,
-                      post_nms_topn, nms_thresh, workspace, workspace_bytes, rois, roi_scores,
-                      num_rois, tie_flag, stream);
+  return run_proposal(kStepHead | kStepRest, scores, bbox, im_info, anchors, A, H, W, feat_stride,
+                      min_size, pre_nms_topn, post_nms_topn, nms_thresh, workspace, workspace_bytes,
+                      rois, roi_scores, num_rois, tie_flag, 1, stream);
+}
+
+int mcProposalHead(const float* scores, const float* bbox, const float* im_info, const float* anchors,
+                   int A, int H, int W, int feat_stride, float min_size, int pre_nms_topn,
+                   int post_nms_topn, float nms_thresh, void* workspace, size_t workspace_bytes,
+                   float* rois, float* roi_scores, int* num_rois, int* state, void* stream) {
+  MC_REQUIRE(state, "mcProposalHead: null argument");
+  return run_proposal(kStepHead, scores, bbox, im_info, anchors, A, H, W, feat_stride, min_size,
+                      pre_nms_topn, post_nms_topn, nms_thresh, workspace, workspace_bytes, rois,
+                      roi_scores, num_rois, state, 2, stream);
+}
+
+int mcProposalRest(const float* scores, const float* bbox, const float* im_info, const float* anchors,
+                   int A, int H, int W, int feat_stride, float min_size, int pre_nms_topn,
+                   int post_nms_topn, float nms_thresh, void* workspace, size_t workspace_bytes,
+                   float* rois, float* roi_scores, int* num_rois, int* state, void* stream) {
+  return run_proposal(kStepRest, scores, bbox, im_info, anchors, A, H, W, feat_stride, min_size,
+                      pre_nms_topn, post_nms_topn, nms_thresh, workspace, workspace_bytes, rois,
+                      roi_scores, num_rois, state, 2, stream);
 }
 
 int mcProposalForceGeneralReplay(int on) {
@@ -1585,9 +1940,9 @@ int mcProposalStatic(const float* scores, const float* bbox, const float* im_inf
              need, kStaticScratchBytes);
   void* ws = nullptr;
   if (static_scratch(&ws) != 0) return -1;
-  return run_proposal(scores, bbox, im_info, anchors, A, H, W, feat_stride, min_size, pre_nms_topn,
-                      post_nms_topn, nms_thresh, ws, kStaticScratchBytes, rois, roi_scores, num_rois,
-                      tie_flag, stream);
+  return run_proposal(kStepHead | kStepRest, scores, bbox, im_info, anchors, A, H, W, feat_stride,
+                      min_size, pre_nms_topn, post_nms_topn, nms_thresh, ws, kStaticScratchBytes, rois,
+                      roi_scores, num_rois, tie_flag, 1, stream);
 }
 
 }  // extern "C"

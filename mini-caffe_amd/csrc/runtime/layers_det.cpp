@@ -78,20 +78,27 @@ class ProposalLayer : public Layer {
     size_t bytes = 0;
     MC_CHECK(mcProposalWorkspaceSize(n, pre_nms_topn_, post_nms_topn_, &bytes));
     workspace_.Reshape(vector<int>{static_cast<int>((bytes + 3) / 4)});
-    counters_.Reshape(vector<int>{2});
+    counters_.Reshape(vector<int>{3});
     // full-size tops while the kernels run; shrunk to the roi count afterwards
     top[0]->Reshape(vector<int>{post_nms_topn_, 5});
     if (top.size() > 1) top[1]->Reshape(vector<int>{post_nms_topn_});
-    int* counters = counters_.mutable_gpu_data();
-    MC_CHECK(mcProposal(bottom[0]->gpu_data(), bottom[1]->gpu_data(), bottom[2]->gpu_data(),
-                        anchors_.gpu_data(), A, H, W, feat_stride_, static_cast<float>(min_size_),
-                        pre_nms_topn_, post_nms_topn_, nms_thresh_, workspace_.mutable_gpu_data(),
-                        bytes, top[0]->mutable_gpu_data(),
-                        top.size() > 1 ? top[1]->mutable_gpu_data() : nullptr, counters,
-                        counters + 1, cur_stream()));
-    // The top's shape depends on the data (proposal_layer.cpp:313-320): the one
-    // value that has to come back to the host.
-    const int num_rois = counters_.cpu_data()[0];
+    // The top's shape depends on the data (proposal_layer.cpp:313-320), so the roi count
+    // has to come back to the host; with it comes the word that says whether the head of
+    // the proposal table settled the result.  Only if it did not is the full-size path
+    // queued (counters: roi count, equal-score replay flag, result final).
+    int num_rois = 0;
+    for (int step = 0; step < 2; ++step) {
+      int* counters = counters_.mutable_gpu_data();
+      MC_CHECK((step == 0 ? mcProposalHead : mcProposalRest)(
+          bottom[0]->gpu_data(), bottom[1]->gpu_data(), bottom[2]->gpu_data(), anchors_.gpu_data(), A,
+          H, W, feat_stride_, static_cast<float>(min_size_), pre_nms_topn_, post_nms_topn_,
+          nms_thresh_, workspace_.mutable_gpu_data(), bytes, top[0]->mutable_gpu_data(),
+          top.size() > 1 ? top[1]->mutable_gpu_data() : nullptr, counters, counters + 1,
+          cur_stream()));
+      const int* host = counters_.cpu_data();
+      num_rois = host[0];
+      if (host[2] != 0) break;
+    }
     top[0]->Reshape(vector<int>{num_rois, 5});
     if (top.size() > 1) top[1]->Reshape(vector<int>{num_rois});
   }

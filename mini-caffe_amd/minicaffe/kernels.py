@@ -84,6 +84,8 @@ LIB.mcProposalWorkspaceSize.argtypes = [c_int, c_int, c_int, ctypes.POINTER(ctyp
 LIB.mcProposal.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                            c_float, c_int, c_int, c_float, c_void_p, ctypes.c_size_t, c_void_p,
                            c_void_p, c_void_p, c_void_p, c_void_p]
+LIB.mcProposalHead.argtypes = LIB.mcProposal.argtypes
+LIB.mcProposalRest.argtypes = LIB.mcProposal.argtypes
 LIB.mcProposalTimingEnable.argtypes = [c_int]
 LIB.mcProposalForceGeneralReplay.argtypes = [c_int]
 LIB.mcProposalTimingCollect.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(c_long)]

@@ -789,7 +789,12 @@ def test_normalize(K, shape):
         assert np.abs(yd.cpu().numpy() - want).max() < 1e-6
 
 
-def run_proposal(K, scores, bbox, im_info, param):
+def run_proposal(K, scores, bbox, im_info, param, mode="both"):
+    """mode "both": mcProposal (head of the table, then the full-size path, which skips itself
+    on the device when the head settled the result); "rest": the full-size path alone
+    (mcProposalRest); "steps": the layer's way, mcProposalHead, then mcProposalRest only if
+    the head's state word says the result is not final.  Returns rois, scores, the
+    equal-score replay flag and whether the head step alone gave the result."""
     anchors = oracle.generate_anchors()
     A, H, W = 9, scores.shape[2], scores.shape[3]
     pre, post = param["pre_nms_topn"], param["post_nms_topn"]
@@ -799,15 +804,30 @@ def run_proposal(K, scores, bbox, im_info, param):
     sd, bd, idv, ad = dev(scores), dev(bbox), dev(im_info), dev(anchors)
     rois = torch.full((post, 5), float("nan"), device="cuda")
     rs = torch.zeros(post, device="cuda")
-    cnt = torch.zeros(2, dtype=torch.int32, device="cuda")
-    K.check_mc(K.LIB.mcProposal(fptr(sd), fptr(bd), fptr(idv), fptr(ad), A, H, W, 16,
-                                ctypes.c_float(param.get("min_size", 16)), pre, post,
-                                ctypes.c_float(param["nms_thresh"]), fptr(ws), sz.value, fptr(rois),
-                                fptr(rs), ctypes.c_void_p(cnt.data_ptr()),
-                                ctypes.c_void_p(cnt.data_ptr() + 4), None))
-    torch.cuda.synchronize()
+    cnt = torch.zeros(3, dtype=torch.int32, device="cuda")
+
+    def call(fn):
+        K.check_mc(fn(fptr(sd), fptr(bd), fptr(idv), fptr(ad), A, H, W, 16,
+                      ctypes.c_float(param.get("min_size", 16)), pre, post,
+                      ctypes.c_float(param["nms_thresh"]), fptr(ws), sz.value, fptr(rois),
+                      fptr(rs), ctypes.c_void_p(cnt.data_ptr()),
+                      ctypes.c_void_p(cnt.data_ptr() + 4), None))
+        torch.cuda.synchronize()
+
+    head_final = False
+    if mode == "both":
+        call(K.LIB.mcProposal)
+    elif mode == "rest":
+        call(K.LIB.mcProposalRest)
+        assert int(cnt[2].item()) == 1
+    else:
+        call(K.LIB.mcProposalHead)
+        head_final = int(cnt[2].item()) == 1
+        if not head_final:
+            call(K.LIB.mcProposalRest)
+            assert int(cnt[2].item()) == 1
     n, ties = int(cnt[0].item()), int(cnt[1].item())
-    return rois[:n].cpu().numpy(), rs[:n].cpu().numpy(), ties
+    return rois[:n].cpu().numpy(), rs[:n].cpu().numpy(), ties, head_final
 
 
 @pytest.mark.parametrize("hw,pre,post,thr,quant", [
@@ -841,11 +861,12 @@ def test_proposal_bit_exact(K, hw, pre, post, thr, quant):
     im_info = np.array([H * 16, W * 16, 1.0], np.float32)
     param = {"pre_nms_topn": pre, "post_nms_topn": post, "nms_thresh": thr}
     want_rois, want_scores = oracle.proposal(param, scores, bbox, im_info, 2)
-    rois, rs, ties = run_proposal(K, scores, bbox, im_info, param)
-    assert np.array_equal(rois, want_rois)
-    assert np.array_equal(rs, want_scores)
-    if quant:
-        assert ties & 1
+    for mode in ("rest", "both", "steps"):
+        rois, rs, ties, _ = run_proposal(K, scores, bbox, im_info, param, mode)
+        assert np.array_equal(rois, want_rois), mode
+        assert np.array_equal(rs, want_scores), mode
+        if quant and mode == "rest":
+            assert ties & 1
 
 
 @pytest.mark.parametrize("hw,pre,post,thr,pairs,seed", [
@@ -888,11 +909,12 @@ def test_proposal_with_few_equal_scores(K, hw, pre, post, thr, pairs, seed, gene
     want_rois, want_scores = oracle.proposal(param, scores, bbox, im_info, 2)
     K.check_mc(K.LIB.mcProposalForceGeneralReplay(int(general)))
     try:
-        rois, rs, ties = run_proposal(K, scores, bbox, im_info, param)
+        for mode in ("both", "steps", "rest"):
+            rois, rs, ties, _ = run_proposal(K, scores, bbox, im_info, param, mode)
+            assert np.array_equal(rois, want_rois), mode
+            assert np.array_equal(rs, want_scores), mode
     finally:
         K.check_mc(K.LIB.mcProposalForceGeneralReplay(0))
-    assert np.array_equal(rois, want_rois)
-    assert np.array_equal(rs, want_scores)
     # which kernel did it: 3 = the few-ties one (at most 22 528 proposals and 500 equal
     # neighbour pairs among the best pre_nms_topn + 1 sorted scores), 1 = the general one
     props = oracle.generate_proposals(scores[0, A:], bbox[0], oracle.generate_anchors(), float(im_info[0]),
@@ -901,6 +923,46 @@ def test_proposal_with_few_equal_scores(K, hw, pre, post, thr, pairs, seed, gene
     counted = int((skey[:-1] == skey[1:])[:min(pre, n)].sum())
     assert counted > 0
     assert ties == (3 if (not general and n <= 22528 and counted <= 500) else 1)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_proposal_head_with_equal_scores_among_the_best(K, seed):
+    """The head step (best 512 proposals) may only call its result final when the order of
+    equal scores cannot matter.  Equal scores are planted among the best few hundred
+    proposals, half of the groups on proposals of one anchor position and shape (boxes
+    that overlap: one suppresses the other, which one depends on the reference's order),
+    half on proposals far apart (both kept: the order of the rows depends on it), some
+    below a box that suppresses them (dead: no order matters).  Whatever the head decides,
+    the rows must equal the reference's bit for bit; over the seeds both outcomes occur."""
+    rng = np.random.default_rng(500 + seed)
+    A, H, W = 9, 38, 63
+    n = A * H * W
+    fg = (rng.permutation(n).astype(np.float32) / n * 0.9 + 0.05).reshape(H, W, A)
+    bbox = (rng.standard_normal((1, 4 * A, H, W)) * 0.05).astype(np.float32)
+    flat = fg.reshape(-1)
+    best = np.argsort(-flat)[:400]
+    groups = int(rng.integers(0, 4)) if seed % 3 else 0
+    for g in range(groups):
+        i = int(rng.choice(best[20:]))
+        h, w, k = np.unravel_index(i, (H, W, A))
+        if g % 2 == 0:      # neighbour position, same anchor shape: heavy overlap
+            j = np.ravel_multi_index((h, min(w + 1, W - 1) if w + 1 < W else w - 1, k), (H, W, A))
+        else:               # far away
+            j = np.ravel_multi_index(((h + H // 2) % H, (w + W // 2) % W, k), (H, W, A))
+        flat[j] = flat[i]
+    scores = rng.random((1, 2 * A, H, W)).astype(np.float32)
+    scores[0, A:] = fg.transpose(2, 0, 1)
+    im_info = np.array([H * 16, W * 16, 1.0], np.float32)
+    param = {"pre_nms_topn": 6000, "post_nms_topn": int(rng.choice([50, 300])), "nms_thresh": 0.7}
+    want_rois, want_scores = oracle.proposal(param, scores, bbox, im_info, 2)
+    outcomes = []
+    for mode in ("steps", "both"):
+        rois, rs, ties, head_final = run_proposal(K, scores, bbox, im_info, param, mode)
+        assert np.array_equal(rois, want_rois), (mode, head_final)
+        assert np.array_equal(rs, want_scores), (mode, head_final)
+        outcomes.append(head_final)
+    if groups == 0:
+        assert outcomes[0]          # distinct scores: the head settles it
 
 
 def test_detection_output_shared_locations_without_background_fail(K):

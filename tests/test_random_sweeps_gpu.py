@@ -140,7 +140,7 @@ def test_random_proposals(K):
     """Map sizes, pre / post_nms_topn around the scan's 512-box super-blocks, thresholds
     from 0.05 to 0.99, tight and loose boxes, with and without equal scores."""
     rng = np.random.default_rng(123)
-    for _ in range(120):
+    for case in range(120):
         H, W = int(rng.integers(3, 45)), int(rng.integers(3, 64))
         A = 9
         n = A * H * W
@@ -157,7 +157,7 @@ def test_random_proposals(K):
         im_info = np.array([H * 16, W * 16, 1.0], np.float32)
         param = {"pre_nms_topn": pre, "post_nms_topn": post, "nms_thresh": thr}
         want_rois, want_scores = oracle.proposal(param, scores, bbox, im_info, 2)
-        rois, rs, _ = T.run_proposal(K, scores, bbox, im_info, param)
+        rois, rs, _, _ = T.run_proposal(K, scores, bbox, im_info, param, ("both", "steps", "rest")[case % 3])
         assert np.array_equal(rois, want_rois) and np.array_equal(rs, want_scores), (H, W, pre, post, thr, spread, quant)
 
 
