@@ -165,6 +165,176 @@ __device__ inline void block_sort_desc_lds(uint32_t* keys, VT* vals, int n, Bloc
   }
 }
 
+// ---- the `want` smallest keys of a table, in order, without sorting the table --------
+//
+// For want <= kSortThreads (the candidates of a greedy pass that looks at a few hundred
+// entries of a table of thousands).  Every thread holds PER keys in registers, entry
+// tid + j * kSortThreads in rk[j]; the all-ones key marks "no entry".
+//   1. First cut: every thread has a smallest key, and the largest of those has at least
+//      one key per thread at or below it, kSortThreads >= want in all; the threads hold
+//      strided samples of the table, so usually a few thousand keys pass: the candidates
+//      (kSelectCandPer per thread at most, else the call fails and the caller sorts).
+//   2. tau = the want-th smallest candidate by bisection on the key bits, two bits per
+//      round from the top (three trial values, one count over the workgroup each: ballots
+//      and scalar population counts within a wavefront, the wavefronts' counts through
+//      LDS); bits that are the same in every candidate are skipped.
+//   3. The m >= want candidates at or below tau (more than want only if keys equal to tau
+//      hang over) go one to a thread through a compare-exchange network on (key, index):
+//      all pairs differ, so the order is that of a stable sort by key.
+// Returns m, and in thread t < m the entry of rank t; 0 when step 1 or 3 does not fit
+// (crowds of equal keys).  All threads of the workgroup must call it.
+constexpr int kSelectCandPer = 8;
+struct BlockSelectLds {
+  uint32_t ckey[kSelectCandPer * kSortThreads];
+  unsigned short cidx[kSelectCandPer * kSortThreads];
+  uint32_t x[2 * kSortThreads];
+  int cnt[2][3][kSortThreads / 64];
+  uint32_t red[kSortThreads / 64];
+  uint32_t wave_sum[kSortThreads / 64];
+  int tot;
+};
+
+template <int K, int J>
+__device__ __forceinline__ void bitonic_step(uint32_t& key, uint32_t& idx, uint32_t* xk, uint32_t* xi) {
+  const int tid = threadIdx.x;
+  uint32_t ok, oi;
+  if constexpr (J >= 64) {
+    __syncthreads();
+    xk[tid] = key;
+    xi[tid] = idx;
+    __syncthreads();
+    ok = xk[tid ^ J];
+    oi = xi[tid ^ J];
+  } else {
+    ok = __shfl_xor(key, J, 64);
+    oi = __shfl_xor(idx, J, 64);
+  }
+  const bool up = (tid & K) == 0;          // this run sorts ascending
+  const bool lower = (tid & J) == 0;       // this thread keeps the smaller of the two
+  const bool other_less = ok < key || (ok == key && oi < idx);
+  const bool take = (lower == up) ? other_less : !other_less;
+  key = take ? ok : key;
+  idx = take ? oi : idx;
+  if constexpr (J > 1) bitonic_step<K, J / 2>(key, idx, xk, xi);
+}
+// Ascending by (key, idx) over one pair per thread of a kSortThreads workgroup; fully
+// unrolled, so every lane shuffle has a constant distance.
+template <int K>
+__device__ __forceinline__ void bitonic_sort_block(uint32_t& key, uint32_t& idx, uint32_t* xk, uint32_t* xi) {
+  if constexpr (K > 2) bitonic_sort_block<K / 2>(key, idx, xk, xi);
+  bitonic_step<K, K / 2>(key, idx, xk, xi);
+}
+
+template <int PER>
+__device__ __forceinline__ int block_select_smallest(const uint32_t (&rk)[PER], int want, BlockSelectLds* s,
+                                            uint32_t* key_out, uint32_t* idx_out) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  uint32_t lowest = 0xffffffffu;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) lowest = min(lowest, rk[j]);
+  uint32_t cut = lowest;  // (a thread without entries holds all ones: every entry passes)
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) cut = max(cut, static_cast<uint32_t>(__shfl_xor(cut, o, 64)));
+  __syncthreads();  // (the caller may still be reading what `s` overlays)
+  if (lane == 0) s->red[wave] = cut;
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < kSortThreads / 64; ++w) cut = max(cut, s->red[w]);
+  int mine = 0;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) mine += (rk[j] != 0xffffffffu && rk[j] <= cut) ? 1 : 0;
+  uint32_t base = block_exclusive_scan(static_cast<uint32_t>(mine), s->wave_sum);
+  if (tid == kSortThreads - 1) s->tot = static_cast<int>(base) + mine;
+  __syncthreads();
+  const int ncand = s->tot;
+  if (ncand > kSelectCandPer * kSortThreads || ncand < want) return 0;  // uniform
+  {
+    int at = static_cast<int>(base);
+#pragma unroll
+    for (int j = 0; j < PER; ++j)
+      if (rk[j] != 0xffffffffu && rk[j] <= cut) {
+        s->ckey[at] = rk[j];
+        s->cidx[at] = static_cast<unsigned short>(tid + j * kSortThreads);
+        ++at;
+      }
+  }
+  __syncthreads();
+  uint32_t ck[kSelectCandPer];
+  uint32_t diff = 0;
+  const uint32_t first = s->ckey[0];
+#pragma unroll
+  for (int j = 0; j < kSelectCandPer; ++j) {
+    const int i = tid + j * kSortThreads;
+    ck[j] = i < ncand ? s->ckey[i] : 0xffffffffu;
+    diff |= (i < ncand ? ck[j] : first) ^ first;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) diff |= __shfl_xor(diff, o, 64);
+  if (lane == 0) s->red[wave] = diff;  // (all reads of the cut are behind two barriers)
+  __syncthreads();
+  diff = 0;
+#pragma unroll
+  for (int w = 0; w < kSortThreads / 64; ++w) diff |= s->red[w];
+  diff = __builtin_amdgcn_readfirstlane(diff);
+  // Of the four values of a bit pair the smallest whose trial (prefix | pair | all lower
+  // bits set) has enough candidates at or below.  (An absent entry, all ones, is never at
+  // or below a trial value that has a zero bit; the all-ones trial is not counted.)
+  uint32_t tau = first & ~diff;
+  for (int bit = 31; bit >= 1; bit -= 2) {
+    if (!((diff >> (bit - 1)) & 3u)) continue;  // uniform
+    const uint32_t pair = 3u << (bit - 1), low = (1u << (bit - 1)) - 1u;
+    const uint32_t prefix = tau & ~pair;
+    const uint32_t t0 = prefix | low, t1 = prefix | (1u << (bit - 1)) | low, t2 = prefix | (1u << bit) | low;
+    int c0 = 0, c1 = 0, c2 = 0;
+#pragma unroll
+    for (int j = 0; j < kSelectCandPer; ++j) {
+      c0 += __popcll(__ballot(ck[j] <= t0));  // scalar: the wavefront's count
+      c1 += __popcll(__ballot(ck[j] <= t1));
+      c2 += __popcll(__ballot(ck[j] <= t2));
+    }
+    const int slot = (bit >> 1) & 1;
+    if (lane == 0) {
+      s->cnt[slot][0][wave] = c0;
+      s->cnt[slot][1][wave] = c1;
+      s->cnt[slot][2][wave] = c2;
+    }
+    __syncthreads();
+    int n0 = 0, n1 = 0, n2 = 0;
+#pragma unroll
+    for (int w = 0; w < kSortThreads / 64; ++w) {
+      n0 += s->cnt[slot][0][w];
+      n1 += s->cnt[slot][1][w];
+      n2 += s->cnt[slot][2][w];
+    }
+    tau = prefix | (n0 >= want ? 0u : n1 >= want ? (1u << (bit - 1)) : n2 >= want ? (1u << bit) : pair);
+  }
+  mine = 0;
+#pragma unroll
+  for (int j = 0; j < kSelectCandPer; ++j) mine += (ck[j] != 0xffffffffu && ck[j] <= tau) ? 1 : 0;
+  base = block_exclusive_scan(static_cast<uint32_t>(mine), s->wave_sum);
+  if (tid == kSortThreads - 1) s->tot = static_cast<int>(base) + mine;
+  __syncthreads();
+  const int m = s->tot;
+  if (m > kSortThreads) return 0;  // uniform: keys equal to tau in a crowd
+  {
+    int at = static_cast<int>(base);
+#pragma unroll
+    for (int j = 0; j < kSelectCandPer; ++j)
+      if (ck[j] != 0xffffffffu && ck[j] <= tau) {
+        s->x[at] = ck[j];
+        s->x[kSortThreads + at] = s->cidx[tid + j * kSortThreads];
+        ++at;
+      }
+  }
+  __syncthreads();
+  uint32_t key = tid < m ? s->x[tid] : 0xffffffffu;
+  uint32_t idx = tid < m ? s->x[kSortThreads + tid] : 0xffffffffu;
+  bitonic_sort_block<kSortThreads>(key, idx, s->x, s->x + kSortThreads);
+  *key_out = key;
+  *idx_out = idx;
+  return m;
+}
+
 }  // namespace mchip
 
 #endif  // MCHIP_EXACT_BLOCK_SORT_H_

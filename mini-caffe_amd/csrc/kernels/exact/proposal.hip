@@ -153,44 +153,9 @@ __global__ __launch_bounds__(256) void proposal_order_gather_kernel(
 // the order would also decide who is in, counts as not settled), and only then reports
 // the result as complete.
 constexpr int kHeadWant = 512;                        // = kScanRows, one super-block of the scan
-constexpr int kHeadThreads = 512;
+constexpr int kHeadThreads = kSortThreads;
 constexpr int kHeadPer = 44;                          // keys per thread
 constexpr int kHeadMaxN = kHeadPer * kHeadThreads;    // 22528 proposals
-constexpr int kHeadCandPer = 8;                       // candidates per thread after the first cut
-constexpr int kHeadCand = kHeadCandPer * kHeadThreads;
-
-// Compare-exchange network over one (key, index) pair per thread of the workgroup
-// (kHeadThreads entries, the unused ones hold the largest pair): ascending by key, then
-// index.  Partners closer than a wavefront are reached by lane shuffles, the others
-// through LDS.  Fully unrolled: every shuffle has a constant distance.
-template <int K, int J>
-__device__ __forceinline__ void bitonic_step(uint32_t& key, uint32_t& idx, uint32_t* xk, uint32_t* xi) {
-  const int tid = threadIdx.x;
-  uint32_t ok, oi;
-  if constexpr (J >= 64) {
-    __syncthreads();
-    xk[tid] = key;
-    xi[tid] = idx;
-    __syncthreads();
-    ok = xk[tid ^ J];
-    oi = xi[tid ^ J];
-  } else {
-    ok = __shfl_xor(key, J, 64);
-    oi = __shfl_xor(idx, J, 64);
-  }
-  const bool up = (tid & K) == 0;          // this run sorts ascending
-  const bool lower = (tid & J) == 0;       // this thread keeps the smaller of the two
-  const bool other_less = ok < key || (ok == key && oi < idx);
-  const bool take = (lower == up) ? other_less : !other_less;
-  key = take ? ok : key;
-  idx = take ? oi : idx;
-  if constexpr (J > 1) bitonic_step<K, J / 2>(key, idx, xk, xi);
-}
-template <int K>
-__device__ __forceinline__ void bitonic_merge_up_to(uint32_t& key, uint32_t& idx, uint32_t* xk, uint32_t* xi) {
-  if constexpr (K > 2) bitonic_merge_up_to<K / 2>(key, idx, xk, xi);
-  bitonic_step<K, K / 2>(key, idx, xk, xi);
-}
 
 // info[0] = number of ordered entries m >= want (the keys at or below the want-th smallest),
 // 0 when the head could not be ordered here (more candidates than the kernel holds: equal
@@ -202,137 +167,23 @@ __global__ __launch_bounds__(kHeadThreads) void proposal_head_kernel(
     int* __restrict__ out_order, int* __restrict__ info, const float4* __restrict__ boxes,
     const float* __restrict__ scores, float4* __restrict__ sorted_boxes,
     float* __restrict__ sorted_scores) {
-  __shared__ uint32_t s_ckey[kHeadCand];
-  __shared__ unsigned short s_cidx[kHeadCand];
-  __shared__ uint32_t s_x[2 * kHeadThreads];
-  __shared__ int s_cnt[2][3][kHeadThreads / 64];
-  __shared__ uint32_t s_red[kHeadThreads / 64];
-  __shared__ uint32_t s_wave_sum[kHeadThreads / 64];
-  __shared__ int s_tot;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  __shared__ BlockSelectLds sel;
+  const int tid = threadIdx.x;
   // any thread may hold any key: coalesced loads, key i in thread i % threads (no branches
   // around the loads: all of them are in flight together)
   uint32_t rk[kHeadPer];
 #pragma unroll
-  for (int j = 0; j < kHeadPer; ++j) {
-    const int i = tid + j * kHeadThreads;
-    const uint32_t k = keys[min(i, n - 1)];
-    rk[j] = i < n ? k : 0xffffffffu;
-  }
-  // First cut.  Every thread has a smallest key; the largest of those has at least one key
-  // per thread at or below it, kHeadThreads >= want in all, and (the threads hold strided
-  // samples of the table) usually a few thousand: the candidates.
-  uint32_t lowest = 0xffffffffu;
+  for (int j = 0; j < kHeadPer; ++j) rk[j] = keys[min(tid + j * kHeadThreads, n - 1)];
+  __builtin_amdgcn_sched_barrier(0);  // (or each load is waited for before the next is issued)
 #pragma unroll
-  for (int j = 0; j < kHeadPer; ++j) lowest = min(lowest, rk[j]);
-  uint32_t cut = lowest;  // a thread without keys (n < threads) holds all ones: every key passes
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) cut = max(cut, __shfl_xor(cut, o, 64));
-  if (lane == 0) s_red[wave] = cut;
-  __syncthreads();
-#pragma unroll
-  for (int w = 0; w < kHeadThreads / 64; ++w) cut = max(cut, s_red[w]);
-  int mine = 0;
-#pragma unroll
-  for (int j = 0; j < kHeadPer; ++j) mine += (tid + j * kHeadThreads < n && rk[j] <= cut) ? 1 : 0;
-  uint32_t base = block_exclusive_scan(static_cast<uint32_t>(mine), s_wave_sum);
-  if (tid == kHeadThreads - 1) s_tot = static_cast<int>(base) + mine;
-  __syncthreads();
-  const int ncand = s_tot;
-  if (ncand > kHeadCand) {  // uniform
+  for (int j = 0; j < kHeadPer; ++j)
+    rk[j] = tid + j * kHeadThreads < n ? min(rk[j], 0xfffffffeu) : 0xffffffffu;  // (all ones: no entry)
+  uint32_t key, idx;
+  const int m = block_select_smallest<kHeadPer>(rk, want, &sel, &key, &idx);
+  if (m == 0) {  // uniform
     if (tid == 0) info[0] = 0;
     return;
   }
-  {
-    int at = static_cast<int>(base);
-#pragma unroll
-    for (int j = 0; j < kHeadPer; ++j)
-      if (tid + j * kHeadThreads < n && rk[j] <= cut) {
-        s_ckey[at] = rk[j];
-        s_cidx[at] = static_cast<unsigned short>(tid + j * kHeadThreads);
-        ++at;
-      }
-  }
-  __syncthreads();
-  uint32_t ck[kHeadCandPer];
-  uint32_t diff = 0;
-  const uint32_t first = s_ckey[0];
-#pragma unroll
-  for (int j = 0; j < kHeadCandPer; ++j) {
-    const int i = tid + j * kHeadThreads;
-    ck[j] = i < ncand ? s_ckey[i] : 0xffffffffu;
-    diff |= (i < ncand ? ck[j] : first) ^ first;
-  }
-  // bits that are the same in every candidate are tau's as well: their rounds are skipped
-  // (the best scores share sign, exponent and often the first bits of the mantissa)
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) diff |= __shfl_xor(diff, o, 64);
-  if (lane == 0) s_red[wave] = diff;  // (all reads of the cut are behind two barriers)
-  __syncthreads();
-  diff = 0;
-#pragma unroll
-  for (int w = 0; w < kHeadThreads / 64; ++w) diff |= s_red[w];
-  diff = __builtin_amdgcn_readfirstlane(diff);
-  // tau = the smallest value with at least `want` candidates <= tau, two bits per round from
-  // the top: of the four values of the pair the smallest whose trial (prefix | pair | all
-  // lower bits set) has enough candidates at or below.  (A padding entry, all ones, is
-  // never at or below a trial value that has a zero bit; the all-ones trial is not counted.)
-  uint32_t tau = first & ~diff;
-  for (int bit = 31; bit >= 1; bit -= 2) {
-    if (!((diff >> (bit - 1)) & 3u)) continue;  // uniform
-    const uint32_t pair = 3u << (bit - 1), low = (1u << (bit - 1)) - 1u;
-    const uint32_t prefix = tau & ~pair;
-    const uint32_t t0 = prefix | low, t1 = prefix | (1u << (bit - 1)) | low, t2 = prefix | (1u << bit) | low;
-    int c0 = 0, c1 = 0, c2 = 0;
-#pragma unroll
-    for (int j = 0; j < kHeadCandPer; ++j) {
-      c0 += __popcll(__ballot(ck[j] <= t0));  // scalar: the wavefront's count
-      c1 += __popcll(__ballot(ck[j] <= t1));
-      c2 += __popcll(__ballot(ck[j] <= t2));
-    }
-    const int slot = (bit >> 1) & 1;
-    if (lane == 0) {
-      s_cnt[slot][0][wave] = c0;
-      s_cnt[slot][1][wave] = c1;
-      s_cnt[slot][2][wave] = c2;
-    }
-    __syncthreads();
-    int n0 = 0, n1 = 0, n2 = 0;
-#pragma unroll
-    for (int w = 0; w < kHeadThreads / 64; ++w) {
-      n0 += s_cnt[slot][0][w];
-      n1 += s_cnt[slot][1][w];
-      n2 += s_cnt[slot][2][w];
-    }
-    tau = prefix | (n0 >= want ? 0u : n1 >= want ? (1u << (bit - 1)) : n2 >= want ? (1u << bit) : pair);
-  }
-  // the candidates at or below tau, at most one per thread from here on
-  mine = 0;
-#pragma unroll
-  for (int j = 0; j < kHeadCandPer; ++j) mine += ck[j] <= tau ? 1 : 0;  // (padding: tau < all ones, or no padding passes below)
-  base = block_exclusive_scan(static_cast<uint32_t>(mine), s_wave_sum);
-  if (tid == kHeadThreads - 1) s_tot = static_cast<int>(base) + mine;
-  __syncthreads();
-  const int m = s_tot;
-  if (m > kHeadThreads) {  // uniform: equal scores hang over the end of the head
-    if (tid == 0) info[0] = 0;
-    return;
-  }
-  {
-    int at = static_cast<int>(base);
-#pragma unroll
-    for (int j = 0; j < kHeadCandPer; ++j)
-      if (ck[j] <= tau) {
-        s_x[at] = ck[j];
-        s_x[kHeadThreads + at] = s_cidx[tid + j * kHeadThreads];
-        ++at;
-      }
-  }
-  __syncthreads();
-  uint32_t key = tid < m ? s_x[tid] : 0xffffffffu;
-  uint32_t idx = tid < m ? s_x[kHeadThreads + tid] : 0xffffffffu;
-  // ((key, index) pairs are all different, so the network's order is the stable one)
-  bitonic_merge_up_to<kHeadThreads>(key, idx, s_x, s_x + kHeadThreads);
   if (tid < m) {
     out_keys[tid] = key;
     out_order[tid] = static_cast<int>(idx);

@@ -156,6 +156,52 @@ def test_nms_pixel_brute_force(thr, max_keep):
     assert np.array_equal(got, brute_nms_pixel(boxes, thr, max_keep))
 
 
+def test_order_of_equal_scores_is_irrelevant_with_one_live_member():
+    """The rule the device's head step relies on: a group of equal scores may stand in any
+    order when at most one of its members is alive where the greedy pass reaches the group
+    (alive: overlaps no box kept before the group by more than the threshold).  Checked on
+    the CPU against every order of planted groups; and the converse happens: with two live
+    members some order changes the kept rows."""
+    import itertools
+    r = rng(9)
+    changed_with_two_live = 0
+    checked_with_one_live = 0
+    for trial in range(120):
+        n = 60
+        c = r.random((n, 2)) * 120
+        wh = r.random((n, 2)) * 60 + 10
+        boxes = np.round(np.concatenate([c, c + wh], 1)).astype(np.float32)
+        scores = np.sort(r.random(n).astype(np.float32))[::-1].copy()
+        start, size = int(r.integers(5, 40)), int(r.integers(2, 4))
+        scores[start:start + size] = scores[start]
+        thr, max_keep = float(r.choice([0.3, 0.5])), int(r.choice([8, 60]))
+        table = np.concatenate([boxes, scores[:, None]], 1).astype(np.float32)
+        kept_before = [k for k in brute_nms_pixel(table, thr, n) if k < start]
+
+        def iou(a, b):
+            w = min(a[2], b[2]) - max(a[0], b[0]) + 1
+            h = min(a[3], b[3]) - max(a[1], b[1]) + 1
+            if w <= 0 or h <= 0:
+                return 0.0
+            inter = w * h
+            return inter / ((a[2] - a[0] + 1) * (a[3] - a[1] + 1) + (b[2] - b[0] + 1) * (b[3] - b[1] + 1) - inter)
+
+        live = [z for z in range(start, start + size)
+                if not any(iou(boxes[k], boxes[z]) > thr for k in kept_before)]
+        results = set()
+        for perm in itertools.permutations(range(start, start + size)):
+            order = list(range(start)) + list(perm) + list(range(start + size, n))
+            kept = brute_nms_pixel(table[order], thr, max_keep)
+            results.add(tuple(map(tuple, table[order][kept])))
+        reached = len(kept_before) < max_keep
+        if len(live) <= 1 or not reached:
+            assert len(results) == 1, (trial, live)
+            checked_with_one_live += 1
+        elif len(results) > 1:
+            changed_with_two_live += 1
+    assert checked_with_one_live > 20 and changed_with_two_live > 20
+
+
 def test_proposal_end_to_end_small():
     r = rng(4)
     A, H, W = 9, 5, 6
