@@ -158,6 +158,13 @@ int mcConvTimingCollect(double* total_ms, long* launches, double* flops);
 int mcConvTimingCollectDetail(double* total_ms, long* launches, double* flops, double* issued_flops,
                               long* winograd);
 
+/* Frees the calling thread's kernel scratch (the partial sums and arrival counters of
+ * contractions whose channel loop is cut into slices, BatchNorm's per-part statistics):
+ * grow-only device buffers, one per stream the thread has launched on, that the thread
+ * owns.  They are also freed when the thread ends, and by MemPoolClear / CaffeMemPoolClear.
+ * Waits for the device.  No counterpart in the reference. */
+int mcReleaseScratch(void);
+
 /* HIP stream of the calling thread's Mini-Caffe context (created on first use);
  * lets a harness record events around Net::Forward.  NULL if no device. */
 void* mcCurrentStream(void);

@@ -466,6 +466,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
     // stores and loads that go past the per-XCD L2, which is not coherent with
     // the other seven), so no cache write-back or invalidation is needed: a
     // workgroup waits until its own stores have completed and then counts.
+    // What this rests on is particular to the parts it is built for: a store with
+    // device scope (sc1) is written through to the memory side, where all XCDs meet,
+    // and vmcnt counts it down only when that write has been acknowledged; an
+    // atomic on the counter issued after the wait is therefore ordered behind the
+    // partial sums at the one place every later device-scope load reads from.  The
+    // language's memory model promises none of this for relaxed accesses.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx942__) && !defined(__gfx950__)
+#error "the in-launch sum of K slices relies on gfx942 / gfx950 device-scope write-through"
+#endif
     const int tile_id = (sub_index * gridDim.y + g) * gridDim.x + blockIdx.x;
     constexpr int kRegs = TM * TN * 16;  // accumulator registers per thread
     float* mine = a.partial +

@@ -389,7 +389,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // The partial sums and the counter are accessed with device-scope atomic operations
     // only (relaxed stores and loads that go past the per-XCD L2, which is not coherent
     // with the other seven), so no cache write-back or invalidation is needed: a
-    // workgroup waits until its own stores have completed and then counts.
+    // workgroup waits until its own stores have completed and then counts.  (A
+    // device-scope store is written through to the memory side and counted down by vmcnt
+    // when acknowledged there; the relaxed accesses alone promise nothing of the kind.)
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx942__) && !defined(__gfx950__)
+#error "the in-launch sum of channel slices relies on gfx942 / gfx950 device-scope write-through"
+#endif
     const int tile_id = blockIdx.x;
     const size_t slice_elems = static_cast<size_t>(gridDim.x) * (64 * 256);
     float* mine = a.partial + blockIdx.y * slice_elems + static_cast<size_t>(tile_id) * (64 * 256) + tid;

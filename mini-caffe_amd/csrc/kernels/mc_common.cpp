@@ -15,21 +15,37 @@ struct Workspace {
   float* ptr = nullptr;
   size_t bytes = 0;
 };
-thread_local std::vector<std::pair<hipStream_t, Workspace>> g_workspaces[2];
 struct Counters {
   int* ptr = nullptr;
   size_t count = 0;
 };
-thread_local std::vector<std::pair<hipStream_t, Counters>> g_counters;
+// The calling thread's scratch buffers, one per stream it has launched on.  They belong to
+// the thread: released when it ends (and by mcReleaseScratch), so a thread that runs one
+// net and exits leaves no device memory behind.
+struct ThreadScratch {
+  std::vector<std::pair<hipStream_t, Workspace>> workspaces;
+  std::vector<std::pair<hipStream_t, Counters>> counters;
+  void release() {
+    // hipFree waits for the device: no kernel still reads what is freed
+    for (auto& e : workspaces)
+      if (e.second.ptr) (void)hipFree(e.second.ptr);
+    for (auto& e : counters)
+      if (e.second.ptr) (void)hipFree(e.second.ptr);
+    workspaces.clear();
+    counters.clear();
+  }
+  ~ThreadScratch() { release(); }
+};
+thread_local ThreadScratch g_scratch;
 }  // namespace
 
 int stream_counters(hipStream_t st, size_t count, int** out) {
   Counters* c = nullptr;
-  for (auto& e : g_counters)
+  for (auto& e : g_scratch.counters)
     if (e.first == st) c = &e.second;
   if (!c) {
-    g_counters.emplace_back(st, Counters());
-    c = &g_counters.back().second;
+    g_scratch.counters.emplace_back(st, Counters());
+    c = &g_scratch.counters.back().second;
   }
   if (c->count < count) {
     if (c->ptr) MC_HIP(hipFree(c->ptr));  // waits for the device: every user has put its zeros back
@@ -45,14 +61,13 @@ int stream_counters(hipStream_t st, size_t count, int** out) {
   return 0;
 }
 
-int stream_workspace(hipStream_t st, size_t bytes, float** out, int slot) {
+int stream_workspace(hipStream_t st, size_t bytes, float** out) {
   Workspace* ws = nullptr;
-  auto& all = g_workspaces[slot != 0];
-  for (auto& e : all)
+  for (auto& e : g_scratch.workspaces)
     if (e.first == st) ws = &e.second;
   if (!ws) {
-    all.emplace_back(st, Workspace());
-    ws = &all.back().second;
+    g_scratch.workspaces.emplace_back(st, Workspace());
+    ws = &g_scratch.workspaces.back().second;
   }
   if (ws->bytes < bytes) {
     if (ws->ptr) MC_HIP(hipFree(ws->ptr));  // waits for the device
@@ -67,3 +82,8 @@ int stream_workspace(hipStream_t st, size_t bytes, float** out, int slot) {
 }  // namespace mchip
 
 extern "C" const char* mcLastError(void) { return mchip::last_error().c_str(); }
+
+extern "C" int mcReleaseScratch(void) {
+  mchip::g_scratch.release();
+  return 0;
+}

@@ -58,10 +58,10 @@ inline int ew_blocks(long n, int threads, int per_thread = 1) {
 
 // Device scratch for partial results that one call writes and reads back (the
 // slices of a split-K contraction, per-part statistics): one grow-only buffer per
-// (host thread, stream).  Work on one stream is ordered, so consecutive calls
-// share it.  Growing frees the old buffer, which waits for the device.  A caller
-// that keeps its buffer across a call that takes one itself uses another slot.
-int stream_workspace(hipStream_t st, size_t bytes, float** out, int slot = 0);
+// (host thread, stream), owned by the thread: freed when the thread ends or calls
+// mcReleaseScratch.  Work on one stream is ordered, so consecutive calls share it.
+// Growing frees the old buffer, which waits for the device.
+int stream_workspace(hipStream_t st, size_t bytes, float** out);
 
 // Arrival counters for kernels whose workgroups hand work to the last one to
 // finish: one grow-only array of ints per (host thread, stream), zero when it is

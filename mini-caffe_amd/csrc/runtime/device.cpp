@@ -85,6 +85,7 @@ MemPoolState MemPoolGetState() {
 void MemPoolClear() {
   Context::Get().Sync();
   Context::Get().pool()->Clear();
+  (void)mcReleaseScratch();  // the kernels' own scratch of this thread
 }
 
 // ---------------------------------------------------------------------------

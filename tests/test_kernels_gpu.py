@@ -524,6 +524,66 @@ def test_conv_slices_summed_in_launch_over_many_launches(K):
         assert netrun.rel_err(whole.cpu().numpy(), plain.cpu().numpy()) < 1e-4, it
 
 
+SLICED_IN_THE_CONFIGS = [
+    # cin, h, w, cout, k, s, p, d, transposed, batch: the launches of the five configurations
+    # (and their sizes) that leave workgroup slots empty and so cut their channel loop
+    (64, 56, 56, 64, 3, 1, 1, 1, False, 1),          # config 1
+    (1024, 14, 14, 256, 1, 1, 0, 1, False, 64),      # ResNet-50 b64, 784 tiles
+    (512, 28, 28, 256, 1, 2, 0, 1, False, 64),
+    (2048, 7, 7, 512, 1, 1, 0, 1, False, 64),        # 392 tiles
+    (1024, 14, 14, 512, 1, 2, 0, 1, False, 64),
+    (2048, 1, 1, 1000, 1, 1, 0, 1, False, 64),       # the classifier
+    (512, 7, 7, 512, 3, 1, 1, 1, False, 64),         # Winograd path, two slices
+    (512, 19, 19, 1024, 3, 1, 6, 6, False, 8),       # SSD300 b8: fc6 (dilated), fc7, the extra layers
+    (1024, 19, 19, 1024, 1, 1, 0, 1, False, 8),
+    (1024, 19, 19, 256, 1, 1, 0, 1, False, 8),
+    (256, 19, 19, 512, 3, 2, 1, 1, False, 8),
+    (512, 10, 10, 128, 1, 1, 0, 1, False, 8),
+    (128, 10, 10, 256, 3, 2, 1, 1, False, 8),
+    (128, 5, 5, 256, 3, 1, 0, 1, False, 8),
+    (128, 3, 3, 256, 3, 1, 0, 1, False, 8),
+    (512, 19, 19, 512, 3, 1, 1, 1, False, 8),        # conv5_x: Winograd path, sliced
+    (1024, 38, 63, 512, 3, 1, 1, 1, False, 1),       # RPN head: Winograd path, three slices
+    (1024, 4, 4, 512, 4, 2, 1, 1, True, 128),        # DCGAN b128: first deconvolution
+]
+
+
+def test_conv_sliced_launches_of_the_configurations_in_rotation(K):
+    """Every launch of the five configurations whose channel loop the library cuts into
+    slices (summed inside the launch out of a workspace and arrival counters that all
+    sliced launches of a stream share), by the library's own choice of slices, three
+    rounds in rotation: the three results of a geometry must be the same bit for bit (a
+    partial sum read before it arrived, or left over from another launch, would differ)
+    and agree with the unsliced launch (summation order only: two fp32 sums over up to
+    9216 terms, bar 3e-4 against 1e-4 for a result against the oracle)."""
+    gen = torch.Generator(device="cuda").manual_seed(15)
+    work = []
+    for cin, h, w, cout, k, st, p, d, tr, n in SLICED_IN_THE_CONFIGS:
+        plan = K.ConvPlan(K.conv_geom(cin, h, w, cout, k, st, p, d, 1, tr))
+        plain = K.ConvPlan(K.conv_geom(cin, h, w, cout, k, st, p, d, 1, tr))
+        plain.force_split(1)
+        wshape = (cin, cout, k, k) if tr else (cout, cin, k, k)
+        wd = torch.randn(*wshape, device="cuda", generator=gen) * (2.0 / (cin * k * k)) ** 0.5
+        plan.set_weights(wd.data_ptr())
+        plain.set_weights(wd.data_ptr())
+        ho, wo = plan.output_shape()
+        xd = torch.randn(n, cin, h, w, device="cuda", generator=gen)
+        bd = torch.randn(cout, device="cuda", generator=gen)
+        work.append((plan, plain, wd, xd, bd, (n, cout, ho, wo), []))
+    for _ in range(3):
+        for plan, plain, wd, xd, bd, ys, outs in work:
+            y = torch.full(ys, float("nan"), device="cuda")
+            plan.forward(ys[0], xd.data_ptr(), y.data_ptr(), shift=bd.data_ptr(), activation=K_ACT_RELU)
+            outs.append(y)
+    torch.cuda.synchronize()
+    for (plan, plain, wd, xd, bd, ys, outs), geom in zip(work, SLICED_IN_THE_CONFIGS):
+        assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2]), geom
+        ref = torch.full(ys, float("nan"), device="cuda")
+        plain.forward(ys[0], xd.data_ptr(), ref.data_ptr(), shift=bd.data_ptr(), activation=K_ACT_RELU)
+        torch.cuda.synchronize()
+        assert netrun.rel_err(outs[0].cpu().numpy(), ref.cpu().numpy()) < 3e-4, geom
+
+
 @pytest.mark.parametrize("act,slope", [("none", 0.0), ("relu", 0.0), ("relu", 0.2), ("tanh", 0.0),
                                        ("sigmoid", 0.0)])
 def test_conv_epilogue_activations_full_channel_blocks(K, act, slope):

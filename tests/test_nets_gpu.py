@@ -189,6 +189,43 @@ def test_three_threads_each_with_their_own_net(gpu_mode):
         assert netrun.rel_err(got[t], jobs[t][2]) < 1e-3, t
 
 
+def test_short_lived_thread_leaves_no_device_memory(gpu_mode):
+    """A thread that builds a net, runs it (contractions whose channel loop is cut into
+    slices take partial-sum scratch and arrival counters from the kernel library, blobs
+    come from the thread's pool) and ends WITHOUT clearing anything: what it allocated
+    belongs to the thread and goes back to the device when the thread ends."""
+    import threading
+    import torch
+    from minicaffe import zoo
+    spec, inputs = zoo.resnet50_spec(batch=4, size=64, stages=(1, 1, 1, 1), width=32, num_classes=7,
+                                     bn_seed=3, seed=4)
+    errors = []
+
+    def work():
+        try:
+            gpu_mode.set_runtime_mode(1, 0)
+            net = run_net(gpu_mode, spec, inputs)
+            for _ in range(2):
+                net.forward()
+            del net
+        except Exception as e:           # noqa: BLE001 - reported by the main thread
+            errors.append(repr(e))
+
+    def one_thread():
+        th = threading.Thread(target=work)
+        th.start()
+        th.join(timeout=100)
+        assert not errors, errors
+        torch.cuda.synchronize()
+        return torch.cuda.mem_get_info()[0]
+
+    one_thread()                          # (first use: code objects, the runtime's own pools)
+    free_before = one_thread()
+    for _ in range(3):
+        free_after = one_thread()
+    assert free_before - free_after < (4 << 20), (free_before, free_after)
+
+
 def test_flatten_and_reshape_as_views(gpu_mode):
     """Flatten and Reshape take over their bottom's memory when they are its last
     reader; a bottom that is read again, is a net input or is a marked output is
