@@ -135,7 +135,6 @@ struct WinogradArgs {
 // which two physical K rows form a step is free as long as both operands agree,
 // so half-wave h reads the stage's channels 2 h and 2 h + 1 with one 8-byte LDS read
 // and step e multiplies channels {e, 2 + e}.
-template <int DIAG>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void winograd_fused_kernel(
     const WinogradArgs a) {
   // K loop: As[2][f 16][kp 2][m 64][e 2], Bs[2][2][f 16][kp 2][t 32][e 2]  (64 KB);
@@ -224,12 +223,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
   float4 areg[4];
   float ereg[4][4];
-  const float sgv = a.slope + lane;  // (diagnosis builds only)
 
 #define MC_LOADF(res, voff, soff) \
   __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(res, voff, soff, 0))
 #define MC_LOAD_A(kt)                                                                           \
-  if (!(DIAG & 2)) {                                                                            \
+  {                                                                                             \
     const unsigned a_soff = static_cast<unsigned>((mt * a.KT + (kt)) * kAStage) * 4u;           \
     _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                             \
       const u32x4 w4 = __builtin_amdgcn_raw_buffer_load_b128(ures, a_voff, a_soff + i * 4096u, 0); \
@@ -237,20 +235,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }                                                                                           \
   }
 #define MC_LOAD_B(s)                                                                            \
-  if (!(DIAG & 1)) {                                                                            \
+  {                                                                                             \
     const unsigned b_soff = static_cast<unsigned>(s) * round_bytes;                             \
     _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                             \
       _Pragma("unroll") for (int j = 0; j < 4; ++j) ereg[i][j] = MC_LOADF(xres, boff[i][j], b_soff); \
     }                                                                                           \
   }
 #define MC_STORE_A(buf)                                                                         \
-  if (!(DIAG & 4)) {                                                                            \
+  {                                                                                             \
     _Pragma("unroll") for (int i = 0; i < 4; ++i)                                               \
       *reinterpret_cast<float4*>(As + (buf)*kAStage + a_st + i * 1024) = areg[i];               \
   }
   // V = B^T d B, B^T = [1 0 -1 0; 0 1 1 0; 0 -1 1 0; 0 1 0 -1]
-#define MC_STORE_B()                                                                       \
-  if (!(DIAG & 4)) {                                                                            \
+#define MC_STORE_B()                                                                            \
+  {                                                                                             \
     float* bw = Bs + (b_st ^ (2 * kBStage));                                                    \
     _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                             \
       const float r0 = ereg[0][j] - ereg[2][j], r1 = ereg[1][j] + ereg[2][j];                   \
@@ -270,7 +268,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #define MC_COMPUTE(abuf, sub)                                                             \
   {                                                                                             \
     f32x2 av[4][2], bv[4];                                                                      \
-    if (DIAG & 8) { _Pragma("unroll") for (int j = 0; j < 4; ++j) { av[j][0] = av[j][1] = bv[j] = f32x2{sgv, sgv}; } } else \
     _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                             \
       _Pragma("unroll") for (int mb = 0; mb < 2; ++mb) av[j][mb] = *reinterpret_cast<const f32x2*>( \
           As + (abuf)*kAStage + a_rd + j * (kTileM * kStageC) + mb * 64);                       \
@@ -323,7 +320,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     MC_COMPUTE(0, 0);                                                    \
     MC_STORE_A(1);                                                       \
     MC_ORDER_FIRST();                                                    \
-    if (!(DIAG & 16)) __syncthreads();                                   \
+    __syncthreads();                                                     \
     __builtin_amdgcn_sched_barrier(0);                                   \
     MC_LOAD_A(2 * s_next);                                               \
     MC_COMPUTE(1, 1);                                                    \
@@ -332,7 +329,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     b_st ^= 2 * kBStage;                                                 \
     b_rd ^= 2 * kBStage;                                                 \
     MC_ORDER_SECOND();                                                   \
-    if (!(DIAG & 16)) __syncthreads();                                   \
+    __syncthreads();                                                     \
     __builtin_amdgcn_sched_barrier(0);                                   \
   }
 
@@ -672,19 +669,8 @@ int winograd_forward(WinogradState* w, int num, const float* bottom, float* top,
       if (stream_workspace(st, sizeof(float) * tiles * slices * 64 * 256, &a.partial)) return -1;
       if (stream_counters(st, static_cast<size_t>(tiles), &a.counters)) return -1;
     }
-    static const int diag = getenv("MC_WINO_DIAG") ? atoi(getenv("MC_WINO_DIAG")) : 0;
     const dim3 grid(static_cast<unsigned>(tiles), slices);
-    switch (diag) {
-      case 1: winograd_fused_kernel<1><<<grid, 256, 0, st>>>(a); break;
-      case 2: winograd_fused_kernel<2><<<grid, 256, 0, st>>>(a); break;
-      case 3: winograd_fused_kernel<3><<<grid, 256, 0, st>>>(a); break;
-      case 4: winograd_fused_kernel<4><<<grid, 256, 0, st>>>(a); break;
-      case 7: winograd_fused_kernel<7><<<grid, 256, 0, st>>>(a); break;
-      case 15: winograd_fused_kernel<15><<<grid, 256, 0, st>>>(a); break;
-      case 20: winograd_fused_kernel<20><<<grid, 256, 0, st>>>(a); break;
-      case 31: winograd_fused_kernel<31><<<grid, 256, 0, st>>>(a); break;
-      default: winograd_fused_kernel<0><<<grid, 256, 0, st>>>(a);
-    }
+    winograd_fused_kernel<<<grid, 256, 0, st>>>(a);
     MC_LAUNCH_CHECK();
   }
   return 0;
