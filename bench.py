@@ -170,6 +170,20 @@ def main():
                 "mfma_issued_gflop_per_step": round(issued.value / steps / 1e9, 1),
                 "mfma_issued_tflops": round(issued_tflops, 2),
                 "mfma_issued_frac": round(issued_tflops / FP32_MFMA_PEAK_TFLOPS, 4)}
+    # The same step with the input handed over as a host buffer every time, as a caller of
+    # CaffeNetForward with fresh images does: the copy over PCIe is inside the time.
+    n_h2d = max(5, min(args.steps, 20))
+    net.forward(**inputs)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(n_h2d):
+        net.forward(**inputs)
+    torch.cuda.synchronize()
+    el_h2d = time.perf_counter() - t0
+    with_h2d = {"value_with_h2d": round(args.batch * n_h2d / el_h2d, 1),
+                "ms_per_step_with_h2d": round(1e3 * el_h2d / n_h2d, 3), "steps_with_h2d": n_h2d,
+                "h2d_bytes_per_step": int(sum(v.nbytes for v in inputs.values()))}
+
     # The same net with every convolution on the direct path (no Winograd), shorter: what
     # the implicit-GEMM kernel alone gives, for comparison with the figures above.
     direct = None
@@ -230,16 +244,18 @@ def main():
            "roofline": roofline, "cpu_baseline": cpu,
            "conv_mfma_util_pct": mfma_util, "conv_mfma_util_source": mfma_note,
            "direct_path_only": direct}
+    out.update(with_h2d)
     out.update(tails)
     print(json.dumps(out))
 
 
 def detection_tails(mc, craft, zoo, LIB):
-    """NMS / Proposal / DetectionOutput device time at the sizes of configurations 4 and 3.
-    The nets run once to produce the tails' real inputs (RPN scores and deltas; SSD
-    locations, softmaxed confidences, priors); the tails are then called alone through the
-    kernel-level C ABI, 5 warm-up + 30 calls, each call timed with HIP events on its
-    stream; medians in microseconds."""
+    """NMS / Proposal / DetectionOutput device time at the sizes of configurations 4 and 3,
+    medians in microseconds.  Proposal: the layer inside the RPN net, through its stage hook.
+    DetectionOutput: the SSD net runs once for locations and priors, the confidences are the
+    softmax of N(0, sigma = 2) logits as configuration 3 states (the net's own confidences
+    give a second figure); the tail is called alone through the kernel-level C ABI, 5 warm-up
+    + 30 calls, each call between HIP events on its stream."""
     import statistics
     import numpy as np
     import torch
@@ -253,48 +269,42 @@ def detection_tails(mc, craft, zoo, LIB):
     spec, inputs = zoo.rpn_spec(seed=0)
     net = mc.Net.from_buffers(craft.to_prototxt(spec, "rpn"))
     craft.load_weights(net, spec)
-    for m in ("rpn_cls_prob_reshape", "rpn_bbox_pred"):
-        net.mark_output(m)
+    net.mark_output("rpn_bbox_pred")
     net.forward(**inputs)
-    prob = net.get_blob("rpn_cls_prob_reshape").data.copy()
-    bbox = net.get_blob("rpn_bbox_pred").data.copy()
-    del net
+    bbox = net.get_blob("rpn_bbox_pred").data
     pp = spec[-1]["proposal_param"]
     pre, post, thr = pp.get("pre_nms_topn", 6000), pp.get("post_nms_topn", 300), pp.get("nms_thresh", 0.7)
     A, H, W = bbox.shape[1] // 4, bbox.shape[2], bbox.shape[3]
-    import oracle
-    sd, bd, idv, ad = dev(prob), dev(bbox), dev(inputs["im_info"]), dev(oracle.generate_anchors())
-    sz = ctypes.c_size_t()
-    K.check_mc(LIB.mcProposalWorkspaceSize(A * H * W, pre, post, ctypes.byref(sz)))
-    ws = torch.empty(sz.value, dtype=torch.uint8, device="cuda")
-    rois = torch.empty((post, 5), device="cuda")
-    cnt = torch.zeros(2, dtype=torch.int32, device="cuda")
-
-    def proposal():
-        K.check_mc(LIB.mcProposal(P(sd.data_ptr()), P(bd.data_ptr()), P(idv.data_ptr()), P(ad.data_ptr()), A, H, W, 16,
-                                  ctypes.c_float(16), pre, post, ctypes.c_float(thr), P(ws.data_ptr()), sz.value,
-                                  P(rois.data_ptr()), None, P(cnt.data_ptr()), P(cnt.data_ptr() + 4), P(stream)))
-
+    # The Proposal layer of the net itself is what is timed (its own anchor table, its own
+    # sequence of calls: the head of the score table first, the counters read back, the
+    # full-size path only if the head did not settle the result).  The stage hook records
+    # HIP events inside every call the layer makes.
     for _ in range(5):
-        proposal()
-    torch.cuda.synchronize()
-    stages = []
+        net.forward()
+    stages, calls_seen = [], set()
     for _ in range(30):
         LIB.mcProposalTimingEnable(1)
-        proposal()
+        net.forward()
         LIB.mcProposalTimingEnable(0)
         ms, calls = (ctypes.c_double * 4)(), ctypes.c_long()
         K.check_mc(LIB.mcProposalTimingCollect(ms, ctypes.byref(calls)))
         stages.append([1e3 * v for v in ms])
+        calls_seen.add(calls.value)
+    kept = int(net.get_blob(spec[-1]["top"][0]).data.shape[0])
+    del net
     med = [statistics.median(s[k] for s in stages) for k in range(4)]
-    out["nms_us"] = round(med[2], 1)
+    out["nms_us"] = round(med[1] + med[3], 1)
     out["proposal_us"] = round(statistics.median(sum(s) for s in stages), 1)
     out["proposal_detail"] = {
-        "workload": "config 4: %d anchors -> best %d -> NMS %.1f -> <= %d rois (kept %d, equal scores in the "
-                    "best %d: %s)" % (A * H * W, pre, thr, post, int(cnt[0]), pre, "yes" if int(cnt[1]) else "no"),
-        "decode_sort_us": round(med[0], 1), "tie_order_replay_us": round(med[1], 1),
-        "nms_mask_scan_us": round(med[2], 1), "gather_us": round(med[3], 1),
-        "method": "mcProposal alone on the net's own scores, HIP events between stages, median of 30 calls"}
+        "workload": "config 4: %d anchors -> best %d -> NMS %.1f -> <= %d rois (kept %d; the layer made %s "
+                    "call(s) per forward: 1 = the head of the table settled the result, 2 = the full-size path "
+                    "ran too)" % (A * H * W, pre, thr, post, kept, "/".join(str(c) for c in sorted(calls_seen))),
+        "decode_head_order_us": round(med[0], 1), "head_nms_check_gather_us": round(med[1], 1),
+        "full_sort_replay_us": round(med[2], 1), "full_nms_gather_us": round(med[3], 1),
+        "nms_us_is": "head_nms_check_gather_us + full_nms_gather_us",
+        "method": "the net's Proposal layer on the net's own scores, HIP events between the stages of each "
+                  "call the layer makes (device time; the read-back between the calls is not in it), median of "
+                  "30 forwards"}
 
     # configuration 3: SSD300 b8, 8732 priors x 21 classes, top_k 400, NMS 0.45, keep 200
     spec, inputs = zoo.ssd300_spec(batch=8, seed=0)
@@ -309,35 +319,49 @@ def detection_tails(mc, craft, zoo, LIB):
     num, Pn, C = loc.shape[0], prior.shape[2] // 4, dp["num_classes"]
     nmsp = dp["nms_param"]
     code = {"CORNER": 1, "CENTER_SIZE": 2, "CORNER_SIZE": 3}[str(dp.get("code_type", "CORNER"))]
+    sz = ctypes.c_size_t()
+    cnt = torch.zeros(2, dtype=torch.int32, device="cuda")
     K.check_mc(LIB.mcDetectionOutputWorkspaceSize(num, Pn, C, 1, nmsp["top_k"], ctypes.byref(sz)))
     max_rows = LIB.mcDetectionOutputMaxRows(num, Pn, C, nmsp["top_k"], dp["keep_top_k"])
     ws = torch.empty(sz.value, dtype=torch.uint8, device="cuda")
     rows = torch.empty((max_rows, 7), device="cuda")
 
+    thr_conf = dp.get("confidence_threshold", -3.4028234663852886e38)
+
     def detect():
         K.check_mc(LIB.mcDetectionOutput(
             P(loc.data_ptr()), P(conf.data_ptr()), P(prior.data_ptr()), num, Pn, C, 1, dp.get("background_label_id", 0),
-            code, 0, dp["keep_top_k"], ctypes.c_float(dp.get("confidence_threshold", -3.4028234663852886e38)),
+            code, 0, dp["keep_top_k"], ctypes.c_float(thr_conf),
             ctypes.c_float(nmsp["nms_threshold"]), ctypes.c_float(nmsp.get("eta", 1.0)), nmsp["top_k"],
             P(ws.data_ptr()), sz.value, P(rows.data_ptr()), max_rows, P(cnt.data_ptr()), P(cnt.data_ptr() + 4),
             P(stream)))
 
-    for _ in range(5):
-        detect()
-    torch.cuda.synchronize()
-    spans = []
-    for _ in range(30):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        detect()
-        e1.record()
-        spans.append((e0, e1))
-    torch.cuda.synchronize()
-    out["detection_output_us"] = round(1e3 * statistics.median(a.elapsed_time(b) for a, b in spans), 1)
+    def timed_detect():
+        for _ in range(5):
+            detect()
+        torch.cuda.synchronize()
+        spans = []
+        for _ in range(30):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            detect()
+            e1.record()
+            spans.append((e0, e1))
+        torch.cuda.synchronize()
+        return round(1e3 * statistics.median(a.elapsed_time(b) for a, b in spans), 1), int(cnt[0])
+
+    own_us, own_rows = timed_detect()
+    # configuration 3's confidences: logits ~ N(0, sigma = 2) per (image, prior, class), softmax over classes
+    logits = torch.randn((num, Pn, C), generator=torch.Generator().manual_seed(3)) * 2.0
+    conf = torch.softmax(logits, dim=2).reshape(num, Pn * C).contiguous().cuda()
+    us, rows_n = timed_detect()
+    out["detection_output_us"] = us
     out["detection_output_detail"] = {
-        "workload": "config 3: %d images x %d priors x %d classes, top_k %d, NMS %.2f, keep %d (rows %d)"
-                    % (num, Pn, C, nmsp["top_k"], nmsp["nms_threshold"], dp["keep_top_k"], int(cnt[0])),
-        "method": "mcDetectionOutput alone on the net's own tail inputs, HIP events on the launch stream, "
+        "workload": "config 3: %d images x %d priors x %d classes, confidences = softmax of N(0, sigma=2) logits, "
+                    "confidence_threshold %.2f, top_k %d, NMS %.2f, keep %d (rows %d)"
+                    % (num, Pn, C, thr_conf, nmsp["top_k"], nmsp["nms_threshold"], dp["keep_top_k"], rows_n),
+        "on_the_nets_own_confidences_us": own_us, "on_the_nets_own_confidences_rows": own_rows,
+        "method": "mcDetectionOutput alone (locations and priors from the net), HIP events on the launch stream, "
                   "median of 30 calls"}
     return out
 
@@ -361,9 +385,9 @@ def configs_report(path, mc, craft, zoo, LIB):
              # not a BASELINE configuration: the depthwise-separable graph of the reference's ssd example
              ("+  MobileNet-SSD b32", zoo.mobilenet_ssd_spec(batch=32, seed=0), ("detection_out",), 32,
               zoo.mobilenet_ssd_spec(batch=2, seed=0), 2)]
-    lines = ["%-30s %10s %10s %12s %10s %8s %12s %12s  %s"
-             % ("configuration", "ms/forward", "GFLOP", "contr. ms", "TFLOP/s", "of peak", "GPU img/s",
-                "CPU img/s", "tail layers (us, device time)")]
+    lines = ["%-30s %10s %10s %12s %12s %10s %8s %12s %12s  %s"
+             % ("configuration", "ms/forward", "GFLOP", "contr. ms", "dir-eq TF/s", "issued TF/s", "of peak",
+                "GPU img/s", "CPU img/s", "tail layers (us, device time)")]
     for name, (spec, inputs), tails, batch, (cspec, cinputs), cbatch in cases:
         net = mc.Net.from_buffers(craft.to_prototxt(spec, "net"))
         craft.load_weights(net, spec)
@@ -379,7 +403,9 @@ def configs_report(path, mc, craft, zoo, LIB):
         for _ in range(reps):
             net.forward()
         tot_ms, launches, fl = ctypes.c_double(), ctypes.c_long(), ctypes.c_double()
-        LIB.mcConvTimingCollect(ctypes.byref(tot_ms), ctypes.byref(launches), ctypes.byref(fl))
+        issued, wino = ctypes.c_double(), ctypes.c_long()
+        LIB.mcConvTimingCollectDetail(ctypes.byref(tot_ms), ctypes.byref(launches), ctypes.byref(fl),
+                                      ctypes.byref(issued), ctypes.byref(wino))
         LIB.mcConvTimingEnable(0)
         tail_txt = ""
         if tails:
@@ -403,16 +429,20 @@ def configs_report(path, mc, craft, zoo, LIB):
                                  for t, v in last.items())
         cms = tot_ms.value / reps
         tf_s = fl.value / (tot_ms.value * 1e-3) / 1e12 if tot_ms.value else 0.0
+        is_s = issued.value / (tot_ms.value * 1e-3) / 1e12 if tot_ms.value else 0.0
         # CPU path (oracle restatement of the reference, OpenBLAS sgemm, all host cores): one
         # pass at the reduced batch
         last = cspec[-1]["top"][0]
         t0 = time.perf_counter()
         netrun.oracle_forward(cspec, cinputs, keep={last})
         cpu_rate = cbatch / (time.perf_counter() - t0)
-        lines.append("%-30s %10.3f %10.2f %12.3f %10.1f %7.1f%% %12.1f %12.2f  %s"
-                     % (name, ms, fl.value / reps / 1e9, cms, tf_s, 100 * tf_s / FP32_MFMA_PEAK_TFLOPS,
+        lines.append("%-30s %10.3f %10.2f %12.3f %12.1f %10.1f %7.1f%% %12.1f %12.2f  %s"
+                     % (name, ms, fl.value / reps / 1e9, cms, tf_s, is_s, 100 * is_s / FP32_MFMA_PEAK_TFLOPS,
                         batch / (ms * 1e-3), cpu_rate, tail_txt))
         del net
+    lines.append("dir-eq TF/s: the contractions' direct-sum FLOPs over the device time of their launches (a 3x3 layer on "
+                 "the Winograd path counts with its direct-sum FLOPs, so this rate can pass the matrix peak); issued "
+                 "TF/s / of peak: what the matrix pipe was handed in the same time, against 157.3 TFLOP/s.")
     lines.append("CPU column: one pass of the oracle (reference algorithm: per-image im2col + OpenBLAS sgemm, "
                  "unfused layers) on %d host threads at batch 1/4/1/1/8/2." % oracle.openblas_threads())
     with open(path, "w") as f:
@@ -462,7 +492,7 @@ def layer_scaling(path):
             del x, y, w, plan
         lines.append("%-22s" % ("%d->%d %dx%d @%d%s" % (cin, cout, k, k, h, " W" if mode else "")) + "".join(cells))
     lines.append("cells: time per launch (10 back-to-back launches between two events) and TFLOP/s; W = the layer as "
-                 "F(2x2,3x3) Winograd (three launches, TFLOP/s in the direct sum's FLOPs)")
+                 "F(2x2,3x3) Winograd (one fused launch; TFLOP/s in the direct sum's FLOPs, which can exceed the matrix peak)")
     with open(path, "w") as f:
         f.write("\n".join(lines) + "\n")
 
@@ -470,9 +500,14 @@ def layer_scaling(path):
 def layer_roofline(path, batch):
     """Every distinct convolution of ResNet-50 v1 alone (ReLU epilogue, no residual), one
     launch at a time through the kernel-level C ABI: which roofline binds it and how close
-    the launch comes.  Bytes = bottom + top + filter, each once."""
+    the launch comes.  Bytes = bottom + top + filter, each once.  Two rates per layer: the
+    direct sum's FLOPs over the time (what the layer is worth; a Winograd launch can exceed
+    the matrix peak on this scale, so no fraction is printed for it) and the FLOPs the matrix
+    pipe was handed (padding of tiles included, 2.25 times fewer products on the Winograd
+    path) with their share of the fp32 peak."""
     import torch
     from minicaffe import kernels as K
+    from minicaffe.base import LIB
     # cin, height = width, cout, kernel, stride, pad, number of layers of this shape
     shapes = [(3, 224, 64, 7, 2, 3, 1), (64, 56, 256, 1, 1, 0, 4), (64, 56, 64, 1, 1, 0, 1), (64, 56, 64, 3, 1, 1, 3),
               (256, 56, 64, 1, 1, 0, 2), (256, 56, 512, 1, 2, 0, 1), (256, 56, 128, 1, 2, 0, 1), (128, 28, 128, 3, 1, 1, 4),
@@ -481,9 +516,12 @@ def layer_roofline(path, batch):
               (1024, 14, 2048, 1, 2, 0, 1), (1024, 14, 512, 1, 2, 0, 1), (512, 7, 512, 3, 1, 1, 3),
               (512, 7, 2048, 1, 1, 0, 3), (2048, 7, 512, 1, 1, 0, 2)]
     stream = torch.cuda.current_stream().cuda_stream
-    lines = ["%-24s %3s %8s %9s %8s %6s %9s %9s %9s %7s" % ("convolution (batch %d)" % batch, "x", "GFLOP", "MB", "FLOP/B",
-                                                           "bound", "roof us", "meas. us", "TFLOP/s", "of roof")]
-    sum_roof = sum_meas = 0.0
+    lines = ["%-24s %3s %8s %9s %8s %6s %9s %9s %11s %9s %8s" % (
+        "convolution (batch %d)" % batch, "x", "GFLOP", "MB", "FLOP/B", "bound", "roof us", "meas. us",
+        "direct-eq.", "issued", "issued")]
+    lines.append("%-24s %3s %8s %9s %8s %6s %9s %9s %11s %9s %8s" % (
+        "", "", "", "", "", "", "", "", "TFLOP/s", "TFLOP/s", "of peak"))
+    sum_roof = sum_meas = sum_issued = 0.0
     for cin, h, cout, k, s_, p_, cnt in shapes:
         plan = K.ConvPlan(K.conv_geom(cin, h, h, cout, k, s_, p_))
         ho, wo = plan.output_shape()
@@ -510,17 +548,29 @@ def layer_roofline(path, batch):
             e1.record()
             torch.cuda.synchronize()
             us = e0.elapsed_time(e1) / reps * 1e3
+            # what the launch hands the matrix pipe: from the library's own count
+            LIB.mcConvTimingEnable(1)
+            plan.forward(batch, x.data_ptr(), y.data_ptr(), activation=K.ACT_RELU, stream=stream)
+            tot_ms, launches, fl_c = ctypes.c_double(), ctypes.c_long(), ctypes.c_double()
+            issued, wino = ctypes.c_double(), ctypes.c_long()
+            LIB.mcConvTimingCollectDetail(ctypes.byref(tot_ms), ctypes.byref(launches), ctypes.byref(fl_c),
+                                          ctypes.byref(issued), ctypes.byref(wino))
+            LIB.mcConvTimingEnable(0)
             if mode == -1:
                 sum_roof += roof * cnt
                 sum_meas += us * cnt
-            lines.append("%-24s %3d %8.2f %9.1f %8.1f %6s %9.1f %9.1f %9.1f %6.1f%%  %s" % (
+                sum_issued += issued.value * cnt
+            lines.append("%-24s %3d %8.2f %9.1f %8.1f %6s %9.1f %9.1f %11.1f %9.1f %7.1f%%  %s" % (
                 "%d->%d %dx%d/%d @%d" % (cin, cout, k, k, s_, h), cnt, fl / 1e9, nbytes / 1e6, fl / nbytes,
-                "mfma" if t_mfma >= t_hbm else "hbm", roof, us, fl / us / 1e6, 100 * roof / us,
-                "" if not winograd else ("Winograd F(2x2,3x3): transforms + 16 products" if mode == -1
+                "mfma" if t_mfma >= t_hbm else "hbm", roof, us, fl / us / 1e6, issued.value / us / 1e6,
+                100 * issued.value / us / 1e6 / FP32_MFMA_PEAK_TFLOPS,
+                "" if not winograd else ("Winograd F(2x2,3x3), one fused launch" if mode == -1
                                          else "(same layer pinned to the direct path; not in the total)")))
         del x, y, w, plan
-    lines.append("all 53 convolutions: roofline %.0f us, measured %.0f us = %.1f%% of the per-layer roofline"
-                 % (sum_roof, sum_meas, 100 * sum_roof / sum_meas))
+    lines.append("all 53 convolutions: direct-sum roofline %.0f us, measured %.0f us (direct-sum equivalent %.1f%% of the "
+                 "per-layer roofline); issued to the matrix pipe: %.1f%% of the fp32 peak over the same time"
+                 % (sum_roof, sum_meas, 100 * sum_roof / sum_meas,
+                    100 * sum_issued / sum_meas / 1e6 / FP32_MFMA_PEAK_TFLOPS))
     lines.append("roof us = max(FLOP / 157.3 TFLOP/s, bytes / 8 TB/s) with the FLOPs and bytes of the direct sum; 20 "
                  "back-to-back calls between two events.")
     with open(path, "w") as f:
