@@ -708,6 +708,13 @@ def bandwidth_report(path):
         timed("depthwise 3x3/%d + ReLU, 32x%dx%dx%d (MobileNet)" % (s_, cin, h, h),
               4 * 32 * cin * (h * h + ho * wo), make)
         del plan
+    # the plain copy at the sizes of the small launches above: what a launch of that size can reach at all
+    for label, nel in (("the 19x19 depthwise launch", 32 * 512 * 19 * 19), ("Normalize", 8 * 512 * 38 * 38),
+                       ("LRN", 64 * 96 * 55 * 55)):
+        def make(nel=nel):
+            a, y = dev(nel), dev(nel)
+            return (lambda: LIB.mcCopy2D(P(a.data_ptr()), nel, P(y.data_ptr()), nel, nel, 1, P(stream))), (a, y)
+        timed("copy of the size of %s" % label, 4 * 2 * nel, make)
     head = ["%-58s %12s %8s %12s %13s %8s %14s" % ("kernel, shape", "alg. bytes", "operands", "cold", "achieved",
                                                   "of 8 TB/s", "one launch")]
     tail = ["cold: 40 back-to-back launches between two HIP events, rotating over `operands` sets (more than 512 MB",
