@@ -381,6 +381,12 @@ int mcDetectionOutput(const float* loc, const float* conf, const float* prior, i
                       float confidence_threshold, float nms_threshold, float eta, int top_k,
                       void* workspace, size_t workspace_bytes, float* out_rows, int max_rows,
                       int* num_rows, int* cut_tie_flag, void* stream);
+/* Test knob (process-wide): with a constant threshold (eta 1), at most 512 candidates
+ * per class and at most 12 288 priors, the per-class work runs as three launches
+ * (candidate selection, pairwise overlap bits spread over the whole chip, greedy scan);
+ * 0 keeps such inputs on the one-launch-per-class kernel that every other input takes,
+ * 1 restores the automatic choice.  Results are the same. */
+int mcDetectionOutputSplit(int on);
 
 /* ROIPoolingLayer::Forward (roi_pooling_layer.cpp:37-110; .cu:13-81): max pooling of
  * bottom [num, channels, height, width] over num_rois regions, rois rows of

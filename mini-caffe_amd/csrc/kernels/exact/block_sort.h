@@ -16,8 +16,8 @@ namespace mchip {
 constexpr int kSortThreads = 512;
 
 // Monotone map float -> uint32 such that a > b  <=>  key(a) < key(b); -0 == +0.
-__device__ __forceinline__ uint32_t desc_key(float f) {
-  uint32_t u = __float_as_uint(f);
+__host__ __device__ __forceinline__ uint32_t desc_key(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
   if (u == 0x80000000u) u = 0u;
   const uint32_t asc = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
   return ~asc;
@@ -170,10 +170,11 @@ __device__ inline void block_sort_desc_lds(uint32_t* keys, VT* vals, int n, Bloc
 // For want <= kSortThreads (the candidates of a greedy pass that looks at a few hundred
 // entries of a table of thousands).  Every thread holds PER keys in registers, entry
 // tid + j * kSortThreads in rk[j]; the all-ones key marks "no entry".
-//   1. First cut: every thread has a smallest key, and the largest of those has at least
-//      one key per thread at or below it, kSortThreads >= want in all; the threads hold
-//      strided samples of the table, so usually a few thousand keys pass: the candidates
-//      (kSelectCandPer per thread at most, else the call fails and the caller sorts).
+//   1. First cut: every thread has a smallest key; in each wavefront the ceil(want / 8)-th
+//      smallest of those has that many keys at or below it, so the largest of the eight
+//      wavefronts' values has at least `want`.  The threads hold strided samples of the
+//      table, so usually a thousand or two keys pass: the candidates (kSelectCandPer per
+//      thread at most, else the call fails and the caller sorts).
 //   2. tau = the want-th smallest candidate by bisection on the key bits, two bits per
 //      round from the top (three trial values, one count over the workgroup each: ballots
 //      and scalar population counts within a wavefront, the wavefronts' counts through
@@ -232,9 +233,20 @@ __device__ __forceinline__ int block_select_smallest(const uint32_t (&rk)[PER], 
   uint32_t lowest = 0xffffffffu;
 #pragma unroll
   for (int j = 0; j < PER; ++j) lowest = min(lowest, rk[j]);
-  uint32_t cut = lowest;  // (a thread without entries holds all ones: every entry passes)
+  // the wavefront's share of the cut: the ceil(want / 8)-th smallest of its 64 thread
+  // minima (eight wavefronts: at least `want` entries lie at or below the largest share)
+  uint32_t cut = lowest;  // (a thread without entries holds all ones)
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) cut = max(cut, static_cast<uint32_t>(__shfl_xor(cut, o, 64)));
+  for (int k = 2; k <= 64; k <<= 1) {
+#pragma unroll
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      const uint32_t other = static_cast<uint32_t>(__shfl_xor(cut, j, 64));
+      const bool up = (lane & k) == 0 || k == 64, lower = (lane & j) == 0;
+      cut = (lower == up) ? min(cut, other) : max(cut, other);
+    }
+  }
+  static_assert(kSortThreads / 64 == 8, "eight wavefronts share the cut");
+  cut = static_cast<uint32_t>(__shfl(cut, (want + 7) / 8 - 1, 64));
   __syncthreads();  // (the caller may still be reading what `s` overlays)
   if (lane == 0) s->red[wave] = cut;
   __syncthreads();

@@ -35,11 +35,23 @@ __device__ __forceinline__ float dbox_size(float xmin, float ymin, float xmax, f
 __global__ __launch_bounds__(256) void det_decode_kernel(
     const float* __restrict__ loc, const float* __restrict__ prior, int num, int P,
     int loc_classes, int code_type, int var_in_target, DBox* __restrict__ out,
-    int* __restrict__ cut_tie_flag) {
+    int* __restrict__ cut_tie_flag, const float* __restrict__ conf, int C,
+    uint32_t* __restrict__ keys_by_class) {
   const long total = (long)num * loc_classes * P;
   const long t = blockIdx.x * 256L + threadIdx.x;
   if (t == 0 && cut_tie_flag) *cut_tie_flag = 0;  // raised by det_select_kernel, two launches on
-  if (t >= total) return;
+  if (t >= total) {
+    // The threads behind the boxes (keys_by_class != null): one per (image, prior) turns the
+    // prior's C confidences into sort keys and stores them class by class, [image][class]
+    // [prior], so that the launch that orders a class reads its keys front to back.
+    const long t2 = t - total;
+    if (keys_by_class == nullptr || t2 >= (long)num * P) return;
+    const int p = static_cast<int>(t2 % P);
+    const int i = static_cast<int>(t2 / P);
+    const float* cp = conf + ((long)i * P + p) * C;
+    for (int c = 0; c < C; ++c) keys_by_class[((long)i * C + c) * P + p] = desc_key(cp[c]);
+    return;
+  }
   const int p = static_cast<int>(t % P);
   const int c = static_cast<int>((t / P) % loc_classes);
   const int i = static_cast<int>(t / ((long)P * loc_classes));
@@ -127,6 +139,31 @@ __device__ __forceinline__ float jaccard(const DBox& a, const DBox& b) {
 __device__ __forceinline__ bool overlap_rejects(const DBox& a, const DBox& b, float thr) {
   const float iw = fminf(a.xmax, b.xmax) - fmaxf(a.xmin, b.xmin);
   const float ih = fminf(a.ymax, b.ymax) - fmaxf(a.ymin, b.ymin);
+  const float isz = iw * ih;
+  const float q = isz / (a.size + b.size - isz);
+  const float overlap = (iw > 0.f && ih > 0.f) ? q : 0.f;
+  return !(overlap <= thr);
+}
+
+// The same for the many-pairs kernel, whose second box `b` is the same in every lane (it
+// sits in scalar registers).  fmaxf / fminf first quiet a possible signalling NaN in each
+// operand the compiler cannot prove clean, one more vector instruction per coordinate of
+// `b` and pair; v_max_f32 / v_min_f32 written out take the operands as they are.  For
+// ordered operands both give the larger / smaller one; with a NaN coordinate (a NaN location
+// prediction) the reference's overlap is not defined either.
+__device__ __forceinline__ float vmax_vs(float v, float s) {
+  float r;
+  asm("v_max_f32 %0, %2, %1" : "=v"(r) : "v"(v), "s"(s));
+  return r;
+}
+__device__ __forceinline__ float vmin_vs(float v, float s) {
+  float r;
+  asm("v_min_f32 %0, %2, %1" : "=v"(r) : "v"(v), "s"(s));
+  return r;
+}
+__device__ __forceinline__ bool overlap_rejects_uniform_b(const DBox& a, const DBox& b, float thr) {
+  const float iw = vmin_vs(a.xmax, b.xmax) - vmax_vs(a.xmin, b.xmin);
+  const float ih = vmin_vs(a.ymax, b.ymax) - vmax_vs(a.ymin, b.ymin);
   const float isz = iw * ih;
   const float q = isz / (a.size + b.size - isz);
   const float overlap = (iw > 0.f && ih > 0.f) ? q : 0.f;
@@ -449,6 +486,223 @@ __global__ __launch_bounds__(kSortThreads) void det_class_nms_lds_kernel(
                                   &kept_count[seg]);
 }
 
+// ---- constant threshold, top_k <= 512, P <= kDetLdsMax: the per-class work in three launches
+//
+// det_candidates_kernel (one workgroup per image and class) picks and orders the class's
+// top_k candidates; det_overlap_kernel forms the candidates' pairwise "rejects" bits with
+// one wavefront per 64 x 64 block of pairs, so the quadratic part of the work spreads
+// over the whole chip instead of one CU per class; det_scan_kernel (one wavefront per
+// image and class) makes the greedy decisions from those bits alone.
+constexpr int kDetSplitTopK = kSortThreads;          // candidates per class at most
+constexpr int kDetSplitWords = kDetSplitTopK / 64;   // 64-candidate blocks per class at most
+
+// The candidates by a sort of the whole key table in LDS, for tables the selection gives up
+// on.  Kept out of line: inlined, its register arrays spill the selection's.
+__device__ __noinline__ int det_candidates_by_sort(const uint32_t* __restrict__ keys, int P, uint32_t key_thr,
+                                                   int want, uint32_t* s_key, unsigned short* s_val,
+                                                   BlockSortLds16* lds, int* s_valid, uint32_t* key_out,
+                                                   uint32_t* idx_out) {
+  const int tid = threadIdx.x;
+  if (tid == 0) *s_valid = 0;
+  __syncthreads();
+  int valid = 0;
+  for (int p = tid; p < P; p += kSortThreads) {
+    const uint32_t k = keys[p];
+    const bool ok = k < key_thr;
+    valid += ok;
+    s_key[p] = ok ? k : 0xffffffffu;  // below-threshold scores sort last
+    s_val[p] = static_cast<unsigned short>(p);
+  }
+  if (valid) atomicAdd(s_valid, valid);
+  __syncthreads();
+  // squeeze the scores above the threshold to the front in prior order and sort those
+  const int nvalid = *s_valid;
+  if (nvalid < P) {
+    const int per = (P + kSortThreads - 1) / kSortThreads;
+    const int begin = min(tid * per, P), end = min(begin + per, P);
+    uint32_t run[kDetLdsPer];
+    uint32_t mine = 0;
+#pragma unroll
+    for (int j = 0; j < kDetLdsPer; ++j) {
+      run[j] = 0xffffffffu;
+      if (begin + j < end) run[j] = s_key[begin + j];
+      mine += run[j] != 0xffffffffu;
+    }
+    uint32_t pos = block_exclusive_scan(mine, lds->wave_sum);  // synchronises before returning
+#pragma unroll
+    for (int j = 0; j < kDetLdsPer; ++j)
+      if (run[j] != 0xffffffffu) {
+        s_key[pos] = run[j];
+        s_val[pos] = static_cast<unsigned short>(begin + j);
+        ++pos;
+      }
+    __syncthreads();
+  }
+  block_sort_desc_lds<kDetLdsPer, unsigned short>(s_key, s_val, nvalid, lds);
+  const int ncand = min(nvalid, want);
+  if (tid < ncand) {
+    *key_out = s_key[tid];
+    *idx_out = s_val[tid];
+  }
+  return ncand;
+}
+
+// Candidates of one (image, class): the top_k best scores above the threshold in (score
+// descending, prior ascending) order, what GetMaxScoreIndex leaves (bbox_util.cpp:523-540).
+// The keys come class by class from det_decode_kernel; a score is above the threshold
+// exactly if its key is below the threshold's key.  First the selection that does not sort
+// the table; if it gives up (crowds of equal scores), the sort in LDS.
+__global__ __launch_bounds__(kSortThreads) void det_candidates_kernel(
+    const uint32_t* __restrict__ keys_by_class, const DBox* __restrict__ boxes, int P, int C,
+    int loc_classes, int background, uint32_t key_thr, int top_k, int cand_stride,
+    uint32_t* __restrict__ cand_key, int* __restrict__ cand_idx, DBox* __restrict__ cand_box,
+    int* __restrict__ ncand_out) {
+  __shared__ BlockSortLds16 lds;
+  __shared__ __attribute__((aligned(16))) uint32_t s_key[kDetLdsMax];
+  __shared__ unsigned short s_val[kDetLdsMax];
+  __shared__ int s_valid;
+  static_assert(sizeof(BlockSelectLds) <= sizeof(uint32_t) * kDetLdsMax, "the selection's scratch overlays the key table");
+  const int c = blockIdx.x, i = blockIdx.y;
+  const int seg = i * C + c;
+  const int tid = threadIdx.x;
+  if (c == background) {
+    if (tid == 0) ncand_out[seg] = 0;
+    return;
+  }
+  const uint32_t* __restrict__ keys = keys_by_class + (size_t)seg * P;
+  uint32_t rk[kDetLdsPer];
+#pragma unroll
+  for (int j = 0; j < kDetLdsPer; ++j) {
+    const int p = tid + j * kSortThreads;
+    rk[j] = p < P ? keys[p] : 0xffffffffu;
+  }
+  const int want = min(top_k, P);
+  uint32_t key = 0xffffffffu, idx = 0;
+  int ncand;
+  const int m = block_select_smallest<kDetLdsPer>(rk, want, reinterpret_cast<BlockSelectLds*>(s_key), &key, &idx);
+  if (m > 0) {  // uniform
+    ncand = __syncthreads_count(tid < want && key < key_thr);
+  } else {
+    ncand = det_candidates_by_sort(keys, P, key_thr, want, s_key, s_val, &lds, &s_valid, &key, &idx);
+  }
+  if (tid < ncand) {
+    const DBox* cls_boxes = boxes + ((size_t)i * loc_classes + (loc_classes == 1 ? 0 : c)) * P;
+    const size_t at = (size_t)seg * cand_stride + tid;
+    cand_key[at] = key;
+    cand_idx[at] = static_cast<int>(idx);
+    cand_box[at] = cls_boxes[idx];
+  }
+  if (tid == 0) ncand_out[seg] = ncand;
+}
+
+// One wavefront per pair of 64-candidate blocks (bi <= bj) of one (image, class): lane l
+// holds candidate 64 bi + l (the earlier box of a pair) and candidate 64 bj + l; the later
+// boxes go round as scalar broadcasts, and a ballot over the earlier ones is the word the
+// scan needs: col_rejects[candidate 64 bj + k][bi] = the candidates of block bi that
+// candidate 64 bj + k is rejected against (JaccardOverlap is symmetric in its two boxes:
+// bbox_util.cpp:184-204).
+constexpr int kOverlapWaves = 4;
+__global__ __launch_bounds__(64 * kOverlapWaves) void det_overlap_kernel(
+    const DBox* __restrict__ cand_box, const int* __restrict__ ncand_in, int cand_stride, float nms_thr,
+    unsigned long long* __restrict__ col_rejects) {
+  const int seg = blockIdx.y;
+  const int lane = threadIdx.x & 63;
+  // pair index bj (bj + 1) / 2 + bi (the same in every lane: said so, for scalar addressing)
+  const int q = blockIdx.x * kOverlapWaves + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  int bj = 0;
+  while ((bj + 1) * (bj + 2) / 2 <= q) ++bj;
+  const int bi = q - bj * (bj + 1) / 2;
+  const int ncand = ncand_in[seg];
+  if (64 * bj >= ncand) return;  // (uniform over the wavefront; bi <= bj)
+  const DBox* __restrict__ cb = cand_box + (size_t)seg * cand_stride;
+  const int r = 64 * bi + lane, k0 = 64 * bj + lane;
+  const bool row_in = r < ncand;
+  const DBox rb = cb[min(r, ncand - 1)];
+  // The later box of a pair is the same for the whole wavefront: read through the scalar
+  // unit (a uniform address in memory nobody writes during the launch), so the vector unit
+  // only does the arithmetic.  Columns past the last candidate repeat it; their words are
+  // never read.
+  unsigned long long word = 0;
+#pragma unroll 8
+  for (int k = 0; k < 64; ++k) {
+    const DBox kb = cb[min(64 * bj + k, ncand - 1)];
+    const unsigned long long bits =
+        __ballot(static_cast<int>(row_in) & static_cast<int>(overlap_rejects_uniform_b(rb, kb, nms_thr)));
+    word = lane == k ? bits : word;
+  }
+  col_rejects[((size_t)seg * cand_stride + k0) * kDetSplitWords + bi] = word;  // (k0 < 64 words <= cand_stride)
+}
+
+// The greedy pass of ApplyNMSFast for a constant threshold (bbox_util.cpp:681-716) from the
+// bits alone, one wavefront per (image, class), a block of 64 candidates at a time: a
+// candidate is out if a kept candidate of an earlier block rejects it (its words of the
+// earlier blocks against those blocks' kept bits); the block's own candidates settle in
+// rounds as in greedy_nms_blocks.  Every word a lane will need is requested before the
+// first decision, so the pass waits for memory once.
+__global__ __launch_bounds__(64) void det_scan_kernel(
+    const unsigned long long* __restrict__ col_rejects, const int* __restrict__ ncand_in,
+    const int* __restrict__ cand_idx, const uint32_t* __restrict__ cand_key,
+    const DBox* __restrict__ cand_box, int cand_stride, int max_cand, int* __restrict__ kept_idx,
+    uint32_t* __restrict__ kept_key, DBox* __restrict__ kept_box, int* __restrict__ kept_count) {
+  const int seg = blockIdx.x, lane = threadIdx.x;
+  const int ncand = ncand_in[seg];
+  const int words = (ncand + 63) >> 6;
+  unsigned long long w[kDetSplitWords][kDetSplitWords];
+  int prior[kDetSplitWords];
+  uint32_t ckey[kDetSplitWords];
+  DBox cbox[kDetSplitWords];
+#pragma unroll
+  for (int b = 0; b < kDetSplitWords; ++b) {
+    if (b < words) {  // uniform
+      const size_t at = (size_t)seg * cand_stride + 64 * b + lane;
+      const ulonglong2* src = reinterpret_cast<const ulonglong2*>(col_rejects + at * kDetSplitWords);
+#pragma unroll
+      for (int h = 0; h < kDetSplitWords / 2; ++h) {
+        const ulonglong2 v = src[h];
+        w[b][2 * h] = v.x;
+        w[b][2 * h + 1] = v.y;
+      }
+      const size_t mine = (size_t)seg * cand_stride + min(64 * b + lane, ncand - 1);
+      prior[b] = cand_idx[mine];
+      ckey[b] = cand_key[mine];
+      cbox[b] = cand_box[mine];
+    }
+  }
+  unsigned long long keep[kDetSplitWords];
+  int nkept = 0;
+  int* const kept = kept_idx + (size_t)seg * max_cand;
+#pragma unroll
+  for (int b = 0; b < kDetSplitWords; ++b) {
+    if (b < words) {  // uniform
+      const int bn = min(64, ncand - 64 * b);
+      const unsigned long long valid = bn >= 64 ? ~0ull : ((1ull << bn) - 1ull);
+      bool out = false;
+#pragma unroll
+      for (int e = 0; e < b; ++e) out = out || (w[b][e] & keep[e]) != 0;
+      const unsigned long long before = w[b][b] & ((1ull << lane) - 1ull);
+      unsigned long long open = ~__ballot(out) & valid, keep_bits = 0;
+      while (open != 0) {  // wave-uniform
+        const bool is_open = (open >> lane) & 1ull;
+        const bool rejected = (before & keep_bits) != 0;
+        const bool waits = (before & open) != 0;
+        const unsigned long long now_rejected = __ballot(is_open && rejected);
+        const unsigned long long now_kept = __ballot(is_open && !rejected && !waits);
+        keep_bits |= now_kept;
+        open &= ~(now_kept | now_rejected);
+      }
+      keep[b] = keep_bits;
+      if ((keep_bits >> lane) & 1ull) {
+        const int pos = nkept + __popcll(keep_bits & ((1ull << lane) - 1ull));
+        kept[pos] = prior[b];
+        kept_key[(size_t)seg * max_cand + pos] = ckey[b];
+        kept_box[(size_t)seg * max_cand + pos] = cbox[b];
+      }
+      nkept += __popcll(keep_bits);
+    }
+  }
+  if (lane == 0) kept_count[seg] = nkept;
+}
+
 // Sum of one int per thread over the workgroup, returned to every thread.  `slots` has
 // one entry per wavefront and may be reused right after the call returns.
 __device__ __forceinline__ int block_sum(int v, uint32_t* slots) {
@@ -707,6 +961,157 @@ __global__ __launch_bounds__(kSortThreads) void det_select_kernel(
   if (threadIdx.x == kSortThreads - 1) rows_count[i] = static_cast<int>(pos);
 }
 
+// keep_top_k and the output rows of one image from what det_scan_kernel left (keys and
+// boxes of every class's kept candidates in NMS order), for keep_top_k <= 512 and at most
+// kSelLdsMax entries per image; the rows go straight to their place in the output (every
+// workgroup adds up the row counts of the images before its own), so no launch follows.
+// The keep_top_k best entries come from the selection that does not sort the list; ties
+// at the cut go by (label, NMS order), which is entry order.  If the selection gives up,
+// select_short does the image the long way round.
+struct SelectFastLds {
+  BlockSelectLds sel;
+  int rows[1024];  // rows of every image
+  uint32_t skey[kSortThreads];
+  uint32_t sidx[kSortThreads];
+  int before, all;
+};
+__device__ __noinline__ void det_select_slowly(
+    const float* __restrict__ conf, const DBox* __restrict__ boxes, int P, int C, int loc_classes,
+    int keep_top_k, int max_cand, const int* __restrict__ kept_idx, const int* s_off, int total,
+    int i, float* __restrict__ rows_image, int* __restrict__ rows_count,
+    int* __restrict__ cut_tie_flag, SelectShortLds* st) {
+  select_short(conf, boxes, P, C, loc_classes, keep_top_k, max_cand, kept_idx, s_off, total, i,
+               rows_image, rows_count, cut_tie_flag, st);
+}
+__global__ __launch_bounds__(kSortThreads) void det_select_fast_kernel(
+    const float* __restrict__ conf, const DBox* __restrict__ boxes, int P, int loc_classes,
+    const int* __restrict__ kept_idx, const uint32_t* __restrict__ kept_key,
+    const DBox* __restrict__ kept_box, const int* __restrict__ kept_count, int num, int C,
+    int max_cand, int keep_top_k, float* __restrict__ rows_tmp, int* __restrict__ rows_count,
+    int max_rows, float* __restrict__ out, int* __restrict__ num_rows,
+    int* __restrict__ cut_tie_flag) {
+  __shared__ SelectFastLds lds;
+  __shared__ SelectShortLds short_lds;
+  __shared__ int s_off[1024];
+  const int i = blockIdx.x, tid = threadIdx.x;
+  for (int t = tid; t < num; t += kSortThreads) lds.rows[t] = 0;
+  __syncthreads();
+  for (int t = tid; t < num * C; t += kSortThreads) atomicAdd(&lds.rows[t / C], kept_count[t]);
+  for (int c = tid; c < C; c += kSortThreads) s_off[c + 1] = kept_count[i * C + c];
+  __syncthreads();
+  if (tid < 64) {
+    int before = 0, all = 0;
+    for (int t = tid; t < num; t += 64) {
+      int r = lds.rows[t];
+      if (keep_top_k > -1 && r > keep_top_k) r = keep_top_k;
+      all += r;
+      if (t < i) before += r;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      before += __shfl_xor(before, o, 64);
+      all += __shfl_xor(all, o, 64);
+    }
+    if (tid == 0) {
+      lds.before = before;
+      lds.all = all;
+      int off = 0;
+      for (int c = 0; c < C; ++c) {
+        const int cnt = s_off[c + 1];
+        s_off[c] = off;
+        off += cnt;
+      }
+      s_off[C] = off;
+    }
+  }
+  __syncthreads();
+  const int all = lds.all, before = lds.before, total = s_off[C];
+  if (all == 0) {
+    // one row of -1 per image carrying the image index (detection_output_layer.cpp:175-185)
+    if (i == 0) {
+      for (int t = tid; t < num * 7 && t < max_rows * 7; t += kSortThreads)
+        out[t] = (t % 7 == 0) ? static_cast<float>(t / 7) : -1.f;
+      if (tid == 0) *num_rows = num;
+    }
+    return;
+  }
+  if (i == 0 && tid == 0) *num_rows = all < max_rows ? all : max_rows;
+  // entry e of the image = (label, place in that label's NMS order), labels ascending
+  auto label_of = [&](int e) {
+    int lo = 0, hi = C - 1;  // the last label whose entries start at or before e
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (s_off[mid] <= e) lo = mid; else hi = mid - 1;
+    }
+    // (labels without entries share their start with the next one: step over them)
+    while (s_off[lo + 1] <= e) ++lo;
+    return lo;
+  };
+  auto write_row = [&](int row, int e, int c) {
+    if (before + row >= max_rows) return;
+    const size_t at = (size_t)(i * C + c) * max_cand + (e - s_off[c]);
+    const uint32_t asc = ~kept_key[at];
+    const float score = __uint_as_float((asc & 0x80000000u) ? (asc & 0x7fffffffu) : ~asc);
+    const DBox b = kept_box[at];
+    float* r = out + (size_t)(before + row) * 7;
+    r[0] = static_cast<float>(i);
+    r[1] = static_cast<float>(c);
+    r[2] = score;
+    r[3] = b.xmin;
+    r[4] = b.ymin;
+    r[5] = b.xmax;
+    r[6] = b.ymax;
+  };
+  if (keep_top_k < 0 || total <= keep_top_k) {
+    for (int e = tid; e < total; e += kSortThreads) write_row(e, e, label_of(e));
+    return;
+  }
+  uint32_t rk[kSelLdsPer];
+#pragma unroll
+  for (int j = 0; j < kSelLdsPer; ++j) {
+    const int e = tid + j * kSortThreads;
+    rk[j] = 0xffffffffu;
+    if (e < total) {
+      const int c = label_of(e);
+      rk[j] = kept_key[(size_t)(i * C + c) * max_cand + (e - s_off[c])];
+    }
+  }
+  uint32_t key, e_sel;
+  const int m = block_select_smallest<kSelLdsPer>(rk, keep_top_k, &lds.sel, &key, &e_sel);
+  if (m == 0) {  // uniform
+    float* tmp = rows_tmp + (size_t)i * C * max_cand * 7;
+    det_select_slowly(conf, boxes, P, C, loc_classes, keep_top_k, max_cand, kept_idx, s_off, total, i,
+                      tmp, rows_count, cut_tie_flag, &short_lds);
+    __threadfence_block();
+    __syncthreads();
+    for (int t = tid; t < keep_top_k * 7; t += kSortThreads)
+      if (before + t / 7 < max_rows) out[(size_t)before * 7 + t] = tmp[t];
+    return;
+  }
+  // thread t < keep_top_k holds the entry of rank t by (score, entry); its row is its rank
+  // by entry among those
+  const bool mine = tid < keep_top_k;
+  lds.skey[tid] = key;
+  lds.sidx[tid] = mine ? e_sel : 0xffffffffu;
+  __syncthreads();
+  if (cut_tie_flag) {
+    // more entries at the cut's score than places: which of them survive is decided here by
+    // entry order and in the reference by std::sort's internals
+    if (tid == 0 && m > keep_top_k) atomicOr(cut_tie_flag, 1);
+    // equal scores of one label among the kept rows (neighbours in this order: equal scores
+    // are ordered by entry, and a label's entries are contiguous): the reference rebuilds
+    // the label's list in std::sort's order, here they stay in NMS order
+    if (mine && tid + 1 < keep_top_k && lds.skey[tid + 1] == key &&
+        label_of(static_cast<int>(lds.sidx[tid + 1])) == label_of(static_cast<int>(e_sel)))
+      atomicOr(cut_tie_flag, 2);
+  }
+  if (mine) {
+    int row = 0;
+    for (int t = 0; t < keep_top_k; ++t) row += lds.sidx[t] < e_sel;
+    write_row(row, static_cast<int>(e_sel), label_of(static_cast<int>(e_sel)));
+  }
+}
+
 // Concatenates the per-image rows, one workgroup per image; with no detection at
 // all, one row of -1 per image carrying the image index
 // (detection_output_layer.cpp:175-185).
@@ -755,7 +1160,7 @@ __global__ __launch_bounds__(256) void det_emit_kernel(const float* __restrict__
 
 struct DetLayout {
   size_t boxes, k0, v0, k1, v1, kept_idx, kept_count, sk0, sv0, sk1, sv1, selected, rows_tmp,
-      rows_count, total;
+      rows_count, cand_key, cand_idx, cand_box, ncand, col_rejects, kept_key, kept_box, total;
 };
 
 inline size_t det_align(size_t v) { return (v + 255) / 256 * 256; }
@@ -784,11 +1189,24 @@ DetLayout det_layout(int num, int P, int C, int loc_classes, int max_cand) {
   L.selected = take(4 * entries);
   L.rows_tmp = take(4 * 7 * entries);
   L.rows_count = take(4 * (size_t)num);
+  // the three-launch path (top_k <= kDetSplitTopK): candidate lists and their pair bits
+  const size_t cands = segs * (size_t)((max_cand + 63) / 64 * 64);
+  const bool split = max_cand <= kDetSplitTopK;
+  L.cand_key = take(split ? 4 * cands : 0);
+  L.cand_idx = take(split ? 4 * cands : 0);
+  L.cand_box = take(split ? sizeof(DBox) * cands : 0);
+  L.ncand = take(split ? 4 * segs : 0);
+  L.col_rejects = take(split ? 8 * kDetSplitWords * cands : 0);
+  L.kept_key = take(split ? 4 * entries : 0);
+  L.kept_box = take(split ? sizeof(DBox) * entries : 0);
   L.total = off;
   return L;
 }
 
 int det_max_cand(int P, int top_k) { return (top_k > -1 && top_k < P) ? top_k : P; }
+
+// Test knob: 0 keeps every input on the one-launch per-class kernels.
+bool g_det_split = true;
 
 }  // namespace
 }  // namespace mchip
@@ -813,6 +1231,11 @@ int mcDetectionOutputMaxRows(int num, int num_priors, int num_classes, int top_k
   long rows = per_image * num;
   if (rows < num) rows = num;
   return rows > 0x7fffffffL ? 0x7fffffff : static_cast<int>(rows);
+}
+
+int mcDetectionOutputSplit(int on) {
+  g_det_split = on != 0;
+  return 0;
 }
 
 int mcDetectionOutput(const float* loc, const float* conf, const float* prior, int num,
@@ -844,11 +1267,42 @@ int mcDetectionOutput(const float* loc, const float* conf, const float* prior, i
   auto i32 = [&](size_t off) { return reinterpret_cast<int*>(ws + off); };
   hipStream_t st = static_cast<hipStream_t>(stream);
   const long ndec = (long)num * loc_classes * num_priors;
-  det_decode_kernel<<<ceil_div(ndec, 256), 256, 0, st>>>(loc, prior, num, num_priors, loc_classes,
-                                                         code_type, variance_encoded_in_target,
-                                                         boxes, cut_tie_flag);
+  // constant threshold and at most kDetSplitTopK candidates per class: the per-class work
+  // in three launches (candidates, pair bits over the whole chip, scan)
+  const bool split = g_det_split && eta >= 1.f && max_cand <= kDetSplitTopK && num_priors <= kDetLdsMax;
+  det_decode_kernel<<<ceil_div(ndec + (split ? (long)num * num_priors : 0), 256), 256, 0, st>>>(
+      loc, prior, num, num_priors, loc_classes, code_type, variance_encoded_in_target, boxes,
+      cut_tie_flag, conf, num_classes, split ? u32(L.k0) : nullptr);
   MC_LAUNCH_CHECK();
-  if (num_priors <= kDetLdsMax)
+  if (split) {
+    const int cand_stride = (max_cand + 63) / 64 * 64, words = cand_stride / 64;
+    DBox* cand_box = reinterpret_cast<DBox*>(ws + L.cand_box);
+    unsigned long long* col_rejects = reinterpret_cast<unsigned long long*>(ws + L.col_rejects);
+    det_candidates_kernel<<<dim3(num_classes, num), kSortThreads, 0, st>>>(
+        u32(L.k0), boxes, num_priors, num_classes, loc_classes, background_label,
+        desc_key(confidence_threshold), max_cand, cand_stride, u32(L.cand_key), i32(L.cand_idx),
+        cand_box, i32(L.ncand));
+    MC_LAUNCH_CHECK();
+    det_overlap_kernel<<<dim3(ceil_div(words * (words + 1) / 2, kOverlapWaves), num * num_classes),
+                         64 * kOverlapWaves, 0, st>>>(cand_box, i32(L.ncand), cand_stride,
+                                                      nms_threshold, col_rejects);
+    MC_LAUNCH_CHECK();
+    det_scan_kernel<<<num * num_classes, 64, 0, st>>>(
+        col_rejects, i32(L.ncand), i32(L.cand_idx), u32(L.cand_key), cand_box, cand_stride, max_cand,
+        i32(L.kept_idx), u32(L.kept_key), reinterpret_cast<DBox*>(ws + L.kept_box), i32(L.kept_count));
+    MC_LAUNCH_CHECK();
+    // (the background label has no entries)
+    const int labels = num_classes - (background_label >= 0 && background_label < num_classes ? 1 : 0);
+    if (keep_top_k <= kSortThreads && (long)labels * max_cand <= kSelLdsMax) {
+      det_select_fast_kernel<<<num, kSortThreads, 0, st>>>(
+          conf, boxes, num_priors, loc_classes, i32(L.kept_idx), u32(L.kept_key),
+          reinterpret_cast<DBox*>(ws + L.kept_box), i32(L.kept_count), num, num_classes, max_cand,
+          keep_top_k, reinterpret_cast<float*>(ws + L.rows_tmp), i32(L.rows_count), max_rows, out_rows,
+          num_rows, cut_tie_flag);
+      MC_LAUNCH_CHECK();
+      return 0;
+    }
+  } else if (num_priors <= kDetLdsMax)
     det_class_nms_lds_kernel<<<dim3(num_classes, num), kSortThreads, 0, st>>>(
         conf, boxes, num_priors, num_classes, loc_classes, background_label, confidence_threshold,
         nms_threshold, eta, top_k, max_cand, i32(L.kept_idx), i32(L.kept_count));

@@ -60,6 +60,7 @@ LIB.mcConvTimingCollectDetail.argtypes = [ctypes.POINTER(ctypes.c_double), ctype
 LIB.mcDetectionOutputWorkspaceSize.argtypes = [c_int, c_int, c_int, c_int, c_int,
                                                ctypes.POINTER(ctypes.c_size_t)]
 LIB.mcDetectionOutputMaxRows.argtypes = [c_int] * 5
+LIB.mcDetectionOutputSplit.argtypes = [c_int]
 LIB.mcDetectionOutput.argtypes = [c_void_p, c_void_p, c_void_p] + [c_int] * 8 + \
     [c_float, c_float, c_float, c_int, c_void_p, ctypes.c_size_t, c_void_p, c_int, c_void_p, c_void_p,
      c_void_p]

@@ -1110,17 +1110,28 @@ def run_detection_output(K, param, loc, conf, prior):
     max_rows = K.LIB.mcDetectionOutputMaxRows(num, P, C, tk, keep)
     ws = torch.empty(sz.value, dtype=torch.uint8, device="cuda")
     ld, cd, pd = dev(loc), dev(conf), dev(prior)
-    out = torch.full((max_rows, 7), float("nan"), device="cuda")
-    cnt = torch.full((2,), -5, dtype=torch.int32, device="cuda")
     code = {"CORNER": 1, "CENTER_SIZE": 2, "CORNER_SIZE": 3}[str(param.get("code_type", "CORNER"))]
-    K.check_mc(K.LIB.mcDetectionOutput(
-        fptr(ld), fptr(cd), fptr(pd), num, P, C, int(share), param.get("background_label_id", 0), code,
-        int(param.get("variance_encoded_in_target", False)), keep,
-        ctypes.c_float(param.get("confidence_threshold", -3.4028234663852886e38)),
-        ctypes.c_float(nmsp.get("nms_threshold", 0.3)), ctypes.c_float(nmsp.get("eta", 1.0)), tk, fptr(ws),
-        sz.value, fptr(out), max_rows, ctypes.c_void_p(cnt.data_ptr()), ctypes.c_void_p(cnt.data_ptr() + 4), None))
-    torch.cuda.synchronize()
-    return out[:int(cnt[0].item())].cpu().numpy(), int(cnt[1].item())
+    results = []
+    # every input twice: the automatic choice of kernels (three launches per class where the
+    # input allows it), then pinned to the one-launch-per-class kernels; same rows, same flag
+    for split in (1, 0):
+        out = torch.full((max_rows, 7), float("nan"), device="cuda")
+        cnt = torch.full((2,), -5, dtype=torch.int32, device="cuda")
+        K.check_mc(K.LIB.mcDetectionOutputSplit(split))
+        try:
+            K.check_mc(K.LIB.mcDetectionOutput(
+                fptr(ld), fptr(cd), fptr(pd), num, P, C, int(share), param.get("background_label_id", 0), code,
+                int(param.get("variance_encoded_in_target", False)), keep,
+                ctypes.c_float(param.get("confidence_threshold", -3.4028234663852886e38)),
+                ctypes.c_float(nmsp.get("nms_threshold", 0.3)), ctypes.c_float(nmsp.get("eta", 1.0)), tk, fptr(ws),
+                sz.value, fptr(out), max_rows, ctypes.c_void_p(cnt.data_ptr()), ctypes.c_void_p(cnt.data_ptr() + 4),
+                None))
+            torch.cuda.synchronize()
+        finally:
+            K.check_mc(K.LIB.mcDetectionOutputSplit(1))
+        results.append((out[:int(cnt[0].item())].cpu().numpy(), int(cnt[1].item())))
+    assert np.array_equal(results[0][0], results[1][0], equal_nan=True) and results[0][1] == results[1][1]
+    return results[0]
 
 
 def cut_tie_expected(param, loc, conf, prior):
