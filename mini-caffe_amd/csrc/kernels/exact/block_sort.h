@@ -175,6 +175,7 @@ __device__ inline void block_sort_desc_lds(uint32_t* keys, VT* vals, int n, Bloc
 //      wavefronts' values has at least `want`.  The threads hold strided samples of the
 //      table, so usually a thousand or two keys pass: the candidates (kSelectCandPer per
 //      thread at most, else the call fails and the caller sorts).
+//      If they fit one to a thread they all go through step 3 and step 2 is skipped.
 //   2. tau = the want-th smallest candidate by bisection on the key bits, two bits per
 //      round from the top (three trial values, one count over the workgroup each: ballots
 //      and scalar population counts within a wavefront, the wavefronts' counts through
@@ -236,17 +237,23 @@ __device__ __forceinline__ int block_select_smallest(const uint32_t (&rk)[PER], 
   // the wavefront's share of the cut: the ceil(want / 8)-th smallest of its 64 thread
   // minima (eight wavefronts: at least `want` entries lie at or below the largest share)
   uint32_t cut = lowest;  // (a thread without entries holds all ones)
-#pragma unroll
-  for (int k = 2; k <= 64; k <<= 1) {
-#pragma unroll
-    for (int j = k >> 1; j > 0; j >>= 1) {
-      const uint32_t other = static_cast<uint32_t>(__shfl_xor(cut, j, 64));
-      const bool up = (lane & k) == 0 || k == 64, lower = (lane & j) == 0;
-      cut = (lower == up) ? min(cut, other) : max(cut, other);
-    }
-  }
   static_assert(kSortThreads / 64 == 8, "eight wavefronts share the cut");
-  cut = static_cast<uint32_t>(__shfl(cut, (want + 7) / 8 - 1, 64));
+  const int kth = (want + 7) / 8;
+  if (kth >= 64) {  // uniform: the largest of the 64
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) cut = max(cut, static_cast<uint32_t>(__shfl_xor(cut, o, 64)));
+  } else {  // the 64 minima in ascending order over the lanes, then the kth of them
+#pragma unroll
+    for (int k = 2; k <= 64; k <<= 1) {
+#pragma unroll
+      for (int j = k >> 1; j > 0; j >>= 1) {
+        const uint32_t other = static_cast<uint32_t>(__shfl_xor(cut, j, 64));
+        const bool up = (lane & k) == 0 || k == 64, lower = (lane & j) == 0;
+        cut = (lower == up) ? min(cut, other) : max(cut, other);
+      }
+    }
+    cut = static_cast<uint32_t>(__shfl(cut, kth - 1, 64));
+  }
   __syncthreads();  // (the caller may still be reading what `s` overlays)
   if (lane == 0) s->red[wave] = cut;
   __syncthreads();
@@ -271,6 +278,20 @@ __device__ __forceinline__ int block_select_smallest(const uint32_t (&rk)[PER], 
       }
   }
   __syncthreads();
+  if (ncand <= kSortThreads) {  // uniform
+    // the candidates fit one to a thread: order them all; m = those at or below the
+    // want-th of them
+    uint32_t key = tid < ncand ? s->ckey[tid] : 0xffffffffu;
+    uint32_t idx = tid < ncand ? s->cidx[tid] : 0xffffffffu;
+    bitonic_sort_block<kSortThreads>(key, idx, s->x, s->x + kSortThreads);
+    __syncthreads();
+    if (tid == want - 1) s->x[0] = key;
+    __syncthreads();
+    const uint32_t tau = s->x[0];
+    *key_out = key;
+    *idx_out = idx;
+    return __syncthreads_count(tid < ncand && key <= tau);
+  }
   uint32_t ck[kSelectCandPer];
   uint32_t diff = 0;
   const uint32_t first = s->ckey[0];

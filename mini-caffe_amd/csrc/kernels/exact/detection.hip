@@ -49,7 +49,14 @@ __global__ __launch_bounds__(256) void det_decode_kernel(
     const int p = static_cast<int>(t2 % P);
     const int i = static_cast<int>(t2 / P);
     const float* cp = conf + ((long)i * P + p) * C;
-    for (int c = 0; c < C; ++c) keys_by_class[((long)i * C + c) * P + p] = desc_key(cp[c]);
+    for (int c0 = 0; c0 < C; c0 += 8) {  // eight loads in flight before the first store
+      float v[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) v[q] = cp[min(c0 + q, C - 1)];
+#pragma unroll
+      for (int q = 0; q < 8; ++q)
+        if (c0 + q < C) keys_by_class[((long)i * C + c0 + q) * P + p] = desc_key(v[q]);
+    }
     return;
   }
   const int p = static_cast<int>(t % P);
@@ -1067,13 +1074,16 @@ __global__ __launch_bounds__(kSortThreads) void det_select_fast_kernel(
     return;
   }
   uint32_t rk[kSelLdsPer];
+  {
+    int c = label_of(min(tid, total - 1));  // a thread's entries ascend: so do their labels
 #pragma unroll
-  for (int j = 0; j < kSelLdsPer; ++j) {
-    const int e = tid + j * kSortThreads;
-    rk[j] = 0xffffffffu;
-    if (e < total) {
-      const int c = label_of(e);
-      rk[j] = kept_key[(size_t)(i * C + c) * max_cand + (e - s_off[c])];
+    for (int j = 0; j < kSelLdsPer; ++j) {
+      const int e = tid + j * kSortThreads;
+      rk[j] = 0xffffffffu;
+      if (e < total) {
+        while (s_off[c + 1] <= e) ++c;
+        rk[j] = kept_key[(size_t)(i * C + c) * max_cand + (e - s_off[c])];
+      }
     }
   }
   uint32_t key, e_sel;
