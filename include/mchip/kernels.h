@@ -381,12 +381,13 @@ int mcDetectionOutput(const float* loc, const float* conf, const float* prior, i
                       float confidence_threshold, float nms_threshold, float eta, int top_k,
                       void* workspace, size_t workspace_bytes, float* out_rows, int max_rows,
                       int* num_rows, int* cut_tie_flag, void* stream);
-/* Test knob (process-wide): with a constant threshold (eta 1), at most 512 candidates
- * per class and at most 12 288 priors, the per-class work runs as three launches
- * (candidate selection, pairwise overlap bits spread over the whole chip, greedy scan);
- * 0 keeps such inputs on the one-launch-per-class kernel that every other input takes,
- * 1 restores the automatic choice.  Results are the same. */
-int mcDetectionOutputSplit(int on);
+/* Test knob (process-wide).  With a constant threshold (eta 1), at most 512 candidates
+ * per class and at most 12 288 priors, the per-class work can run as three launches
+ * (candidate selection, pairwise overlap bits spread over the whole chip, greedy scan)
+ * followed by one launch for keep_top_k and the rows, instead of one launch per class
+ * that does everything on one CU.  mode 1 (the default) takes that path where it is
+ * faster (4096 priors and more), 2 wherever it fits, 0 never.  Results are the same. */
+int mcDetectionOutputSplit(int mode);
 
 /* ROIPoolingLayer::Forward (roi_pooling_layer.cpp:37-110; .cu:13-81): max pooling of
  * bottom [num, channels, height, width] over num_rois regions, rois rows of

@@ -101,7 +101,7 @@ struct BlockSortLds16 {
 };
 
 template <int MAXPER, typename VT, bool SKIP_CONSTANT_DIGITS = true>
-__device__ inline void block_sort_desc_lds(uint32_t* keys, VT* vals, int n, BlockSortLds16* lds) {
+__device__ __forceinline__ void block_sort_desc_lds(uint32_t* keys, VT* vals, int n, BlockSortLds16* lds) {
   const int tid = threadIdx.x;
   const int per = (n + kSortThreads - 1) / kSortThreads;
   const int begin = min(tid * per, n), end = min(begin + per, n);

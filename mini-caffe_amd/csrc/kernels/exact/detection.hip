@@ -1215,8 +1215,11 @@ DetLayout det_layout(int num, int P, int C, int loc_classes, int max_cand) {
 
 int det_max_cand(int P, int top_k) { return (top_k > -1 && top_k < P) ? top_k : P; }
 
-// Test knob: 0 keeps every input on the one-launch per-class kernels.
-bool g_det_split = true;
+// Who takes the three-launch per-class path: 1 = inputs it fits and pays for (tables of
+// 4096 priors and more: below that the sort of the whole table in LDS is cheap and one
+// launch per class wins, MobileNet-SSD's 32 x 21 lists of 1917 priors 35 against 53 us),
+// 2 = every input it fits, 0 = none (test knob).
+int g_det_split = 1;
 
 }  // namespace
 }  // namespace mchip
@@ -1243,8 +1246,9 @@ int mcDetectionOutputMaxRows(int num, int num_priors, int num_classes, int top_k
   return rows > 0x7fffffffL ? 0x7fffffff : static_cast<int>(rows);
 }
 
-int mcDetectionOutputSplit(int on) {
-  g_det_split = on != 0;
+int mcDetectionOutputSplit(int mode) {
+  MC_REQUIRE(mode >= 0 && mode <= 2, "mcDetectionOutputSplit: bad argument");
+  g_det_split = mode;
   return 0;
 }
 
@@ -1279,7 +1283,8 @@ int mcDetectionOutput(const float* loc, const float* conf, const float* prior, i
   const long ndec = (long)num * loc_classes * num_priors;
   // constant threshold and at most kDetSplitTopK candidates per class: the per-class work
   // in three launches (candidates, pair bits over the whole chip, scan)
-  const bool split = g_det_split && eta >= 1.f && max_cand <= kDetSplitTopK && num_priors <= kDetLdsMax;
+  const bool split = g_det_split != 0 && eta >= 1.f && max_cand <= kDetSplitTopK &&
+                     num_priors <= kDetLdsMax && (g_det_split == 2 || num_priors >= 4096);
   det_decode_kernel<<<ceil_div(ndec + (split ? (long)num * num_priors : 0), 256), 256, 0, st>>>(
       loc, prior, num, num_priors, loc_classes, code_type, variance_encoded_in_target, boxes,
       cut_tie_flag, conf, num_classes, split ? u32(L.k0) : nullptr);

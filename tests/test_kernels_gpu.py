@@ -1112,9 +1112,9 @@ def run_detection_output(K, param, loc, conf, prior):
     ld, cd, pd = dev(loc), dev(conf), dev(prior)
     code = {"CORNER": 1, "CENTER_SIZE": 2, "CORNER_SIZE": 3}[str(param.get("code_type", "CORNER"))]
     results = []
-    # every input twice: the automatic choice of kernels (three launches per class where the
-    # input allows it), then pinned to the one-launch-per-class kernels; same rows, same flag
-    for split in (1, 0):
+    # every input twice: three launches per class wherever the input allows it, then pinned
+    # to the one-launch-per-class kernels; same rows, same flag
+    for split in (2, 0):
         out = torch.full((max_rows, 7), float("nan"), device="cuda")
         cnt = torch.full((2,), -5, dtype=torch.int32, device="cuda")
         K.check_mc(K.LIB.mcDetectionOutputSplit(split))
