@@ -344,7 +344,9 @@ int mcProposalTimingCollect(double* stage_ms, long* calls);
  * (mcProposalWorkspaceSize) exceeds 8 MiB are refused with an error: 1 x 18 x 38 x 63
  * scores with pre_nms_topn 6000 need 6.7 MB.  The call itself allocates and frees
  * nothing.  Every call on a GPU uses that GPU's one buffer: calls that overlap on one
- * GPU (two streams, two threads) race; calls on one stream are ordered and safe. */
+ * GPU (two streams, two threads) race; calls on one stream are ordered and safe.
+ * The first call on a device looks the buffer's address up (hipGetSymbolAddress, which
+ * may load the library's code object): make it once outside any stream capture. */
 int mcProposalStatic(const float* scores, const float* bbox, const float* im_info,
                      const float* anchors, int A, int H, int W, int feat_stride, float min_size,
                      int pre_nms_topn, int post_nms_topn, float nms_thresh, float* rois,

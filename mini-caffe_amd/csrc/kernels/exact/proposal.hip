@@ -1533,7 +1533,8 @@ constexpr size_t kStaticScratchBytes = size_t(8) << 20;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 // Optional stage timing (measurement hook): while enabled on the calling thread every
-// call records five HIP events on its stream.
+// call records up to five HIP events on its stream (a stage that launches nothing shares
+// the event before it and reads as zero).
 struct ProposalTimes {
   hipEvent_t ev[5];
 };
@@ -1694,13 +1695,16 @@ int run_proposal(int steps, const float* scores, const float* bbox, const float*
         sboxes, sscores, kept, num_rois, rois, roi_scores, flags, state, state_ints);
     MC_LAUNCH_CHECK();
   } else {
-    MC_HIP(mark(3));
+    times.ev[3] = times.ev[2];  // (nothing ran in stage 2: no event of its own, zero time)
     if (state && !head_possible) {  // the head step was asked for and cannot run: not final
       zero_ints_kernel<<<1, 64, 0, st>>>(state, state_ints);
       MC_LAUNCH_CHECK();
+      MC_HIP(mark(4));
+    } else {
+      times.ev[4] = times.ev[3];
     }
   }
-  MC_HIP(mark(4));
+  if (steps & kStepRest) MC_HIP(mark(4));
   if (timing) g_prop_timed.push_back(times);
   return 0;
 }
@@ -1766,7 +1770,8 @@ int mcProposalTimingCollect(double* stage_ms, long* calls) {
       MC_HIP(hipEventElapsedTime(&e, t.ev[k], t.ev[k + 1]));
       sum[k] += e;
     }
-    for (int k = 0; k < 5; ++k) (void)hipEventDestroy(t.ev[k]);
+    for (int k = 0; k < 5; ++k)
+      if (k == 0 || t.ev[k] != t.ev[k - 1]) (void)hipEventDestroy(t.ev[k]);  // (an empty stage shares its event)
   }
   if (stage_ms)
     for (int k = 0; k < 4; ++k) stage_ms[k] = sum[k];

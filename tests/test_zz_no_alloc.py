@@ -75,6 +75,29 @@ def test_static_scratch_matches_workspace_entry_point_on_consecutive_calls(K):
         assert np.array_equal(got[2], rois) and np.array_equal(got[3], rs)
 
 
+def test_static_scratch_allocates_nothing(K):
+    """What the entry point is for: after one call on the device (the first looks up the
+    buffer's address, which may load the code object: it must happen outside a capture),
+    further calls leave the device's free memory as it is."""
+    scores, bbox, im_info = _inputs(6, 38, 63, 0)
+    A, H, W, pre, post = 9, 38, 63, 6000, 300
+    dev = [torch.from_numpy(np.ascontiguousarray(a)).cuda()
+           for a in (scores, bbox, im_info, oracle.generate_anchors())]
+    rois = torch.empty((post, 5), device="cuda")
+    rs = torch.empty((post,), device="cuda")
+    cnt = torch.zeros(2, dtype=torch.int32, device="cuda")
+    args = [_ptr(d) for d in dev] + [A, H, W, 16, ctypes.c_float(16), pre, post, ctypes.c_float(0.7), _ptr(rois),
+                                     _ptr(rs), ctypes.c_void_p(cnt.data_ptr()), ctypes.c_void_p(cnt.data_ptr() + 4), None]
+    K.check_mc(K.LIB.mcProposalStatic(*args))
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(5):
+        K.check_mc(K.LIB.mcProposalStatic(*args))
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert int(cnt[0].item()) > 0
+
+
 def test_static_scratch_refuses_what_it_cannot_hold(K):
     scores, bbox, im_info = _inputs(5, 60, 80, 0)          # 43200 proposals
     with pytest.raises(Exception, match="scratch"):
