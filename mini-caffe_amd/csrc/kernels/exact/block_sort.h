@@ -184,7 +184,9 @@ __device__ __forceinline__ void block_sort_desc_lds(uint32_t* keys, VT* vals, in
 //      hang over) go one to a thread through a compare-exchange network on (key, index):
 //      all pairs differ, so the order is that of a stable sort by key.
 // Returns m, and in thread t < m the entry of rank t; 0 when step 1 or 3 does not fit
-// (crowds of equal keys).  All threads of the workgroup must call it.
+// (crowds of equal keys).  All threads of the workgroup must call it.  A caller that already
+// knows a key with at least `want` entries at or below it passes it as `known_cut` (not 0)
+// and step 1 uses that instead of the thread minima.
 constexpr int kSelectCandPer = 8;
 struct BlockSelectLds {
   uint32_t ckey[kSelectCandPer * kSortThreads];
@@ -229,17 +231,18 @@ __device__ __forceinline__ void bitonic_sort_block(uint32_t& key, uint32_t& idx,
 
 template <int PER>
 __device__ __forceinline__ int block_select_smallest(const uint32_t (&rk)[PER], int want, BlockSelectLds* s,
-                                            uint32_t* key_out, uint32_t* idx_out) {
+                                            uint32_t* key_out, uint32_t* idx_out, uint32_t known_cut = 0) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   uint32_t lowest = 0xffffffffu;
 #pragma unroll
   for (int j = 0; j < PER; ++j) lowest = min(lowest, rk[j]);
+  if (known_cut != 0) lowest = known_cut;  // (uniform) the caller knows a key with `want` entries at or below it
   // the wavefront's share of the cut: the ceil(want / 8)-th smallest of its 64 thread
   // minima (eight wavefronts: at least `want` entries lie at or below the largest share)
   uint32_t cut = lowest;  // (a thread without entries holds all ones)
   static_assert(kSortThreads / 64 == 8, "eight wavefronts share the cut");
   const int kth = (want + 7) / 8;
-  if (kth >= 64) {  // uniform: the largest of the 64
+  if (kth >= 64 || known_cut != 0) {  // uniform: the largest of the 64 (all the same with a known cut)
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) cut = max(cut, static_cast<uint32_t>(__shfl_xor(cut, o, 64)));
   } else {  // the 64 minima in ascending order over the lanes, then the kth of them

@@ -1073,8 +1073,38 @@ __global__ __launch_bounds__(kSortThreads) void det_select_fast_kernel(
     for (int e = tid; e < total; e += kSortThreads) write_row(e, e, label_of(e));
     return;
   }
-  uint32_t rk[kSelLdsPer];
-  {
+  uint32_t key = 0xffffffffu, e_sel = 0xffffffffu;
+  int m = 0;
+  // Every label's list is in descending score order, so the image's best entries sit at the
+  // heads of the lists.  First the heads alone: R entries of every label, one to a thread,
+  // ordered by the compare-exchange network.  If no list that goes on behind its head has
+  // its R-th entry at or below the keep_top_k-th key of the heads, nothing further down any
+  // list can be among the best keep_top_k (or tie with the last of them), and the heads hold
+  // the answer.  A label with more than R of the best entries sends the image to the
+  // selection over all entries below, which then starts from the heads' cut.
+  uint32_t cut = 0;  // the heads' keep_top_k-th key when the heads did not settle it: the true one is no larger
+  const int R = kSortThreads / C;
+  if (R >= 1) {  // uniform
+    const int c = tid / R, r = tid - c * R;
+    const int cnt = c < C ? s_off[c + 1] - s_off[c] : 0;
+    if (r < cnt) {
+      key = kept_key[(size_t)(i * C + c) * max_cand + r];
+      e_sel = static_cast<uint32_t>(s_off[c] + r);
+    }
+    const uint32_t head_end = (r == R - 1 && cnt > R) ? key : 0xffffffffu;
+    bitonic_sort_block<kSortThreads>(key, e_sel, lds.sel.x, lds.sel.x + kSortThreads);
+    __syncthreads();
+    if (tid == keep_top_k - 1) lds.sel.x[0] = key;
+    __syncthreads();
+    const uint32_t tau = lds.sel.x[0];
+    // (tau all ones: the heads hold fewer than keep_top_k entries)
+    if (!__syncthreads_or(tau == 0xffffffffu || head_end <= tau))
+      m = __syncthreads_count(key <= tau);
+    else if (tau != 0xffffffffu)
+      cut = tau;
+  }
+  if (m == 0) {  // uniform
+    uint32_t rk[kSelLdsPer];
     int c = label_of(min(tid, total - 1));  // a thread's entries ascend: so do their labels
 #pragma unroll
     for (int j = 0; j < kSelLdsPer; ++j) {
@@ -1085,9 +1115,8 @@ __global__ __launch_bounds__(kSortThreads) void det_select_fast_kernel(
         rk[j] = kept_key[(size_t)(i * C + c) * max_cand + (e - s_off[c])];
       }
     }
+    m = block_select_smallest<kSelLdsPer>(rk, keep_top_k, &lds.sel, &key, &e_sel, cut);
   }
-  uint32_t key, e_sel;
-  const int m = block_select_smallest<kSelLdsPer>(rk, keep_top_k, &lds.sel, &key, &e_sel);
   if (m == 0) {  // uniform
     float* tmp = rows_tmp + (size_t)i * C * max_cand * 7;
     det_select_slowly(conf, boxes, P, C, loc_classes, keep_top_k, max_cand, kept_idx, s_off, total, i,
