@@ -159,6 +159,9 @@ def main():
     steps = max(1, args.steps)
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP32_MFMA_PEAK_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(achieved / FP32_MFMA_PEAK_TFLOPS, 4),
+                "frac_is": "direct-sum FLOPs of all contractions over their device time, against the fp32 MFMA peak: what "
+                           "the layers are worth; the matrix pipe's own utilisation is mfma_issued_frac (the Winograd "
+                           "layers hand it 2.25 times fewer products)",
                 "traffic": traffic, "traffic_source": traffic_note,
                 "kernel": "igemm_f32 / winograd_fused (Convolution + InnerProduct, fused BN/Scale/ReLU epilogue; "
                           "%d of the %d contractions per step are 3x3 stride-1 layers run as F(2x2,3x3) Winograd "
@@ -241,6 +244,8 @@ def main():
                                   "(BASELINE configs[1])" % args.batch,
                       "conv_gflop_per_step": round(flops["conv"] / 1e9, 1),
                       "api": "CaffeNetForward (Net::Forward(reshape=true))"},
+           "timing_note": "the device needs about a second of load to settle: 20 steps after 5 warm-up steps read "
+                          "2-3 % slower than the default 100 after 50 (the same library, the same box)",
            "roofline": roofline, "cpu_baseline": cpu,
            "conv_mfma_util_pct": mfma_util, "conv_mfma_util_source": mfma_note,
            "direct_path_only": direct}
