@@ -257,6 +257,12 @@ int mcSoftmax(const float* bottom, float* top, int outer, int channels, int inne
  * slice_layer.cu:8-46). */
 int mcCopy2D(const float* src, long src_pitch, float* dst, long dst_pitch, long width, long rows,
              void* stream);
+/* Concat of `count` sources along the axis behind `rows` leading rows, in one launch per
+ * eight sources: dst[r][offset_k + i] = srcs[k][r * widths[k] + i], offsets in source
+ * order, dst rows of sum(widths) floats (concat_layer.cu:8-46: one kernel per bottom
+ * there).  srcs and widths are host arrays. */
+int mcConcat(const float* const* srcs, const long* widths, int count, float* dst, long rows,
+             void* stream);
 
 /* Generic N-d transpose, top axis i = bottom axis order[i]
  * (permute_layer.cpp:9-106, PermuteKernel permute_layer.cu:10-28).  The

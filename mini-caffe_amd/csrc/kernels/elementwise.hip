@@ -4,6 +4,8 @@
 // All of them move each element once: one global read per input and one global
 // write per output, 16-byte vector accesses whenever the shape allows it, and a
 // grid of a few waves per CU walking the blob with a grid stride.
+#include <algorithm>
+
 #include "mc_common.h"
 #include "mchip/kernels.h"
 
@@ -310,6 +312,34 @@ __global__ __launch_bounds__(256) void copy2d_kernel(const float* __restrict__ s
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Up to kConcatSources strided copies into one destination in one launch: blockIdx.y is
+// the source, the x extent of the grid covers the largest of them.
+constexpr int kConcatSources = 8;
+struct ConcatArgs {
+  const float* src[kConcatSources];
+  long width[kConcatSources];   // floats per row of the source (its pitch as well)
+  long offset[kConcatSources];  // where its rows start inside a destination row
+  float* dst;
+  long dst_pitch, rows;
+};
+template <int VEC>
+__global__ __launch_bounds__(256) void concat_kernel(const ConcatArgs a) {
+  const int k = blockIdx.y;
+  const float* __restrict__ src = a.src[k];
+  float* __restrict__ dst = a.dst + a.offset[k];
+  const long wv = a.width[k] / VEC;
+  const long n = wv * a.rows;
+  for (long i = blockIdx.x * 256L + threadIdx.x; i < n; i += gridDim.x * 256L) {
+    const long r = i / wv, c = (i - r * wv) * VEC;
+    if (VEC == 4) {
+      *reinterpret_cast<float4*>(dst + r * a.dst_pitch + c) =
+          *reinterpret_cast<const float4*>(src + r * a.width[k] + c);
+    } else {
+      dst[r * a.dst_pitch + c] = src[r * a.width[k] + c];
+    }
+  }
+}
+
 }  // namespace
 }  // namespace mchip
 
@@ -471,6 +501,45 @@ int mcCopy2D(const float* src, long src_pitch, float* dst, long dst_pitch, long 
                                                                    width, rows);
   }
   MC_LAUNCH_CHECK();
+  return 0;
+}
+
+int mcConcat(const float* const* srcs, const long* widths, int count, float* dst, long rows,
+             void* stream) {
+  MC_REQUIRE(srcs && widths && dst && count > 0 && rows >= 0, "mcConcat: bad argument");
+  long pitch = 0;
+  for (int i = 0; i < count; ++i) {
+    MC_REQUIRE(widths[i] >= 0 && (widths[i] == 0 || srcs[i]), "mcConcat: bad source");
+    pitch += widths[i];
+  }
+  if (rows == 0 || pitch == 0) return 0;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  long offset = 0;
+  for (int first = 0; first < count; first += kConcatSources) {
+    ConcatArgs a;
+    a.dst = dst;
+    a.dst_pitch = pitch;
+    a.rows = rows;
+    int n = 0;
+    long widest = 0;
+    bool vec = pitch % 4 == 0 && aligned16(dst);
+    for (int i = first; i < count && i < first + kConcatSources; ++i) {
+      if (widths[i] == 0) continue;
+      a.src[n] = srcs[i];
+      a.width[n] = widths[i];
+      a.offset[n] = offset;
+      vec = vec && widths[i] % 4 == 0 && offset % 4 == 0 && aligned16(srcs[i]);
+      widest = std::max(widest, widths[i]);
+      offset += widths[i];
+      ++n;
+    }
+    if (n == 0) continue;
+    if (vec)
+      concat_kernel<4><<<dim3(ew_blocks(widest / 4 * rows, 256), n), 256, 0, st>>>(a);
+    else
+      concat_kernel<1><<<dim3(ew_blocks(widest * rows, 256), n), 256, 0, st>>>(a);
+    MC_LAUNCH_CHECK();
+  }
   return 0;
 }
 

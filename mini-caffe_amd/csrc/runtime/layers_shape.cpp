@@ -55,16 +55,15 @@ class ConcatLayer : public Layer {
       DeviceCopy(*bottom[0], top[0]);
       return;
     }
-    float* top_data = top[0]->mutable_gpu_data();
-    const long top_pitch = static_cast<long>(top[0]->shape(axis_)) * inner_;
-    long offset = 0;
+    // all bottoms in one launch (per eight of them)
+    vector<const float*> srcs;
+    vector<long> widths;
     for (Blob* b : bottom) {
-      const long width = static_cast<long>(b->shape(axis_)) * inner_;
-      if (width > 0 && outer_ > 0)
-        MC_CHECK(mcCopy2D(b->gpu_data(), width, top_data + offset, top_pitch, width, outer_,
-                          cur_stream()));
-      offset += width;
+      srcs.push_back(b->gpu_data());
+      widths.push_back(static_cast<long>(b->shape(axis_)) * inner_);
     }
+    MC_CHECK(mcConcat(srcs.data(), widths.data(), static_cast<int>(srcs.size()),
+                      top[0]->mutable_gpu_data(), outer_, cur_stream()));
   }
   int axis_ = 1, outer_ = 0, inner_ = 0;
 };

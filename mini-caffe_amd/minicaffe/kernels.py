@@ -46,6 +46,7 @@ LIB.mcEltwise.argtypes = [c_int, c_int, ctypes.POINTER(c_void_p), ctypes.POINTER
                           c_void_p, c_int, c_float, c_void_p]
 LIB.mcSoftmax.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]
 LIB.mcCopy2D.argtypes = [c_void_p, c_long, c_void_p, c_long, c_long, c_long, c_void_p]
+LIB.mcConcat.argtypes = [ctypes.POINTER(c_void_p), ctypes.POINTER(ctypes.c_long), c_int, c_void_p, ctypes.c_long, c_void_p]
 LIB.mcPermute.argtypes = [c_void_p, c_void_p, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int),
                           c_void_p]
 LIB.mcFill.argtypes = [c_void_p, c_long, c_float, c_void_p]

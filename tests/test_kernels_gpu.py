@@ -844,6 +844,23 @@ def test_copy2d_and_fill(K):
     assert np.array_equal(got[:, 10:43], x) and np.all(got[0, :5] == 2.5) and np.all(got[1:, :10] == 0)
 
 
+@pytest.mark.parametrize("widths,rows", [
+    ((4, 8, 12), 5),                                  # every width and offset a multiple of four: 16-byte accesses
+    ((3, 0, 7, 1), 6),                                # ragged widths, an empty source
+    ((16, 24, 24, 24, 16, 16, 84, 126, 126, 126, 84, 84), 8),   # more than eight sources: two launches
+    ((5,), 3), ((34928, 8664, 2400, 600, 144, 16), 8)])        # one source; SSD300's six location heads
+def test_concat_in_one_launch(K, widths, rows):
+    rng = np.random.default_rng(14)
+    xs = [rng.standard_normal((rows, w)).astype(np.float32) for w in widths]
+    keep = [dev(x) if x.size else None for x in xs]
+    srcs = (ctypes.c_void_p * len(xs))(*[k.data_ptr() if k is not None else None for k in keep])
+    ws = (ctypes.c_long * len(xs))(*widths)
+    yd = torch.full((rows, sum(widths)), float("nan"), device="cuda")
+    K.check_mc(K.LIB.mcConcat(srcs, ws, len(xs), fptr(yd), rows, None))
+    torch.cuda.synchronize()
+    assert np.array_equal(yd.cpu().numpy(), np.concatenate(xs, axis=1))
+
+
 @pytest.mark.parametrize("shape", [(2, 12, 5, 7),       # a thread keeps its channels in registers (<= 128)
                                    (2, 512, 9, 11),     # SSD's 512 channels, ragged pixel tile (<= 512)
                                    (1, 130, 6, 6), (1, 515, 3, 5)])   # > 512 channels: read twice
