@@ -71,6 +71,8 @@ def main():
     ap.add_argument("--no-detection-tails", action="store_true",
                     help="skip the NMS / Proposal / DetectionOutput timings (profiling runs of the "
                          "ResNet-50 forward alone)")
+    ap.add_argument("--no-two-threads", action="store_true",
+                    help="skip the run with two host threads, each with its own net and stream")
     ap.add_argument("--configs-report", metavar="PATH",
                     help="also time all five BASELINE configurations (whole forward, contraction "
                          "launches, Proposal / DetectionOutput layers) and write a text table to PATH")
@@ -218,6 +220,9 @@ def main():
                   "note": "same net, mcConvWinogradDefault(0): all 53 convolutions on the direct implicit-GEMM path"}
         del net0
 
+    two_threads = None if args.no_two_threads else two_thread_throughput(mc, craft, zoo, args.batch,
+                                                                         max(10, args.steps // 2))
+
     if args.configs_report:
         configs_report(args.configs_report, mc, craft, zoo, LIB)
     if args.layer_scaling:
@@ -248,10 +253,56 @@ def main():
                           "2-3 % slower than the default 100 after 50 (the same library, the same box)",
            "roofline": roofline, "cpu_baseline": cpu,
            "conv_mfma_util_pct": mfma_util, "conv_mfma_util_source": mfma_note,
-           "direct_path_only": direct}
+           "direct_path_only": direct, "two_host_threads": two_threads}
     out.update(with_h2d)
     out.update(tails)
     print(json.dumps(out))
+
+
+def two_thread_throughput(mc, craft, zoo, batch, steps):
+    """Two host threads, each with its own net of the same batch and its own stream (the
+    runtime's context is per thread, as in the reference: tests/run_net.cpp:238-246 runs
+    three such threads).  Launches of the two streams fill each other's last, partly
+    empty rounds of workgroups.  Reported beside `value`, never as `value`: two batches
+    are in flight and a step takes nearly twice as long."""
+    import threading
+    bar = threading.Barrier(2)
+    took, errors = [0.0, 0.0], []
+
+    def work(idx):
+        try:
+            mc.set_runtime_mode(1, 0)
+            spec, inputs = zoo.resnet50_spec(batch=batch, size=224, seed=idx)
+            net = mc.Net.from_buffers(craft.to_prototxt(spec, "ResNet-50"))
+            craft.load_weights(net, spec)
+            net.forward(**inputs)
+            for _ in range(max(5, steps // 2)):
+                net.forward()
+            bar.wait()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                net.forward()
+            took[idx] = time.perf_counter() - t0
+            bar.wait()
+            prob = net.get_blob("prob").data
+            assert abs(float(prob.sum()) - batch) < 1e-2 * batch
+            del net
+            mc.memory_pool_clear()
+        except Exception as e:  # noqa: BLE001 - reported by the caller
+            errors.append(repr(e))
+            bar.abort()
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    if errors:
+        return {"error": errors[0]}
+    return {"value": round(2 * batch * steps / max(took), 1), "unit": "images/s", "threads": 2,
+            "steps_per_thread": steps, "ms_per_step_per_thread": round(1e3 * max(took) / steps, 3),
+            "note": "two host threads, each its own ResNet-50 b%d net, context and HIP stream, forwards "
+                    "running concurrently; not the headline figure (two batches in flight)" % batch}
 
 
 def detection_tails(mc, craft, zoo, LIB):
