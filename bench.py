@@ -67,7 +67,8 @@ def main():
                     help="keep every convolution on the direct implicit-GEMM path (3x3 stride-1 layers with "
                          "128 or more channels otherwise run as F(2x2,3x3) Winograd)")
     ap.add_argument("--no-direct-comparison", action="store_true",
-                    help="skip the second, shorter measurement with every convolution on the direct path")
+                    help="skip the second, shorter measurement with every convolution on the direct path "
+                         "(and the two-thread run: profiling commands see the one net's launches only)")
     ap.add_argument("--no-detection-tails", action="store_true",
                     help="skip the NMS / Proposal / DetectionOutput timings (profiling runs of the "
                          "ResNet-50 forward alone)")
@@ -220,7 +221,7 @@ def main():
                   "note": "same net, mcConvWinogradDefault(0): all 53 convolutions on the direct implicit-GEMM path"}
         del net0
 
-    two_threads = None if args.no_two_threads else two_thread_throughput(mc, craft, zoo, args.batch,
+    two_threads = None if args.no_two_threads or args.no_direct_comparison else two_thread_throughput(mc, craft, zoo, args.batch,
                                                                          max(10, args.steps // 2))
 
     if args.configs_report:
