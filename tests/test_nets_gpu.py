@@ -189,6 +189,50 @@ def test_three_threads_each_with_their_own_net(gpu_mode):
         assert netrun.rel_err(got[t], jobs[t][2]) < 1e-3, t
 
 
+def test_two_threads_running_forwards_at_the_same_time_keep_their_bits(gpu_mode):
+    """Two threads, each with its own net (different sizes and weights), run forty forwards
+    each at the same time on their own streams: launches of the two streams share the chip,
+    and the partial sums and arrival counters of sliced contractions belong to the (thread,
+    stream) pair.  Every forward must give the bits the same net gave when it ran alone."""
+    import threading
+    from minicaffe import zoo
+    jobs = [zoo.resnet50_spec(batch=6, size=96, stages=(1, 2, 1, 1), width=64, num_classes=9, bn_seed=5, seed=6),
+            zoo.resnet50_spec(batch=4, size=128, stages=(2, 1, 1, 1), width=32, num_classes=11, bn_seed=7, seed=8)]
+    alone = []
+    for spec, inputs in jobs:
+        net = run_net(gpu_mode, spec, inputs)
+        alone.append({k: net.get_blob(k).data.copy() for k in ("prob", "fc1000")})
+        del net
+    bar = threading.Barrier(2)
+    errors = []
+
+    def work(t):
+        try:
+            gpu_mode.set_runtime_mode(1, 0)
+            spec, inputs = jobs[t]
+            net = run_net(gpu_mode, spec, inputs)
+            bar.wait(timeout=60)
+            for it in range(40):
+                net.forward()
+                for k, want in alone[t].items():
+                    got = net.get_blob(k).data
+                    if not np.array_equal(got, want):
+                        errors.append((t, it, k, float(np.abs(got - want).max())))
+                        return
+            del net
+            gpu_mode.memory_pool_clear()
+        except Exception as e:           # noqa: BLE001 - reported by the main thread
+            errors.append((t, repr(e)))
+            bar.abort()
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=100)
+    assert not errors, errors
+
+
 def test_short_lived_thread_leaves_no_device_memory(gpu_mode):
     """A thread that builds a net, runs it (contractions whose channel loop is cut into
     slices take partial-sum scratch and arrival counters from the kernel library, blobs
