@@ -220,16 +220,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
     // PW4: thread = (K row tid % 16, pixel quad tid / 16); the plane is a multiple of four
     // pixels, so a quad never straddles two images
     const int p = PW4 ? nt * BN + 4 * (tid >> 4) : nt * BN + pj;
-    if (p < a.P) {
-      const int n = fast_div(p, a.div_hw_mul, a.div_hw_shift);
-      const int rem = p - n * a.HqWq;
-      const int qh = fast_div(rem, a.div_w_mul, a.div_w_shift);
-      const int qw = rem - qh * a.Wq;
-      const int hi0 = qh * a.q_sh + a.in_oh;
-      const int wi0 = qw * a.q_sw + a.in_ow;
-      xvoff = static_cast<unsigned>(
-          ((n * a.x_nstride + g * a.x_gstride + hi0 * a.W + wi0) << 2) + a.pix_shift);
-      if constexpr (PW4) xvoff += static_cast<unsigned>(tid & 15) * (static_cast<unsigned>(a.x_cstride) * 4u);
+    // (the divisions are prepared for every column of the last tile, also those past the
+    // last pixel: the pointwise modes compute first and pick afterwards, without a branch)
+    const int n = fast_div(p, a.div_hw_mul, a.div_hw_shift);
+    const int rem = p - n * a.HqWq;
+    const int qh = fast_div(rem, a.div_w_mul, a.div_w_shift);
+    const int qw = rem - qh * a.Wq;
+    const int hi0 = qh * a.q_sh + a.in_oh;
+    const int wi0 = qw * a.q_sw + a.in_ow;
+    unsigned origin = static_cast<unsigned>(
+        ((n * a.x_nstride + g * a.x_gstride + hi0 * a.W + wi0) << 2) + a.pix_shift);
+    if constexpr (PW4) origin += static_cast<unsigned>(tid & 15) * (static_cast<unsigned>(a.x_cstride) * 4u);
+    if constexpr (PW) xvoff = p < a.P ? origin : kNoElement;
+    if (!PW && p < a.P) {
+      xvoff = origin;
       if constexpr (!PW) {
         row_bad = 0x80000000u;  // bit 31: the tap of K padding rows, never valid
         col_bad = 0u;
@@ -271,7 +275,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
   }
   const unsigned wt_kt_bytes = static_cast<unsigned>(a.Mpad) * BK * 4;
   const unsigned wt_g_bytes = static_cast<unsigned>(g) * (a.Kpad / BK) * wt_kt_bytes;
-  const unsigned x_cbytes = static_cast<unsigned>(a.x_cstride) * 4;
+  // (said to be uniform: the compiler otherwise merges this load with the one inside the
+  // divergent branch above into a vector register, and every pixel-quad load of the K
+  // loop, whose scalar offset is a multiple of it, gets wrapped in a loop over lanes)
+  const unsigned x_cbytes = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(a.x_cstride) * 4);
   const int kmax = a.K - 1;
 
   float4 areg[KS][A_VEC];
@@ -414,13 +421,30 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
   // loop they pass through the then idle A tile so that a lane reads the four
   // consecutive rows of an accumulator group with one 16-byte LDS read instead
   // of eight buffer loads.
+  // Through buffer descriptors with scalar bases (a null vector has no records and reads
+  // as zero; lanes with no row to fetch carry the out-of-range offset).  Picking between
+  // the two pointers per lane instead costs a memory round trip before the first tile is
+  // even requested: the compiler then selects between the *addresses of the two fields*
+  // in the argument block and fetches the pointer with a vector load, and the access
+  // through it is a flat one, which the next wait for scalar loads waits for as well.
   float ep_val = tid < BM ? 1.f : 0.f;
-  {
-    const float* src = tid < BM ? a.scale : a.shift;
-    const int row = mt * BM + (tid < BM ? tid : tid - BM);
-    if (tid < 2 * BM && src != nullptr && row < a.M) ep_val = src[g * a.M + row];
+  // Both pointers as scalars first: picking between the two *fields* makes the compiler
+  // pick between their addresses in the argument block and fetch the pointer with a
+  // vector load, a memory round trip every wavefront then waits for before it has
+  // requested its first tile.  The load itself follows the requests for the first tile
+  // (it is a flat access, which the next wait for scalar loads waits for as well).
+  const float* scale_ptr = a.scale;
+  const float* shift_ptr = a.shift;
+  asm("" : "+s"(scale_ptr), "+s"(shift_ptr));
+#define MC_LOAD_FACTORS()                                                              \
+  {                                                                                    \
+    const float* src = tid < BM ? scale_ptr : shift_ptr;                               \
+    const int row = mt * BM + (tid < BM ? tid : tid - BM);                             \
+    if (tid < 2 * BM && src != nullptr && row < a.M) ep_val = src[g * a.M + row];      \
   }
 
+  MC_LOAD_FACTORS();
+#undef MC_LOAD_FACTORS
   if (kt_end > kt_begin) {
     // Tile kt_begin + t sits in LDS buffer t % 2; the loads of the next tile
     // are in flight while the MFMA block of the current one runs.
@@ -460,7 +484,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 #undef MC_COMPUTE
 #undef MC_INTERLEAVE
 
-  if (a.counters != nullptr) {
+  // What the epilogue reads from the argument block is fetched here in one batch:
+  // fetched where it is first used, the fields cost the wavefront four or five
+  // scalar-memory round trips after the last MFMA, one after the other.  (Before the K
+  // loop they would not fit the scalar registers the loop needs.)
+  struct {
+    int* counters;
+    const float* residual;
+    unsigned y_bytes, div_hw_mul, div_hw_shift, div_w_mul, div_w_shift;
+    int y_cstride, y_nstride, Wo, out_sh, out_sw, out_oh, out_ow, M, P, HqWq, Wq, act;
+    float slope;
+  } e = {a.counters, a.residual, a.y_bytes, a.div_hw_mul, a.div_hw_shift, a.div_w_mul, a.div_w_shift,
+         a.y_cstride, a.y_nstride, a.Wo, a.out_sh, a.out_sw, a.out_oh, a.out_ow, a.M, a.P, a.HqWq, a.Wq,
+         a.act, a.slope};
+  asm volatile("" ::"s"(e.counters), "s"(e.residual), "s"(e.y_bytes), "s"(e.div_hw_mul), "s"(e.div_hw_shift),
+               "s"(e.div_w_mul), "s"(e.div_w_shift), "s"(e.y_cstride), "s"(e.y_nstride), "s"(e.Wo),
+               "s"(e.out_sh), "s"(e.out_sw), "s"(e.out_oh), "s"(e.out_ow), "s"(e.M), "s"(e.P), "s"(e.HqWq),
+               "s"(e.Wq), "s"(e.act), "s"(e.slope));
+
+  if (e.counters != nullptr) {
     // K slices summed here: see IgemmArgs::partial.  The partial sums and the
     // counter are accessed with device-scope atomic operations only (relaxed
     // stores and loads that go past the per-XCD L2, which is not coherent with
@@ -491,13 +533,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
     __syncthreads();  // ... every thread's, and every wave is done with the tiles in LDS
     int* arrived = reinterpret_cast<int*>(&As[0][0][0][0]);
     if (tid == 0)
-      arrived[0] = __hip_atomic_fetch_add(&a.counters[tile_id], 1, __ATOMIC_RELAXED,
+      arrived[0] = __hip_atomic_fetch_add(&e.counters[tile_id], 1, __ATOMIC_RELAXED,
                                           __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (arrived[0] != batch.slices - 1) return;  // uniform over the workgroup
     // the next launch on this stream starts from zero
     if (tid == 0)
-      __hip_atomic_store(&a.counters[tile_id], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&e.counters[tile_id], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const float* part = a.partial + static_cast<size_t>(tile_id) * (kRegs * 256) + tid;
     const size_t slice_elems = static_cast<size_t>(a.partial_tiles) * (kRegs * 256);
 #pragma unroll
@@ -528,18 +570,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
   // pixel, which drops its stores), the row as a scalar offset.  Per-channel
   // factors and residual values are fetched eight rows at a time, all loads of
   // a batch issued before the first use.
-  const bool has_scale = a.scale != nullptr;
-  const bool has_shift = a.shift != nullptr;
-  const bool has_res = a.residual != nullptr;
+  const bool has_scale = scale_ptr != nullptr;
+  const bool has_shift = shift_ptr != nullptr;
+  const bool has_res = e.residual != nullptr;
   const __amdgpu_buffer_rsrc_t yres =
-      __builtin_amdgcn_make_buffer_rsrc(yout, 0, a.y_bytes, kBufferFlags);
+      __builtin_amdgcn_make_buffer_rsrc(yout, 0, e.y_bytes, kBufferFlags);
   const __amdgpu_buffer_rsrc_t rres = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<float*>(a.residual), 0, has_res ? a.y_bytes : 0, kBufferFlags);
+      const_cast<float*>(e.residual), 0, has_res ? e.y_bytes : 0, kBufferFlags);
   // 0: none, 1: ReLU (max with 0), 2: leaky ReLU, 3: TanH / Sigmoid
-  const int act_mode = a.act == MC_ACT_NONE ? 0
-                       : a.act == MC_ACT_RELU ? (a.slope == 0.f ? 1 : 2)
+  const int act_mode = e.act == MC_ACT_NONE ? 0
+                       : e.act == MC_ACT_RELU ? (e.slope == 0.f ? 1 : 2)
                                               : 3;
-  const unsigned cs4 = static_cast<unsigned>(a.y_cstride) * 4;
+  const unsigned cs4 = static_cast<unsigned>(e.y_cstride) * 4;
   float* ep = &As[0][0][0][0];
   static_assert(2 * BM <= 256 && 2 * BM <= 2 * KS * BM * LDK, "factors must fit the A tile");
   if (has_scale | has_shift) {
@@ -559,21 +601,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int p = nt * BN + wn0 + j * 32 + l32;
-    const int n = fast_div(p, a.div_hw_mul, a.div_hw_shift);
-    const int rem = p - n * a.HqWq;
-    const int qh = fast_div(rem, a.div_w_mul, a.div_w_shift);
-    const int qw = rem - qh * a.Wq;
+    const int n = fast_div(p, e.div_hw_mul, e.div_hw_shift);
+    const int rem = p - n * e.HqWq;
+    const int qh = fast_div(rem, e.div_w_mul, e.div_w_shift);
+    const int qw = rem - qh * e.Wq;
     const int ybase =
-        n * a.y_nstride + (qh * a.out_sh + a.out_oh) * a.Wo + qw * a.out_sw + a.out_ow;
+        n * e.y_nstride + (qh * e.out_sh + e.out_oh) * e.Wo + qw * e.out_sw + e.out_ow;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const int mblock = mt * BM + wm0 + i * 32;  // wave-uniform
       const int m0 = mblock + 4 * lhi;
-      if (mblock + 32 <= a.M) {
+      if (mblock + 32 <= e.M) {
         // All 32 rows are real channels.
-        const unsigned c0 = g * a.M + m0;
+        const unsigned c0 = g * e.M + m0;
         const unsigned y_voff =
-            p < a.P ? static_cast<unsigned>(ybase + c0 * a.y_cstride) * 4 : kNoElement;
+            p < e.P ? static_cast<unsigned>(ybase + c0 * e.y_cstride) * 4 : kNoElement;
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
           if (has_scale | has_shift) {
@@ -602,24 +644,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
           } else if (act_mode == 1) {
             MC_STORE_ROWS(fmaxf(v, 0.f))
           } else if (act_mode == 2) {
-            MC_STORE_ROWS(v > 0.f ? v : v * a.slope)
+            MC_STORE_ROWS(v > 0.f ? v : v * e.slope)
           } else {
-            MC_STORE_ROWS(apply_act(v, a.act, a.slope))
+            MC_STORE_ROWS(apply_act(v, e.act, e.slope))
           }
         }
-      } else if (p < a.P) {
+      } else if (p < e.P) {
         // Block straddles the last channel: row by row, skipping rows >= M.
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int m = m0 + MC_ROW(r);
-          if (m < a.M) {
-            const int c = g * a.M + m;
+          if (m < e.M) {
+            const int c = g * e.M + m;
             float v = acc[i][j][r];
             if (has_scale) v *= a.scale[c];
             if (has_shift) v += a.shift[c];
-            const int yo = ybase + c * a.y_cstride;
-            if (has_res) v += a.residual[yo];
-            yout[yo] = apply_act(v, a.act, a.slope);
+            const int yo = ybase + c * e.y_cstride;
+            if (has_res) v += e.residual[yo];
+            yout[yo] = apply_act(v, e.act, e.slope);
           }
         }
       }

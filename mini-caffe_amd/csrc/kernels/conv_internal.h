@@ -47,7 +47,12 @@ inline void make_fast_div(unsigned d, unsigned long long n_max, unsigned* mul, u
 
 // n / d for the d the host prepared (mul, shift) for; shift == 32 means d == 1.
 __device__ __forceinline__ int fast_div(int n, unsigned mul, unsigned shift) {
-  return shift == 32 ? n : static_cast<int>(__umulhi(static_cast<unsigned>(n), mul) >> shift);
+  // both sides computed and picked by a mask: as a conditional expression on the uniform
+  // `shift` this becomes a branch, which splits a kernel's prologue into blocks and
+  // leaves its argument loads waiting one after the other
+  const unsigned q = __umulhi(static_cast<unsigned>(n), mul) >> (shift & 31);
+  const unsigned keep = shift == 32 ? 0xFFFFFFFFu : 0u;
+  return static_cast<int>((static_cast<unsigned>(n) & keep) | (q & ~keep));
 }
 
 // 3x3 stride-1 convolution as F(2x2, 3x3) Winograd in one launch: the input
