@@ -136,18 +136,28 @@ __device__ __forceinline__ float apply_act(float v, int act, float slope) {
 // Pointwise: every row k of the gather is channel k of the bottom blob
 // at the thread's own pixel (1x1 kernel, no padding), so the K loop needs no
 // tap table and no bounds handling at all.
-template <int BM, int BN, int WM, int WN, int OCC, int MODE, int KS>
+// ONE_SUB: the launch holds one sub-problem (every Convolution): its arguments then sit
+// at fixed places of the argument block and are fetched in one batch at the top, instead
+// of after the number of slices has arrived and said which sub-problem this workgroup
+// belongs to.
+template <int BM, int BN, int WM, int WN, int OCC, int MODE, int KS, bool ONE_SUB = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void igemm_kernel(
     const IgemmBatch batch) {
   static_assert(WM * WN == 4, "four wavefronts per workgroup");
   int sub_index = 0, kslice = blockIdx.z;
-  while (kslice >= batch.slices) {  // at most kMaxSubs - 1 rounds, on the scalar unit
-    kslice -= batch.slices;
-    ++sub_index;
+  if constexpr (!ONE_SUB) {
+    while (kslice >= batch.slices) {  // at most kMaxSubs - 1 rounds, on the scalar unit
+      kslice -= batch.slices;
+      ++sub_index;
+    }
   }
   const IgemmArgs& a = batch.sub[sub_index];
   // sub-problems of one launch may differ in tile count: the grid is the largest
-  if (static_cast<int>(blockIdx.x) >= a.MT * a.NT) return;
+  // (a single sub-problem's grid is exact: no test, and no branch that keeps the argument
+  // fetches behind it from being issued together)
+  if constexpr (!ONE_SUB) {
+    if (static_cast<int>(blockIdx.x) >= a.MT * a.NT) return;
+  }
   static_assert(BN >= 64 && 256 % BN == 0, "BN must be 64, 128 or 256");
   constexpr int TM = BM / WM / 32;
   constexpr int TN = BN / WN / 32;
@@ -839,6 +849,7 @@ struct TileConfig {
   int ks;  // 16-row K tiles per stage
   const char* name;
   void (*kernel[4])(const IgemmBatch);  // indexed by mode; [3] (pixel-quad pointwise) may be null
+  void (*one_sub[4])(const IgemmBatch);  // the same for launches of one sub-problem, or null
 };
 
 const TileConfig kConfigs[] = {
@@ -853,7 +864,10 @@ const TileConfig kConfigs[] = {
       igemm_kernel<64, 128, 2, 2, 5, kModePointwise, 1>}},
     {64, 64, 1, "igemm_f32_64x64",
      {igemm_kernel<64, 64, 2, 2, 8, kModeMasks, 1>, igemm_kernel<64, 64, 2, 2, 8, kModeOneMask, 1>,
-      igemm_kernel<64, 64, 2, 2, 8, kModePointwise, 1>, igemm_kernel<64, 64, 2, 2, 8, kModePointwiseQuad, 1>}},
+      igemm_kernel<64, 64, 2, 2, 8, kModePointwise, 1>, igemm_kernel<64, 64, 2, 2, 8, kModePointwiseQuad, 1>},
+     {igemm_kernel<64, 64, 2, 2, 8, kModeMasks, 1, true>, igemm_kernel<64, 64, 2, 2, 8, kModeOneMask, 1, true>,
+      igemm_kernel<64, 64, 2, 2, 8, kModePointwise, 1, true>,
+      igemm_kernel<64, 64, 2, 2, 8, kModePointwiseQuad, 1, true>}},
     {32, 128, 1, "igemm_f32_32x128",
      {igemm_kernel<32, 128, 1, 4, 4, kModeMasks, 1>, igemm_kernel<32, 128, 1, 4, 4, kModeOneMask, 1>,
       igemm_kernel<32, 128, 1, 4, 4, kModePointwise, 1>}},
@@ -1494,7 +1508,8 @@ int conv_forward_images(const mcConvPlan* plan, int num, const float* bottom, fl
       }
       int mode = pointwise ? kModePointwise : (one_mask ? kModeOneMask : kModeMasks);
       if (pointwise && quad_ok && cfg.kernel[kModePointwiseQuad]) mode = kModePointwiseQuad;
-      cfg.kernel[mode]<<<grid, 256, extra_lds, st>>>(batch);
+      auto kernel = (nsub == 1 && cfg.one_sub[mode]) ? cfg.one_sub[mode] : cfg.kernel[mode];
+      kernel<<<grid, 256, extra_lds, st>>>(batch);
     }
     MC_LAUNCH_CHECK();
   }
