@@ -426,23 +426,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
   const int l32 = lane & 31;
   const int lhi = lane >> 5;
 
-  // Per-channel factors of the epilogue: thread t < BM fetches the scale of
-  // row t of this tile, thread BM + t its shift, before the K loop; after the
-  // loop they pass through the then idle A tile so that a lane reads the four
-  // consecutive rows of an accumulator group with one 16-byte LDS read instead
-  // of eight buffer loads.
-  // Through buffer descriptors with scalar bases (a null vector has no records and reads
-  // as zero; lanes with no row to fetch carry the out-of-range offset).  Picking between
-  // the two pointers per lane instead costs a memory round trip before the first tile is
-  // even requested: the compiler then selects between the *addresses of the two fields*
-  // in the argument block and fetches the pointer with a vector load, and the access
-  // through it is a flat one, which the next wait for scalar loads waits for as well.
+  // Per-channel factors of the epilogue: thread t < BM fetches the scale of row t of this
+  // tile, thread BM + t its shift, before the K loop, and leaves them in the padding of
+  // the first A buffer (columns BK and BK + 1 of row t, which no tile store and no
+  // operand read touches) together with the first tile: the first barrier of the K loop
+  // publishes them, and after the last MFMA a wavefront reads the (scale, shift) pairs of
+  // its rows from there without another barrier and without waiting for the other three.
   float ep_val = tid < BM ? 1.f : 0.f;
   // Both pointers as scalars first: picking between the two *fields* makes the compiler
   // pick between their addresses in the argument block and fetch the pointer with a
   // vector load, a memory round trip every wavefront then waits for before it has
-  // requested its first tile.  The load itself follows the requests for the first tile
-  // (it is a flat access, which the next wait for scalar loads waits for as well).
+  // requested its first tile.
   const float* scale_ptr = a.scale;
   const float* shift_ptr = a.shift;
   asm("" : "+s"(scale_ptr), "+s"(shift_ptr));
@@ -455,12 +449,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 
   MC_LOAD_FACTORS();
 #undef MC_LOAD_FACTORS
+  static_assert(2 * BM <= 256 && LDK >= BK + 2, "factors go to the padding of the first A buffer");
+#define MC_STORE_FACTORS() \
+  if (tid < 2 * BM) As[0][0][tid & (BM - 1)][BK + (tid >= BM ? 1 : 0)] = ep_val
   if (kt_end > kt_begin) {
     // Tile kt_begin + t sits in LDS buffer t % 2; the loads of the next tile
     // are in flight while the MFMA block of the current one runs.
     const int nk = kt_end - kt_begin;
     MC_LOAD_TILES(kt_begin);
     MC_STORE_TILES(0);
+    MC_STORE_FACTORS();
     __syncthreads();
     int t = 0;
     for (; t + 2 < nk; t += 2) {
@@ -486,7 +484,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
     } else {
       MC_COMPUTE(0);
     }
+  } else {
+    // (a slice past the last K tile of a short sub-problem: zeros, but it may be the one
+    // that sums the slices and runs the epilogue)
+    MC_STORE_FACTORS();
+    __syncthreads();
   }
+#undef MC_STORE_FACTORS
 #undef MC_LOADF
 #undef MC_GATHER1
 #undef MC_LOAD_TILES
@@ -592,13 +596,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
                        : e.act == MC_ACT_RELU ? (e.slope == 0.f ? 1 : 2)
                                               : 3;
   const unsigned cs4 = static_cast<unsigned>(e.y_cstride) * 4;
-  float* ep = &As[0][0][0][0];
-  static_assert(2 * BM <= 256 && 2 * BM <= 2 * KS * BM * LDK, "factors must fit the A tile");
-  if (has_scale | has_shift) {
-    __syncthreads();  // every wave is done reading the last A tile
-    if (tid < 2 * BM) ep[tid] = ep_val;
-    __syncthreads();
-  }
 #define MC_ROW(r) (8 * ((r) / 4) + ((r) % 4))
 #define MC_LOADF(res, voff, soff) \
   __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(res, voff, soff, 0))
@@ -631,12 +628,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
           if (has_scale | has_shift) {
             float sc[8], sh[8];
 #pragma unroll
-            for (int qq = 0; qq < 2; ++qq) {
-              const int lrow = wm0 + i * 32 + 4 * lhi + 8 * (half * 2 + qq);
-              const float4 s4 = *reinterpret_cast<const float4*>(ep + lrow);
-              const float4 h4 = *reinterpret_cast<const float4*>(ep + BM + lrow);
-              sc[qq * 4 + 0] = s4.x; sc[qq * 4 + 1] = s4.y; sc[qq * 4 + 2] = s4.z; sc[qq * 4 + 3] = s4.w;
-              sh[qq * 4 + 0] = h4.x; sh[qq * 4 + 1] = h4.y; sh[qq * 4 + 2] = h4.z; sh[qq * 4 + 3] = h4.w;
+            for (int q = 0; q < 8; ++q) {
+              const int lrow = wm0 + i * 32 + 4 * lhi + MC_ROW(half * 8 + q);
+              const float2 f = *reinterpret_cast<const float2*>(&As[0][0][lrow][BK]);
+              sc[q] = f.x;
+              sh[q] = f.y;
             }
 #pragma unroll
             for (int q = 0; q < 8; ++q)
