@@ -657,7 +657,8 @@ __global__ __launch_bounds__(64) void det_scan_kernel(
   unsigned long long w[kDetSplitWords][kDetSplitWords];
   int prior[kDetSplitWords];
   uint32_t ckey[kDetSplitWords];
-  DBox cbox[kDetSplitWords];
+  float cbox[kDetSplitWords][5];  // (five floats each: an array of DBox would live in scratch memory)
+  static_assert(sizeof(DBox) == 5 * sizeof(float), "a box is five floats");
 #pragma unroll
   for (int b = 0; b < kDetSplitWords; ++b) {
     if (b < words) {  // uniform
@@ -672,7 +673,9 @@ __global__ __launch_bounds__(64) void det_scan_kernel(
       const size_t mine = (size_t)seg * cand_stride + min(64 * b + lane, ncand - 1);
       prior[b] = cand_idx[mine];
       ckey[b] = cand_key[mine];
-      cbox[b] = cand_box[mine];
+      const float* box = reinterpret_cast<const float*>(cand_box + mine);
+#pragma unroll
+      for (int k = 0; k < 5; ++k) cbox[b][k] = box[k];
     }
   }
   unsigned long long keep[kDetSplitWords];
@@ -702,7 +705,9 @@ __global__ __launch_bounds__(64) void det_scan_kernel(
         const int pos = nkept + __popcll(keep_bits & ((1ull << lane) - 1ull));
         kept[pos] = prior[b];
         kept_key[(size_t)seg * max_cand + pos] = ckey[b];
-        kept_box[(size_t)seg * max_cand + pos] = cbox[b];
+        float* box = reinterpret_cast<float*>(kept_box + (size_t)seg * max_cand + pos);
+#pragma unroll
+        for (int k = 0; k < 5; ++k) box[k] = cbox[b][k];
       }
       nkept += __popcll(keep_bits);
     }
