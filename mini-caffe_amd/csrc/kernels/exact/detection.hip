@@ -590,7 +590,13 @@ __global__ __launch_bounds__(kSortThreads) void det_candidates_kernel(
   if (m > 0) {  // uniform
     ncand = __syncthreads_count(tid < want && key < key_thr);
   } else {
-    ncand = det_candidates_by_sort(keys, P, key_thr, want, s_key, s_val, &lds, &s_valid, &key, &idx);
+    // (its results through variables of their own: a variable whose address goes to a
+    // function that is not inlined lives in scratch memory for the whole kernel)
+    uint32_t sorted_key = 0xffffffffu, sorted_idx = 0;
+    ncand = det_candidates_by_sort(keys, P, key_thr, want, s_key, s_val, &lds, &s_valid, &sorted_key,
+                                   &sorted_idx);
+    key = sorted_key;
+    idx = sorted_idx;
   }
   if (tid < ncand) {
     const DBox* cls_boxes = boxes + ((size_t)i * loc_classes + (loc_classes == 1 ? 0 : c)) * P;
