@@ -265,9 +265,11 @@ def test_short_lived_thread_leaves_no_device_memory(gpu_mode):
 
     one_thread()                          # (first use: code objects, the runtime's own pools)
     free_before = one_thread()
-    for _ in range(3):
+    for _ in range(6):
         free_after = one_thread()
-    assert free_before - free_after < (4 << 20), (free_before, free_after)
+    # the net, its weights and its scratch are some 20 MB per thread; the HIP runtime's own
+    # pools grow in steps of 2 MiB now and then (seen: 4 MiB over three threads, once)
+    assert free_before - free_after < (8 << 20), (free_before, free_after)
 
 
 def test_flatten_and_reshape_as_views(gpu_mode):
