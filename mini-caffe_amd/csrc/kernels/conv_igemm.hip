@@ -234,12 +234,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
     // last pixel: the pointwise modes compute first and pick afterwards, without a branch)
     const int n = fast_div(p, a.div_hw_mul, a.div_hw_shift);
     const int rem = p - n * a.HqWq;
-    const int qh = fast_div(rem, a.div_w_mul, a.div_w_shift);
-    const int qw = rem - qh * a.Wq;
+    // (the pixel-quad mode runs only where pixel `rem` of the iteration grid is element
+    // `rem` of the bottom plane and of the top plane: no row and column needed)
+    const int qh = PW4 ? 0 : fast_div(rem, a.div_w_mul, a.div_w_shift);
+    const int qw = PW4 ? 0 : rem - qh * a.Wq;
     const int hi0 = qh * a.q_sh + a.in_oh;
     const int wi0 = qw * a.q_sw + a.in_ow;
     unsigned origin = static_cast<unsigned>(
-        ((n * a.x_nstride + g * a.x_gstride + hi0 * a.W + wi0) << 2) + a.pix_shift);
+        ((n * a.x_nstride + g * a.x_gstride + (PW4 ? rem : hi0 * a.W + wi0)) << 2) + a.pix_shift);
     if constexpr (PW4) origin += static_cast<unsigned>(tid & 15) * (static_cast<unsigned>(a.x_cstride) * 4u);
     if constexpr (PW) xvoff = p < a.P ? origin : kNoElement;
     if (!PW && p < a.P) {
@@ -610,10 +612,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
     const int p = nt * BN + wn0 + j * 32 + l32;
     const int n = fast_div(p, e.div_hw_mul, e.div_hw_shift);
     const int rem = p - n * e.HqWq;
-    const int qh = fast_div(rem, e.div_w_mul, e.div_w_shift);
-    const int qw = rem - qh * e.Wq;
-    const int ybase =
-        n * e.y_nstride + (qh * e.out_sh + e.out_oh) * e.Wo + qw * e.out_sw + e.out_ow;
+    int ybase;
+    if constexpr (PW4) {
+      ybase = n * e.y_nstride + rem;
+    } else {
+      const int qh = fast_div(rem, e.div_w_mul, e.div_w_shift);
+      const int qw = rem - qh * e.Wq;
+      ybase = n * e.y_nstride + (qh * e.out_sh + e.out_oh) * e.Wo + qw * e.out_sw + e.out_ow;
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const int mblock = mt * BM + wm0 + i * 32;  // wave-uniform
@@ -1356,7 +1362,11 @@ int conv_forward_images(const mcConvPlan* plan, int num, const float* bottom, fl
     if (s->Kpad > 0) min_kt = std::min(min_kt, s->Kpad / (BK * cfg.ks));
     pointwise = pointwise && s->pointwise;
     quad_ok = quad_ok && s->q_sh == 1 && s->q_sw == 1 && s->Hq == g.height_in && s->Wq == g.width_in &&
-              (s->Hq * s->Wq) % 4 == 0 && s->K % 16 == 0 && s->in_oh == 0 && s->in_ow == 0;
+              (s->Hq * s->Wq) % 4 == 0 && s->K % 16 == 0 && s->in_oh == 0 && s->in_ow == 0 &&
+              // ... and pixel p of an image is element p of its top plane as well (the kernel
+              // then needs no row / column of a pixel on either side)
+              s->out_sh == 1 && s->out_sw == 1 && s->out_oh == 0 && s->out_ow == 0 && s->Hq == plan->Ho &&
+              s->Wq == plan->Wo;
     one_mask = one_mask && s->one_mask;
     flops += 2.0 * pixels * plan->M * g.group * s->K;
   }
